@@ -1,0 +1,76 @@
+"""ctypes bindings of include/et_sampler.h (the C ABI of libet_sampler.so).
+
+The library is loaded from this package's directory; there is no fallback: if it has not been
+built (``python -m executorch_amd.build``) loading raises.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libet_sampler.so")
+
+OK, INTERNAL, INVALID_STATE, NOT_SUPPORTED, INVALID_ARGUMENT, MEMORY_ALLOCATION_FAILED = 0x00, 0x01, 0x02, 0x10, 0x12, 0x21
+DTYPE_HALF, DTYPE_FLOAT, DTYPE_BFLOAT16, DTYPE_UINT16 = 5, 6, 15, 27
+
+
+class RowDebug(C.Structure):
+    _fields_ = [
+        ("max_val", C.c_float),
+        ("sum", C.c_float),
+        ("coin", C.c_float),
+        ("cumulative", C.c_float),
+        ("r", C.c_float),
+        ("n_candidates", C.c_int32),
+        ("last_idx", C.c_int32),
+        ("position", C.c_int32),
+    ]
+
+
+# name -> (restype, argtypes); every symbol declared in include/et_sampler.h
+SIGNATURES = {
+    "ets_sampler_create": (C.c_int32, [C.c_int32, C.c_float, C.c_float, C.c_uint64, C.c_int32, C.POINTER(C.c_void_p)]),
+    "ets_sampler_create_default": (C.c_int32, [C.c_int32, C.c_float, C.c_int32, C.POINTER(C.c_void_p)]),
+    "ets_sampler_destroy": (C.c_int32, [C.c_void_p]),
+    "ets_sampler_set_temperature": (C.c_int32, [C.c_void_p, C.c_float]),
+    "ets_sampler_set_topk": (C.c_int32, [C.c_void_p, C.c_int32]),
+    "ets_sampler_set_topp": (C.c_int32, [C.c_void_p, C.c_float]),
+    "ets_sampler_sample": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int32, C.POINTER(C.c_int32)]),
+    "ets_sampler_sample_batch": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int64, C.c_void_p, C.c_void_p]),
+    "ets_sampler_sample_batch_debug": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int64, C.c_void_p,
+                                                   C.c_void_p, C.c_void_p, C.c_void_p]),
+    "ets_sampler_set_rng_states": (C.c_int32, [C.c_void_p, C.c_int32, C.c_int32, C.c_void_p]),
+    "ets_sampler_get_rng_states": (C.c_int32, [C.c_void_p, C.c_int32, C.c_int32, C.c_void_p]),
+    "ets_sample_from_logits": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.POINTER(C.c_int64), C.POINTER(C.c_int32)]),
+    "ets_logits_to_token": (C.c_int32, [C.c_void_p, C.c_int32, C.c_int32, C.POINTER(C.c_int64), C.c_float, C.POINTER(C.c_int32)]),
+    "ets_random_u32": (C.c_uint32, [C.POINTER(C.c_uint64)]),
+    "ets_random_f32": (C.c_float, [C.POINTER(C.c_uint64)]),
+    "ets_sampler_last_error": (C.c_char_p, [C.c_void_p]),
+    "ets_version": (C.c_char_p, []),
+}
+
+# csrc/ets_test_hooks.h
+TEST_HOOKS = {
+    "ets_test_expf": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p]),
+    "ets_test_seq_sum": (C.c_int32, [C.c_void_p, C.c_int32, C.c_float, C.c_float, C.c_void_p, C.c_void_p, C.c_void_p]),
+}
+
+_lib = None
+
+
+def lib() -> C.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with `python -m executorch_amd.build` "
+                "(there is no CPU fallback for the sampler)")
+        L = C.CDLL(LIB_PATH)
+        for table in (SIGNATURES, TEST_HOOKS):
+            for name, (res, args) in table.items():
+                f = getattr(L, name)
+                f.restype = res
+                f.argtypes = args
+        _lib = L
+    return _lib

@@ -1,0 +1,408 @@
+// Host side of the C ABI declared in include/et_sampler.h: handle bookkeeping, argument
+// checks and kernel launches.  Compiled with hipcc for gfx950 only.
+#include "../../include/et_sampler.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <cstring>
+#include <ctime>
+#include <mutex>
+#include <new>
+#include <string>
+
+#include "ets_kernels.h"
+#include "ets_test_hooks.h"
+
+namespace {
+
+thread_local std::string g_thread_error;
+
+struct ErrorSink {
+  std::string* where;
+};
+
+}  // namespace
+
+struct ets_sampler {
+  int32_t vocab = 0;
+  float inv_temperature = 0.0f;
+  float topp = 0.9f;
+  int32_t topk = 0;
+  int32_t max_batch = 0;
+  int device = 0;
+  int lds_keys = 0;            // keys that fit in the dynamic LDS sort buffer (power of two)
+  size_t lds_bytes = 0;
+  int64_t scratch_stride = 0;  // keys per row of candidate scratch (power of two >= vocab)
+  uint64_t* d_rng = nullptr;       // [max_batch]
+  uint64_t* d_scratch = nullptr;   // [max_batch, scratch_stride], allocated on first stochastic use
+  uint64_t* d_partials = nullptr;  // [max_batch, kMaxSplits] argmax partial results
+  uint32_t* d_counters = nullptr;  // [max_batch] argmax arrival counters (zero between launches)
+  void* d_row = nullptr;           // staging for one host row (vocab * 4 bytes)
+  int32_t* d_token = nullptr;      // staging for one token
+  std::string last_error;
+};
+
+namespace {
+
+constexpr int kMaxSplits = 64;
+
+ets_status fail(ets_sampler* s, ets_status code, const std::string& msg) {
+  if (s) {
+    s->last_error = msg;
+  } else {
+    g_thread_error = msg;
+  }
+  return code;
+}
+
+ets_status hip_fail(ets_sampler* s, hipError_t e, const char* what) {
+  return fail(s, e == hipErrorOutOfMemory ? ETS_MEMORY_ALLOCATION_FAILED : ETS_INTERNAL,
+              std::string(what) + ": " + hipGetErrorString(e));
+}
+
+#define ETS_HIP(s, call)                                  \
+  do {                                                    \
+    hipError_t e_ = (call);                               \
+    if (e_ != hipSuccess) return hip_fail(s, e_, #call);  \
+  } while (0)
+
+bool dtype_ok(int32_t dtype) {
+  return dtype == ETS_DTYPE_FLOAT || dtype == ETS_DTYPE_HALF || dtype == ETS_DTYPE_BFLOAT16 ||
+         dtype == ETS_DTYPE_UINT16;
+}
+
+size_t dtype_size(int32_t dtype) { return dtype == ETS_DTYPE_FLOAT ? 4 : 2; }
+
+// Device guard: the handle's buffers live on the device that was current at creation.
+struct DeviceGuard {
+  int prev = -1;
+  bool switched = false;
+  explicit DeviceGuard(int dev) {
+    if (hipGetDevice(&prev) == hipSuccess && prev != dev) switched = (hipSetDevice(dev) == hipSuccess);
+  }
+  ~DeviceGuard() {
+    if (switched) (void)hipSetDevice(prev);
+  }
+};
+
+template <int DT>
+ets_status launch_argmax(ets_sampler* s, const void* d_logits, int32_t batch, int64_t stride, int32_t* d_tokens,
+                         hipStream_t stream) {
+  // Enough workgroups to fill 256 CUs several times over, but no segment under 2048 entries.
+  int splits = (2048 + batch - 1) / batch;
+  const int max_by_len = (s->vocab + 2047) / 2048;
+  if (splits > max_by_len) splits = max_by_len;
+  if (splits > kMaxSplits) splits = kMaxSplits;
+  if (splits < 1) splits = 1;
+  dim3 grid(splits, batch);
+  hipLaunchKernelGGL((ets::argmax_kernel<DT>), grid, dim3(ets::kArgmaxBlock), 0, stream, d_logits, stride, s->vocab,
+                     s->d_partials, s->d_counters, d_tokens);
+  ETS_HIP(s, hipGetLastError());
+  return ETS_OK;
+}
+
+template <int DT>
+ets_status launch_rows(ets_sampler* s, const ets::RowParams& p, int32_t batch, hipStream_t stream) {
+  static std::once_flag once;
+  static hipError_t attr_err = hipSuccess;
+  const size_t lds = s->lds_bytes;
+  std::call_once(once, [&] {
+    attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(&ets::sample_rows_kernel<DT>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+  });
+  if (attr_err != hipSuccess) return hip_fail(s, attr_err, "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
+  hipLaunchKernelGGL((ets::sample_rows_kernel<DT>), dim3(batch), dim3(ets::kBlock), lds, stream, p);
+  ETS_HIP(s, hipGetLastError());
+  return ETS_OK;
+}
+
+ets_status ensure_scratch(ets_sampler* s) {
+  if (s->d_scratch) return ETS_OK;
+  const size_t bytes = static_cast<size_t>(s->max_batch) * static_cast<size_t>(s->scratch_stride) * sizeof(uint64_t);
+  ETS_HIP(s, hipMalloc(reinterpret_cast<void**>(&s->d_scratch), bytes));
+  return ETS_OK;
+}
+
+ets_status sample_device(ets_sampler* s, const void* d_logits, int32_t dtype, int32_t batch, int64_t stride,
+                         int32_t* d_tokens, float* d_probs, ets_row_debug* d_debug, hipStream_t stream) {
+  if (s->inv_temperature == 0.0f) {
+    // greedy: no coin is consumed (sampler.cpp:226-228)
+    switch (dtype) {
+      case ETS_DTYPE_FLOAT:
+        return launch_argmax<ets::kDtypeFloat>(s, d_logits, batch, stride, d_tokens, stream);
+      case ETS_DTYPE_HALF:
+        return launch_argmax<ets::kDtypeHalf>(s, d_logits, batch, stride, d_tokens, stream);
+      case ETS_DTYPE_BFLOAT16:
+        return launch_argmax<ets::kDtypeBFloat16>(s, d_logits, batch, stride, d_tokens, stream);
+      default:
+        return launch_argmax<ets::kDtypeUInt16>(s, d_logits, batch, stride, d_tokens, stream);
+    }
+  }
+  if (dtype == ETS_DTYPE_UINT16) {
+    return fail(s, ETS_NOT_SUPPORTED,
+                "stochastic sampling of UInt16 logits is not supported (integer softmax of the reference "
+                "degenerates to 0/1 weights); use temperature 0 or dequantise first");
+  }
+  ets_status st = ensure_scratch(s);
+  if (st != ETS_OK) return st;
+  ets::RowParams p;
+  p.logits = d_logits;
+  p.row_stride = stride;
+  p.vocab = s->vocab;
+  p.inv_temperature = s->inv_temperature;
+  p.topp = s->topp;
+  p.topk = s->topk;
+  p.rng = s->d_rng;
+  p.tokens = d_tokens;
+  p.probs = d_probs;
+  p.debug = reinterpret_cast<ets::RowDebug*>(d_debug);
+  p.scratch = s->d_scratch;
+  p.scratch_stride = s->scratch_stride;
+  p.lds_keys = s->lds_keys;
+  switch (dtype) {
+    case ETS_DTYPE_FLOAT:
+      return launch_rows<ets::kDtypeFloat>(s, p, batch, stream);
+    case ETS_DTYPE_HALF:
+      return launch_rows<ets::kDtypeHalf>(s, p, batch, stream);
+    default:
+      return launch_rows<ets::kDtypeBFloat16>(s, p, batch, stream);
+  }
+}
+
+float inverse_temperature_ctor(float temperature) {
+  // sampler.cpp:178: static_cast<bool>(temperature) ? 1.0f / temperature : 0
+  return (temperature != 0.0f) ? 1.0f / temperature : 0.0f;
+}
+
+}  // namespace
+
+static_assert(sizeof(ets_row_debug) == sizeof(ets::RowDebug), "debug record layouts must agree");
+
+extern "C" {
+
+ets_status ets_sampler_create(int32_t vocab_size, float temperature, float topp, uint64_t rng_seed,
+                              int32_t max_batch, ets_sampler** out) {
+  if (!out) return fail(nullptr, ETS_INVALID_ARGUMENT, "ets_sampler_create: out is null");
+  *out = nullptr;
+  if (vocab_size < 1) return fail(nullptr, ETS_INVALID_ARGUMENT, "ets_sampler_create: vocab_size must be >= 1");
+  if (max_batch < 1) return fail(nullptr, ETS_INVALID_ARGUMENT, "ets_sampler_create: max_batch must be >= 1");
+  ets_sampler* s = new (std::nothrow) ets_sampler();
+  if (!s) return fail(nullptr, ETS_MEMORY_ALLOCATION_FAILED, "ets_sampler_create: out of host memory");
+  s->vocab = vocab_size;
+  s->inv_temperature = inverse_temperature_ctor(temperature);
+  s->topp = topp;
+  s->topk = 0;
+  s->max_batch = max_batch;
+  auto bail = [&](hipError_t e, const char* what) {
+    ets_status st = hip_fail(nullptr, e, what);
+    ets_sampler_destroy(s);
+    return st;
+  };
+  hipError_t e = hipGetDevice(&s->device);
+  if (e != hipSuccess) return bail(e, "hipGetDevice");
+  int lds_limit = 0;
+  e = hipDeviceGetAttribute(&lds_limit, hipDeviceAttributeMaxSharedMemoryPerBlock, s->device);
+  if (e != hipSuccess) return bail(e, "hipDeviceGetAttribute(MaxSharedMemoryPerBlock)");
+  // static LDS of the row kernel (BlockScratch) is well under 2 KiB
+  int keys = 1;
+  while (static_cast<size_t>(keys) * 2 * sizeof(uint64_t) + 2048 <= static_cast<size_t>(lds_limit)) keys *= 2;
+  if (keys < 64) {
+    ets_sampler_destroy(s);
+    return fail(nullptr, ETS_INTERNAL, "ets_sampler_create: device reports too little LDS per workgroup");
+  }
+  s->lds_keys = keys;
+  s->lds_bytes = static_cast<size_t>(keys) * sizeof(uint64_t);
+  s->scratch_stride = 2;
+  while (s->scratch_stride < vocab_size) s->scratch_stride *= 2;
+
+  e = hipMalloc(reinterpret_cast<void**>(&s->d_rng), sizeof(uint64_t) * max_batch);
+  if (e != hipSuccess) return bail(e, "hipMalloc(rng states)");
+  e = hipMalloc(reinterpret_cast<void**>(&s->d_partials), sizeof(uint64_t) * max_batch * kMaxSplits);
+  if (e != hipSuccess) return bail(e, "hipMalloc(argmax partials)");
+  e = hipMalloc(reinterpret_cast<void**>(&s->d_counters), sizeof(uint32_t) * max_batch);
+  if (e != hipSuccess) return bail(e, "hipMalloc(argmax counters)");
+  e = hipMemset(s->d_counters, 0, sizeof(uint32_t) * max_batch);
+  if (e != hipSuccess) return bail(e, "hipMemset(argmax counters)");
+  e = hipMalloc(&s->d_row, static_cast<size_t>(vocab_size) * 4);
+  if (e != hipSuccess) return bail(e, "hipMalloc(row staging)");
+  e = hipMalloc(reinterpret_cast<void**>(&s->d_token), sizeof(int32_t));
+  if (e != hipSuccess) return bail(e, "hipMalloc(token staging)");
+  // row b's stream starts at rng_seed + b
+  uint64_t* seeds = new (std::nothrow) uint64_t[max_batch];
+  if (!seeds) {
+    ets_sampler_destroy(s);
+    return fail(nullptr, ETS_MEMORY_ALLOCATION_FAILED, "ets_sampler_create: out of host memory");
+  }
+  for (int32_t b = 0; b < max_batch; ++b) seeds[b] = rng_seed + static_cast<uint64_t>(b);
+  e = hipMemcpy(s->d_rng, seeds, sizeof(uint64_t) * max_batch, hipMemcpyHostToDevice);
+  delete[] seeds;
+  if (e != hipSuccess) return bail(e, "hipMemcpy(rng states)");
+  *out = s;
+  return ETS_OK;
+}
+
+ets_status ets_sampler_create_default(int32_t vocab_size, float temperature, int32_t max_batch, ets_sampler** out) {
+  return ets_sampler_create(vocab_size, temperature, 0.9f, static_cast<uint64_t>(std::time(nullptr)), max_batch, out);
+}
+
+ets_status ets_sampler_destroy(ets_sampler* s) {
+  if (!s) return ETS_OK;
+  {
+    DeviceGuard g(s->device);
+    (void)hipFree(s->d_rng);
+    (void)hipFree(s->d_scratch);
+    (void)hipFree(s->d_partials);
+    (void)hipFree(s->d_counters);
+    (void)hipFree(s->d_row);
+    (void)hipFree(s->d_token);
+  }
+  delete s;
+  return ETS_OK;
+}
+
+ets_status ets_sampler_set_temperature(ets_sampler* s, float temperature) {
+  if (!s) return fail(nullptr, ETS_INVALID_ARGUMENT, "ets_sampler_set_temperature: null handle");
+  if (temperature < 0.0f) temperature = 0.0f;
+  s->inv_temperature = (temperature != 0.0f) ? 1.0f / temperature : 0.0f;
+  return ETS_OK;
+}
+
+ets_status ets_sampler_set_topk(ets_sampler* s, int32_t topk) {
+  if (!s) return fail(nullptr, ETS_INVALID_ARGUMENT, "ets_sampler_set_topk: null handle");
+  s->topk = topk;
+  return ETS_OK;
+}
+
+ets_status ets_sampler_set_topp(ets_sampler* s, float topp) {
+  if (!s) return fail(nullptr, ETS_INVALID_ARGUMENT, "ets_sampler_set_topp: null handle");
+  s->topp = topp;
+  return ETS_OK;
+}
+
+ets_status ets_sampler_sample_batch_debug(ets_sampler* s, const void* d_logits, int32_t dtype, int32_t batch,
+                                          int64_t row_stride_elems, int32_t* d_tokens, float* d_probs,
+                                          ets_row_debug* d_debug, void* hip_stream) {
+  if (!s) return fail(nullptr, ETS_INVALID_ARGUMENT, "ets_sampler_sample_batch: null handle");
+  s->last_error.clear();
+  if (!d_logits || !d_tokens) return fail(s, ETS_INVALID_ARGUMENT, "ets_sampler_sample_batch: null pointer");
+  if (!dtype_ok(dtype)) return fail(s, ETS_INVALID_ARGUMENT, "ets_sampler_sample_batch: unsupported dtype");
+  if (batch < 0 || batch > s->max_batch)
+    return fail(s, ETS_INVALID_ARGUMENT, "ets_sampler_sample_batch: batch exceeds the handle's max_batch");
+  if (row_stride_elems < s->vocab)
+    return fail(s, ETS_INVALID_ARGUMENT, "ets_sampler_sample_batch: row stride smaller than vocab_size");
+  if (batch == 0) return ETS_OK;
+  DeviceGuard g(s->device);
+  return sample_device(s, d_logits, dtype, batch, row_stride_elems, d_tokens, d_probs, d_debug,
+                       static_cast<hipStream_t>(hip_stream));
+}
+
+ets_status ets_sampler_sample_batch(ets_sampler* s, const void* d_logits, int32_t dtype, int32_t batch,
+                                    int64_t row_stride_elems, int32_t* d_tokens, void* hip_stream) {
+  return ets_sampler_sample_batch_debug(s, d_logits, dtype, batch, row_stride_elems, d_tokens, nullptr, nullptr,
+                                        hip_stream);
+}
+
+ets_status ets_sampler_sample(ets_sampler* s, const void* logits, int32_t dtype, int32_t* token_out) {
+  if (!s) return fail(nullptr, ETS_INVALID_ARGUMENT, "ets_sampler_sample: null handle");
+  s->last_error.clear();
+  if (!logits || !token_out) return fail(s, ETS_INVALID_ARGUMENT, "ets_sampler_sample: null pointer");
+  if (!dtype_ok(dtype)) return fail(s, ETS_INVALID_ARGUMENT, "ets_sampler_sample: unsupported dtype");
+  DeviceGuard g(s->device);
+  ETS_HIP(s, hipMemcpy(s->d_row, logits, static_cast<size_t>(s->vocab) * dtype_size(dtype), hipMemcpyHostToDevice));
+  ets_status st = sample_device(s, s->d_row, dtype, 1, s->vocab, s->d_token, nullptr, nullptr, nullptr);
+  if (st != ETS_OK) return st;
+  ETS_HIP(s, hipMemcpy(token_out, s->d_token, sizeof(int32_t), hipMemcpyDeviceToHost));
+  return ETS_OK;
+}
+
+ets_status ets_sampler_set_rng_states(ets_sampler* s, int32_t first_row, int32_t count, const uint64_t* states) {
+  if (!s) return fail(nullptr, ETS_INVALID_ARGUMENT, "ets_sampler_set_rng_states: null handle");
+  if (!states || first_row < 0 || count < 0 || first_row + count > s->max_batch)
+    return fail(s, ETS_INVALID_ARGUMENT, "ets_sampler_set_rng_states: bad range or null pointer");
+  if (count == 0) return ETS_OK;
+  DeviceGuard g(s->device);
+  ETS_HIP(s, hipMemcpy(s->d_rng + first_row, states, sizeof(uint64_t) * count, hipMemcpyHostToDevice));
+  return ETS_OK;
+}
+
+ets_status ets_sampler_get_rng_states(ets_sampler* s, int32_t first_row, int32_t count, uint64_t* states) {
+  if (!s) return fail(nullptr, ETS_INVALID_ARGUMENT, "ets_sampler_get_rng_states: null handle");
+  if (!states || first_row < 0 || count < 0 || first_row + count > s->max_batch)
+    return fail(s, ETS_INVALID_ARGUMENT, "ets_sampler_get_rng_states: bad range or null pointer");
+  if (count == 0) return ETS_OK;
+  DeviceGuard g(s->device);
+  ETS_HIP(s, hipMemcpy(states, s->d_rng + first_row, sizeof(uint64_t) * count, hipMemcpyDeviceToHost));
+  return ETS_OK;
+}
+
+ets_status ets_sample_from_logits(ets_sampler* s, const void* data, int32_t dtype, int32_t rank, const int64_t* sizes,
+                                  int32_t* token_out) {
+  if (!s) return fail(nullptr, ETS_INVALID_ARGUMENT, "ets_sample_from_logits: null handle");
+  s->last_error.clear();
+  if (!data || !sizes || !token_out || rank < 1)
+    return fail(s, ETS_INVALID_ARGUMENT, "ets_sample_from_logits: null pointer or rank < 1");
+  if (!dtype_ok(dtype)) return fail(s, ETS_INVALID_ARGUMENT, "Unsupported dtype in sample_from_logits");
+  const int64_t vocab = sizes[rank - 1];
+  if (vocab != s->vocab)
+    return fail(s, ETS_INVALID_ARGUMENT, "ets_sample_from_logits: last dimension differs from the sampler's vocab_size");
+  const char* p = static_cast<const char*>(data);
+  if (rank == 3) {
+    if (sizes[1] < 1) return fail(s, ETS_INVALID_ARGUMENT, "ets_sample_from_logits: empty sequence dimension");
+    p += static_cast<size_t>((sizes[1] - 1) * vocab) * dtype_size(dtype);  // last position of batch 0 (util.h:48-51)
+  }
+  return ets_sampler_sample(s, p, dtype, token_out);
+}
+
+ets_status ets_logits_to_token(const void* data, int32_t dtype, int32_t rank, const int64_t* sizes, float temperature,
+                               int32_t* token_out) {
+  if (!data || !sizes || !token_out || rank < 1)
+    return fail(nullptr, ETS_INVALID_ARGUMENT, "ets_logits_to_token: null pointer or rank < 1");
+  const int64_t vocab = sizes[rank - 1];
+  if (vocab < 1 || vocab > INT32_MAX) return fail(nullptr, ETS_INVALID_ARGUMENT, "ets_logits_to_token: bad vocab size");
+  ets_sampler* s = nullptr;
+  ets_status st = ets_sampler_create_default(static_cast<int32_t>(vocab), temperature, 1, &s);
+  if (st != ETS_OK) return st;
+  st = ets_sample_from_logits(s, data, dtype, rank, sizes, token_out);
+  if (st != ETS_OK) g_thread_error = s->last_error;
+  ets_sampler_destroy(s);
+  return st;
+}
+
+uint32_t ets_random_u32(uint64_t* state) {
+  uint64_t s = *state;
+  s ^= s >> 12;
+  s ^= s << 25;
+  s ^= s >> 27;
+  *state = s;
+  return static_cast<uint32_t>((s * 0x2545F4914F6CDD1Dull) >> 32);
+}
+
+float ets_random_f32(uint64_t* state) { return static_cast<float>(ets_random_u32(state) >> 8) / 16777216.0f; }
+
+const char* ets_sampler_last_error(const ets_sampler* s) { return s ? s->last_error.c_str() : g_thread_error.c_str(); }
+
+const char* ets_version(void) { return "et_sampler 0.1 (gfx950)"; }
+
+// ---- test hooks (not part of the drop-in surface; declared in csrc/ets_test_hooks.h) ----------
+ets_status ets_test_expf(const float* d_x, float* d_y, int64_t n, void* hip_stream) {
+  if (!d_x || !d_y || n < 0) return fail(nullptr, ETS_INVALID_ARGUMENT, "ets_test_expf: bad arguments");
+  if (n == 0) return ETS_OK;
+  int64_t blocks = (n + 255) / 256;
+  if (blocks > 65536) blocks = 65536;
+  hipLaunchKernelGGL(ets::expf_exact_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0,
+                     static_cast<hipStream_t>(hip_stream), d_x, d_y, n);
+  ETS_HIP(nullptr, hipGetLastError());
+  return ETS_OK;
+}
+
+ets_status ets_test_seq_sum(const float* d_a, int32_t n, float s0, float threshold, float* d_sum, int32_t* d_stop,
+                            void* hip_stream) {
+  if (!d_a || !d_sum || !d_stop || n < 0) return fail(nullptr, ETS_INVALID_ARGUMENT, "ets_test_seq_sum: bad arguments");
+  hipLaunchKernelGGL(ets::seq_sum_kernel, dim3(1), dim3(ets::kBlock), 0, static_cast<hipStream_t>(hip_stream), d_a, n,
+                     s0, threshold, d_sum, d_stop);
+  ETS_HIP(nullptr, hipGetLastError());
+  return ETS_OK;
+}
+
+}  // extern "C"

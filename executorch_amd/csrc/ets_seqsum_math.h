@@ -1,0 +1,93 @@
+// Integer arithmetic behind the sequential-float-sum emulation.  No HIP dependency: the
+// includer defines ETS_HD (function qualifiers), so the same code is unit-tested on the host.
+#pragma once
+
+#include <stdint.h>
+
+#ifndef ETS_HD
+#define ETS_HD inline
+#endif
+
+namespace ets {
+
+constexpr uint32_t kSat = 1u << 26;  // saturation value of integer increments (> 2^24)
+
+// ---- sequential float sums as an integer scan --------------------------------------------------
+// A scalar loop `s += a[i]` (a[i] >= 0) rounds after every add.  While s stays inside one
+// binade [2^k, 2^(k+1)) every partial sum is an integer multiple of u = ulp(s): writing
+// s = S*u, adding a gives S + rne(a/u), where the tie case (a/u has fraction exactly 1/2)
+// rounds so that the new S is even.  The increment therefore depends on the incoming state only
+// through the PARITY of S, so a run of elements is summarised by two integers -- the total
+// increment when entered with S even and with S odd -- and such summaries compose
+// associatively.  That turns the loop into a parallel scan.  When a partial sum would leave the
+// binade (S + inc >= 2^24) the summary stops being valid; the caller then lets one lane do the
+// offending adds natively and restarts the scan behind it with the new u.
+
+struct ParityInc {
+  uint32_t even;  // total increment if the run is entered with S even
+  uint32_t odd;   // ... with S odd
+};
+
+ETS_HD uint32_t sat_add(uint32_t a, uint32_t b) {
+  const uint32_t c = a + b;
+  return c < kSat ? c : kSat;
+}
+
+// a followed by b
+ETS_HD ParityInc compose(ParityInc a, ParityInc b) {
+  ParityInc c;
+  c.even = sat_add(a.even, (a.even & 1u) ? b.odd : b.even);
+  c.odd = sat_add(a.odd, ((a.odd + 1u) & 1u) ? b.odd : b.even);
+  return c;
+}
+
+// Integer view of the running sum: s = S * 2^(kb - 150) with kb the biased exponent (>= 1).
+struct SumState {
+  uint32_t S;
+  int kb;
+};
+
+ETS_HD SumState sum_state(float s) {
+  const uint32_t b = __builtin_bit_cast(uint32_t, s);
+  SumState st;
+  const uint32_t e = b >> 23;  // s >= 0, so no sign bit
+  st.kb = e ? static_cast<int>(e) : 1;
+  st.S = e ? ((b & 0x7fffffu) | 0x800000u) : b;
+  return st;
+}
+
+// Inverse of sum_state for S' <= 2^24 (the implicit bit carries into the exponent field).
+ETS_HD float sum_value(uint32_t S, int kb) {
+  return __builtin_bit_cast(float, (static_cast<uint32_t>(kb - 1) << 23) + S);
+}
+
+// Fold element `abits` (float bits, finite, >= 0) into a lane's summary.
+ETS_HD void fold_elem(ParityInc& acc, uint32_t abits, int kb) {
+  uint32_t ea = abits >> 23;
+  uint32_t M = abits & 0x7fffffu;
+  if (ea) {
+    M |= 0x800000u;
+  } else {
+    ea = 1;
+  }
+  const int sh = kb - static_cast<int>(ea);
+  uint32_t n0, up = 0, tie = 0;
+  if (sh <= 0) {
+    n0 = (sh < -2) ? kSat : (M << (-sh));  // a >= 2^k: certainly leaves the binade
+  } else if (sh >= 25) {
+    n0 = 0;  // a < u/2: absorbed
+  } else {
+    n0 = M >> sh;
+    const uint32_t rem = M & ((1u << sh) - 1u);
+    const uint32_t half = 1u << (sh - 1);
+    up = rem > half ? 1u : 0u;
+    tie = rem == half ? 1u : 0u;
+  }
+  const uint32_t base = n0 + up;
+  const uint32_t inc_even = base + (tie & ((acc.even + n0) & 1u));
+  const uint32_t inc_odd = base + (tie & ((acc.odd + n0 + 1u) & 1u));
+  acc.even = sat_add(acc.even, inc_even);
+  acc.odd = sat_add(acc.odd, inc_odd);
+}
+
+}  // namespace ets

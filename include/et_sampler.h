@@ -1,0 +1,155 @@
+/*
+ * et_sampler.h -- C ABI of the MI355X (gfx950) LLM token sampler.
+ *
+ * A drop-in for ExecuTorch's `extension/llm/sampler` path: every entry point below names the
+ * reference interface it replaces (paths relative to the ExecuTorch tree).  Plain pointers
+ * and sizes only; no C++ or torch types cross this boundary.  The C++ class
+ * `executorch::extension::llm::Sampler` in include/executorch_amd/sampler.h and the Python
+ * class `executorch_amd.Sampler` are thin wrappers over these functions.
+ *
+ * Semantics shared by all sampling entry points (Sampler::sample<T>, sampler.cpp:222-251):
+ *   temperature == 0          -> arg-max, lowest index wins ties, no coin is drawn;
+ *   otherwise                 -> logits * (1/temperature), softmax, ONE xorshift64* coin, then
+ *     0 < topk < vocab        -> top-k draw            (sampler.cpp:72-120)
+ *     topp <= 0 || topp >= 1  -> multinomial draw      (sampler.cpp:58-70)
+ *     else                    -> top-p (nucleus) draw  (sampler.cpp:122-171)
+ * Arithmetic: rows of every dtype are converted to fp32 (exactly) and the fp32 instantiation
+ * of the reference is followed bit for bit, including the order of its sequential float
+ * additions; fp16/bf16 rows therefore give what the reference gives after the "convert the
+ * row to float, then sample<float>" step several of its own runners perform
+ * (examples/models/gemma4/runner/gemma4_runner.cpp:166-182).  Among candidates whose
+ * probabilities are exactly equal the lower token index is ordered first (the reference
+ * leaves that order to std::sort).  The logits buffer is never written: the reference's
+ * side effect of leaving probabilities in it (sampler.cpp:231-235) is not reproduced.
+ *
+ * Every function returns an ets_status; none aborts.  Calls on one handle must be serialized
+ * by the caller (as for the reference, text_decoder_runner.h:81-82); distinct handles are
+ * independent.
+ */
+#ifndef ET_SAMPLER_H_
+#define ET_SAMPLER_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#if defined(_WIN32)
+#define ETS_API
+#else
+#define ETS_API __attribute__((visibility("default")))
+#endif
+
+/* Status codes: numeric values of executorch::runtime::Error (runtime/core/error.h:35-61). */
+typedef int32_t ets_status;
+#define ETS_OK 0x00
+#define ETS_INTERNAL 0x01          /* a HIP call failed; see ets_sampler_last_error()       */
+#define ETS_INVALID_STATE 0x02
+#define ETS_NOT_SUPPORTED 0x10     /* e.g. stochastic sampling of UInt16 rows               */
+#define ETS_INVALID_ARGUMENT 0x12  /* null pointer, bad size, unknown dtype, batch too big  */
+#define ETS_MEMORY_ALLOCATION_FAILED 0x21
+
+/* Element types: numeric values of executorch ScalarType
+ * (runtime/core/portable_type/scalar_type.h:98-125); the four that
+ * sample_from_logits() accepts (util.h:36-43). */
+#define ETS_DTYPE_HALF 5
+#define ETS_DTYPE_FLOAT 6
+#define ETS_DTYPE_BFLOAT16 15
+#define ETS_DTYPE_UINT16 27
+
+typedef struct ets_sampler ets_sampler;
+
+/* Intermediate values of one row's draw, written by the *_debug entry point (tests only). */
+typedef struct {
+  float max_val;        /* row maximum of logits * inv_temperature                          */
+  float sum;            /* softmax normaliser, accumulated like the reference (index order) */
+  float coin;           /* the row's xorshift64* coin                                        */
+  float cumulative;     /* mass of the nucleus / of the top-k set                            */
+  float r;              /* coin scaled into that mass                                        */
+  int32_t n_candidates; /* entries >= the top-p cutoff (vocab for top-k)                     */
+  int32_t last_idx;     /* last sorted position inside the nucleus                           */
+  int32_t position;     /* sorted position of the returned token                             */
+} ets_row_debug;
+
+/* Sampler::Sampler(int32_t vocab_size, float temperature, float topp, unsigned long long
+ * rng_seed)  -- sampler.cpp:173-181.  No clamping of temperature (a negative value gives a
+ * negative inverse, as there).  `max_batch` (>= 1) is the largest batch later passed to
+ * ets_sampler_sample_batch(); row b starts with xorshift64* state rng_seed + b, so row 0 is
+ * the reference object's own stream.  The handle lives on the current HIP device. */
+ETS_API ets_status ets_sampler_create(int32_t vocab_size, float temperature, float topp, uint64_t rng_seed,
+                                      int32_t max_batch, ets_sampler** out);
+
+/* Sampler::Sampler(int32_t vocab_size, float temperature)  -- sampler.cpp:183-187:
+ * topp = kTopp = 0.9f (sampler.h:29), seed = time(NULL). */
+ETS_API ets_status ets_sampler_create_default(int32_t vocab_size, float temperature, int32_t max_batch,
+                                              ets_sampler** out);
+
+/* Sampler's implicit destructor. */
+ETS_API ets_status ets_sampler_destroy(ets_sampler* s);
+
+/* Sampler::set_temperature  -- sampler.h:48-53 (negative values are reset to 0). */
+ETS_API ets_status ets_sampler_set_temperature(ets_sampler* s, float temperature);
+
+/* Sampler::set_topk  -- sampler.h:58-60 (k <= 0 or k >= vocab disables top-k). */
+ETS_API ets_status ets_sampler_set_topk(ets_sampler* s, int32_t topk);
+
+/* No counterpart: the reference fixes top-p at construction (sampler.h:78).  Provided so one
+ * handle can serve requests with different nucleus sizes. */
+ETS_API ets_status ets_sampler_set_topp(ets_sampler* s, float topp);
+
+/* Sampler::sample<T>(T* logits)  -- sampler.cpp:222-251, instantiations :253-258.
+ * `logits` is a HOST pointer to vocab_size elements of `dtype`; the row is copied to the
+ * device, sampled there and the token copied back (synchronous).  Consumes row 0's coin. */
+ETS_API ets_status ets_sampler_sample(ets_sampler* s, const void* logits, int32_t dtype, int32_t* token_out);
+
+/* Batched form of Sampler::sample<T> (no counterpart; the reference is batch-1, util.h:48-51).
+ * `d_logits` is a DEVICE pointer to `batch` rows of vocab_size elements, row b starting at
+ * element b * row_stride_elems (>= vocab_size); `d_tokens` is a DEVICE pointer to `batch`
+ * int32.  Row b uses and advances its own coin stream, so the result equals `batch`
+ * reference objects seeded rng_seed + b and does not depend on how rows are batched.
+ * Asynchronous on `hip_stream` (a hipStream_t, NULL = the default stream). */
+ETS_API ets_status ets_sampler_sample_batch(ets_sampler* s, const void* d_logits, int32_t dtype, int32_t batch,
+                                           int64_t row_stride_elems, int32_t* d_tokens, void* hip_stream);
+
+/* As above, plus per-row intermediates for the parity tests: `d_probs` (nullable) receives the
+ * fp32 softmax probabilities [batch, vocab_size] that the reference would leave in its buffer,
+ * `d_debug` (nullable) one ets_row_debug per row.  Both are DEVICE pointers. */
+ETS_API ets_status ets_sampler_sample_batch_debug(ets_sampler* s, const void* d_logits, int32_t dtype,
+                                                 int32_t batch, int64_t row_stride_elems, int32_t* d_tokens,
+                                                 float* d_probs, ets_row_debug* d_debug, void* hip_stream);
+
+/* Per-row xorshift64* states (sampler.h:82 `rng_state_`, one per row here).  HOST pointers to
+ * `count` values for rows [first_row, first_row + count).  Lets a run be replayed or resumed. */
+ETS_API ets_status ets_sampler_set_rng_states(ets_sampler* s, int32_t first_row, int32_t count,
+                                              const uint64_t* states);
+ETS_API ets_status ets_sampler_get_rng_states(ets_sampler* s, int32_t first_row, int32_t count, uint64_t* states);
+
+/* sample_from_logits(const Tensor&, Sampler&)  -- util.h:25-55.  The tensor is passed as
+ * (HOST data, dtype, rank, sizes[rank]); rank 3 samples the last position of batch 0, the
+ * last dimension must equal the handle's vocab_size.  An unsupported dtype returns
+ * ETS_INVALID_ARGUMENT where the reference aborts (util.h:30-34). */
+ETS_API ets_status ets_sample_from_logits(ets_sampler* s, const void* data, int32_t dtype, int32_t rank,
+                                          const int64_t* sizes, int32_t* token_out);
+
+/* logits_to_token(const Tensor&, float temperature = 0)  -- util.h:64-71: a temporary
+ * 2-argument Sampler over the tensor's last dimension. */
+ETS_API ets_status ets_logits_to_token(const void* data, int32_t dtype, int32_t rank, const int64_t* sizes,
+                                       float temperature, int32_t* token_out);
+
+/* random_u32 / random_f32  -- sampler.cpp:210-220, on the host (exported so callers can
+ * predict or replay a row's coins). */
+ETS_API uint32_t ets_random_u32(uint64_t* state);
+ETS_API float ets_random_f32(uint64_t* state);
+
+/* Text of the last error on this handle ("" if none); valid until the next call on it.
+ * With s == NULL: the last error of a failed create / handle-less call on this thread. */
+ETS_API const char* ets_sampler_last_error(const ets_sampler* s);
+
+/* Library version string. */
+ETS_API const char* ets_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ET_SAMPLER_H_ */

@@ -1,0 +1,141 @@
+// Host check of the integer scan that emulates a sequential fp32 sum (the arithmetic in
+// executorch_amd/csrc/ets_seqsum_math.h).  A serial simulation of the workgroup algorithm --
+// lanes own runs of consecutive elements, run summaries are composed in order, the first run
+// that leaves the binade or crosses the threshold is redone with native adds -- is compared
+// with the plain loop `s += a[i]` on adversarial and random inputs.  Exit code 0 iff every
+// case matches bit for bit.  Built and run by tests/test_seqsum_host.py.
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+#include <random>
+#include <vector>
+
+#include "ets_seqsum_math.h"
+
+using namespace ets;
+
+struct Result {
+  float sum;
+  int stop;
+};
+
+static Result plain(const std::vector<float>& a, float s0, float thr) {
+  volatile float s = s0;
+  for (size_t i = 0; i < a.size(); ++i) {
+    s = s + a[i];
+    if (s > thr) return {s, (int)i};
+  }
+  return {s, -1};
+}
+
+static Result simulated(const std::vector<float>& a, float s0, float thr, int lanes, int run) {
+  const int n = (int)a.size();
+  const int chunk = lanes * run;
+  float s = s0;
+  for (int base = 0; base < n; base += chunk) {
+    int resume = 0;
+    while (true) {
+      SumState st = sum_state(s);
+      std::vector<ParityInc> mine(lanes), incl(lanes), excl(lanes);
+      ParityInc acc = {0, 0};
+      for (int t = 0; t < lanes; ++t) {
+        ParityInc m = {0, 0};
+        if (t >= resume)
+          for (int e = 0; e < run; ++e) {
+            int i = base + t * run + e;
+            uint32_t bits = 0;
+            if (i < n) std::memcpy(&bits, &a[i], 4);
+            fold_elem(m, bits, st.kb);
+          }
+        mine[t] = m;
+        excl[t] = acc;
+        acc = compose(acc, m);
+        incl[t] = acc;
+      }
+      bool odd = st.S & 1u;
+      int j = lanes;
+      for (int t = 0; t < lanes; ++t) {
+        uint32_t Si = st.S + (odd ? incl[t].odd : incl[t].even);
+        bool special = Si >= (1u << 24);
+        if (!special) special = sum_value(Si, st.kb) > thr;
+        if (special) {
+          j = t;
+          break;
+        }
+      }
+      if (j == lanes) {
+        s = sum_value(st.S + (odd ? acc.odd : acc.even), st.kb);
+        break;
+      }
+      volatile float sj = sum_value(st.S + (odd ? excl[j].odd : excl[j].even), st.kb);
+      for (int e = 0; e < run; ++e) {
+        int i = base + j * run + e;
+        if (i < n) {
+          sj = sj + a[i];
+          if (sj > thr) return {sj, i};
+        }
+      }
+      s = sj;
+      resume = j + 1;
+    }
+  }
+  return {s, -1};
+}
+
+static int check(const std::vector<float>& a, float s0, float thr, const char* what) {
+  Result p = plain(a, s0, thr);
+  int bad = 0;
+  const int shapes[][2] = {{1024, 4}, {64, 4}, {7, 3}, {1, 1}, {256, 8}};
+  for (auto& sh : shapes) {
+    Result q = simulated(a, s0, thr, sh[0], sh[1]);
+    if (std::memcmp(&p.sum, &q.sum, 4) != 0 || p.stop != q.stop) {
+      std::printf("MISMATCH %s lanes=%d run=%d: plain (%a,%d) simulated (%a,%d)\n", what, sh[0], sh[1], p.sum,
+                  p.stop, q.sum, q.stop);
+      ++bad;
+    }
+  }
+  return bad;
+}
+
+int main() {
+  std::mt19937_64 rng(12345);
+  int bad = 0, cases = 0;
+  const float inf = INFINITY;
+  auto uni = [&](double lo, double hi) { return lo + (hi - lo) * (rng() >> 11) * (1.0 / 9007199254740992.0); };
+  for (int rep = 0; rep < 400; ++rep) {
+    int n = 1 + (int)(rng() % 20000);
+    std::vector<float> a(n);
+    int kind = rep % 8;
+    for (int i = 0; i < n; ++i) {
+      switch (kind) {
+        case 0: a[i] = (float)std::exp(uni(-30, 0)); break;                      // wide dynamic range
+        case 1: a[i] = (float)std::exp(uni(-18, -15)); break;                    // near the absorption edge
+        case 2: a[i] = std::ldexp(1.0f, -(int)(rng() % 40)); break;              // powers of two: ties galore
+        case 3: a[i] = std::ldexp((float)(1 + rng() % 7), -(int)(rng() % 30)); break;  // few-bit values
+        case 4: a[i] = (rng() % 50 == 0) ? (float)uni(0.1, 1.0) : (float)std::exp(uni(-25, -14)); break;  // peaked
+        case 5: a[i] = (rng() % 3 == 0) ? 0.0f : std::ldexp((float)(rng() % 4096), -149 + (int)(rng() % 30)); break;  // denormals
+        case 6: a[i] = 1.0f / (float)n; break;                                   // flat
+        default: a[i] = (float)uni(0, 1e-3); break;
+      }
+    }
+    float s0 = (rep % 5 == 0) ? (float)uni(0, 2) : 0.0f;
+    bad += check(a, s0, inf, "sum");
+    Result tot = plain(a, s0, inf);
+    float thr = tot.sum * (float)uni(0, 1.05);
+    bad += check(a, s0, thr, "threshold");
+    bad += check(a, s0, 0.0f, "threshold0");
+    cases += 3;
+  }
+  // half-ulp ties against an odd and an even running sum
+  for (int k = 0; k < 64; ++k) {
+    std::vector<float> a(5000, std::ldexp(1.0f, -24));
+    a[0] = 1.0f + std::ldexp((float)(k & 1), -23);
+    a[17] = std::ldexp(3.0f, -24);
+    a[k + 20] = std::ldexp(1.0f, -23);
+    bad += check(a, 0.0f, inf, "ties");
+    ++cases;
+  }
+  std::printf("seqsum_host_check: %d cases, %d mismatches\n", cases, bad);
+  return bad != 0;
+}
