@@ -1,0 +1,187 @@
+"""Benchmark of the token-sampling hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2]
+
+A step is one batched sampling call over one [B, vocab] matrix of synthetic logits already
+resident in HBM.  Steps walk a ring of distinct matrices larger than the 256 MB Infinity Cache so
+that every step reads its logits from HBM.  Prints one JSON line (rows/s, roofline of the
+dominant kernel, the CPU baseline timed on this box's host cores).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+from concurrent.futures import ThreadPoolExecutor
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+
+
+def synth_logits_device(w, count, torch, dev):
+    """`count` matrices of workload `w`'s distribution generated on the device (same shape,
+    dtype and statistics as executorch_amd.workloads, torch's generator instead of numpy's)."""
+    from executorch_amd import workloads as W
+
+    tdt = {W.DTYPE_FLOAT: torch.float32, W.DTYPE_HALF: torch.float16, W.DTYPE_BFLOAT16: torch.bfloat16}[w.dtype]
+    g = torch.Generator(device=dev).manual_seed(w.data_seed)
+    ring = []
+    for _ in range(count):
+        if w.kind == "peaked":
+            x = torch.randn((w.batch, w.vocab), generator=g, device=dev)
+            ids = torch.rand((w.batch, w.vocab), generator=g, device=dev).topk(20, dim=1).indices
+            x.scatter_add_(1, ids, torch.full_like(ids, 8.0, dtype=torch.float32))
+        elif w.kind == "flat":
+            x = torch.randn((w.batch, w.vocab), generator=g, device=dev) * 0.5
+        elif w.kind == "normal2":
+            x = torch.randn((w.batch, w.vocab), generator=g, device=dev) * 2.0
+        elif w.kind == "normal15":
+            x = torch.randn((w.batch, w.vocab), generator=g, device=dev) * 1.5
+        elif w.kind == "mixed":
+            x = torch.randn((w.batch, w.vocab), generator=g, device=dev)
+            u = torch.rand((w.batch // 2, w.vocab), generator=g, device=dev).clamp_(1e-7, 1 - 1e-7)
+            gum = -torch.log(-torch.log(u))
+            hot = torch.randint(0, w.vocab, (w.batch // 2, 1), generator=g, device=dev)
+            gum.scatter_add_(1, hot, torch.full_like(hot, 12.0, dtype=torch.float32))
+            x[1::2] = gum
+        else:
+            raise ValueError(w.kind)
+        ring.append(x.to(tdt))
+    return ring
+
+
+def cpu_baseline(w, seconds_budget=12.0):
+    """The reference sampler on this box's host cores, on a bounded sample of the workload:
+    `sampler.cpp` itself (oracle/_ref) when it was built, else the oracle's restatement."""
+    import numpy as np
+
+    from executorch_amd import workloads as W
+    from oracle import oracle as O
+
+    rows = min(w.batch, 64)
+    x = W.logits(w, 0, rows)
+    cores = max(1, min(16, os.cpu_count() or 1))
+    use_ref = O.have_ref()
+
+    def one_row(b, reps):
+        if use_ref:
+            s = O.RefSampler(w.vocab, w.temperature, w.topp, w.coin_seed + b)
+        else:
+            s = O.Sampler(w.vocab, w.temperature, w.topp, w.coin_seed + b, mode=O.MODE_NATIVE)
+        for _ in range(reps):
+            s.sample(x[b].copy(), w.dtype)
+
+    t0 = time.perf_counter()
+    one_row(0, 3)
+    per_row = (time.perf_counter() - t0) / 3
+    reps = max(1, int(seconds_budget * cores / (per_row * rows)))
+    reps = min(reps, 5000)
+    t0 = time.perf_counter()
+    with ThreadPoolExecutor(cores) as pool:
+        list(pool.map(lambda b: one_row(b, reps), range(rows)))
+    dt = time.perf_counter() - t0
+    t0 = time.perf_counter()
+    one_row(1 % rows, 5)
+    one_core = 5 / (time.perf_counter() - t0)
+    return {
+        "value": rows * reps / dt,
+        "unit": "rows/s",
+        "cores": cores,
+        "kind": "reference" if use_ref else "port",
+        "sample": f"{rows} rows of {w.name} step 0, each sampled {reps} times by its own Sampler, native "
+                  f"{W.DTYPE_NAMES[w.dtype]} sample<T>, {cores} threads ({dt:.1f} s)",
+        "rows_per_s_one_core": one_core,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="cfg2")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU; rows are independent, so more GPUs would each take "
+              "a slice of the batch with no communication.  Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+
+    import executorch_amd as ea
+    from executorch_amd import workloads as W
+    from oracle import oracle as O
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    w = W.WORKLOADS[args.workload]
+    step_bytes = w.bytes_per_step
+    ring_len = max(2, -(-(576 << 20) // step_bytes))  # >= 576 MiB of distinct logits
+    ring = synth_logits_device(w, ring_len, torch, dev)
+    s = ea.Sampler(w.vocab, w.temperature, w.topp, w.coin_seed, max_batch=w.batch)
+    out = torch.empty(w.batch, dtype=torch.int32, device=dev)
+
+    # parity spot check on host-generated rows before timing anything
+    rows = min(w.batch, 64)
+    hx = W.logits(w, 0, rows)
+    if w.dtype == W.DTYPE_BFLOAT16:
+        dx = torch.from_numpy(hx.view(np.int16)).to(dev).view(torch.bfloat16)
+    else:
+        dx = torch.from_numpy(hx).to(dev)
+    chk = ea.Sampler(w.vocab, w.temperature, w.topp, w.coin_seed, max_batch=rows)
+    got = chk.sample_batch(dx).cpu().numpy()
+    want, _ = O.sample_rows(hx, w.dtype, O.inv_temperature(w.temperature), w.topp, 0, W.coin_seeds(w, rows).copy(),
+                            mode=O.MODE_UPCAST, tie=O.TIE_STABLE, threads=8)
+    mismatches = int((got != want).sum())
+
+    for i in range(args.warmup):
+        s.sample_batch(ring[i % ring_len], out=out)
+    torch.cuda.synchronize()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    ev0.record()
+    for i in range(args.steps):
+        s.sample_batch(ring[i % ring_len], out=out)
+    ev1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    kernel_ms = ev0.elapsed_time(ev1) / args.steps  # events on the launch stream; one kernel per step
+    ms_per_step = wall * 1e3 / args.steps
+    achieved = step_bytes / (kernel_ms * 1e-3) / 1e9
+
+    line = {
+        "metric": f"sampled rows/sec at vocab {w.vocab}, B={w.batch}, {W.DTYPE_NAMES[w.dtype]}, "
+                  f"T={w.temperature}, top-p {w.topp}",
+        "value": w.batch * args.steps / wall,
+        "unit": "rows/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": f"{w.name}: vocab {w.vocab}, batch {w.batch}, {W.DTYPE_NAMES[w.dtype]} logits ({w.kind}), "
+                               f"temperature {w.temperature}, top-p {w.topp}, per-row xorshift64* coins; "
+                               f"ring of {ring_len} distinct matrices ({ring_len * step_bytes >> 20} MiB)"},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None, "kernel": "sample_rows_kernel",
+                     "kernel_ms": kernel_ms, "algorithmic_bytes_per_launch": step_bytes},
+        "parity": {"rows_checked": rows, "token_mismatches_vs_oracle": mismatches},
+    }
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline(w)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

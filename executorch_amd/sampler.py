@@ -158,19 +158,17 @@ def debug_records(debug_out: torch.Tensor) -> np.ndarray:
     return raw.view(dt).reshape(-1)
 
 
-def _host_tensor_args(logits):
+def _host_tensor_args(logits, dtype):
     if isinstance(logits, torch.Tensor):
         t = logits.contiguous().cpu()
-        return t, t.data_ptr(), dtype_code(t), list(t.shape)
+        return t, t.data_ptr(), dtype_code(t) if dtype is None else dtype, list(t.shape)
     a = np.ascontiguousarray(logits)
-    return a, a.ctypes.data, dtype_code(a), list(a.shape)
+    return a, a.ctypes.data, dtype_code(a) if dtype is None else dtype, list(a.shape)
 
 
 def sample_from_logits(logits, sampler: Sampler, dtype: int | None = None) -> int:
     """util.h:25-55: rank 3 ``[1, S, V]`` samples the last position of batch 0."""
-    keep, ptr, code, shape = _host_tensor_args(logits)
-    if dtype is not None:
-        code = dtype
+    keep, ptr, code, shape = _host_tensor_args(logits, dtype)
     sizes = (C.c_int64 * len(shape))(*shape)
     tok = C.c_int32(-1)
     sampler._check(_capi.lib().ets_sample_from_logits(sampler._h, ptr, code, len(shape), sizes, C.byref(tok)))
@@ -179,9 +177,7 @@ def sample_from_logits(logits, sampler: Sampler, dtype: int | None = None) -> in
 
 def logits_to_token(logits, temperature: float = 0.0, dtype: int | None = None) -> int:
     """util.h:64-71: a temporary 2-argument Sampler over the tensor's last dimension."""
-    keep, ptr, code, shape = _host_tensor_args(logits)
-    if dtype is not None:
-        code = dtype
+    keep, ptr, code, shape = _host_tensor_args(logits, dtype)
     sizes = (C.c_int64 * len(shape))(*shape)
     tok = C.c_int32(-1)
     L = _capi.lib()

@@ -1,0 +1,145 @@
+"""Stochastic path of the HIP sampler against the CPU oracle, through the C ABI.
+
+The oracle runs in "convert the row to fp32, then sample<float>" mode (the arithmetic the HIP
+sampler implements for every dtype) with exactly tied probabilities ordered by token index (the
+HIP sampler's tie rule).  Under those two conventions the bar is bit-exact: tokens, the per-row
+xorshift64* states, the softmax probabilities and the intermediate sums.  Agreement with the
+reference's own tie order (whatever std::sort leaves) is measured next to it: the two may differ
+only on rows where the two candidates' probabilities are exactly equal.
+"""
+import numpy as np
+import pytest
+import torch
+
+import executorch_amd as ea
+from executorch_amd import workloads as W
+from util import f32_bits, to_device
+
+pytestmark = pytest.mark.gpu
+
+
+def run_case(oracle, dev, w, rows, steps, topk=0, probs=False, topp=None, temperature=None):
+    topp = w.topp if topp is None else topp
+    temperature = w.temperature if temperature is None else temperature
+    s = ea.Sampler(w.vocab, temperature, topp, w.coin_seed, max_batch=rows)
+    if topk:
+        s.set_topk(topk)
+    states = W.coin_seeds(w, rows).copy()
+    inv = oracle.inv_temperature(temperature)
+    tie_rows = total = 0
+    for st in range(steps):
+        x = W.logits(w, st, rows)
+        dx = to_device(x, w.dtype, dev)
+        dprobs = torch.empty((rows, w.vocab), dtype=torch.float32, device=dev) if probs else None
+        ddbg = torch.zeros((rows, 8), dtype=torch.int32, device=dev)
+        got = s.sample_batch(dx, probs_out=dprobs, debug_out=ddbg).cpu().numpy()
+        lib_states = states.copy()
+        want, ex = oracle.sample_rows(x, w.dtype, inv, topp, topk, states, mode=oracle.MODE_UPCAST, tie=oracle.TIE_STABLE,
+                                      explain=True, threads=8)
+        ref, _ = oracle.sample_rows(x, w.dtype, inv, topp, topk, lib_states, mode=oracle.MODE_UPCAST,
+                                    tie=oracle.TIE_LIBSTDCXX, threads=8)
+        assert np.array_equal(got, want), (w.name, st, np.nonzero(got != want)[0][:8])
+        dbg = ea.debug_records(ddbg)
+        for b in range(rows):
+            e = ex[b]
+            assert f32_bits(dbg["max_val"][b]) == f32_bits(e.max_val)
+            assert f32_bits(dbg["sum"][b]) == f32_bits(e.sum)
+            assert f32_bits(dbg["coin"][b]) == f32_bits(e.coin)
+            if e.branch in (oracle.BRANCH_TOPP, oracle.BRANCH_TOPK):
+                assert dbg["n_candidates"][b] == e.n_candidates
+                assert dbg["last_idx"][b] == e.last_idx
+                assert f32_bits(dbg["cumulative"][b]) == f32_bits(e.cumulative)
+                assert f32_bits(dbg["r"][b]) == f32_bits(e.r)
+                assert dbg["position"][b] == e.position
+        if probs:
+            p = dprobs.cpu().numpy()
+            for b in range(min(rows, 4)):
+                po = np.empty(w.vocab, dtype=np.float32)
+                o = oracle.Sampler(w.vocab, temperature, topp, 1, mode=oracle.MODE_UPCAST)
+                o.sample(x[b].copy(), w.dtype, probs_out=po)
+                assert np.array_equal(f32_bits(p[b]), f32_bits(po))
+        # vs the reference's own tie order: differences only between equal probabilities
+        diff = np.nonzero(ref != want)[0]
+        for b in diff:
+            po = np.empty(w.vocab, dtype=np.float32)
+            o = oracle.Sampler(w.vocab, temperature, topp, 1, mode=oracle.MODE_UPCAST)
+            o.set_topk(topk)
+            o.sample(x[b].copy(), w.dtype, probs_out=po)
+            assert po[ref[b]] == po[want[b]]
+        tie_rows += len(diff)
+        total += rows
+        assert np.array_equal(s.get_rng_states(rows), states)
+    return tie_rows, total
+
+
+@pytest.mark.parametrize("name,rows,steps", [("cfg1", 1, 60), ("cfg2", 64, 3), ("cfg3", 6, 1), ("cfg4", 32, 2), ("cfg5", 8, 1)])
+def test_workloads_bit_exact(oracle, dev, name, rows, steps):
+    ties, total = run_case(oracle, dev, W.WORKLOADS[name], rows, steps, probs=(name in ("cfg1", "cfg2")))
+    print(f"{name}: {ties}/{total} rows differ from the reference's tie order (all tie-equivalent)")
+
+
+@pytest.mark.parametrize("name,rows", [("cfg2", 16), ("cfg1", 1), ("cfg3", 2)])
+@pytest.mark.parametrize("topk", [1, 5, 40])
+def test_topk_bit_exact(oracle, dev, name, rows, topk):
+    run_case(oracle, dev, W.WORKLOADS[name], rows, 1, topk=topk)
+
+
+@pytest.mark.parametrize("topp,temperature", [(0.0, 1.0), (1.0, 0.7), (0.5, 0.3), (0.99, 1.0), (0.05, 1.0), (0.9, 0.05)])
+def test_parameter_sweep_bit_exact(oracle, dev, topp, temperature):
+    for name, rows in (("cfg1", 2), ("cfg2", 8)):
+        run_case(oracle, dev, W.WORKLOADS[name], rows, 1, topp=topp, temperature=temperature)
+
+
+def test_small_and_ragged_vocabularies(oracle, dev):
+    rng = np.random.default_rng(12)
+    for V in (2, 3, 5, 63, 64, 65, 1023, 1025, 4095, 4097, 8193, 50257):
+        for dtype in (W.DTYPE_FLOAT, W.DTYPE_HALF, W.DTYPE_BFLOAT16):
+            B = 5
+            x = W.to_storage((rng.standard_normal((B, V)) * 1.5).astype(np.float32), dtype)
+            for topp, topk in ((0.9, 0), (1.0, 0), (0.9, 2)):
+                if topk >= V:
+                    continue
+                s = ea.Sampler(V, 0.8, topp, 900, max_batch=B)
+                s.set_topk(topk)
+                states = (np.uint64(900) + np.arange(B, dtype=np.uint64)).astype(np.uint64)
+                got = s.sample_batch(to_device(x, dtype, dev)).cpu().numpy()
+                want, _ = oracle.sample_rows(x, dtype, oracle.inv_temperature(0.8), topp, topk, states,
+                                             mode=oracle.MODE_UPCAST, tie=oracle.TIE_STABLE)
+                assert np.array_equal(got, want), (V, dtype, topp, topk)
+
+
+def test_batch_split_invariance_and_replay(dev):
+    """Row b's token depends only on its own logits and coin stream: sampling the batch whole,
+    in two halves, or row by row gives the same tokens; restoring the states replays them."""
+    w = W.WORKLOADS["cfg2"]
+    rows = 32
+    x = to_device(W.logits(w, 0, rows), w.dtype, dev)
+    a = ea.Sampler(w.vocab, w.temperature, w.topp, 77, max_batch=rows)
+    whole = a.sample_batch(x).cpu().numpy()
+    after = a.get_rng_states()
+    b = ea.Sampler(w.vocab, w.temperature, w.topp, 77, max_batch=rows)
+    seeds = b.get_rng_states()
+    halves = np.empty(rows, dtype=np.int32)
+    for lo, hi in ((0, 16), (16, 32)):
+        c = ea.Sampler(w.vocab, w.temperature, w.topp, 0, max_batch=hi - lo)
+        c.set_rng_states(seeds[lo:hi])
+        halves[lo:hi] = c.sample_batch(x[lo:hi]).cpu().numpy()
+    assert np.array_equal(whole, halves)
+    a.set_rng_states(seeds)
+    assert np.array_equal(a.sample_batch(x).cpu().numpy(), whole)
+    assert np.array_equal(a.get_rng_states(), after)
+    single = ea.Sampler(w.vocab, w.temperature, w.topp, 77 + 5)
+    assert single.sample(x[5].cpu()) == whole[5]
+
+
+def test_total_variation_of_draws(dev):
+    """20 000 draws from softmax(log [.5 .3 .15 .05]) through the batched entry: within 0.02
+    total variation of the target, and of the renormalised nucleus for top-p 0.9."""
+    rows = 2000
+    x = torch.log(torch.tensor([0.5, 0.3, 0.15, 0.05])).repeat(rows, 1).to(dev)
+    for topp, target in ((1.0, [0.5, 0.3, 0.15, 0.05]), (0.9, [0.5 / 0.95, 0.3 / 0.95, 0.15 / 0.95, 0.0])):
+        s = ea.Sampler(4, 1.0, topp, 31337, max_batch=rows)
+        counts = np.zeros(4)
+        for _ in range(10):
+            counts += np.bincount(s.sample_batch(x).cpu().numpy(), minlength=4)
+        assert 0.5 * np.abs(counts / counts.sum() - np.array(target)).sum() < 0.02
