@@ -102,19 +102,27 @@ ets_status launch_argmax(ets_sampler* s, const void* d_logits, int32_t batch, in
   return ETS_OK;
 }
 
-template <int DT>
-ets_status launch_rows(ets_sampler* s, const ets::RowParams& p, int32_t batch, hipStream_t stream) {
+template <int DT, bool ALIGNED>
+ets_status launch_rows_impl(ets_sampler* s, const ets::RowParams& p, int32_t batch, hipStream_t stream) {
   static std::once_flag once;
   static hipError_t attr_err = hipSuccess;
   const size_t lds = s->lds_bytes;
   std::call_once(once, [&] {
-    attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(&ets::sample_rows_kernel<DT>),
+    attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(&ets::sample_rows_kernel<DT, ALIGNED>),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
   });
   if (attr_err != hipSuccess) return hip_fail(s, attr_err, "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
-  hipLaunchKernelGGL((ets::sample_rows_kernel<DT>), dim3(batch), dim3(ets::kBlock), lds, stream, p);
+  hipLaunchKernelGGL((ets::sample_rows_kernel<DT, ALIGNED>), dim3(batch), dim3(ets::kBlock), lds, stream, p);
   ETS_HIP(s, hipGetLastError());
   return ETS_OK;
+}
+
+template <int DT>
+ets_status launch_rows(ets_sampler* s, const ets::RowParams& p, int32_t batch, hipStream_t stream) {
+  // 128-bit loads need a 16-byte aligned base and row pitch
+  const size_t esz = ets::ElemSize<DT>::value;
+  const bool aligned = (reinterpret_cast<uintptr_t>(p.logits) % 16 == 0) && ((static_cast<size_t>(p.row_stride) * esz) % 16 == 0);
+  return aligned ? launch_rows_impl<DT, true>(s, p, batch, stream) : launch_rows_impl<DT, false>(s, p, batch, stream);
 }
 
 ets_status ensure_scratch(ets_sampler* s) {
@@ -204,9 +212,9 @@ ets_status ets_sampler_create(int32_t vocab_size, float temperature, float topp,
   int lds_limit = 0;
   e = hipDeviceGetAttribute(&lds_limit, hipDeviceAttributeMaxSharedMemoryPerBlock, s->device);
   if (e != hipSuccess) return bail(e, "hipDeviceGetAttribute(MaxSharedMemoryPerBlock)");
-  // static LDS of the row kernel (BlockScratch) is well under 2 KiB
+  // the row kernel's static LDS (reduction scratch, selection buffer, histogram) stays under 16 KiB
   int keys = 1;
-  while (static_cast<size_t>(keys) * 2 * sizeof(uint64_t) + 2048 <= static_cast<size_t>(lds_limit)) keys *= 2;
+  while (static_cast<size_t>(keys) * 2 * sizeof(uint64_t) + 16384 <= static_cast<size_t>(lds_limit)) keys *= 2;
   if (keys < 64) {
     ets_sampler_destroy(s);
     return fail(nullptr, ETS_INTERNAL, "ets_sampler_create: device reports too little LDS per workgroup");

@@ -11,12 +11,20 @@
 
 namespace ets {
 
-constexpr int kBlock = 1024;           // lanes per workgroup in the row kernels
-constexpr int kWaves = kBlock / 64;    // wave64 wavefronts per workgroup
-constexpr int kRun = 4;                // consecutive elements owned by one lane per chunk
-constexpr int kChunk = kBlock * kRun;  // elements a workgroup consumes per step
+constexpr int kBlock = 1024;         // lanes per workgroup in the row kernels
+constexpr int kWaves = kBlock / 64;  // wave64 wavefronts per workgroup
 
 constexpr int kDtypeHalf = 5, kDtypeFloat = 6, kDtypeBFloat16 = 15, kDtypeUInt16 = 27;
+
+template <int DT>
+struct ElemSize {
+  static constexpr int value = (DT == kDtypeFloat) ? 4 : 2;
+};
+// Elements per 16-byte vector load.
+template <int DT>
+struct VecElems {
+  static constexpr int value = 16 / ElemSize<DT>::value;
+};
 
 // ---- element loads: every storage type converts to fp32 exactly -----------------------------
 template <int DT>
@@ -39,10 +47,57 @@ __device__ __forceinline__ float load_elem<kDtypeUInt16>(const void* row, int64_
   return static_cast<float>(static_cast<const uint16_t*>(row)[i]);
 }
 
+__device__ __forceinline__ float half_bits_to_float(uint32_t h16) {
+  union {
+    uint16_t u;
+    _Float16 f;
+  } cvt;
+  cvt.u = static_cast<uint16_t>(h16);
+  return static_cast<float>(cvt.f);
+}
+
+// Decode one 16-byte vector into VecElems<DT> floats.
 template <int DT>
-struct ElemSize {
-  static constexpr int value = (DT == kDtypeFloat) ? 4 : 2;
-};
+__device__ __forceinline__ void decode_vec(const uint4& raw, float* out) {
+  const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+  if (DT == kDtypeFloat) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) out[k] = __uint_as_float(w[k]);
+  } else if (DT == kDtypeBFloat16) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      out[2 * k] = __uint_as_float(w[k] << 16);
+      out[2 * k + 1] = __uint_as_float(w[k] & 0xffff0000u);
+    }
+  } else if (DT == kDtypeHalf) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      out[2 * k] = half_bits_to_float(w[k] & 0xffffu);
+      out[2 * k + 1] = half_bits_to_float(w[k] >> 16);
+    }
+  } else {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      out[2 * k] = static_cast<float>(w[k] & 0xffffu);
+      out[2 * k + 1] = static_cast<float>(w[k] >> 16);
+    }
+  }
+}
+
+// Elements [first, first + VecElems) of a row as floats; positions >= n read as `fill`.
+// ALIGNED rows (16-byte aligned base and pitch) use one 128-bit load for interior vectors.
+template <int DT, bool ALIGNED>
+__device__ __forceinline__ void load_run(const void* row, int first, int n, float fill, float* out) {
+  constexpr int VE = VecElems<DT>::value;
+  if (ALIGNED && first + VE <= n) {
+    const uint4 raw = *reinterpret_cast<const uint4*>(static_cast<const char*>(row) +
+                                                      static_cast<int64_t>(first) * ElemSize<DT>::value);
+    decode_vec<DT>(raw, out);
+  } else {
+#pragma unroll
+    for (int e = 0; e < VE; ++e) out[e] = (first + e < n) ? load_elem<DT>(row, first + e) : fill;
+  }
+}
 
 // ---- expf, bit-identical to glibc's (sysdeps/ieee754/flt-32/e_expf.c, FMA build) ------------
 // exp(x) = 2^(k/32) * 2^(r/32), k = round(x * 32/ln2): 2^(k/32) from a 32-entry table of
@@ -60,7 +115,32 @@ __device__ __constant__ uint64_t kExp2Table[32] = {
     0x3fef5818dcfba487ull, 0x3fef7c97337b9b5full, 0x3fefa4afa2a490daull, 0x3fefd0765b6e4540ull,
 };
 
-// `tab` is a copy of kExp2Table in LDS (lanes index it divergently).
+// The table-and-cubic core for |x| < 104 (no special cases).  `tab` is a copy of kExp2Table in
+// LDS (lanes index it divergently).
+__device__ __forceinline__ float expf_core(float x, const uint64_t* tab) {
+  const double kInvLn2N = 0x1.71547652b82fep+0 * 32.0;
+  const double kShift = 0x1.8p+52;
+  const double kC0 = 0x1.c6af84b912394p-5 / 32.0 / 32.0 / 32.0;
+  const double kC1 = 0x1.ebfce50fac4f3p-3 / 32.0 / 32.0;
+  const double kC2 = 0x1.62e42ff0c52d6p-1 / 32.0;
+  const double xd = static_cast<double>(x);
+  double kd = __builtin_fma(kInvLn2N, xd, kShift);
+  const uint32_t ki_lo = static_cast<uint32_t>(__double_as_longlong(kd));  // round(x*32/ln2) mod 2^32
+  kd -= kShift;
+  const double r = __builtin_fma(kInvLn2N, xd, -kd);
+  // t = tab[k % 32] + (k << 47): the shifted term only touches the high word
+  const uint64_t te = tab[ki_lo & 31u];
+  const uint32_t t_hi = static_cast<uint32_t>(te >> 32) + (ki_lo << 15);
+  const double s = __hiloint2double(static_cast<int>(t_hi), static_cast<int>(static_cast<uint32_t>(te)));
+  const double z = __builtin_fma(kC0, r, kC1);
+  const double r2 = r * r;
+  double y = __builtin_fma(kC2, r, 1.0);
+  y = __builtin_fma(z, r2, y);
+  y = y * s;
+  return static_cast<float>(y);
+}
+
+// Full expf (every float input).
 __device__ __forceinline__ float expf_exact(float x, const uint64_t* tab) {
   const uint32_t ux = __float_as_uint(x);
   const uint32_t abstop = (ux >> 20) & 0x7ffu;
@@ -70,26 +150,19 @@ __device__ __forceinline__ float expf_exact(float x, const uint64_t* tab) {
     if (x > 0x1.62e42ep6f) return __uint_as_float(0x7f800000u);
     if (x < -0x1.9fe368p6f) return 0.0f;
   }
-  const double kInvLn2N = 0x1.71547652b82fep+0 * 32.0;
-  const double kShift = 0x1.8p+52;
-  const double kC0 = 0x1.c6af84b912394p-5 / 32.0 / 32.0 / 32.0;
-  const double kC1 = 0x1.ebfce50fac4f3p-3 / 32.0 / 32.0;
-  const double kC2 = 0x1.62e42ff0c52d6p-1 / 32.0;
-  const double xd = static_cast<double>(x);
-  double kd = __builtin_fma(kInvLn2N, xd, kShift);
-  const uint64_t ki = static_cast<uint64_t>(__double_as_longlong(kd));
-  kd -= kShift;
-  const double r = __builtin_fma(kInvLn2N, xd, -kd);
-  const uint64_t t = tab[ki & 31u] + (ki << 47);
-  const double s = __longlong_as_double(static_cast<long long>(t));
-  const double z = __builtin_fma(kC0, r, kC1);
-  const double r2 = r * r;
-  double y = __builtin_fma(kC2, r, 1.0);
-  y = __builtin_fma(z, r2, y);
-  y = y * s;
-  return static_cast<float>(y);
+  return expf_core(x, tab);
 }
 
+// expf for the softmax argument d = x - max, i.e. d <= 0 or NaN.  Branch-free: below
+// ln(2^-150) = -103.972 the result is 0, which is also what the core returns at -104, so
+// clamping there is exact.  A NaN argument comes back as NaN.
+__device__ __forceinline__ float expf_nonpositive(float d, const uint64_t* tab) {
+  const float dc = (d > -104.0f) ? d : -104.0f;  // also maps NaN to -104
+  const float e = expf_core(dc, tab);
+  return (d != d) ? d : e;
+}
+
+// ---- workgroup-wide primitives ------------------------------------------------------------------
 __device__ __forceinline__ ParityInc wave_scan_inclusive(ParityInc v, int lane) {
 #pragma unroll
   for (int d = 1; d < 64; d <<= 1) {
@@ -101,111 +174,12 @@ __device__ __forceinline__ ParityInc wave_scan_inclusive(ParityInc v, int lane) 
   return v;
 }
 
-// LDS scratch shared by the workgroup-wide primitives.
-struct BlockScratch {
-  uint64_t exp2tab[32];
-  ParityInc wave_total[kWaves];
-  int first_flag[kWaves];
-  float red_f[kWaves];
-  uint32_t red_u[kWaves];
-  float bc_sum;
-  int bc_found;
-  uint32_t counter;
-  int flag;
-};
-
-struct SeqSumResult {
-  float sum;      // value of s after the last element consumed
-  int stop_index; // first i with s > threshold after adding a[i]; -1 if none
-};
-
-// Emulates, with all kBlock lanes of the workgroup,
-//     s = s0; for (i = 0; i < n; ++i) { s += a(i); if (s > threshold) return {s, i}; }
-// bit for bit in fp32.  `a(i)` must return a finite, non-negative float and is evaluated once
-// per element; pass threshold = +inf to sum everything.  Must be called by every lane.
-template <typename Fetch>
-__device__ SeqSumResult seq_sum_block(Fetch a, int n, float s0, float threshold, BlockScratch& sm) {
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = tid >> 6;
-  float s = s0;
-  for (int base = 0; base < n; base += kChunk) {
-    uint32_t bits[kRun];
-    const int first = base + tid * kRun;
+__device__ __forceinline__ uint32_t wave_sum_u32(uint32_t v) {
 #pragma unroll
-    for (int e = 0; e < kRun; ++e) {
-      const int i = first + e;
-      bits[e] = (i < n) ? __float_as_uint(a(i)) : 0u;
-    }
-    int resume = 0;  // chunk-relative lane index from which elements are still unconsumed
-    while (true) {
-      const SumState st = sum_state(s);
-      ParityInc mine = {0u, 0u};
-      if (tid >= resume) {
-#pragma unroll
-        for (int e = 0; e < kRun; ++e) fold_elem(mine, bits[e], st.kb);
-      }
-      const ParityInc incl_w = wave_scan_inclusive(mine, lane);
-      if (lane == 63) sm.wave_total[wave] = incl_w;
-      __syncthreads();
-      ParityInc prefix = {0u, 0u};
-      ParityInc total = {0u, 0u};
-      for (int w = 0; w < kWaves; ++w) {
-        if (w == wave) prefix = total;
-        total = compose(total, sm.wave_total[w]);
-      }
-      ParityInc excl_w;
-      excl_w.even = __shfl_up(incl_w.even, 1);
-      excl_w.odd = __shfl_up(incl_w.odd, 1);
-      if (lane == 0) excl_w = {0u, 0u};
-      const ParityInc excl = compose(prefix, excl_w);
-      const ParityInc incl = compose(excl, mine);
-      const bool odd = st.S & 1u;
-      const uint32_t S_excl = st.S + (odd ? excl.odd : excl.even);
-      const uint32_t S_incl = st.S + (odd ? incl.odd : incl.even);
-      // A lane needs scalar treatment if its run leaves the binade or crosses the threshold.
-      bool special = S_incl >= (1u << 24);
-      if (!special) special = sum_value(S_incl, st.kb) > threshold;
-      const uint64_t ballot = __ballot(special);
-      if (lane == 0) sm.first_flag[wave] = ballot ? (wave * 64 + __ffsll(static_cast<long long>(ballot)) - 1) : kBlock;
-      __syncthreads();
-      int j = kBlock;
-      for (int w = 0; w < kWaves; ++w) {
-        const int f = sm.first_flag[w];
-        if (f < kBlock) {
-          j = f;
-          break;
-        }
-      }
-      if (j == kBlock) {  // whole chunk consumed inside the binade
-        s = sum_value(st.S + (odd ? total.odd : total.even), st.kb);
-        break;
-      }
-      if (tid == j) {
-        float sj = sum_value(S_excl, st.kb);
-        int found = -1;
-#pragma unroll
-        for (int e = 0; e < kRun; ++e) {
-          const int i = first + e;
-          if (i < n && found < 0) {
-            sj = sj + __uint_as_float(bits[e]);
-            if (sj > threshold) found = i;
-          }
-        }
-        sm.bc_sum = sj;
-        sm.bc_found = found;
-      }
-      __syncthreads();
-      s = sm.bc_sum;
-      const int found = sm.bc_found;
-      if (found >= 0) return {s, found};
-      resume = j + 1;
-    }
-  }
-  return {s, -1};
+  for (int d = 32; d > 0; d >>= 1) v += __shfl_xor(v, d);
+  return v;
 }
 
-// ---- small workgroup reductions ----------------------------------------------------------------
 __device__ __forceinline__ float wave_max_ignoring_nan(float v) {
 #pragma unroll
   for (int d = 32; d > 0; d >>= 1) {
@@ -213,6 +187,168 @@ __device__ __forceinline__ float wave_max_ignoring_nan(float v) {
     v = (o > v) ? o : v;
   }
   return v;
+}
+
+// LDS scratch shared by the workgroup-wide primitives.
+struct BlockScratch {
+  uint64_t exp2tab[32];
+  ParityInc wave_total[kWaves];
+  int first_flag[kWaves];
+  uint32_t fast_total[2][kWaves];  // double-buffered: one barrier per fast chunk
+  float red_f[kWaves];
+  uint32_t red_u[kWaves];
+  float bc_sum;
+  int bc_found;
+  uint32_t counter;
+  uint32_t counter2;
+  int flag;
+};
+
+struct SeqSumResult {
+  float sum;       // value of s after the last element consumed
+  int stop_index;  // first i with s > threshold after adding a[i]; -1 if none
+};
+
+// Running state of a sequential sum that a workgroup advances chunk by chunk.
+struct SeqSum {
+  float s;
+  int stop_index;
+  uint32_t parity_buf;  // which fast_total buffer the next fast chunk uses
+};
+
+// Consumes one chunk: lane `tid` owns elements first .. first + R - 1 (global positions, in
+// lane order), given as float bit patterns in bits[] (finite, >= 0; positions >= n must hold 0).
+// Emulates  for each element: s += a; if (s > threshold) stop  in fp32, bit for bit.
+// Fast path: when the whole chunk stays inside the current binade of s, below the threshold
+// and has no half-ulp tie, the chunk's contribution is the plain sum of the lanes' rounded
+// increments (one workgroup reduction).  Otherwise the chunk is redone with the ordered scan:
+// the first lane whose run leaves the binade or crosses the threshold adds its elements
+// natively and the scan restarts behind it.  Must be called by all lanes; returns true when the
+// threshold was crossed (st.stop_index set).
+template <int R>
+__device__ bool seq_sum_chunk(SeqSum& st, const uint32_t (&bits)[R], int first, int n, float threshold,
+                              BlockScratch& sm) {
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  // ---- fast path
+  {
+    const SumState ss = sum_state(st.s);
+    uint32_t inc = 0;
+    bool tie = false;
+    if (ss.kb >= 64) {
+#pragma unroll
+      for (int e = 0; e < R; ++e) inc += fast_inc(bits[e], ss.kb, tie);
+    } else {
+      tie = true;  // tiny running sums (start of a row) always take the ordered path
+    }
+    // saturate at 2^25 (anything >= 2^24 forces the ordered path) so that the sums below
+    // cannot wrap: 64 lanes * 2^25 = 2^31, 16 waves * 2^25 = 2^29
+    constexpr uint32_t kFastSat = 1u << 25;
+    if (tie) inc = kFastSat;
+    inc = inc < kFastSat ? inc : kFastSat;
+    uint32_t wsum = wave_sum_u32(inc);
+    wsum = wsum < kFastSat ? wsum : kFastSat;
+    const uint32_t buf = st.parity_buf;
+    st.parity_buf ^= 1u;
+    if (lane == 0) sm.fast_total[buf][wave] = wsum;
+    __syncthreads();
+    uint32_t total = 0;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) total += sm.fast_total[buf][w];
+    const uint32_t S_new = ss.S + total;
+    if (S_new < (1u << 24)) {
+      const float s_new = sum_value(S_new, ss.kb);
+      if (!(s_new > threshold)) {
+        st.s = s_new;
+        return false;
+      }
+    }
+  }
+  // ---- ordered path
+  int resume = 0;  // lanes below `resume` have been consumed
+  while (true) {
+    const SumState ss = sum_state(st.s);
+    ParityInc mine = {0u, 0u};
+    if (tid >= resume) {
+#pragma unroll
+      for (int e = 0; e < R; ++e) fold_elem(mine, bits[e], ss.kb);
+    }
+    const ParityInc incl_w = wave_scan_inclusive(mine, lane);
+    if (lane == 63) sm.wave_total[wave] = incl_w;
+    __syncthreads();
+    ParityInc prefix = {0u, 0u};
+    ParityInc total = {0u, 0u};
+    for (int w = 0; w < kWaves; ++w) {
+      if (w == wave) prefix = total;
+      total = compose(total, sm.wave_total[w]);
+    }
+    ParityInc excl_w;
+    excl_w.even = __shfl_up(incl_w.even, 1);
+    excl_w.odd = __shfl_up(incl_w.odd, 1);
+    if (lane == 0) excl_w = {0u, 0u};
+    const ParityInc excl = compose(prefix, excl_w);
+    const ParityInc incl = compose(excl, mine);
+    const bool odd = ss.S & 1u;
+    const uint32_t S_excl = ss.S + (odd ? excl.odd : excl.even);
+    const uint32_t S_incl = ss.S + (odd ? incl.odd : incl.even);
+    bool special = S_incl >= (1u << 24);
+    if (!special) special = sum_value(S_incl, ss.kb) > threshold;
+    const uint64_t ballot = __ballot(special);
+    if (lane == 0) sm.first_flag[wave] = ballot ? (wave * 64 + __ffsll(static_cast<long long>(ballot)) - 1) : kBlock;
+    __syncthreads();
+    int j = kBlock;
+    for (int w = 0; w < kWaves; ++w) {
+      const int f = sm.first_flag[w];
+      if (f < kBlock) {
+        j = f;
+        break;
+      }
+    }
+    if (j == kBlock) {
+      st.s = sum_value(ss.S + (odd ? total.odd : total.even), ss.kb);
+      return false;
+    }
+    if (tid == j) {
+      float sj = sum_value(S_excl, ss.kb);
+      int found = -1;
+#pragma unroll
+      for (int e = 0; e < R; ++e) {
+        const int i = first + e;
+        if (i < n && found < 0) {
+          sj = sj + __uint_as_float(bits[e]);
+          if (sj > threshold) found = i;
+        }
+      }
+      sm.bc_sum = sj;
+      sm.bc_found = found;
+    }
+    __syncthreads();
+    st.s = sm.bc_sum;
+    const int found = sm.bc_found;
+    if (found >= 0) {
+      st.stop_index = found;
+      return true;
+    }
+    resume = j + 1;
+  }
+}
+
+// Whole-array form:  s = s0; for (i < n) { s += a(i); if (s > threshold) return {s, i}; }
+// with lane `tid` owning R consecutive elements per chunk.  `a(i)` must return a finite,
+// non-negative float; pass threshold = +inf to sum everything.  Must be called by every lane.
+template <int R, typename Fetch>
+__device__ SeqSumResult seq_sum_block(Fetch a, int n, float s0, float threshold, BlockScratch& sm) {
+  SeqSum st = {s0, -1, 0u};
+  for (int base = 0; base < n; base += kBlock * R) {
+    uint32_t bits[R];
+    const int first = base + static_cast<int>(threadIdx.x) * R;
+#pragma unroll
+    for (int e = 0; e < R; ++e) bits[e] = (first + e < n) ? __float_as_uint(a(first + e)) : 0u;
+    if (seq_sum_chunk<R>(st, bits, first, n, threshold, sm)) break;
+  }
+  __syncthreads();  // callers reuse the scratch right away
+  return {st.s, st.stop_index};
 }
 
 }  // namespace ets

@@ -5,7 +5,7 @@
 //                        (sampler.cpp:58-171, 189-251), one workgroup per row
 //
 // Everything that the reference computes with a sequential fp32 loop (the softmax sum, the
-// nucleus mass, the CDF walks) goes through seq_sum_block(), so the results carry the same
+// nucleus mass, the CDF walks) goes through seq_sum_chunk(), so the results carry the same
 // rounding as the scalar loops they replace.
 #pragma once
 
@@ -29,7 +29,7 @@ struct RowParams {
   int32_t* tokens;    // [batch]
   float* probs;       // [batch, vocab] or null
   RowDebug* debug;    // [batch] or null
-  uint64_t* scratch;  // [batch, scratch_stride] candidate keys
+  uint64_t* scratch;  // [batch, scratch_stride] candidate keys (rows that overflow LDS)
   int64_t scratch_stride;
   int32_t lds_keys;   // power of two: keys that fit in the dynamic LDS buffer
 };
@@ -130,8 +130,13 @@ __device__ void lds_merge_stages(uint64_t* t, int T, int gbase, int k, int j_sta
   }
 }
 
+// Ascending sort of N keys (a power of two) that already sit in LDS.
+__device__ void sort_keys_lds(uint64_t* lds, int N) {
+  for (int k = 2; k <= N; k <<= 1) lds_merge_stages(lds, N, 0, k, k >> 1);
+}
+
 // Ascending sort of keys[0, N), N a power of two, by one workgroup.  `keys` is global memory;
-// `lds` holds T keys (T a power of two).  N <= T sorts entirely in LDS.
+// `lds` holds T keys (T a power of two).  N <= T leaves the sorted keys in LDS as well.
 __device__ void sort_keys_block(uint64_t* keys, int N, uint64_t* lds, int T) {
   const int tid = threadIdx.x;
   if (T > N) T = N;
@@ -180,11 +185,67 @@ __device__ __forceinline__ int pow2_ceil(int n) {
   return p;
 }
 
+// Wave-aggregated append: lanes with `keep` get consecutive slots from *counter.
+__device__ __forceinline__ uint32_t wave_append_slot(bool keep, uint32_t* counter, int lane) {
+  const uint64_t mask = __ballot(keep);
+  uint32_t slot0 = 0;
+  if (mask) {
+    const int leader = __ffsll(static_cast<long long>(mask)) - 1;
+    if (lane == leader) slot0 = atomicAdd(counter, static_cast<uint32_t>(__popcll(mask)));
+    slot0 = __shfl(slot0, leader);
+  }
+  return slot0 + static_cast<uint32_t>(__popcll(mask & ((1ull << lane) - 1ull)));
+}
+
+constexpr int kSelCap = 1024;   // small selection buffer for peaked rows
+constexpr int kHistBins = 512;  // probability histogram used to pre-select the nucleus
+
+struct NucleusScratch {
+  uint64_t sel[kSelCap];
+  float hist_mass[kHistBins];
+  uint32_t hist_count[kHistBins];
+};
+
+// The two CDF walks over candidates sorted by descending probability (sampler.cpp:150-170,
+// :103-119 for top-k).  Returns the sorted position of the draw, or -2 when `n_sorted` entries
+// were not enough to decide where the nucleus ends (top-p only, when more candidates exist).
+template <typename Keys>
+__device__ int draw_from_sorted(Keys keys, int n_sorted, int n_total, bool use_topk, int topk, float topp, float coin,
+                                RowDebug& dbg, BlockScratch& sm) {
+  const float kInf = __uint_as_float(0x7f800000u);
+  auto sorted_prob = [&](int i) -> float { return cand_prob(keys[i]); };
+  int last_idx;
+  float mass;
+  if (use_topk) {
+    last_idx = topk - 1;
+    mass = seq_sum_block<1>(sorted_prob, topk, 0.0f, kInf, sm).sum;
+  } else {
+    const SeqSumResult res = seq_sum_block<1>(sorted_prob, n_sorted, 0.0f, topp, sm);
+    if (res.stop_index < 0 && n_sorted < n_total) return -2;
+    last_idx = res.stop_index >= 0 ? res.stop_index : n_sorted - 1;
+    mass = res.sum;
+  }
+  const float r = coin * mass;  // sampler.cpp:109 / :162
+  const SeqSumResult walk = seq_sum_block<1>(sorted_prob, last_idx + 1, 0.0f, r, sm);
+  const int pos = walk.stop_index >= 0 ? walk.stop_index : last_idx;
+  dbg.last_idx = last_idx;
+  dbg.cumulative = mass;
+  dbg.r = r;
+  dbg.position = pos;
+  return pos;
+}
+
 // ---- the stochastic path: one workgroup per row -------------------------------------------------
-template <int DT>
+// Pass 1 reads the row from HBM: row maximum of x = logit * inv_temperature, plus an estimate of
+// the softmax normaliser (fast exp, any order) that is only used to pre-filter top-p candidates.
+// Pass 2 re-reads the row (L2 / Infinity Cache): exact expf, the sequential sum in index order,
+// and the candidates' (exp, index) pairs into LDS.  Then the coin and the draw.
+template <int DT, bool ALIGNED>
 __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
   extern __shared__ __align__(16) uint64_t lds_keys[];
   __shared__ BlockScratch sm;
+  __shared__ NucleusScratch ns;
+  constexpr int VE = VecElems<DT>::value;
   const int row = blockIdx.x;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -196,38 +257,151 @@ __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
   uint64_t* scratch = p.scratch + static_cast<int64_t>(row) * p.scratch_stride;
   const float kInf = __uint_as_float(0x7f800000u);
   const float kNaN = __uint_as_float(0x7fc00000u);
+  const int cap = p.lds_keys;
 
   if (tid < 32) sm.exp2tab[tid] = kExp2Table[tid];
-
-  // ---- row maximum of x = logit * inv_temperature (sampler.cpp:231-233, 191-197)
-  float m = -kInf;
-  for (int i = tid; i < V; i += kBlock) {
-    const float x = load_elem<DT>(logits, i) * inv;
-    if (x > m) m = x;
+  if (tid == 0) {
+    sm.counter = 0u;
+    sm.counter2 = 0u;
   }
-  m = wave_max_ignoring_nan(m);
-  if (lane == 0) sm.red_f[wave] = m;
-  __syncthreads();
-  m = sm.red_f[0];
-  for (int w = 1; w < kWaves; ++w) m = (sm.red_f[w] > m) ? sm.red_f[w] : m;
+
+  const bool use_topk = p.topk > 0 && p.topk < V;
+  const bool use_mult = !use_topk && (p.topp <= 0.0f || p.topp >= 1.0f);
+  const bool use_topp = !use_topk && !use_mult;
+
+  // ---- pass 1: row maximum (sampler.cpp:231-233, 191-197) and normaliser estimate
+  float m = -kInf;    // lane-local running maximum
+  float est = 0.0f;   // lane-local sum of exp(x - m), fast exp
   {
+    auto visit = [&](float l) {
+      const float x = l * inv;
+      if (x > m) {
+        est = est * __expf(m - x);  // m == -inf: est is still 0
+        m = x;
+      }
+      est += (x > -kInf) ? __expf(x - m) : 0.0f;  // NaN and -inf contribute nothing
+    };
+    if (ALIGNED) {
+      const int nvec = V / VE;
+      const uint4* vec = reinterpret_cast<const uint4*>(logits);
+      int j = tid;
+      for (; j + 3 * kBlock < nvec; j += 4 * kBlock) {
+        const uint4 r0 = vec[j], r1 = vec[j + kBlock], r2 = vec[j + 2 * kBlock], r3 = vec[j + 3 * kBlock];
+        float v[VE];
+        decode_vec<DT>(r0, v);
+#pragma unroll
+        for (int e = 0; e < VE; ++e) visit(v[e]);
+        decode_vec<DT>(r1, v);
+#pragma unroll
+        for (int e = 0; e < VE; ++e) visit(v[e]);
+        decode_vec<DT>(r2, v);
+#pragma unroll
+        for (int e = 0; e < VE; ++e) visit(v[e]);
+        decode_vec<DT>(r3, v);
+#pragma unroll
+        for (int e = 0; e < VE; ++e) visit(v[e]);
+      }
+      for (; j < nvec; j += kBlock) {
+        float v[VE];
+        decode_vec<DT>(vec[j], v);
+#pragma unroll
+        for (int e = 0; e < VE; ++e) visit(v[e]);
+      }
+      for (int i = nvec * VE + tid; i < V; i += kBlock) visit(load_elem<DT>(logits, i));
+    } else {
+      for (int i = tid; i < V; i += kBlock) visit(load_elem<DT>(logits, i));
+    }
+  }
+  float S_est;
+  {
+    const float wm = wave_max_ignoring_nan(m);
+    float scaled = (m > -kInf) ? est * __expf(m - wm) : 0.0f;
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1) scaled += __shfl_xor(scaled, d);
+    if (lane == 0) {
+      sm.red_f[wave] = wm;
+      sm.red_u[wave] = __float_as_uint(scaled);
+    }
+    __syncthreads();
+    m = sm.red_f[0];
+    for (int w = 1; w < kWaves; ++w) m = (sm.red_f[w] > m) ? sm.red_f[w] : m;
+    S_est = 0.0f;
+    for (int w = 0; w < kWaves; ++w) {
+      const float wmax = sm.red_f[w];
+      if (wmax > -kInf) S_est += __uint_as_float(sm.red_u[w]) * __expf(wmax - m);
+    }
     const float x0 = load_elem<DT>(logits, 0) * inv;
     if (x0 != x0) m = x0;  // max_val starts at x[0]; nothing compares greater than NaN
+    __syncthreads();
   }
-  __syncthreads();
 
-  // ---- softmax normaliser: sum of expf(x - max) in index order (sampler.cpp:199-203)
+  // ---- pass 2: softmax normaliser, sequential in index order (sampler.cpp:199-203), and the
+  // top-p candidates.  An entry survives the reference's cutoff when fl(e / S) >= cutoff, which
+  // implies e >= cutoff * S * (1 - 2^-24); S_est stands in for S with 1 % slack and the
+  // inequality is re-checked against the exact S below.
+  const float cutoff = use_topp ? (1.0f - p.topp) / static_cast<float>(V - 1) : 0.0f;  // sampler.cpp:136
+  const float cut_lo = cutoff * S_est * 0.99f;
+  const bool collect = use_topp && (S_est == S_est) && S_est < kInf;
   bool saw_nan = false;
-  auto fetch_e = [&](int i) -> float {
-    const float x = load_elem<DT>(logits, i) * inv;
-    const float e = expf_exact(x - m, sm.exp2tab);
-    if (e != e) {
-      saw_nan = true;
-      return 0.0f;
+  SeqSum st = {0.0f, -1, 0u};
+  {
+    const int chunk = kBlock * VE;
+    uint4 raw = make_uint4(0, 0, 0, 0);
+    const uint4* vec = reinterpret_cast<const uint4*>(logits);
+    if (ALIGNED && tid * VE + VE <= V) raw = vec[tid];
+    for (int base = 0; base < V; base += chunk) {
+      const int first = base + tid * VE;
+      float v[VE];
+      if (ALIGNED && first + VE <= V) {
+        decode_vec<DT>(raw, v);
+      } else {
+#pragma unroll
+        for (int e = 0; e < VE; ++e) v[e] = (first + e < V) ? load_elem<DT>(logits, first + e) : 0.0f;
+      }
+      {
+        const int nfirst = first + chunk;  // prefetch the next chunk's vector
+        if (ALIGNED && nfirst + VE <= V) raw = vec[nfirst / VE];
+      }
+      uint32_t bits[VE];
+      uint32_t cand_mask = 0;
+#pragma unroll
+      for (int e = 0; e < VE; ++e) {
+        const bool valid = first + e < V;
+        const float x = v[e] * inv;
+        float ex = expf_nonpositive(x - m, sm.exp2tab);
+        if (valid && ex != ex) saw_nan = true;
+        ex = (valid && ex == ex) ? ex : 0.0f;
+        bits[e] = __float_as_uint(ex);
+        if (collect && valid && ex >= cut_lo) cand_mask |= 1u << e;
+      }
+      if (collect) {
+        // slots for this lane's candidates: wave prefix over the per-lane counts
+        const uint32_t mine = static_cast<uint32_t>(__popc(cand_mask));
+        uint32_t incl = mine;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+          const uint32_t o = __shfl_up(incl, d);
+          if (lane >= d) incl += o;
+        }
+        const uint32_t wave_total = __shfl(incl, 63);
+        uint32_t slot = 0;
+        if (wave_total) {
+          if (lane == 63) slot = atomicAdd(&sm.counter, wave_total);
+          slot = __shfl(slot, 63) + incl - mine;
+#pragma unroll
+          for (int e = 0; e < VE; ++e) {
+            if (cand_mask & (1u << e)) {
+              if (slot < static_cast<uint32_t>(cap))
+                lds_keys[slot] = (static_cast<uint64_t>(bits[e]) << 32) | static_cast<uint32_t>(first + e);
+              ++slot;
+            }
+          }
+        }
+      }
+      seq_sum_chunk<VE>(st, bits, first, V, kInf, sm);
     }
-    return e;
-  };
-  float S = seq_sum_block(fetch_e, V, 0.0f, kInf, sm).sum;
+  }
+  float S = st.s;
   {
     const uint64_t any = __ballot(saw_nan);
     if (lane == 0) sm.red_u[wave] = any ? 1u : 0u;
@@ -235,35 +409,33 @@ __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
     uint32_t nan_row = 0;
     for (int w = 0; w < kWaves; ++w) nan_row |= sm.red_u[w];
     if (nan_row) S = kNaN;  // one NaN addend poisons the running sum for good
-    __syncthreads();
   }
 
   // ---- one coin per call (sampler.cpp:237, 210-220)
   if (tid == 0) {
-    uint64_t st = p.rng[row];
-    st ^= st >> 12;
-    st ^= st << 25;
-    st ^= st >> 27;
-    p.rng[row] = st;
-    const uint32_t u = static_cast<uint32_t>((st * 0x2545F4914F6CDD1Dull) >> 32);
+    uint64_t rs = p.rng[row];
+    rs ^= rs >> 12;
+    rs ^= rs << 25;
+    rs ^= rs >> 27;
+    p.rng[row] = rs;
+    const uint32_t u = static_cast<uint32_t>((rs * 0x2545F4914F6CDD1Dull) >> 32);
     sm.red_f[0] = static_cast<float>(u >> 8) / 16777216.0f;
   }
   __syncthreads();
   const float coin = sm.red_f[0];
+  const int n_listed = static_cast<int>(sm.counter);
   __syncthreads();
 
   auto prob_at = [&](int i) -> float {
     const float x = load_elem<DT>(logits, i) * inv;
-    return expf_exact(x - m, sm.exp2tab) / S;  // sampler.cpp:205-207: a true division
+    return expf_nonpositive(x - m, sm.exp2tab) / S;  // sampler.cpp:205-207: a true division
   };
   if (probs) {
     for (int i = tid; i < V; i += kBlock) probs[i] = prob_at(i);
   }
 
   RowDebug dbg = {m, S, coin, 0.0f, 0.0f, 0, 0, 0};
-  int32_t token;
-  const bool use_topk = p.topk > 0 && p.topk < V;
-  const bool use_mult = !use_topk && (p.topp <= 0.0f || p.topp >= 1.0f);
+  int32_t token = -1;
 
   if (S != S) {
     // Every probability is NaN.  The multinomial walk never fires and returns the last
@@ -271,72 +443,190 @@ __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
     // reference does not define: report -1.
     token = use_mult ? V - 1 : -1;
   } else if (use_mult) {
-    // ---- sampler.cpp:58-70
-    const SeqSumResult res = seq_sum_block(prob_at, V, 0.0f, coin, sm);
-    token = res.stop_index >= 0 ? res.stop_index : V - 1;
-    dbg.cumulative = res.sum;
+    // ---- sampler.cpp:58-70: first index whose running sum of probabilities exceeds the coin
+    SeqSum walk = {0.0f, -1, 0u};
+    for (int base = 0; base < V; base += kBlock * VE) {
+      const int first = base + tid * VE;
+      float v[VE];
+      load_run<DT, ALIGNED>(logits, first, V, 0.0f, v);
+      uint32_t bits[VE];
+#pragma unroll
+      for (int e = 0; e < VE; ++e) {
+        const float x = v[e] * inv;
+        const float pi = expf_nonpositive(x - m, sm.exp2tab) / S;
+        bits[e] = (first + e < V) ? __float_as_uint(pi) : 0u;
+      }
+      if (seq_sum_chunk<VE>(walk, bits, first, V, coin, sm)) break;
+    }
+    token = walk.stop_index >= 0 ? walk.stop_index : V - 1;
+    dbg.cumulative = walk.s;
     dbg.position = token;
   } else {
-    // ---- candidates: top-p keeps p >= (1 - topp) / (V - 1) (sampler.cpp:136-143); top-k
-    // ranks the whole row (sampler.cpp:87-92)
-    const float cutoff = use_topk ? 0.0f : (1.0f - p.topp) / static_cast<float>(V - 1);
-    if (tid == 0) sm.counter = 0u;
-    __syncthreads();
-    for (int base = 0; base < V; base += kBlock) {
-      const int i = base + tid;
-      float pi = 0.0f;
-      bool keep = false;
-      if (i < V) {
-        pi = prob_at(i);
-        keep = pi >= cutoff;
+    bool done = false;
+    const bool list_ok = collect && n_listed <= cap && cut_lo <= cutoff * S * 0.9999f;
+    if (use_topp && list_ok) {
+      // ---- exact filter p >= cutoff over the listed entries (sampler.cpp:137-143) and a
+      // histogram of probability mass by magnitude to find where the nucleus must end
+      for (int b = tid; b < kHistBins; b += kBlock) {
+        ns.hist_mass[b] = 0.0f;
+        ns.hist_count[b] = 0u;
       }
-      const uint64_t mask = __ballot(keep);
-      if (mask) {
-        uint32_t slot0 = 0;
-        const int leader = __ffsll(static_cast<long long>(mask)) - 1;
-        if (lane == leader) slot0 = atomicAdd(&sm.counter, static_cast<uint32_t>(__popcll(mask)));
-        slot0 = __shfl(slot0, leader);
-        if (keep) {
-          const uint32_t slot = slot0 + static_cast<uint32_t>(__popcll(mask & ((1ull << lane) - 1ull)));
-          scratch[slot] = cand_key(pi, i);
+      __syncthreads();
+      const int bin0 = static_cast<int>(__float_as_uint(cutoff) >> 19);
+      for (int j = tid; j < n_listed; j += kBlock) {
+        const uint64_t ent = lds_keys[j];
+        const float pj = __uint_as_float(static_cast<uint32_t>(ent >> 32)) / S;
+        uint64_t key = ~0ull;
+        if (pj >= cutoff) {
+          key = cand_key(pj, static_cast<int>(static_cast<uint32_t>(ent)));
+          int bin = static_cast<int>(__float_as_uint(pj) >> 19) - bin0;
+          bin = bin < 0 ? 0 : (bin >= kHistBins ? kHistBins - 1 : bin);
+          atomicAdd(&ns.hist_mass[bin], pj);
+          atomicAdd(&ns.hist_count[bin], 1u);
         }
+        lds_keys[j] = key;
+      }
+      __syncthreads();
+      // wave 0: walk the bins from the largest probabilities down until the mass is safely
+      // above topp; everything in those bins is selected for sorting
+      if (wave == 0) {
+        constexpr int per = kHistBins / 64;
+        float mass[per];
+        uint32_t cnt[per];
+        float lane_mass = 0.0f;
+        uint32_t lane_cnt = 0;
+#pragma unroll
+        for (int q = 0; q < per; ++q) {
+          const int bin = kHistBins - 1 - (lane * per + q);
+          mass[q] = ns.hist_mass[bin];
+          cnt[q] = ns.hist_count[bin];
+          lane_mass += mass[q];
+          lane_cnt += cnt[q];
+        }
+        float incl_m = lane_mass;
+        uint32_t incl_c = lane_cnt;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+          const float om = __shfl_up(incl_m, d);
+          const uint32_t oc = __shfl_up(incl_c, d);
+          if (lane >= d) {
+            incl_m += om;
+            incl_c += oc;
+          }
+        }
+        const float target = p.topp * 1.004f + 1e-6f;
+        const uint64_t hit = __ballot(incl_m >= target);
+        const uint32_t total_cnt = __shfl(incl_c, 63);
+        if (hit) {
+          const int hl = __ffsll(static_cast<long long>(hit)) - 1;
+          if (lane == hl) {
+            float run_m = incl_m - lane_mass;
+            uint32_t run_c = incl_c - lane_cnt;
+            int q = 0;
+#pragma unroll
+            for (; q < per; ++q) {
+              run_m += mass[q];
+              run_c += cnt[q];
+              if (run_m >= target) break;
+            }
+            q = q < per ? q : per - 1;
+            sm.flag = kHistBins - 1 - (lane * per + q);
+            sm.counter2 = run_c;
+          }
+        } else if (lane == 0) {
+          sm.flag = 0;
+          sm.counter2 = total_cnt;
+        }
+        if (lane == 0) sm.red_u[0] = total_cnt;
+      }
+      __syncthreads();
+      const int sel_bin = sm.flag;
+      int n_sel = static_cast<int>(sm.counter2);
+      const int n0 = static_cast<int>(sm.red_u[0]);
+      dbg.n_candidates = n0;
+      __syncthreads();
+      if (n0 == 0) {
+        token = -1;  // the reference reads probindex[-1] here
+        done = true;
+      } else {
+        const uint64_t* sorted = nullptr;
+        if (n_sel <= kSelCap) {
+          // peaked row: move the few selected keys to the small buffer and sort them there
+          if (tid == 0) sm.counter = 0u;
+          __syncthreads();
+          for (int base = 0; base < n_listed; base += kBlock) {
+            const int j = base + tid;
+            uint64_t key = ~0ull;
+            if (j < n_listed) key = lds_keys[j];
+            bool keep = false;
+            if (key != ~0ull) {
+              int bin = static_cast<int>(__float_as_uint(cand_prob(key)) >> 19) - bin0;
+              bin = bin < 0 ? 0 : (bin >= kHistBins ? kHistBins - 1 : bin);
+              keep = bin >= sel_bin;
+            }
+            const uint32_t slot = wave_append_slot(keep, &sm.counter, lane);
+            if (keep) ns.sel[slot] = key;
+          }
+          __syncthreads();
+          const int N = pow2_ceil(n_sel);
+          for (int i = n_sel + tid; i < N; i += kBlock) ns.sel[i] = ~0ull;
+          __syncthreads();
+          sort_keys_lds(ns.sel, N);
+          sorted = ns.sel;
+        } else {
+          // broad row: sort the whole list in place (entries that failed the cutoff are ~0)
+          n_sel = n0;
+          const int N = pow2_ceil(n_listed);
+          for (int i = n_listed + tid; i < N; i += kBlock) lds_keys[i] = ~0ull;
+          __syncthreads();
+          sort_keys_lds(lds_keys, N);
+          sorted = lds_keys;
+        }
+        int pos = draw_from_sorted(sorted, n_sel, n0, false, 0, p.topp, coin, dbg, sm);
+        if (pos == -2) {
+          // the pre-selected bins did not reach topp after all: sort every candidate
+          const int N = pow2_ceil(n_listed);
+          for (int i = n_listed + tid; i < N; i += kBlock) lds_keys[i] = ~0ull;
+          __syncthreads();
+          sort_keys_lds(lds_keys, N);
+          sorted = lds_keys;
+          pos = draw_from_sorted(sorted, n0, n0, false, 0, p.topp, coin, dbg, sm);
+        }
+        token = static_cast<int32_t>(static_cast<uint32_t>(sorted[pos]));
+        done = true;
       }
     }
-    __syncthreads();
-    const int n0 = static_cast<int>(sm.counter);
-    dbg.n_candidates = n0;
-    if (n0 == 0) {
-      token = -1;  // the reference reads probindex[-1] here
-    } else {
-      const int N = pow2_ceil(n0);
-      for (int i = n0 + tid; i < N; i += kBlock) scratch[i] = ~0ull;
+    if (!done) {
+      // ---- general path: candidates to global memory, full sort.  Top-p rows whose list does
+      // not fit in LDS, and top-k (which ranks the whole row, sampler.cpp:87-100).
+      const float cut = use_topk ? 0.0f : cutoff;
+      if (tid == 0) sm.counter = 0u;
       __syncthreads();
-      sort_keys_block(scratch, N, lds_keys, p.lds_keys);
-      const uint64_t* keys = scratch;
-      if (N <= p.lds_keys) {  // the sorted tile is still in LDS
-        keys = lds_keys;
+      for (int base = 0; base < V; base += kBlock) {
+        const int i = base + tid;
+        float pi = 0.0f;
+        bool keep = false;
+        if (i < V) {
+          pi = prob_at(i);
+          keep = pi >= cut;
+        }
+        const uint32_t slot = wave_append_slot(keep, &sm.counter, lane);
+        if (keep) scratch[slot] = cand_key(pi, i);
       }
-      auto sorted_prob = [&](int i) -> float { return cand_prob(keys[i]); };
-      int last_idx;
-      float mass;
-      if (use_topk) {
-        // ---- sampler.cpp:103-119: float accumulators over the k best
-        last_idx = p.topk - 1;
-        mass = seq_sum_block(sorted_prob, p.topk, 0.0f, kInf, sm).sum;
+      __syncthreads();
+      const int n0 = static_cast<int>(sm.counter);
+      dbg.n_candidates = n0;
+      if (n0 == 0) {
+        token = -1;
       } else {
-        // ---- sampler.cpp:150-159: first position where the running mass exceeds topp
-        const SeqSumResult res = seq_sum_block(sorted_prob, n0, 0.0f, p.topp, sm);
-        last_idx = res.stop_index >= 0 ? res.stop_index : n0 - 1;
-        mass = res.sum;
+        const int N = pow2_ceil(n0);
+        for (int i = n0 + tid; i < N; i += kBlock) scratch[i] = ~0ull;
+        __syncthreads();
+        sort_keys_block(scratch, N, lds_keys, cap);
+        const uint64_t* keys = (N <= cap) ? lds_keys : scratch;
+        const int pos = draw_from_sorted(keys, n0, n0, use_topk, p.topk, p.topp, coin, dbg, sm);
+        token = static_cast<int32_t>(static_cast<uint32_t>(keys[pos]));
       }
-      const float r = coin * mass;  // sampler.cpp:109 / :162
-      const SeqSumResult walk = seq_sum_block(sorted_prob, last_idx + 1, 0.0f, r, sm);
-      const int pos = walk.stop_index >= 0 ? walk.stop_index : last_idx;
-      token = static_cast<int32_t>(static_cast<uint32_t>(keys[pos]));
-      dbg.last_idx = last_idx;
-      dbg.cumulative = mass;
-      dbg.r = r;
-      dbg.position = pos;
     }
   }
   if (tid == 0) {
@@ -350,7 +640,11 @@ __global__ void __launch_bounds__(256) expf_exact_kernel(const float* x, float* 
   __shared__ uint64_t tab[32];
   if (threadIdx.x < 32) tab[threadIdx.x] = kExp2Table[threadIdx.x];
   __syncthreads();
-  for (int64_t i = blockIdx.x * 256ll + threadIdx.x; i < n; i += 256ll * gridDim.x) y[i] = expf_exact(x[i], tab);
+  for (int64_t i = blockIdx.x * 256ll + threadIdx.x; i < n; i += 256ll * gridDim.x) {
+    const float v = x[i];
+    // non-positive arguments go through the branch-free form the sampler uses
+    y[i] = (v <= 0.0f) ? expf_nonpositive(v, tab) : expf_exact(v, tab);
+  }
 }
 
 // Sequential float sum of an array by one workgroup (test hook for seq_sum_block).
@@ -358,7 +652,7 @@ __global__ void __launch_bounds__(kBlock)
 seq_sum_kernel(const float* a, int32_t n, float s0, float threshold, float* sum_out, int32_t* stop_out) {
   __shared__ BlockScratch sm;
   auto fetch = [&](int i) -> float { return a[i]; };
-  const SeqSumResult r = seq_sum_block(fetch, n, s0, threshold, sm);
+  const SeqSumResult r = seq_sum_block<4>(fetch, n, s0, threshold, sm);
   if (threadIdx.x == 0) {
     *sum_out = r.sum;
     *stop_out = r.stop_index;

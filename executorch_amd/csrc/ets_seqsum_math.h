@@ -90,4 +90,17 @@ ETS_HD void fold_elem(ParityInc& acc, uint32_t abits, int kb) {
   acc.odd = sat_add(acc.odd, inc_odd);
 }
 
+// Order-free shortcut used while a whole chunk stays inside the binade of s (biased exponent
+// kb >= 64) and no element sits on a half-ulp tie: the increment of `abits` is rne(a / ulp(s)),
+// computed with an exact power-of-two scaling in float.  Sets `tie` when the fraction is exactly
+// 1/2 (the caller must then fall back to the ordered scan) and saturates at kSat.
+ETS_HD uint32_t fast_inc(uint32_t abits, int kb, bool& tie) {
+  const float scale = __builtin_bit_cast(float, static_cast<uint32_t>(277 - kb) << 23);  // 2^(150 - kb)
+  float t = __builtin_bit_cast(float, abits) * scale;
+  t = t < 67108864.0f ? t : 67108864.0f;
+  const float r = __builtin_rintf(t);
+  tie = tie || (__builtin_fabsf(t - r) == 0.5f);
+  return static_cast<uint32_t>(r);
+}
+
 }  // namespace ets
