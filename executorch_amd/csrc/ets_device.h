@@ -192,9 +192,9 @@ __device__ __forceinline__ float wave_max_ignoring_nan(float v) {
 // LDS scratch shared by the workgroup-wide primitives.
 struct BlockScratch {
   uint64_t exp2tab[32];
-  ParityInc wave_total[kWaves];
+  ParityInc wave_total[2][kWaves];  // double-buffered, like group_total
   int first_flag[kWaves];
-  uint32_t fast_total[2][kWaves];  // double-buffered: one barrier per fast chunk
+  float group_total[2][kWaves];    // same, for seq_sum_group
   float red_f[kWaves];
   uint32_t red_u[kWaves];
   float bc_sum;
@@ -213,115 +213,147 @@ struct SeqSumResult {
 struct SeqSum {
   float s;
   int stop_index;
-  uint32_t parity_buf;  // which fast_total buffer the next fast chunk uses
+  uint32_t parity_buf;  // which half of the double-buffered LDS totals the next round uses
 };
+
+// Lane-local summary of the order-free shortcut, accumulated in float while the elements are
+// produced: inc = sum of rne(a / ulp(s)) (exact while below 2^24), tie = max |t - rne(t)|, which is
+// 0.5 exactly when some element sits on a half-ulp tie.
+struct FastAcc {
+  float inc;
+  float tie;
+};
+
+// Scale that maps an addend to units of ulp(s); 0 when s is too small for the shortcut.
+__device__ __forceinline__ float fast_scale(float s) {
+  const SumState ss = sum_state(s);
+  return ss.kb >= 64 ? __uint_as_float(static_cast<uint32_t>(277 - ss.kb) << 23) : 0.0f;
+}
+
+__device__ __forceinline__ void fast_fold(FastAcc& a, float e, float scale) {
+  const float t = e * scale;
+  const float r = __builtin_rintf(t);
+  a.inc += r;
+  a.tie = __builtin_fmaxf(a.tie, __builtin_fabsf(t - r));
+}
+
+// Summary of a lane's run of R elements for the running sum s (see ets_seqsum_math.h).
+template <int R>
+__device__ __forceinline__ ParityInc fold_run(const uint32_t (&bits)[R], float s) {
+  const SumState ss = sum_state(s);
+  ParityInc acc = {0u, 0u};
+  if (ss.kb >= 64) {
+    const float scale = __uint_as_float(static_cast<uint32_t>(277 - ss.kb) << 23);  // 2^(150 - kb)
+#pragma unroll
+    for (int e = 0; e < R; ++e) fold_elem_scaled(acc, __uint_as_float(bits[e]), scale);
+  } else {
+#pragma unroll
+    for (int e = 0; e < R; ++e) fold_elem(acc, bits[e], ss.kb);
+  }
+  return acc;
+}
+
+// One wavefront consumes its own 64 runs exactly, starting from running sum s: a wave-level scan
+// of the run summaries finds the first lane whose run leaves the binade of s or crosses the
+// threshold; that lane adds its elements natively and the scan restarts behind it with the new
+// ulp.  No barriers: only this wave takes part.  On return s is the running sum after the wave's
+// last element, or `found` is the position where the threshold was crossed.
+template <int R>
+__device__ void wave_resolve(float& s, int& found, const uint32_t (&bits)[R], int first, int n, float threshold) {
+  const int lane = threadIdx.x & 63;
+  int consumed = 0;  // lanes below this have been consumed
+  found = -1;
+  while (true) {
+    ParityInc mine = {0u, 0u};
+    if (lane >= consumed) mine = fold_run<R>(bits, s);
+    const ParityInc incl = wave_scan_inclusive(mine, lane);
+    ParityInc excl;
+    excl.even = __shfl_up(incl.even, 1);
+    excl.odd = __shfl_up(incl.odd, 1);
+    if (lane == 0) excl = {0u, 0u};
+    const SumState ss = sum_state(s);
+    const bool odd = ss.S & 1u;
+    const uint32_t S_incl = ss.S + (odd ? incl.odd : incl.even);
+    const uint32_t S_excl = ss.S + (odd ? excl.odd : excl.even);
+    bool special = S_incl >= (1u << 24);
+    if (!special) special = sum_value(S_incl, ss.kb) > threshold;
+    const uint64_t ballot = __ballot(special);
+    if (!ballot) {
+      const uint32_t S_end = __shfl(S_incl, 63);
+      s = sum_value(S_end, ss.kb);
+      return;
+    }
+    const int j = __ffsll(static_cast<long long>(ballot)) - 1;
+    float sj = 0.0f;
+    int fj = -1;
+    if (lane == j) {
+      sj = sum_value(S_excl, ss.kb);
+#pragma unroll
+      for (int e = 0; e < R; ++e) {
+        const int i = first + e;
+        if (i < n && fj < 0) {
+          sj = sj + __uint_as_float(bits[e]);
+          if (sj > threshold) fj = i;
+        }
+      }
+    }
+    s = __shfl(sj, j);
+    fj = __shfl(fj, j);
+    if (fj >= 0) {
+      found = fj;
+      return;
+    }
+    consumed = j + 1;
+  }
+}
 
 // Consumes one chunk: lane `tid` owns elements first .. first + R - 1 (global positions, in
 // lane order), given as float bit patterns in bits[] (finite, >= 0; positions >= n must hold 0).
 // Emulates  for each element: s += a; if (s > threshold) stop  in fp32, bit for bit.
-// Fast path: when the whole chunk stays inside the current binade of s, below the threshold
-// and has no half-ulp tie, the chunk's contribution is the plain sum of the lanes' rounded
-// increments (one workgroup reduction).  Otherwise the chunk is redone with the ordered scan:
-// the first lane whose run leaves the binade or crosses the threshold adds its elements
-// natively and the scan restarts behind it.  Must be called by all lanes; returns true when the
-// threshold was crossed (st.stop_index set).
+// Each round composes the waves' summaries in order and finds the first wave in which the sum
+// leaves its binade or crosses the threshold; the waves in front of it are committed, that wave
+// resolves its own 512 or so elements with wave_resolve(), and the next round restarts behind it
+// with the new ulp.  Two barriers per round, one when nothing happens.  Must be called by all
+// lanes; returns true when the threshold was crossed (st.stop_index set).
 template <int R>
 __device__ bool seq_sum_chunk(SeqSum& st, const uint32_t (&bits)[R], int first, int n, float threshold,
                               BlockScratch& sm) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  // ---- fast path
-  {
-    const SumState ss = sum_state(st.s);
-    uint32_t inc = 0;
-    bool tie = false;
-    if (ss.kb >= 64) {
-#pragma unroll
-      for (int e = 0; e < R; ++e) inc += fast_inc(bits[e], ss.kb, tie);
-    } else {
-      tie = true;  // tiny running sums (start of a row) always take the ordered path
-    }
-    // saturate at 2^25 (anything >= 2^24 forces the ordered path) so that the sums below
-    // cannot wrap: 64 lanes * 2^25 = 2^31, 16 waves * 2^25 = 2^29
-    constexpr uint32_t kFastSat = 1u << 25;
-    if (tie) inc = kFastSat;
-    inc = inc < kFastSat ? inc : kFastSat;
-    uint32_t wsum = wave_sum_u32(inc);
-    wsum = wsum < kFastSat ? wsum : kFastSat;
+  int resume_wave = 0;  // waves below this have been consumed
+  while (true) {
+    ParityInc mine = {0u, 0u};
+    if (wave >= resume_wave) mine = fold_run<R>(bits, st.s);
+    const ParityInc incl = wave_scan_inclusive(mine, lane);
     const uint32_t buf = st.parity_buf;
     st.parity_buf ^= 1u;
-    if (lane == 0) sm.fast_total[buf][wave] = wsum;
+    if (lane == 63) sm.wave_total[buf][wave] = incl;
     __syncthreads();
-    uint32_t total = 0;
-#pragma unroll
-    for (int w = 0; w < kWaves; ++w) total += sm.fast_total[buf][w];
-    const uint32_t S_new = ss.S + total;
-    if (S_new < (1u << 24)) {
-      const float s_new = sum_value(S_new, ss.kb);
-      if (!(s_new > threshold)) {
-        st.s = s_new;
-        return false;
-      }
-    }
-  }
-  // ---- ordered path
-  int resume = 0;  // lanes below `resume` have been consumed
-  while (true) {
+    // every wave redoes the small scan over the 16 wave totals in its first 16 lanes
+    ParityInc wt = {0u, 0u};
+    if (lane < kWaves) wt = sm.wave_total[buf][lane];
+    const ParityInc upto = wave_scan_inclusive(wt, lane);
     const SumState ss = sum_state(st.s);
-    ParityInc mine = {0u, 0u};
-    if (tid >= resume) {
-#pragma unroll
-      for (int e = 0; e < R; ++e) fold_elem(mine, bits[e], ss.kb);
-    }
-    const ParityInc incl_w = wave_scan_inclusive(mine, lane);
-    if (lane == 63) sm.wave_total[wave] = incl_w;
-    __syncthreads();
-    ParityInc prefix = {0u, 0u};
-    ParityInc total = {0u, 0u};
-    for (int w = 0; w < kWaves; ++w) {
-      if (w == wave) prefix = total;
-      total = compose(total, sm.wave_total[w]);
-    }
-    ParityInc excl_w;
-    excl_w.even = __shfl_up(incl_w.even, 1);
-    excl_w.odd = __shfl_up(incl_w.odd, 1);
-    if (lane == 0) excl_w = {0u, 0u};
-    const ParityInc excl = compose(prefix, excl_w);
-    const ParityInc incl = compose(excl, mine);
     const bool odd = ss.S & 1u;
-    const uint32_t S_excl = ss.S + (odd ? excl.odd : excl.even);
-    const uint32_t S_incl = ss.S + (odd ? incl.odd : incl.even);
-    bool special = S_incl >= (1u << 24);
-    if (!special) special = sum_value(S_incl, ss.kb) > threshold;
-    const uint64_t ballot = __ballot(special);
-    if (lane == 0) sm.first_flag[wave] = ballot ? (wave * 64 + __ffsll(static_cast<long long>(ballot)) - 1) : kBlock;
-    __syncthreads();
-    int j = kBlock;
-    for (int w = 0; w < kWaves; ++w) {
-      const int f = sm.first_flag[w];
-      if (f < kBlock) {
-        j = f;
-        break;
-      }
-    }
-    if (j == kBlock) {
-      st.s = sum_value(ss.S + (odd ? total.odd : total.even), ss.kb);
+    const uint32_t S_upto = ss.S + (odd ? upto.odd : upto.even);
+    bool event = S_upto >= (1u << 24);
+    if (!event) event = sum_value(S_upto, ss.kb) > threshold;
+    const uint64_t ballot = __ballot(event && lane < kWaves);
+    if (!ballot) {
+      st.s = sum_value(__shfl(S_upto, kWaves - 1), ss.kb);
       return false;
     }
-    if (tid == j) {
-      float sj = sum_value(S_excl, ss.kb);
+    const int wstar = __ffsll(static_cast<long long>(ballot)) - 1;
+    if (wave == wstar) {
+      const uint32_t S_front = wstar ? __shfl(S_upto, wstar - 1) : ss.S;
+      float s = sum_value(S_front, ss.kb);
       int found = -1;
-#pragma unroll
-      for (int e = 0; e < R; ++e) {
-        const int i = first + e;
-        if (i < n && found < 0) {
-          sj = sj + __uint_as_float(bits[e]);
-          if (sj > threshold) found = i;
-        }
+      wave_resolve<R>(s, found, bits, first, n, threshold);
+      if (lane == 0) {
+        sm.bc_sum = s;
+        sm.bc_found = found;
       }
-      sm.bc_sum = sj;
-      sm.bc_found = found;
     }
     __syncthreads();
     st.s = sm.bc_sum;
@@ -330,8 +362,52 @@ __device__ bool seq_sum_chunk(SeqSum& st, const uint32_t (&bits)[R], int first, 
       st.stop_index = found;
       return true;
     }
-    resume = j + 1;
+    resume_wave = wstar + 1;
   }
+}
+
+// ---- several chunks per barrier -------------------------------------------------------------------
+// Consumes U chunks (chunk u: lane `tid` owns elements first[u] .. first[u] + R - 1, chunks in
+// increasing position) with ONE barrier when all of them stay inside the binade of s, below the
+// threshold and free of ties; `acc` must have been folded over the same elements with
+// fast_scale(st.s).  Otherwise the chunks go through seq_sum_chunk one after the other.
+template <int U, int R>
+__device__ bool seq_sum_group(SeqSum& st, const uint32_t (&bits)[U][R], FastAcc acc, float scale,
+                              const int (&first)[U], int n, float threshold, BlockScratch& sm) {
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  float inc = acc.inc;
+  float tie = acc.tie;
+#pragma unroll
+  for (int d = 32; d > 0; d >>= 1) {
+    inc += __shfl_xor(inc, d);
+    tie = __builtin_fmaxf(tie, __shfl_xor(tie, d));
+  }
+  const float kBig = 67108864.0f;  // 2^26: "take the ordered path"
+  if (tie == 0.5f || scale == 0.0f || !(inc < kBig)) inc = kBig;
+  const uint32_t buf = st.parity_buf;
+  st.parity_buf ^= 1u;
+  if (lane == 0) sm.group_total[buf][wave] = inc;
+  __syncthreads();
+  float total = 0.0f;
+#pragma unroll
+  for (int w = 0; w < kWaves; ++w) total += sm.group_total[buf][w];
+  if (total < 16777216.0f) {
+    const SumState ss = sum_state(st.s);
+    const uint32_t S_new = ss.S + static_cast<uint32_t>(total);
+    if (S_new < (1u << 24)) {
+      const float s_new = sum_value(S_new, ss.kb);
+      if (!(s_new > threshold)) {
+        st.s = s_new;
+        return false;
+      }
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    if (seq_sum_chunk<R>(st, bits[u], first[u], n, threshold, sm)) return true;
+  }
+  return false;
 }
 
 // Whole-array form:  s = s0; for (i < n) { s += a(i); if (s > threshold) return {s, i}; }

@@ -197,14 +197,30 @@ __device__ __forceinline__ uint32_t wave_append_slot(bool keep, uint32_t* counte
   return slot0 + static_cast<uint32_t>(__popcll(mask & ((1ull << lane) - 1ull)));
 }
 
-constexpr int kSelCap = 1024;   // small selection buffer for peaked rows
-constexpr int kHistBins = 512;  // probability histogram used to pre-select the nucleus
+// Single-lane form of the CDF walk for short lists (the nucleus of a peaked row is a handful of
+// entries; a workgroup-wide scan would spend its time in barriers).
+template <typename Keys>
+__device__ SeqSumResult seq_sum_small(Keys keys, int n, float threshold, BlockScratch& sm) {
+  if (threadIdx.x == 0) {
+    float s = 0.0f;
+    int found = -1;
+    for (int i = 0; i < n; ++i) {
+      s = s + cand_prob(keys[i]);
+      if (s > threshold) {
+        found = i;
+        break;
+      }
+    }
+    sm.bc_sum = s;
+    sm.bc_found = found;
+  }
+  __syncthreads();
+  const SeqSumResult r = {sm.bc_sum, sm.bc_found};
+  __syncthreads();
+  return r;
+}
 
-struct NucleusScratch {
-  uint64_t sel[kSelCap];
-  float hist_mass[kHistBins];
-  uint32_t hist_count[kHistBins];
-};
+constexpr int kSmallWalk = 192;
 
 // The two CDF walks over candidates sorted by descending probability (sampler.cpp:150-170,
 // :103-119 for top-k).  Returns the sorted position of the draw, or -2 when `n_sorted` entries
@@ -218,15 +234,27 @@ __device__ int draw_from_sorted(Keys keys, int n_sorted, int n_total, bool use_t
   float mass;
   if (use_topk) {
     last_idx = topk - 1;
-    mass = seq_sum_block<1>(sorted_prob, topk, 0.0f, kInf, sm).sum;
+    mass = (topk <= kSmallWalk) ? seq_sum_small(keys, topk, kInf, sm).sum
+                                : seq_sum_block<1>(sorted_prob, topk, 0.0f, kInf, sm).sum;
   } else {
-    const SeqSumResult res = seq_sum_block<1>(sorted_prob, n_sorted, 0.0f, topp, sm);
+    // a short prefix usually holds the whole nucleus
+    SeqSumResult res = {0.0f, -1};
+    bool decided = false;
+    if (n_sorted <= kSmallWalk) {
+      res = seq_sum_small(keys, n_sorted, topp, sm);
+      decided = true;
+    } else {
+      res = seq_sum_small(keys, kSmallWalk, topp, sm);
+      decided = res.stop_index >= 0;
+    }
+    if (!decided) res = seq_sum_block<1>(sorted_prob, n_sorted, 0.0f, topp, sm);
     if (res.stop_index < 0 && n_sorted < n_total) return -2;
     last_idx = res.stop_index >= 0 ? res.stop_index : n_sorted - 1;
     mass = res.sum;
   }
   const float r = coin * mass;  // sampler.cpp:109 / :162
-  const SeqSumResult walk = seq_sum_block<1>(sorted_prob, last_idx + 1, 0.0f, r, sm);
+  const SeqSumResult walk = (last_idx < kSmallWalk) ? seq_sum_small(keys, last_idx + 1, r, sm)
+                                                    : seq_sum_block<1>(sorted_prob, last_idx + 1, 0.0f, r, sm);
   const int pos = walk.stop_index >= 0 ? walk.stop_index : last_idx;
   dbg.last_idx = last_idx;
   dbg.cumulative = mass;
@@ -235,11 +263,347 @@ __device__ int draw_from_sorted(Keys keys, int n_sorted, int n_total, bool use_t
   return pos;
 }
 
+// What one pass over the row accumulates.
+//   kScanSum   e_i = expf(x_i - max), sequential sum; optionally lists top-p candidates
+//   kScanWalk  p_i = e_i / S, sequential sum until it exceeds the coin (multinomial draw)
+constexpr int kScanSum = 0, kScanWalk = 1;
+
+struct ScanArgs {
+  const char* logits;
+  int V;
+  float inv;
+  float m;          // row maximum of x
+  float S;          // kScanWalk: normaliser
+  float threshold;  // kScanWalk: the coin; kScanSum: +inf
+  float cutoff;     // kScanSum with listing: the reference's top-p cutoff
+  uint64_t* list;   // kScanSum with listing: (exp bits << 32 | index) of possible candidates
+};
+
+constexpr int kGroup = 2;  // 16-byte vectors per lane between two barriers of the main loop
+
+// One pass over the row in index order.  The main loop handles kGroup * kBlock full vectors per
+// iteration without bounds checks (loads for the next iteration are issued before the current one
+// is processed); the remainder goes through a bounds-checked loop.  Returns true if the threshold
+// was crossed.  With LIST, entries whose exp could still reach the cutoff once the normaliser is
+// known (exp >= cutoff * max(1, running sum), with slack) are appended to args.list and counted
+// in sm.counter.
+template <int DT, bool ALIGNED, int MODE, bool LIST>
+__device__ __forceinline__ bool scan_row(const ScanArgs& a, SeqSum& st, BlockScratch& sm) {
+  constexpr int VE = VecElems<DT>::value;
+  const int tid = threadIdx.x;
+  const int V = a.V;
+  const float inv = a.inv, m = a.m;
+  const uint64_t* tab = sm.exp2tab;
+  int done_elems = 0;
+  auto value_of = [&](float l) -> float {
+    const float x = l * inv;
+    float d = x - m;
+    d = __builtin_fmaxf(d, -104.0f);  // expf is 0 below ln(2^-150); the core gives 0 at -104 too
+    const float e = expf_core(d, tab);
+    return MODE == kScanWalk ? e / a.S : e;  // sampler.cpp:205-207: a true division
+  };
+  if (ALIGNED) {
+    const int nvec = V / VE;
+    const uint4* vec = reinterpret_cast<const uint4*>(a.logits);
+    constexpr int per_iter = kBlock * kGroup;
+    uint4 raw[kGroup];
+    if (per_iter <= nvec) {
+#pragma unroll
+      for (int u = 0; u < kGroup; ++u) raw[u] = vec[u * kBlock + tid];
+    }
+    int vbase = 0;
+    for (; vbase + per_iter <= nvec; vbase += per_iter) {
+      const float scale = fast_scale(st.s);
+      const float cut_lo = LIST ? a.cutoff * __builtin_fmaxf(st.s, 1.0f) * 0.999f : 0.0f;
+      FastAcc acc = {0.0f, 0.0f};
+      uint32_t bits[kGroup][VE];
+      int first[kGroup];
+      const bool more = vbase + 2 * per_iter <= nvec;
+#pragma unroll
+      for (int u = 0; u < kGroup; ++u) {
+        float v[VE];
+        decode_vec<DT>(raw[u], v);
+        if (more) raw[u] = vec[vbase + per_iter + u * kBlock + tid];
+        first[u] = (vbase + u * kBlock + tid) * VE;
+        uint32_t cmask = 0;
+#pragma unroll
+        for (int e = 0; e < VE; ++e) {
+          const float val = value_of(v[e]);
+          bits[u][e] = __float_as_uint(val);
+          fast_fold(acc, val, scale);
+          if (LIST && val >= cut_lo) cmask |= 1u << e;
+        }
+        if (LIST) {
+          while (cmask) {
+            const int e = __ffs(static_cast<int>(cmask)) - 1;
+            cmask &= cmask - 1u;
+            const uint32_t slot = atomicAdd(&sm.counter, 1u);
+            uint32_t eb = bits[u][0];
+#pragma unroll
+            for (int q = 1; q < VE; ++q) eb = (e == q) ? bits[u][q] : eb;
+            a.list[slot] = (static_cast<uint64_t>(eb) << 32) | static_cast<uint32_t>(first[u] + e);
+          }
+        }
+      }
+      if (seq_sum_group<kGroup, VE>(st, bits, acc, scale, first, V, a.threshold, sm)) return true;
+    }
+    done_elems = vbase * VE;
+  }
+  // remainder (and rows whose base or pitch is not 16-byte aligned)
+  for (int base = done_elems; base < V; base += kBlock * VE) {
+    const int first = base + tid * VE;
+    const float cut_lo = LIST ? a.cutoff * __builtin_fmaxf(st.s, 1.0f) * 0.999f : 0.0f;
+    uint32_t bits[VE];
+#pragma unroll
+    for (int e = 0; e < VE; ++e) {
+      const int i = first + e;
+      float val = 0.0f;
+      if (i < V) {
+        val = value_of(load_elem<DT>(a.logits, i));
+        if (LIST && val >= cut_lo) {
+          const uint32_t slot = atomicAdd(&sm.counter, 1u);
+          a.list[slot] = (static_cast<uint64_t>(__float_as_uint(val)) << 32) | static_cast<uint32_t>(i);
+        }
+      }
+      bits[e] = __float_as_uint(val);
+    }
+    if (seq_sum_chunk<VE>(st, bits, first, V, a.threshold, sm)) return true;
+  }
+  return false;
+}
+
+constexpr int kSelCap = 1024;   // small selection buffer for peaked rows
+constexpr int kHistBins = 512;  // probability histogram used to pre-select the nucleus
+
+struct NucleusScratch {
+  uint64_t sel[kSelCap];
+  float hist_mass[kHistBins];
+  uint32_t hist_count[kHistBins];
+};
+
+__device__ __forceinline__ int prob_bin(float p, int bin0) {
+  int bin = static_cast<int>(__float_as_uint(p) >> 19) - bin0;
+  return bin < 0 ? 0 : (bin >= kHistBins ? kHistBins - 1 : bin);
+}
+
+// General path: every candidate (top-p: p >= cutoff; top-k: the whole row, sampler.cpp:87-100)
+// goes to global memory as a sort key and the full list is sorted.  Used by top-k and by top-p
+// rows whose candidates do not fit in LDS.
+template <int DT>
+__device__ int32_t draw_general(const char* logits, int V, float inv, float m, float S, bool use_topk,
+                                             int topk, float topp, float cutoff, float coin, uint64_t* scratch,
+                                             uint64_t* lds_keys, int cap, RowDebug& dbg, BlockScratch& sm) {
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const float cut = use_topk ? 0.0f : cutoff;
+  if (tid == 0) sm.counter = 0u;
+  __syncthreads();
+  for (int base = 0; base < V; base += kBlock) {
+    const int i = base + tid;
+    float pi = 0.0f;
+    bool keep = false;
+    if (i < V) {
+      const float x = load_elem<DT>(logits, i) * inv;
+      pi = expf_nonpositive(x - m, sm.exp2tab) / S;
+      keep = pi >= cut;
+    }
+    const uint32_t slot = wave_append_slot(keep, &sm.counter, lane);
+    if (keep) scratch[slot] = cand_key(pi, i);
+  }
+  __syncthreads();
+  const int n0 = static_cast<int>(sm.counter);
+  dbg.n_candidates = n0;
+  if (n0 == 0) return -1;  // the reference reads probindex[-1] here
+  const int N = pow2_ceil(n0);
+  for (int i = n0 + tid; i < N; i += kBlock) scratch[i] = ~0ull;
+  __syncthreads();
+  sort_keys_block(scratch, N, lds_keys, cap);
+  const uint64_t* keys = (N <= cap) ? lds_keys : scratch;
+  const int pos = draw_from_sorted(keys, n0, n0, use_topk, topk, topp, coin, dbg, sm);
+  return static_cast<int32_t>(static_cast<uint32_t>(keys[pos]));
+}
+
+// Top-p draw from the listed possible candidates (sampler.cpp:122-171).  Returns false when the
+// true candidates do not fit in LDS (the caller then takes the general path).
+__device__ bool draw_topp_listed(const uint64_t* list, int n_listed, float S, float cutoff, float topp,
+                                              float coin, uint64_t* scratch, uint64_t* lds_keys, int cap,
+                                              RowDebug& dbg, int32_t& token, BlockScratch& sm, NucleusScratch& ns) {
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  // ---- exact filter p >= cutoff (sampler.cpp:137-143) into LDS, and a histogram of probability
+  // mass by magnitude that tells where the nucleus must end
+  for (int b = tid; b < kHistBins; b += kBlock) {
+    ns.hist_mass[b] = 0.0f;
+    ns.hist_count[b] = 0u;
+  }
+  if (tid == 0) sm.counter2 = 0u;
+  __syncthreads();
+  const int bin0 = static_cast<int>(__float_as_uint(cutoff) >> 19);
+  for (int base = 0; base < n_listed; base += kBlock) {
+    const int j = base + tid;
+    bool keep = false;
+    float pj = 0.0f;
+    uint32_t idx = 0;
+    if (j < n_listed) {
+      const uint64_t ent = list[j];
+      pj = __uint_as_float(static_cast<uint32_t>(ent >> 32)) / S;
+      idx = static_cast<uint32_t>(ent);
+      keep = pj >= cutoff;
+    }
+    const uint32_t slot = wave_append_slot(keep, &sm.counter2, lane);
+    if (keep) {
+      if (slot < static_cast<uint32_t>(cap)) lds_keys[slot] = cand_key(pj, static_cast<int>(idx));
+      const int bin = prob_bin(pj, bin0);
+      atomicAdd(&ns.hist_mass[bin], pj);
+      atomicAdd(&ns.hist_count[bin], 1u);
+    }
+  }
+  __syncthreads();
+  const int n0 = static_cast<int>(sm.counter2);
+  dbg.n_candidates = n0;
+  if (n0 > cap) return false;
+  if (n0 == 0) {
+    token = -1;  // the reference reads probindex[-1] here
+    return true;
+  }
+  // ---- wave 0 walks the bins from the largest probabilities down until the mass is safely above
+  // topp; everything in those bins is selected for sorting
+  if (wave == 0) {
+    constexpr int per = kHistBins / 64;
+    float mass[per];
+    uint32_t cnt[per];
+    float lane_mass = 0.0f;
+    uint32_t lane_cnt = 0;
+#pragma unroll
+    for (int q = 0; q < per; ++q) {
+      const int bin = kHistBins - 1 - (lane * per + q);
+      mass[q] = ns.hist_mass[bin];
+      cnt[q] = ns.hist_count[bin];
+      lane_mass += mass[q];
+      lane_cnt += cnt[q];
+    }
+    float incl_m = lane_mass;
+    uint32_t incl_c = lane_cnt;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const float om = __shfl_up(incl_m, d);
+      const uint32_t oc = __shfl_up(incl_c, d);
+      if (lane >= d) {
+        incl_m += om;
+        incl_c += oc;
+      }
+    }
+    const float target = topp * 1.004f + 1e-6f;
+    const uint64_t hit = __ballot(incl_m >= target);
+    if (hit) {
+      const int hl = __ffsll(static_cast<long long>(hit)) - 1;
+      if (lane == hl) {
+        float run_m = incl_m - lane_mass;
+        uint32_t run_c = incl_c - lane_cnt;
+        int q_hit = per - 1;
+        uint32_t c_hit = incl_c;
+        bool got = false;
+#pragma unroll
+        for (int q = 0; q < per; ++q) {
+          run_m += mass[q];
+          run_c += cnt[q];
+          if (!got && run_m >= target) {
+            got = true;
+            q_hit = q;
+            c_hit = run_c;
+          }
+        }
+        sm.flag = kHistBins - 1 - (lane * per + q_hit);
+        sm.counter = c_hit;
+      }
+    } else if (lane == 0) {
+      sm.flag = 0;
+      sm.counter = static_cast<uint32_t>(n0);
+    }
+  }
+  __syncthreads();
+  const int sel_bin = sm.flag;
+  int n_sel = static_cast<int>(sm.counter);
+  __syncthreads();
+  const uint64_t* sorted = nullptr;
+  if (n_sel < n0) {
+    // compact the selected keys: into the small buffer when they fit, else through global memory
+    // and back to the front of the LDS list
+    uint64_t* dst = (n_sel <= kSelCap) ? ns.sel : scratch;
+    if (tid == 0) sm.counter2 = 0u;
+    __syncthreads();
+    for (int base = 0; base < n0; base += kBlock) {
+      const int j = base + tid;
+      uint64_t key = 0;
+      bool keep = false;
+      if (j < n0) {
+        key = lds_keys[j];
+        keep = prob_bin(cand_prob(key), bin0) >= sel_bin;
+      }
+      const uint32_t slot = wave_append_slot(keep, &sm.counter2, lane);
+      if (keep) dst[slot] = key;
+    }
+    __syncthreads();
+    const int N = pow2_ceil(n_sel);
+    if (n_sel <= kSelCap) {
+      for (int i = n_sel + tid; i < N; i += kBlock) ns.sel[i] = ~0ull;
+      __syncthreads();
+      sort_keys_lds(ns.sel, N);
+      sorted = ns.sel;
+    } else {
+      // the unselected keys are still needed if the selection turns out too small: park them
+      // behind the selected ones in global memory before LDS is overwritten
+      for (int base = 0; base < n0; base += kBlock) {
+        const int j = base + tid;
+        uint64_t key = 0;
+        bool rest = false;
+        if (j < n0) {
+          key = lds_keys[j];
+          rest = prob_bin(cand_prob(key), bin0) < sel_bin;
+        }
+        const uint32_t slot = wave_append_slot(rest, &sm.counter2, lane);
+        if (rest) scratch[slot] = key;
+      }
+      __syncthreads();
+      // selected keys to the front of the LDS list, padded to a power of two with ~0 (the rest
+      // stays parked in global memory)
+      for (int i = tid; i < n_sel; i += kBlock) lds_keys[i] = scratch[i];
+      for (int i = n_sel + tid; i < N; i += kBlock) lds_keys[i] = ~0ull;
+      __syncthreads();
+      sort_keys_lds(lds_keys, N);
+      sorted = lds_keys;
+    }
+  } else {
+    n_sel = n0;
+    const int N = pow2_ceil(n0);
+    for (int i = n0 + tid; i < N; i += kBlock) lds_keys[i] = ~0ull;
+    __syncthreads();
+    sort_keys_lds(lds_keys, N);
+    sorted = lds_keys;
+  }
+  int pos = draw_from_sorted(sorted, n_sel, n0, false, 0, topp, coin, dbg, sm);
+  if (pos == -2) {
+    // the pre-selected bins did not reach topp after all: sort every candidate
+    if (n_sel > kSelCap) {
+      for (int i = tid; i < n0; i += kBlock) lds_keys[i] = scratch[i];  // selected + parked rest
+      __syncthreads();
+    }
+    const int N = pow2_ceil(n0);
+    for (int i = n0 + tid; i < N; i += kBlock) lds_keys[i] = ~0ull;
+    __syncthreads();
+    sort_keys_lds(lds_keys, N);
+    sorted = lds_keys;
+    pos = draw_from_sorted(sorted, n0, n0, false, 0, topp, coin, dbg, sm);
+  }
+  token = static_cast<int32_t>(static_cast<uint32_t>(sorted[pos]));
+  return true;
+}
+
 // ---- the stochastic path: one workgroup per row -------------------------------------------------
-// Pass 1 reads the row from HBM: row maximum of x = logit * inv_temperature, plus an estimate of
-// the softmax normaliser (fast exp, any order) that is only used to pre-filter top-p candidates.
-// Pass 2 re-reads the row (L2 / Infinity Cache): exact expf, the sequential sum in index order,
-// and the candidates' (exp, index) pairs into LDS.  Then the coin and the draw.
+// Pass 1 reads the row from HBM: maximum of x = logit * inv_temperature and whether any x is NaN.
+// Pass 2 re-reads it (L2 / Infinity Cache): exact expf, the sequential sum in index order, and
+// the list of possible top-p candidates.  Then the coin and the draw.
 template <int DT, bool ALIGNED>
 __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
   extern __shared__ __align__(16) uint64_t lds_keys[];
@@ -253,33 +617,25 @@ __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
   const int V = p.vocab;
   const float inv = p.inv_temperature;
   const char* logits = static_cast<const char*>(p.logits) + static_cast<int64_t>(row) * p.row_stride * ElemSize<DT>::value;
-  float* probs = p.probs ? p.probs + static_cast<int64_t>(row) * V : nullptr;
   uint64_t* scratch = p.scratch + static_cast<int64_t>(row) * p.scratch_stride;
   const float kInf = __uint_as_float(0x7f800000u);
   const float kNaN = __uint_as_float(0x7fc00000u);
-  const int cap = p.lds_keys;
 
   if (tid < 32) sm.exp2tab[tid] = kExp2Table[tid];
-  if (tid == 0) {
-    sm.counter = 0u;
-    sm.counter2 = 0u;
-  }
+  if (tid == 0) sm.counter = 0u;
 
   const bool use_topk = p.topk > 0 && p.topk < V;
   const bool use_mult = !use_topk && (p.topp <= 0.0f || p.topp >= 1.0f);
   const bool use_topp = !use_topk && !use_mult;
 
-  // ---- pass 1: row maximum (sampler.cpp:231-233, 191-197) and normaliser estimate
-  float m = -kInf;    // lane-local running maximum
-  float est = 0.0f;   // lane-local sum of exp(x - m), fast exp
+  // ---- pass 1: row maximum (sampler.cpp:231-233, 191-197)
+  float m = -kInf;
+  bool any_nan = false;
   {
     auto visit = [&](float l) {
       const float x = l * inv;
-      if (x > m) {
-        est = est * __expf(m - x);  // m == -inf: est is still 0
-        m = x;
-      }
-      est += (x > -kInf) ? __expf(x - m) : 0.0f;  // NaN and -inf contribute nothing
+      m = __builtin_fmaxf(m, x);  // ignores NaN, like `if (x > max)`
+      any_nan = any_nan || (x != x);
     };
     if (ALIGNED) {
       const int nvec = V / VE;
@@ -312,103 +668,41 @@ __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
       for (int i = tid; i < V; i += kBlock) visit(load_elem<DT>(logits, i));
     }
   }
-  float S_est;
+  bool row_nan;
   {
-    const float wm = wave_max_ignoring_nan(m);
-    float scaled = (m > -kInf) ? est * __expf(m - wm) : 0.0f;
-#pragma unroll
-    for (int d = 32; d > 0; d >>= 1) scaled += __shfl_xor(scaled, d);
+    m = wave_max_ignoring_nan(m);
+    const uint64_t nan_ballot = __ballot(any_nan);
     if (lane == 0) {
-      sm.red_f[wave] = wm;
-      sm.red_u[wave] = __float_as_uint(scaled);
+      sm.red_f[wave] = m;
+      sm.red_u[wave] = nan_ballot ? 1u : 0u;
     }
     __syncthreads();
     m = sm.red_f[0];
-    for (int w = 1; w < kWaves; ++w) m = (sm.red_f[w] > m) ? sm.red_f[w] : m;
-    S_est = 0.0f;
-    for (int w = 0; w < kWaves; ++w) {
-      const float wmax = sm.red_f[w];
-      if (wmax > -kInf) S_est += __uint_as_float(sm.red_u[w]) * __expf(wmax - m);
+    uint32_t nan_any = sm.red_u[0];
+    for (int w = 1; w < kWaves; ++w) {
+      m = (sm.red_f[w] > m) ? sm.red_f[w] : m;
+      nan_any |= sm.red_u[w];
     }
     const float x0 = load_elem<DT>(logits, 0) * inv;
     if (x0 != x0) m = x0;  // max_val starts at x[0]; nothing compares greater than NaN
+    // expf(x - m) is NaN for some entry exactly when an x is NaN or m is not finite (then the
+    // maximal entry itself gives inf - inf); one NaN addend poisons the running sum for good
+    row_nan = nan_any != 0u || !(m > -kInf && m < kInf);
     __syncthreads();
   }
 
-  // ---- pass 2: softmax normaliser, sequential in index order (sampler.cpp:199-203), and the
-  // top-p candidates.  An entry survives the reference's cutoff when fl(e / S) >= cutoff, which
-  // implies e >= cutoff * S * (1 - 2^-24); S_est stands in for S with 1 % slack and the
-  // inequality is re-checked against the exact S below.
+  // ---- pass 2: softmax normaliser, sequential in index order (sampler.cpp:199-203)
   const float cutoff = use_topp ? (1.0f - p.topp) / static_cast<float>(V - 1) : 0.0f;  // sampler.cpp:136
-  const float cut_lo = cutoff * S_est * 0.99f;
-  const bool collect = use_topp && (S_est == S_est) && S_est < kInf;
-  bool saw_nan = false;
-  SeqSum st = {0.0f, -1, 0u};
-  {
-    const int chunk = kBlock * VE;
-    uint4 raw = make_uint4(0, 0, 0, 0);
-    const uint4* vec = reinterpret_cast<const uint4*>(logits);
-    if (ALIGNED && tid * VE + VE <= V) raw = vec[tid];
-    for (int base = 0; base < V; base += chunk) {
-      const int first = base + tid * VE;
-      float v[VE];
-      if (ALIGNED && first + VE <= V) {
-        decode_vec<DT>(raw, v);
-      } else {
-#pragma unroll
-        for (int e = 0; e < VE; ++e) v[e] = (first + e < V) ? load_elem<DT>(logits, first + e) : 0.0f;
-      }
-      {
-        const int nfirst = first + chunk;  // prefetch the next chunk's vector
-        if (ALIGNED && nfirst + VE <= V) raw = vec[nfirst / VE];
-      }
-      uint32_t bits[VE];
-      uint32_t cand_mask = 0;
-#pragma unroll
-      for (int e = 0; e < VE; ++e) {
-        const bool valid = first + e < V;
-        const float x = v[e] * inv;
-        float ex = expf_nonpositive(x - m, sm.exp2tab);
-        if (valid && ex != ex) saw_nan = true;
-        ex = (valid && ex == ex) ? ex : 0.0f;
-        bits[e] = __float_as_uint(ex);
-        if (collect && valid && ex >= cut_lo) cand_mask |= 1u << e;
-      }
-      if (collect) {
-        // slots for this lane's candidates: wave prefix over the per-lane counts
-        const uint32_t mine = static_cast<uint32_t>(__popc(cand_mask));
-        uint32_t incl = mine;
-#pragma unroll
-        for (int d = 1; d < 64; d <<= 1) {
-          const uint32_t o = __shfl_up(incl, d);
-          if (lane >= d) incl += o;
-        }
-        const uint32_t wave_total = __shfl(incl, 63);
-        uint32_t slot = 0;
-        if (wave_total) {
-          if (lane == 63) slot = atomicAdd(&sm.counter, wave_total);
-          slot = __shfl(slot, 63) + incl - mine;
-#pragma unroll
-          for (int e = 0; e < VE; ++e) {
-            if (cand_mask & (1u << e)) {
-              if (slot < static_cast<uint32_t>(cap))
-                lds_keys[slot] = (static_cast<uint64_t>(bits[e]) << 32) | static_cast<uint32_t>(first + e);
-              ++slot;
-            }
-          }
-        }
-      }
-      seq_sum_chunk<VE>(st, bits, first, V, kInf, sm);
+  float S = kNaN;
+  if (!row_nan) {
+    ScanArgs a = {logits, V, inv, m, 0.0f, kInf, cutoff, scratch};
+    SeqSum st = {0.0f, -1, 0u};
+    if (use_topp) {
+      scan_row<DT, ALIGNED, kScanSum, true>(a, st, sm);
+    } else {
+      scan_row<DT, ALIGNED, kScanSum, false>(a, st, sm);
     }
-  }
-  float S = st.s;
-  {
-    const uint64_t any = __ballot(saw_nan);
-    if (lane == 0) sm.red_u[wave] = any ? 1u : 0u;
-    __syncthreads();
-    uint32_t nan_row = 0;
-    for (int w = 0; w < kWaves; ++w) nan_row |= sm.red_u[w];
-    if (nan_row) S = kNaN;  // one NaN addend poisons the running sum for good
+    S = st.s;
   }
 
   // ---- one coin per call (sampler.cpp:237, 210-220)
@@ -426,207 +720,35 @@ __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
   const int n_listed = static_cast<int>(sm.counter);
   __syncthreads();
 
-  auto prob_at = [&](int i) -> float {
-    const float x = load_elem<DT>(logits, i) * inv;
-    return expf_nonpositive(x - m, sm.exp2tab) / S;  // sampler.cpp:205-207: a true division
-  };
-  if (probs) {
-    for (int i = tid; i < V; i += kBlock) probs[i] = prob_at(i);
+  if (p.probs) {
+    float* probs = p.probs + static_cast<int64_t>(row) * V;
+    for (int i = tid; i < V; i += kBlock) {
+      const float x = load_elem<DT>(logits, i) * inv;
+      probs[i] = expf_nonpositive(x - m, sm.exp2tab) / S;
+    }
   }
 
   RowDebug dbg = {m, S, coin, 0.0f, 0.0f, 0, 0, 0};
   int32_t token = -1;
-
-  if (S != S) {
-    // Every probability is NaN.  The multinomial walk never fires and returns the last
-    // index; top-p keeps no candidate and top-k's comparisons are all false, which the
-    // reference does not define: report -1.
+  if (row_nan) {
+    // Every probability is NaN.  The multinomial walk never fires and returns the last index;
+    // top-p keeps no candidate and top-k's comparisons are all false, which the reference does
+    // not define: report -1.
     token = use_mult ? V - 1 : -1;
   } else if (use_mult) {
     // ---- sampler.cpp:58-70: first index whose running sum of probabilities exceeds the coin
+    ScanArgs a = {logits, V, inv, m, S, coin, 0.0f, nullptr};
     SeqSum walk = {0.0f, -1, 0u};
-    for (int base = 0; base < V; base += kBlock * VE) {
-      const int first = base + tid * VE;
-      float v[VE];
-      load_run<DT, ALIGNED>(logits, first, V, 0.0f, v);
-      uint32_t bits[VE];
-#pragma unroll
-      for (int e = 0; e < VE; ++e) {
-        const float x = v[e] * inv;
-        const float pi = expf_nonpositive(x - m, sm.exp2tab) / S;
-        bits[e] = (first + e < V) ? __float_as_uint(pi) : 0u;
-      }
-      if (seq_sum_chunk<VE>(walk, bits, first, V, coin, sm)) break;
-    }
+    scan_row<DT, ALIGNED, kScanWalk, false>(a, walk, sm);
     token = walk.stop_index >= 0 ? walk.stop_index : V - 1;
     dbg.cumulative = walk.s;
     dbg.position = token;
   } else {
     bool done = false;
-    const bool list_ok = collect && n_listed <= cap && cut_lo <= cutoff * S * 0.9999f;
-    if (use_topp && list_ok) {
-      // ---- exact filter p >= cutoff over the listed entries (sampler.cpp:137-143) and a
-      // histogram of probability mass by magnitude to find where the nucleus must end
-      for (int b = tid; b < kHistBins; b += kBlock) {
-        ns.hist_mass[b] = 0.0f;
-        ns.hist_count[b] = 0u;
-      }
-      __syncthreads();
-      const int bin0 = static_cast<int>(__float_as_uint(cutoff) >> 19);
-      for (int j = tid; j < n_listed; j += kBlock) {
-        const uint64_t ent = lds_keys[j];
-        const float pj = __uint_as_float(static_cast<uint32_t>(ent >> 32)) / S;
-        uint64_t key = ~0ull;
-        if (pj >= cutoff) {
-          key = cand_key(pj, static_cast<int>(static_cast<uint32_t>(ent)));
-          int bin = static_cast<int>(__float_as_uint(pj) >> 19) - bin0;
-          bin = bin < 0 ? 0 : (bin >= kHistBins ? kHistBins - 1 : bin);
-          atomicAdd(&ns.hist_mass[bin], pj);
-          atomicAdd(&ns.hist_count[bin], 1u);
-        }
-        lds_keys[j] = key;
-      }
-      __syncthreads();
-      // wave 0: walk the bins from the largest probabilities down until the mass is safely
-      // above topp; everything in those bins is selected for sorting
-      if (wave == 0) {
-        constexpr int per = kHistBins / 64;
-        float mass[per];
-        uint32_t cnt[per];
-        float lane_mass = 0.0f;
-        uint32_t lane_cnt = 0;
-#pragma unroll
-        for (int q = 0; q < per; ++q) {
-          const int bin = kHistBins - 1 - (lane * per + q);
-          mass[q] = ns.hist_mass[bin];
-          cnt[q] = ns.hist_count[bin];
-          lane_mass += mass[q];
-          lane_cnt += cnt[q];
-        }
-        float incl_m = lane_mass;
-        uint32_t incl_c = lane_cnt;
-#pragma unroll
-        for (int d = 1; d < 64; d <<= 1) {
-          const float om = __shfl_up(incl_m, d);
-          const uint32_t oc = __shfl_up(incl_c, d);
-          if (lane >= d) {
-            incl_m += om;
-            incl_c += oc;
-          }
-        }
-        const float target = p.topp * 1.004f + 1e-6f;
-        const uint64_t hit = __ballot(incl_m >= target);
-        const uint32_t total_cnt = __shfl(incl_c, 63);
-        if (hit) {
-          const int hl = __ffsll(static_cast<long long>(hit)) - 1;
-          if (lane == hl) {
-            float run_m = incl_m - lane_mass;
-            uint32_t run_c = incl_c - lane_cnt;
-            int q = 0;
-#pragma unroll
-            for (; q < per; ++q) {
-              run_m += mass[q];
-              run_c += cnt[q];
-              if (run_m >= target) break;
-            }
-            q = q < per ? q : per - 1;
-            sm.flag = kHistBins - 1 - (lane * per + q);
-            sm.counter2 = run_c;
-          }
-        } else if (lane == 0) {
-          sm.flag = 0;
-          sm.counter2 = total_cnt;
-        }
-        if (lane == 0) sm.red_u[0] = total_cnt;
-      }
-      __syncthreads();
-      const int sel_bin = sm.flag;
-      int n_sel = static_cast<int>(sm.counter2);
-      const int n0 = static_cast<int>(sm.red_u[0]);
-      dbg.n_candidates = n0;
-      __syncthreads();
-      if (n0 == 0) {
-        token = -1;  // the reference reads probindex[-1] here
-        done = true;
-      } else {
-        const uint64_t* sorted = nullptr;
-        if (n_sel <= kSelCap) {
-          // peaked row: move the few selected keys to the small buffer and sort them there
-          if (tid == 0) sm.counter = 0u;
-          __syncthreads();
-          for (int base = 0; base < n_listed; base += kBlock) {
-            const int j = base + tid;
-            uint64_t key = ~0ull;
-            if (j < n_listed) key = lds_keys[j];
-            bool keep = false;
-            if (key != ~0ull) {
-              int bin = static_cast<int>(__float_as_uint(cand_prob(key)) >> 19) - bin0;
-              bin = bin < 0 ? 0 : (bin >= kHistBins ? kHistBins - 1 : bin);
-              keep = bin >= sel_bin;
-            }
-            const uint32_t slot = wave_append_slot(keep, &sm.counter, lane);
-            if (keep) ns.sel[slot] = key;
-          }
-          __syncthreads();
-          const int N = pow2_ceil(n_sel);
-          for (int i = n_sel + tid; i < N; i += kBlock) ns.sel[i] = ~0ull;
-          __syncthreads();
-          sort_keys_lds(ns.sel, N);
-          sorted = ns.sel;
-        } else {
-          // broad row: sort the whole list in place (entries that failed the cutoff are ~0)
-          n_sel = n0;
-          const int N = pow2_ceil(n_listed);
-          for (int i = n_listed + tid; i < N; i += kBlock) lds_keys[i] = ~0ull;
-          __syncthreads();
-          sort_keys_lds(lds_keys, N);
-          sorted = lds_keys;
-        }
-        int pos = draw_from_sorted(sorted, n_sel, n0, false, 0, p.topp, coin, dbg, sm);
-        if (pos == -2) {
-          // the pre-selected bins did not reach topp after all: sort every candidate
-          const int N = pow2_ceil(n_listed);
-          for (int i = n_listed + tid; i < N; i += kBlock) lds_keys[i] = ~0ull;
-          __syncthreads();
-          sort_keys_lds(lds_keys, N);
-          sorted = lds_keys;
-          pos = draw_from_sorted(sorted, n0, n0, false, 0, p.topp, coin, dbg, sm);
-        }
-        token = static_cast<int32_t>(static_cast<uint32_t>(sorted[pos]));
-        done = true;
-      }
-    }
+    if (use_topp) done = draw_topp_listed(scratch, n_listed, S, cutoff, p.topp, coin, scratch, lds_keys, p.lds_keys, dbg, token, sm, ns);
     if (!done) {
-      // ---- general path: candidates to global memory, full sort.  Top-p rows whose list does
-      // not fit in LDS, and top-k (which ranks the whole row, sampler.cpp:87-100).
-      const float cut = use_topk ? 0.0f : cutoff;
-      if (tid == 0) sm.counter = 0u;
-      __syncthreads();
-      for (int base = 0; base < V; base += kBlock) {
-        const int i = base + tid;
-        float pi = 0.0f;
-        bool keep = false;
-        if (i < V) {
-          pi = prob_at(i);
-          keep = pi >= cut;
-        }
-        const uint32_t slot = wave_append_slot(keep, &sm.counter, lane);
-        if (keep) scratch[slot] = cand_key(pi, i);
-      }
-      __syncthreads();
-      const int n0 = static_cast<int>(sm.counter);
-      dbg.n_candidates = n0;
-      if (n0 == 0) {
-        token = -1;
-      } else {
-        const int N = pow2_ceil(n0);
-        for (int i = n0 + tid; i < N; i += kBlock) scratch[i] = ~0ull;
-        __syncthreads();
-        sort_keys_block(scratch, N, lds_keys, cap);
-        const uint64_t* keys = (N <= cap) ? lds_keys : scratch;
-        const int pos = draw_from_sorted(keys, n0, n0, use_topk, p.topk, p.topp, coin, dbg, sm);
-        token = static_cast<int32_t>(static_cast<uint32_t>(keys[pos]));
-      }
+      token = draw_general<DT>(logits, V, inv, m, S, use_topk, p.topk, p.topp, cutoff, coin, scratch, lds_keys,
+                               p.lds_keys, dbg, sm);
     }
   }
   if (tid == 0) {

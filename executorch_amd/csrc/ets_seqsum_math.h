@@ -90,6 +90,23 @@ ETS_HD void fold_elem(ParityInc& acc, uint32_t abits, int kb) {
   acc.odd = sat_add(acc.odd, inc_odd);
 }
 
+// fold_elem for running sums with biased exponent kb >= 64, where a / ulp(s) is an exact
+// power-of-two scaling in float: `scale` = 2^(150 - kb).  Same result as fold_elem.
+ETS_HD void fold_elem_scaled(ParityInc& acc, float a, float scale) {
+  float t = a * scale;
+  t = t < 67108864.0f ? t : 67108864.0f;  // 2^26 == kSat
+  const float fl = __builtin_floorf(t);
+  const float frac = t - fl;  // exact
+  const uint32_t n0 = static_cast<uint32_t>(fl);
+  const uint32_t up = frac > 0.5f ? 1u : 0u;
+  const uint32_t tie = frac == 0.5f ? 1u : 0u;
+  const uint32_t base = n0 + up;
+  const uint32_t inc_even = base + (tie & ((acc.even + n0) & 1u));
+  const uint32_t inc_odd = base + (tie & ((acc.odd + n0 + 1u) & 1u));
+  acc.even = sat_add(acc.even, inc_even);
+  acc.odd = sat_add(acc.odd, inc_odd);
+}
+
 // Order-free shortcut used while a whole chunk stays inside the binade of s (biased exponent
 // kb >= 64) and no element sits on a half-ulp tie: the increment of `abits` is rne(a / ulp(s)),
 // computed with an exact power-of-two scaling in float.  Sets `tie` when the fraction is exactly
