@@ -106,6 +106,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="cfg2")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run five 256 MiB device copies: a kernel of known traffic that calibrates "
+                         "FETCH_SIZE / WRITE_SIZE when this command runs under rocprofv3 --pmc")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; rows are independent, so more GPUs would each take "
@@ -140,6 +143,14 @@ def main():
     want, _ = O.sample_rows(hx, w.dtype, O.inv_temperature(w.temperature), w.topp, 0, W.coin_seeds(w, rows).copy(),
                             mode=O.MODE_UPCAST, tie=O.TIE_STABLE, threads=8)
     mismatches = int((got != want).sum())
+
+    if args.copy_probe:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_()
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     for i in range(args.warmup):
         s.sample_batch(ring[i % ring_len], out=out)
