@@ -195,6 +195,9 @@ struct BlockScratch {
   ParityInc wave_total[2][kWaves];  // double-buffered, like group_total
   int first_flag[kWaves];
   float group_total[2][kWaves];    // same, for seq_sum_group
+  uint32_t group_flag[2][kWaves];
+  float cross_cur[64];             // seq_sum_group stage 2: (chunk, wave) totals, current binade
+  float cross_next[64];            // ... next binade
   float red_f[kWaves];
   uint32_t red_u[kWaves];
   float bc_sum;
@@ -237,6 +240,39 @@ __device__ __forceinline__ void fast_fold(FastAcc& a, float e, float scale) {
   a.tie = __builtin_fmaxf(a.tie, __builtin_fabsf(t - r));
 }
 
+// ---- wave64 cross-lane helpers on DPP (data-parallel primitives: a VALU operand taken from another
+// lane of the same row of 16, or a row broadcast).  A DPP step costs one VALU issue; a shuffle
+// through ds_bpermute costs an LDS round trip, which dominates single-wave code.
+template <int CTRL, int ROW_MASK, int BANK_MASK>
+__device__ __forceinline__ float dpp_or_zero(float v) {
+  // lanes without a source under CTRL (or masked off) read 0
+  return __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(v), CTRL, ROW_MASK, BANK_MASK, false));
+}
+
+// Inclusive prefix sum over the 64 lanes: Hillis-Steele inside each row of 16 (row_shr 1, 2, 4, 8),
+// then row_bcast:15 into rows 1 and 3 and row_bcast:31 into rows 2 and 3.
+__device__ __forceinline__ float wave_scan_inclusive_f32(float v, int /*lane*/) {
+  v += dpp_or_zero<0x111, 0xf, 0xf>(v);
+  v += dpp_or_zero<0x112, 0xf, 0xf>(v);
+  v += dpp_or_zero<0x114, 0xf, 0xf>(v);
+  v += dpp_or_zero<0x118, 0xf, 0xf>(v);
+  v += dpp_or_zero<0x142, 0xa, 0xf>(v);
+  v += dpp_or_zero<0x143, 0xc, 0xf>(v);
+  return v;
+}
+
+// Value of lane `l` (wave-uniform index) in every lane.
+__device__ __forceinline__ float readlane_f32(float v, int l) {
+  return __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(v), l));
+}
+__device__ __forceinline__ uint32_t readlane_u32(uint32_t v, int l) { return __builtin_amdgcn_readlane(v, l); }
+
+// Sum over the 64 lanes, in every lane.
+__device__ __forceinline__ float wave_sum_f32(float v) { return readlane_f32(wave_scan_inclusive_f32(v, 0), 63); }
+
+// Value of the previous lane (0 in lane 0): wave_shr:1.
+__device__ __forceinline__ float lane_before_f32(float v) { return dpp_or_zero<0x138, 0xf, 0xf>(v); }
+
 // Summary of a lane's run of R elements for the running sum s (see ets_seqsum_math.h).
 template <int R>
 __device__ __forceinline__ ParityInc fold_run(const uint32_t (&bits)[R], float s) {
@@ -253,33 +289,59 @@ __device__ __forceinline__ ParityInc fold_run(const uint32_t (&bits)[R], float s
   return acc;
 }
 
-// One wavefront consumes its own 64 runs exactly, starting from running sum s: a wave-level scan
-// of the run summaries finds the first lane whose run leaves the binade of s or crosses the
-// threshold; that lane adds its elements natively and the scan restarts behind it with the new
-// ulp.  No barriers: only this wave takes part.  On return s is the running sum after the wave's
-// last element, or `found` is the position where the threshold was crossed.
+// One wavefront consumes its own 64 runs exactly, starting from running sum s.  No barriers: only
+// this wave takes part.  On return s is the running sum after the wave's last element, or `found`
+// is the position where the threshold was crossed.
+//
+// Common case (s >= 2^-63): the lanes' increments rne(a / ulp(s)) are summed in float (exact below
+// 2^24).  A lane is an "event" if one of its elements sits on a half-ulp tie (the only case in
+// which an increment depends on the order), or if the prefix sum up to and including it leaves
+// the binade of s or crosses the threshold.  The first event lane adds its elements natively and
+// the scan restarts behind it with the new ulp.  Tiny running sums use the two-hypothesis parity
+// summaries instead (integer arithmetic, any magnitude).
 template <int R>
 __device__ void wave_resolve(float& s, int& found, const uint32_t (&bits)[R], int first, int n, float threshold) {
   const int lane = threadIdx.x & 63;
   int consumed = 0;  // lanes below this have been consumed
   found = -1;
   while (true) {
-    ParityInc mine = {0u, 0u};
-    if (lane >= consumed) mine = fold_run<R>(bits, s);
-    const ParityInc incl = wave_scan_inclusive(mine, lane);
-    ParityInc excl;
-    excl.even = __shfl_up(incl.even, 1);
-    excl.odd = __shfl_up(incl.odd, 1);
-    if (lane == 0) excl = {0u, 0u};
+    const float scale = fast_scale(s);
     const SumState ss = sum_state(s);
-    const bool odd = ss.S & 1u;
-    const uint32_t S_incl = ss.S + (odd ? incl.odd : incl.even);
-    const uint32_t S_excl = ss.S + (odd ? excl.odd : excl.even);
-    bool special = S_incl >= (1u << 24);
-    if (!special) special = sum_value(S_incl, ss.kb) > threshold;
-    const uint64_t ballot = __ballot(special);
+    uint64_t ballot;
+    uint32_t S_excl, S_end;
+    if (scale != 0.0f) {
+      FastAcc acc = {0.0f, 0.0f};
+      if (lane >= consumed) {
+#pragma unroll
+        for (int e = 0; e < R; ++e) fast_fold(acc, __uint_as_float(bits[e]), scale);
+      }
+      const float incl = wave_scan_inclusive_f32(acc.inc, lane);
+      const float room = static_cast<float>((1u << 24) - ss.S);
+      bool special = acc.tie == 0.5f || !(incl < room);
+      if (!special) special = sum_value(ss.S + static_cast<uint32_t>(incl), ss.kb) > threshold;
+      ballot = __ballot(special);
+      // exact for every lane up to the first event (all prefix sums in front of it are below `room`)
+      const float excl = lane_before_f32(incl);
+      S_excl = ss.S + static_cast<uint32_t>(excl < room ? excl : 0.0f);
+      const float total = readlane_f32(incl, 63);
+      S_end = ss.S + static_cast<uint32_t>(total < room ? total : 0.0f);
+    } else {
+      ParityInc mine = {0u, 0u};
+      if (lane >= consumed) mine = fold_run<R>(bits, s);
+      const ParityInc incl = wave_scan_inclusive(mine, lane);
+      ParityInc excl;
+      excl.even = __shfl_up(incl.even, 1);
+      excl.odd = __shfl_up(incl.odd, 1);
+      if (lane == 0) excl = {0u, 0u};
+      const bool odd = ss.S & 1u;
+      const uint32_t S_incl = ss.S + (odd ? incl.odd : incl.even);
+      S_excl = ss.S + (odd ? excl.odd : excl.even);
+      bool special = S_incl >= (1u << 24);
+      if (!special) special = sum_value(S_incl, ss.kb) > threshold;
+      ballot = __ballot(special);
+      S_end = __shfl(S_incl, 63);
+    }
     if (!ballot) {
-      const uint32_t S_end = __shfl(S_incl, 63);
       s = sum_value(S_end, ss.kb);
       return;
     }
@@ -297,8 +359,8 @@ __device__ void wave_resolve(float& s, int& found, const uint32_t (&bits)[R], in
         }
       }
     }
-    s = __shfl(sj, j);
-    fj = __shfl(fj, j);
+    s = readlane_f32(sj, j);
+    fj = static_cast<int>(readlane_u32(static_cast<uint32_t>(fj), j));
     if (fj >= 0) {
       found = fj;
       return;
@@ -310,9 +372,9 @@ __device__ void wave_resolve(float& s, int& found, const uint32_t (&bits)[R], in
 // Consumes one chunk: lane `tid` owns elements first .. first + R - 1 (global positions, in
 // lane order), given as float bit patterns in bits[] (finite, >= 0; positions >= n must hold 0).
 // Emulates  for each element: s += a; if (s > threshold) stop  in fp32, bit for bit.
-// Each round composes the waves' summaries in order and finds the first wave in which the sum
-// leaves its binade or crosses the threshold; the waves in front of it are committed, that wave
-// resolves its own 512 or so elements with wave_resolve(), and the next round restarts behind it
+// Each round sums the waves' increments in order and finds the first wave that contains an event
+// (a tie, leaving the binade, crossing the threshold); the waves in front of it are committed,
+// that wave resolves its own 64 runs with wave_resolve(), and the next round restarts behind it
 // with the new ulp.  Two barriers per round, one when nothing happens.  Must be called by all
 // lanes; returns true when the threshold was crossed (st.stop_index set).
 template <int R>
@@ -321,32 +383,62 @@ __device__ bool seq_sum_chunk(SeqSum& st, const uint32_t (&bits)[R], int first, 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  int resume_wave = 0;  // waves below this have been consumed
+  const float kBig = 67108864.0f;  // 2^26 marks a wave that must be resolved (tie inside)
+  int resume_wave = 0;             // waves below this have been consumed
   while (true) {
-    ParityInc mine = {0u, 0u};
-    if (wave >= resume_wave) mine = fold_run<R>(bits, st.s);
-    const ParityInc incl = wave_scan_inclusive(mine, lane);
+    const float scale = fast_scale(st.s);
+    const SumState ss = sum_state(st.s);
     const uint32_t buf = st.parity_buf;
     st.parity_buf ^= 1u;
-    if (lane == 63) sm.wave_total[buf][wave] = incl;
-    __syncthreads();
-    // every wave redoes the small scan over the 16 wave totals in its first 16 lanes
-    ParityInc wt = {0u, 0u};
-    if (lane < kWaves) wt = sm.wave_total[buf][lane];
-    const ParityInc upto = wave_scan_inclusive(wt, lane);
-    const SumState ss = sum_state(st.s);
-    const bool odd = ss.S & 1u;
-    const uint32_t S_upto = ss.S + (odd ? upto.odd : upto.even);
-    bool event = S_upto >= (1u << 24);
-    if (!event) event = sum_value(S_upto, ss.kb) > threshold;
-    const uint64_t ballot = __ballot(event && lane < kWaves);
-    if (!ballot) {
-      st.s = sum_value(__shfl(S_upto, kWaves - 1), ss.kb);
+    int wstar;
+    uint32_t S_front, S_all;
+    if (scale != 0.0f) {
+      float wave_inc = 0.0f;
+      if (wave >= resume_wave) {
+        FastAcc acc = {0.0f, 0.0f};
+#pragma unroll
+        for (int e = 0; e < R; ++e) fast_fold(acc, __uint_as_float(bits[e]), scale);
+        const float inc = wave_sum_f32(acc.inc);
+        const bool tie = __ballot(acc.tie == 0.5f) != 0ull;
+        wave_inc = (tie || !(inc < kBig)) ? kBig : inc;
+      }
+      if (lane == 0) sm.group_total[buf][wave] = wave_inc;
+      __syncthreads();
+      // every wave redoes the small scan over the 16 wave totals in its first 16 lanes
+      const float wt = lane < kWaves ? sm.group_total[buf][lane] : 0.0f;
+      const float upto = wave_scan_inclusive_f32(wt, lane);
+      const float room = static_cast<float>((1u << 24) - ss.S);
+      bool event = !(upto < room);
+      if (!event) event = sum_value(ss.S + static_cast<uint32_t>(upto), ss.kb) > threshold;
+      const uint64_t ballot = __ballot(event && lane < kWaves);
+      wstar = ballot ? __ffsll(static_cast<long long>(ballot)) - 1 : kWaves;
+      const float front = wstar > 0 && wstar < kWaves ? readlane_f32(upto, wstar - 1) : 0.0f;
+      const float all = readlane_f32(upto, kWaves - 1);
+      S_front = ss.S + static_cast<uint32_t>(front);
+      S_all = ss.S + static_cast<uint32_t>(all < room ? all : 0.0f);
+    } else {
+      ParityInc mine = {0u, 0u};
+      if (wave >= resume_wave) mine = fold_run<R>(bits, st.s);
+      const ParityInc incl = wave_scan_inclusive(mine, lane);
+      if (lane == 63) sm.wave_total[buf][wave] = incl;
+      __syncthreads();
+      ParityInc wt = {0u, 0u};
+      if (lane < kWaves) wt = sm.wave_total[buf][lane];
+      const ParityInc upto = wave_scan_inclusive(wt, lane);
+      const bool odd = ss.S & 1u;
+      const uint32_t S_upto = ss.S + (odd ? upto.odd : upto.even);
+      bool event = S_upto >= (1u << 24);
+      if (!event) event = sum_value(S_upto, ss.kb) > threshold;
+      const uint64_t ballot = __ballot(event && lane < kWaves);
+      wstar = ballot ? __ffsll(static_cast<long long>(ballot)) - 1 : kWaves;
+      S_front = wstar > 0 && wstar < kWaves ? __shfl(S_upto, wstar - 1) : ss.S;
+      S_all = __shfl(S_upto, kWaves - 1);
+    }
+    if (wstar == kWaves) {
+      st.s = sum_value(S_all, ss.kb);
       return false;
     }
-    const int wstar = __ffsll(static_cast<long long>(ballot)) - 1;
     if (wave == wstar) {
-      const uint32_t S_front = wstar ? __shfl(S_upto, wstar - 1) : ss.S;
       float s = sum_value(S_front, ss.kb);
       int found = -1;
       wave_resolve<R>(s, found, bits, first, n, threshold);
@@ -366,43 +458,146 @@ __device__ bool seq_sum_chunk(SeqSum& st, const uint32_t (&bits)[R], int first, 
   }
 }
 
-// ---- several chunks per barrier -------------------------------------------------------------------
+// Folds one element into the lane summaries for the current binade (scale) and for the next one
+// (scale / 2), which is where the sum continues after a binade crossing.
+__device__ __forceinline__ void fast_fold2(FastAcc& cur, FastAcc& next, float e, float scale) {
+  const float t = e * scale;
+  const float r = __builtin_rintf(t);
+  cur.inc += r;
+  cur.tie = __builtin_fmaxf(cur.tie, __builtin_fabsf(t - r));
+  const float t1 = t * 0.5f;
+  const float r1 = __builtin_rintf(t1);
+  next.inc += r1;
+  next.tie = __builtin_fmaxf(next.tie, __builtin_fabsf(t1 - r1));
+}
+
 // Consumes U chunks (chunk u: lane `tid` owns elements first[u] .. first[u] + R - 1, chunks in
-// increasing position) with ONE barrier when all of them stay inside the binade of s, below the
-// threshold and free of ties; `acc` must have been folded over the same elements with
-// fast_scale(st.s).  Otherwise the chunks go through seq_sum_chunk one after the other.
+// increasing position).  cur[u] / next[u] are the lane's fast_fold2 summaries of chunk u for the
+// binade of st.s and the one above it (folded with scale = fast_scale(st.s)).
+//   1. If all chunks stay inside the binade, below the threshold and free of ties: one reduction,
+//      one barrier.
+//   2. If the only thing that happens is ONE binade crossing: a prefix sum of the current-binade
+//      increments locates the lane where it happens, that lane adds its elements natively, and
+//      everything behind it is accounted with the next-binade increments.  Two more barriers.
+//   3. Otherwise the chunks go through seq_sum_chunk one after the other.
 template <int U, int R>
-__device__ bool seq_sum_group(SeqSum& st, const uint32_t (&bits)[U][R], FastAcc acc, float scale,
-                              const int (&first)[U], int n, float threshold, BlockScratch& sm) {
+__device__ bool seq_sum_group(SeqSum& st, const uint32_t (&bits)[U][R], const FastAcc (&cur)[U], const FastAcc (&next)[U],
+                              float scale, const int (&first)[U], int n, float threshold, BlockScratch& sm) {
+  static_assert(U * kWaves <= 64, "the cross-wave scan of stage 2 uses one lane per (chunk, wave)");
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
-  float inc = acc.inc;
-  float tie = acc.tie;
+  const float kBig = 67108864.0f;  // 2^26: "not usable"
+  // ---- stage 1
+  float inc = 0.0f, tie = 0.0f, tie_next = 0.0f;
 #pragma unroll
-  for (int d = 32; d > 0; d >>= 1) {
-    inc += __shfl_xor(inc, d);
-    tie = __builtin_fmaxf(tie, __shfl_xor(tie, d));
+  for (int u = 0; u < U; ++u) {
+    inc += cur[u].inc;
+    tie = __builtin_fmaxf(tie, cur[u].tie);
+    tie_next = __builtin_fmaxf(tie_next, next[u].tie);
   }
-  const float kBig = 67108864.0f;  // 2^26: "take the ordered path"
-  if (tie == 0.5f || scale == 0.0f || !(inc < kBig)) inc = kBig;
+  inc = wave_sum_f32(inc);
+  const bool any_tie = __ballot(tie == 0.5f) != 0ull;
+  const bool any_tie_next = __ballot(tie_next == 0.5f) != 0ull;
+  const bool wave_plain = !(any_tie || scale == 0.0f || !(inc < kBig));  // stage 1 usable
+  const bool wave_cross = wave_plain && !any_tie_next;                   // stage 2 usable
   const uint32_t buf = st.parity_buf;
   st.parity_buf ^= 1u;
-  if (lane == 0) sm.group_total[buf][wave] = inc;
+  if (lane == 0) {
+    sm.group_total[buf][wave] = wave_plain ? inc : kBig;
+    sm.group_flag[buf][wave] = wave_cross ? 0u : 1u;
+  }
   __syncthreads();
   float total = 0.0f;
+  uint32_t no_cross = 0u;
 #pragma unroll
-  for (int w = 0; w < kWaves; ++w) total += sm.group_total[buf][w];
-  if (total < 16777216.0f) {
-    const SumState ss = sum_state(st.s);
-    const uint32_t S_new = ss.S + static_cast<uint32_t>(total);
-    if (S_new < (1u << 24)) {
-      const float s_new = sum_value(S_new, ss.kb);
-      if (!(s_new > threshold)) {
-        st.s = s_new;
-        return false;
-      }
+  for (int w = 0; w < kWaves; ++w) {
+    total += sm.group_total[buf][w];
+    no_cross |= sm.group_flag[buf][w];
+  }
+  const SumState ss = sum_state(st.s);
+  const float room = static_cast<float>((1u << 24) - ss.S);  // increments that still fit in the binade
+  if (total < room) {
+    const float s_new = sum_value(ss.S + static_cast<uint32_t>(total), ss.kb);
+    if (!(s_new > threshold)) {
+      st.s = s_new;
+      return false;
     }
   }
+  // ---- stage 2: exactly one crossing, no ties anywhere
+  if (total < kBig && no_cross == 0u && !(total < room) && ss.kb < 253) {
+    float incl[U];  // inclusive prefix of the current-binade increments inside the wave, per chunk
+#pragma unroll
+    for (int u = 0; u < U; ++u) incl[u] = wave_scan_inclusive_f32(cur[u].inc, lane);
+    float next_wave[U];  // wave totals of the next-binade increments
+#pragma unroll
+    for (int u = 0; u < U; ++u) next_wave[u] = wave_sum_f32(next[u].inc);
+    if (lane == 63) {
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        sm.cross_cur[u * kWaves + wave] = incl[u];
+        sm.cross_next[u * kWaves + wave] = next_wave[u];
+      }
+    }
+    __syncthreads();
+    // lanes 0 .. U*16-1 of every wave: (chunk, wave) totals in position order
+    float tc = 0.0f, tn = 0.0f;
+    if (lane < U * kWaves) {
+      tc = sm.cross_cur[lane];
+      tn = sm.cross_next[lane];
+    }
+    const float upto_c = wave_scan_inclusive_f32(tc, lane);  // exact below `room`
+    const float upto_n = wave_scan_inclusive_f32(tn, lane);
+    const uint64_t over = __ballot(lane < U * kWaves && !(upto_c < room));
+    const int slot = __ffsll(static_cast<long long>(over)) - 1;  // (chunk, wave) that holds the crossing
+    const int ustar = slot / kWaves, wstar = slot % kWaves;
+    if (wave == wstar) {
+      const float front = slot ? readlane_f32(upto_c, slot - 1) : 0.0f;  // increments in front of this wave's run
+      const float behind = readlane_f32(upto_n, U * kWaves - 1) - readlane_f32(upto_n, slot);  // next-binade increments behind it
+      float my_incl = incl[0], my_next = next[0].inc;
+#pragma unroll
+      for (int u = 1; u < U; ++u) {
+        my_incl = (u == ustar) ? incl[u] : my_incl;
+        my_next = (u == ustar) ? next[u].inc : my_next;
+      }
+      const float my_next_incl = wave_scan_inclusive_f32(my_next, lane);
+      const uint64_t hit = __ballot(!(front + my_incl < room));
+      const int j = __ffsll(static_cast<long long>(hit)) - 1;
+      const float before = front + lane_before_f32(my_incl);
+      float sj = 0.0f;
+      if (lane == j) {
+        sj = sum_value(ss.S + static_cast<uint32_t>(before), ss.kb);
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          if (u == ustar) {
+#pragma unroll
+            for (int e = 0; e < R; ++e) sj = sj + __uint_as_float(bits[u][e]);  // positions >= n hold 0
+          }
+        }
+      }
+      sj = readlane_f32(sj, j);
+      // increments (next binade) of this wave's lanes behind j, then of everything behind the wave
+      const float tail = readlane_f32(my_next_incl, 63) - readlane_f32(my_next_incl, j) + behind;
+      const SumState sx = sum_state(sj);
+      // every next-binade partial sum is exact only while their grand total stays below 2^24
+      bool ok = sx.kb == ss.kb + 1 && readlane_f32(upto_n, U * kWaves - 1) < 16777216.0f &&
+                tail < static_cast<float>((1u << 24) - sx.S);
+      float s_new = 0.0f;
+      if (ok) {
+        s_new = sum_value(sx.S + static_cast<uint32_t>(tail), sx.kb);
+        ok = !(s_new > threshold);
+      }
+      if (lane == 0) {
+        sm.bc_sum = s_new;
+        sm.bc_found = ok ? 1 : 0;
+      }
+    }
+    __syncthreads();
+    if (sm.bc_found) {
+      st.s = sm.bc_sum;
+      return false;
+    }
+  }
+  // ---- stage 3
 #pragma unroll
   for (int u = 0; u < U; ++u) {
     if (seq_sum_chunk<R>(st, bits[u], first[u], n, threshold, sm)) return true;

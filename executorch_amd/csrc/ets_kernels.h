@@ -315,7 +315,7 @@ __device__ __forceinline__ bool scan_row(const ScanArgs& a, SeqSum& st, BlockScr
     for (; vbase + per_iter <= nvec; vbase += per_iter) {
       const float scale = fast_scale(st.s);
       const float cut_lo = LIST ? a.cutoff * __builtin_fmaxf(st.s, 1.0f) * 0.999f : 0.0f;
-      FastAcc acc = {0.0f, 0.0f};
+      FastAcc cur[kGroup], next[kGroup];
       uint32_t bits[kGroup][VE];
       int first[kGroup];
       const bool more = vbase + 2 * per_iter <= nvec;
@@ -326,11 +326,13 @@ __device__ __forceinline__ bool scan_row(const ScanArgs& a, SeqSum& st, BlockScr
         if (more) raw[u] = vec[vbase + per_iter + u * kBlock + tid];
         first[u] = (vbase + u * kBlock + tid) * VE;
         uint32_t cmask = 0;
+        cur[u] = {0.0f, 0.0f};
+        next[u] = {0.0f, 0.0f};
 #pragma unroll
         for (int e = 0; e < VE; ++e) {
           const float val = value_of(v[e]);
           bits[u][e] = __float_as_uint(val);
-          fast_fold(acc, val, scale);
+          fast_fold2(cur[u], next[u], val, scale);
           if (LIST && val >= cut_lo) cmask |= 1u << e;
         }
         if (LIST) {
@@ -345,7 +347,7 @@ __device__ __forceinline__ bool scan_row(const ScanArgs& a, SeqSum& st, BlockScr
           }
         }
       }
-      if (seq_sum_group<kGroup, VE>(st, bits, acc, scale, first, V, a.threshold, sm)) return true;
+      if (seq_sum_group<kGroup, VE>(st, bits, cur, next, scale, first, V, a.threshold, sm)) return true;
     }
     done_elems = vbase * VE;
   }
@@ -769,15 +771,46 @@ __global__ void __launch_bounds__(256) expf_exact_kernel(const float* x, float* 
   }
 }
 
-// Sequential float sum of an array by one workgroup (test hook for seq_sum_block).
+// Sequential float sum of an array by one workgroup (test hook).  Same loop structure as
+// scan_row: groups of kGroup chunks of 4 elements per lane through seq_sum_group, the remainder
+// through seq_sum_chunk.
 __global__ void __launch_bounds__(kBlock)
 seq_sum_kernel(const float* a, int32_t n, float s0, float threshold, float* sum_out, int32_t* stop_out) {
   __shared__ BlockScratch sm;
-  auto fetch = [&](int i) -> float { return a[i]; };
-  const SeqSumResult r = seq_sum_block<4>(fetch, n, s0, threshold, sm);
+  constexpr int R = 4;
+  const int tid = threadIdx.x;
+  SeqSum st = {s0, -1, 0u};
+  bool stopped = false;
+  int base = 0;
+  for (; !stopped && base + kGroup * kBlock * R <= n; base += kGroup * kBlock * R) {
+    const float scale = fast_scale(st.s);
+    FastAcc cur[kGroup], next[kGroup];
+    uint32_t bits[kGroup][R];
+    int first[kGroup];
+#pragma unroll
+    for (int u = 0; u < kGroup; ++u) {
+      first[u] = base + (u * kBlock + tid) * R;
+      cur[u] = {0.0f, 0.0f};
+      next[u] = {0.0f, 0.0f};
+#pragma unroll
+      for (int e = 0; e < R; ++e) {
+        const float v = a[first[u] + e];
+        bits[u][e] = __float_as_uint(v);
+        fast_fold2(cur[u], next[u], v, scale);
+      }
+    }
+    stopped = seq_sum_group<kGroup, R>(st, bits, cur, next, scale, first, n, threshold, sm);
+  }
+  for (; !stopped && base < n; base += kBlock * R) {
+    uint32_t bits[R];
+    const int first = base + tid * R;
+#pragma unroll
+    for (int e = 0; e < R; ++e) bits[e] = (first + e < n) ? __float_as_uint(a[first + e]) : 0u;
+    stopped = seq_sum_chunk<R>(st, bits, first, n, threshold, sm);
+  }
   if (threadIdx.x == 0) {
-    *sum_out = r.sum;
-    *stop_out = r.stop_index;
+    *sum_out = st.s;
+    *stop_out = st.stop_index;
   }
 }
 

@@ -79,13 +79,15 @@ def inputs(kind, n, rng):
         return a
     if kind == "flat":
         return np.full(n, np.float32(1.0) / np.float32(n), dtype=np.float32)
+    if kind == "bulk":  # small, similar addends: binade crossings far apart, as in the body of a softmax row
+        return rng.uniform(1e-7, 3e-6, n).astype(np.float32)
     raise ValueError(kind)
 
 
-@pytest.mark.parametrize("kind", ["wide", "edge", "pow2", "fewbits", "peaked", "denormal", "flat"])
+@pytest.mark.parametrize("kind", ["wide", "edge", "pow2", "fewbits", "peaked", "denormal", "flat", "bulk"])
 def test_seq_sum_matches_scalar_loop(dev, kind):
     rng = np.random.default_rng([7, len(kind)])
-    for n in (1, 3, 64, 4095, 4096, 4097, 12345, 40000):
+    for n in (1, 3, 64, 4095, 4096, 4097, 8192, 12345, 40000, 150001):
         a = inputs(kind, n, rng)
         total, _ = seq_sum_f32(a)
         for s0, thr in ((0.0, np.inf), (0.0, float(total) * 0.37), (0.0, 0.0), (0.75, float(total) + 0.5), (0.0, float(total))):
