@@ -195,9 +195,7 @@ struct BlockScratch {
   ParityInc wave_total[2][kWaves];  // double-buffered, like group_total
   int first_flag[kWaves];
   float group_total[2][kWaves];    // same, for seq_sum_group
-  uint32_t group_flag[2][kWaves];
-  float cross_cur[64];             // seq_sum_group stage 2: (chunk, wave) totals, current binade
-  float cross_next[64];            // ... next binade
+  float aux_total[2][kWaves];      // second value of block_sum2
   float red_f[kWaves];
   uint32_t red_u[kWaves];
   float bc_sum;
@@ -458,146 +456,34 @@ __device__ bool seq_sum_chunk(SeqSum& st, const uint32_t (&bits)[R], int first, 
   }
 }
 
-// Folds one element into the lane summaries for the current binade (scale) and for the next one
-// (scale / 2), which is where the sum continues after a binade crossing.
-__device__ __forceinline__ void fast_fold2(FastAcc& cur, FastAcc& next, float e, float scale) {
-  const float t = e * scale;
-  const float r = __builtin_rintf(t);
-  cur.inc += r;
-  cur.tie = __builtin_fmaxf(cur.tie, __builtin_fabsf(t - r));
-  const float t1 = t * 0.5f;
-  const float r1 = __builtin_rintf(t1);
-  next.inc += r1;
-  next.tie = __builtin_fmaxf(next.tie, __builtin_fabsf(t1 - r1));
-}
-
 // Consumes U chunks (chunk u: lane `tid` owns elements first[u] .. first[u] + R - 1, chunks in
-// increasing position).  cur[u] / next[u] are the lane's fast_fold2 summaries of chunk u for the
-// binade of st.s and the one above it (folded with scale = fast_scale(st.s)).
-//   1. If all chunks stay inside the binade, below the threshold and free of ties: one reduction,
-//      one barrier.
-//   2. If the only thing that happens is ONE binade crossing: a prefix sum of the current-binade
-//      increments locates the lane where it happens, that lane adds its elements natively, and
-//      everything behind it is accounted with the next-binade increments.  Two more barriers.
-//   3. Otherwise the chunks go through seq_sum_chunk one after the other.
+// increasing position) with ONE barrier when all of them stay inside the binade of s, below the
+// threshold and free of ties; `acc` must have been folded over the same elements with
+// scale = fast_scale(st.s).  Otherwise the chunks go through seq_sum_chunk one after the other.
 template <int U, int R>
-__device__ bool seq_sum_group(SeqSum& st, const uint32_t (&bits)[U][R], const FastAcc (&cur)[U], const FastAcc (&next)[U],
-                              float scale, const int (&first)[U], int n, float threshold, BlockScratch& sm) {
-  static_assert(U * kWaves <= 64, "the cross-wave scan of stage 2 uses one lane per (chunk, wave)");
+__device__ bool seq_sum_group(SeqSum& st, const uint32_t (&bits)[U][R], FastAcc acc, float scale,
+                              const int (&first)[U], int n, float threshold, BlockScratch& sm) {
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
-  const float kBig = 67108864.0f;  // 2^26: "not usable"
-  // ---- stage 1
-  float inc = 0.0f, tie = 0.0f, tie_next = 0.0f;
-#pragma unroll
-  for (int u = 0; u < U; ++u) {
-    inc += cur[u].inc;
-    tie = __builtin_fmaxf(tie, cur[u].tie);
-    tie_next = __builtin_fmaxf(tie_next, next[u].tie);
-  }
-  inc = wave_sum_f32(inc);
-  const bool any_tie = __ballot(tie == 0.5f) != 0ull;
-  const bool any_tie_next = __ballot(tie_next == 0.5f) != 0ull;
-  const bool wave_plain = !(any_tie || scale == 0.0f || !(inc < kBig));  // stage 1 usable
-  const bool wave_cross = wave_plain && !any_tie_next;                   // stage 2 usable
+  const float kBig = 67108864.0f;  // 2^26: "take the ordered path"
+  float inc = wave_sum_f32(acc.inc);
+  const bool any_tie = __ballot(acc.tie == 0.5f) != 0ull;
+  if (any_tie || scale == 0.0f || !(inc < kBig)) inc = kBig;
   const uint32_t buf = st.parity_buf;
   st.parity_buf ^= 1u;
-  if (lane == 0) {
-    sm.group_total[buf][wave] = wave_plain ? inc : kBig;
-    sm.group_flag[buf][wave] = wave_cross ? 0u : 1u;
-  }
+  if (lane == 0) sm.group_total[buf][wave] = inc;
   __syncthreads();
   float total = 0.0f;
-  uint32_t no_cross = 0u;
 #pragma unroll
-  for (int w = 0; w < kWaves; ++w) {
-    total += sm.group_total[buf][w];
-    no_cross |= sm.group_flag[buf][w];
-  }
+  for (int w = 0; w < kWaves; ++w) total += sm.group_total[buf][w];
   const SumState ss = sum_state(st.s);
-  const float room = static_cast<float>((1u << 24) - ss.S);  // increments that still fit in the binade
-  if (total < room) {
+  if (total < static_cast<float>((1u << 24) - ss.S)) {  // stays inside the binade
     const float s_new = sum_value(ss.S + static_cast<uint32_t>(total), ss.kb);
     if (!(s_new > threshold)) {
       st.s = s_new;
       return false;
     }
   }
-  // ---- stage 2: exactly one crossing, no ties anywhere
-  if (total < kBig && no_cross == 0u && !(total < room) && ss.kb < 253) {
-    float incl[U];  // inclusive prefix of the current-binade increments inside the wave, per chunk
-#pragma unroll
-    for (int u = 0; u < U; ++u) incl[u] = wave_scan_inclusive_f32(cur[u].inc, lane);
-    float next_wave[U];  // wave totals of the next-binade increments
-#pragma unroll
-    for (int u = 0; u < U; ++u) next_wave[u] = wave_sum_f32(next[u].inc);
-    if (lane == 63) {
-#pragma unroll
-      for (int u = 0; u < U; ++u) {
-        sm.cross_cur[u * kWaves + wave] = incl[u];
-        sm.cross_next[u * kWaves + wave] = next_wave[u];
-      }
-    }
-    __syncthreads();
-    // lanes 0 .. U*16-1 of every wave: (chunk, wave) totals in position order
-    float tc = 0.0f, tn = 0.0f;
-    if (lane < U * kWaves) {
-      tc = sm.cross_cur[lane];
-      tn = sm.cross_next[lane];
-    }
-    const float upto_c = wave_scan_inclusive_f32(tc, lane);  // exact below `room`
-    const float upto_n = wave_scan_inclusive_f32(tn, lane);
-    const uint64_t over = __ballot(lane < U * kWaves && !(upto_c < room));
-    const int slot = __ffsll(static_cast<long long>(over)) - 1;  // (chunk, wave) that holds the crossing
-    const int ustar = slot / kWaves, wstar = slot % kWaves;
-    if (wave == wstar) {
-      const float front = slot ? readlane_f32(upto_c, slot - 1) : 0.0f;  // increments in front of this wave's run
-      const float behind = readlane_f32(upto_n, U * kWaves - 1) - readlane_f32(upto_n, slot);  // next-binade increments behind it
-      float my_incl = incl[0], my_next = next[0].inc;
-#pragma unroll
-      for (int u = 1; u < U; ++u) {
-        my_incl = (u == ustar) ? incl[u] : my_incl;
-        my_next = (u == ustar) ? next[u].inc : my_next;
-      }
-      const float my_next_incl = wave_scan_inclusive_f32(my_next, lane);
-      const uint64_t hit = __ballot(!(front + my_incl < room));
-      const int j = __ffsll(static_cast<long long>(hit)) - 1;
-      const float before = front + lane_before_f32(my_incl);
-      float sj = 0.0f;
-      if (lane == j) {
-        sj = sum_value(ss.S + static_cast<uint32_t>(before), ss.kb);
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-          if (u == ustar) {
-#pragma unroll
-            for (int e = 0; e < R; ++e) sj = sj + __uint_as_float(bits[u][e]);  // positions >= n hold 0
-          }
-        }
-      }
-      sj = readlane_f32(sj, j);
-      // increments (next binade) of this wave's lanes behind j, then of everything behind the wave
-      const float tail = readlane_f32(my_next_incl, 63) - readlane_f32(my_next_incl, j) + behind;
-      const SumState sx = sum_state(sj);
-      // every next-binade partial sum is exact only while their grand total stays below 2^24
-      bool ok = sx.kb == ss.kb + 1 && readlane_f32(upto_n, U * kWaves - 1) < 16777216.0f &&
-                tail < static_cast<float>((1u << 24) - sx.S);
-      float s_new = 0.0f;
-      if (ok) {
-        s_new = sum_value(sx.S + static_cast<uint32_t>(tail), sx.kb);
-        ok = !(s_new > threshold);
-      }
-      if (lane == 0) {
-        sm.bc_sum = s_new;
-        sm.bc_found = ok ? 1 : 0;
-      }
-    }
-    __syncthreads();
-    if (sm.bc_found) {
-      st.s = sm.bc_sum;
-      return false;
-    }
-  }
-  // ---- stage 3
 #pragma unroll
   for (int u = 0; u < U; ++u) {
     if (seq_sum_chunk<R>(st, bits[u], first[u], n, threshold, sm)) return true;

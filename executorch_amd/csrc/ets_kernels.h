@@ -315,7 +315,7 @@ __device__ __forceinline__ bool scan_row(const ScanArgs& a, SeqSum& st, BlockScr
     for (; vbase + per_iter <= nvec; vbase += per_iter) {
       const float scale = fast_scale(st.s);
       const float cut_lo = LIST ? a.cutoff * __builtin_fmaxf(st.s, 1.0f) * 0.999f : 0.0f;
-      FastAcc cur[kGroup], next[kGroup];
+      FastAcc acc = {0.0f, 0.0f};
       uint32_t bits[kGroup][VE];
       int first[kGroup];
       const bool more = vbase + 2 * per_iter <= nvec;
@@ -326,13 +326,11 @@ __device__ __forceinline__ bool scan_row(const ScanArgs& a, SeqSum& st, BlockScr
         if (more) raw[u] = vec[vbase + per_iter + u * kBlock + tid];
         first[u] = (vbase + u * kBlock + tid) * VE;
         uint32_t cmask = 0;
-        cur[u] = {0.0f, 0.0f};
-        next[u] = {0.0f, 0.0f};
 #pragma unroll
         for (int e = 0; e < VE; ++e) {
           const float val = value_of(v[e]);
           bits[u][e] = __float_as_uint(val);
-          fast_fold2(cur[u], next[u], val, scale);
+          fast_fold(acc, val, scale);
           if (LIST && val >= cut_lo) cmask |= 1u << e;
         }
         if (LIST) {
@@ -347,7 +345,7 @@ __device__ __forceinline__ bool scan_row(const ScanArgs& a, SeqSum& st, BlockScr
           }
         }
       }
-      if (seq_sum_group<kGroup, VE>(st, bits, cur, next, scale, first, V, a.threshold, sm)) return true;
+      if (seq_sum_group<kGroup, VE>(st, bits, acc, scale, first, V, a.threshold, sm)) return true;
     }
     done_elems = vbase * VE;
   }
@@ -372,20 +370,6 @@ __device__ __forceinline__ bool scan_row(const ScanArgs& a, SeqSum& st, BlockScr
     if (seq_sum_chunk<VE>(st, bits, first, V, a.threshold, sm)) return true;
   }
   return false;
-}
-
-constexpr int kSelCap = 1024;   // small selection buffer for peaked rows
-constexpr int kHistBins = 512;  // probability histogram used to pre-select the nucleus
-
-struct NucleusScratch {
-  uint64_t sel[kSelCap];
-  float hist_mass[kHistBins];
-  uint32_t hist_count[kHistBins];
-};
-
-__device__ __forceinline__ int prob_bin(float p, int bin0) {
-  int bin = static_cast<int>(__float_as_uint(p) >> 19) - bin0;
-  return bin < 0 ? 0 : (bin >= kHistBins ? kHistBins - 1 : bin);
 }
 
 // General path: every candidate (top-p: p >= cutoff; top-k: the whole row, sampler.cpp:87-100)
@@ -425,181 +409,129 @@ __device__ int32_t draw_general(const char* logits, int V, float inv, float m, f
   return static_cast<int32_t>(static_cast<uint32_t>(keys[pos]));
 }
 
-// Top-p draw from the listed possible candidates (sampler.cpp:122-171).  Returns false when the
-// true candidates do not fit in LDS (the caller then takes the general path).
-__device__ bool draw_topp_listed(const uint64_t* list, int n_listed, float S, float cutoff, float topp,
-                                              float coin, uint64_t* scratch, uint64_t* lds_keys, int cap,
-                                              RowDebug& dbg, int32_t& token, BlockScratch& sm, NucleusScratch& ns) {
+// Workgroup sum of two floats per lane (DPP inside the wave, LDS across waves, one barrier).
+__device__ __forceinline__ void block_sum2(float& x, float& y, BlockScratch& sm, uint32_t& buf) {
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  x = wave_sum_f32(x);
+  y = wave_sum_f32(y);
+  if (lane == 0) {
+    sm.group_total[buf][wave] = x;
+    sm.aux_total[buf][wave] = y;
+  }
+  __syncthreads();
+  x = 0.0f;
+  y = 0.0f;
+#pragma unroll
+  for (int w = 0; w < kWaves; ++w) {
+    x += sm.group_total[buf][w];
+    y += sm.aux_total[buf][w];
+  }
+  buf ^= 1u;
+}
+
+// Top-p draw from the listed possible candidates (sampler.cpp:122-171).
+//   A. exact filter p = fl(e / S) >= cutoff (sampler.cpp:137-143); the list is rewritten in place
+//      as (p_bits << 32 | index), 0 for dropped entries;
+//   B. a probability threshold tau = p_max / 4^k is lowered until the entries above it carry
+//      safely more than topp (any-order float sums with a 0.4 % margin): the nucleus is among them;
+//   C. only those entries are sorted (bitonic, in LDS) and the reference's two CDF walks run over
+//      them; if they turn out not to reach topp after all, every candidate is sorted instead.
+// Returns false when the entries to sort do not fit in LDS (the caller takes the general path).
+__device__ bool draw_topp_listed(uint64_t* list, int n_listed, float S, float cutoff, float topp, float coin,
+                                 uint64_t* lds_keys, int cap, RowDebug& dbg, int32_t& token, BlockScratch& sm) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
-  // ---- exact filter p >= cutoff (sampler.cpp:137-143) into LDS, and a histogram of probability
-  // mass by magnitude that tells where the nucleus must end
-  for (int b = tid; b < kHistBins; b += kBlock) {
-    ns.hist_mass[b] = 0.0f;
-    ns.hist_count[b] = 0u;
+  uint32_t buf = 0u;
+  // ---- A
+  float cnt = 0.0f, mass = 0.0f;
+  for (int j = tid; j < n_listed; j += kBlock) {
+    const uint64_t ent = list[j];
+    const float pj = __uint_as_float(static_cast<uint32_t>(ent >> 32)) / S;
+    const bool keep = pj >= cutoff;
+    list[j] = keep ? ((static_cast<uint64_t>(__float_as_uint(pj)) << 32) | static_cast<uint32_t>(ent)) : 0ull;
+    cnt += keep ? 1.0f : 0.0f;
+    mass += keep ? pj : 0.0f;
   }
-  if (tid == 0) sm.counter2 = 0u;
-  __syncthreads();
-  const int bin0 = static_cast<int>(__float_as_uint(cutoff) >> 19);
-  for (int base = 0; base < n_listed; base += kBlock) {
-    const int j = base + tid;
-    bool keep = false;
-    float pj = 0.0f;
-    uint32_t idx = 0;
-    if (j < n_listed) {
-      const uint64_t ent = list[j];
-      pj = __uint_as_float(static_cast<uint32_t>(ent >> 32)) / S;
-      idx = static_cast<uint32_t>(ent);
-      keep = pj >= cutoff;
-    }
-    const uint32_t slot = wave_append_slot(keep, &sm.counter2, lane);
-    if (keep) {
-      if (slot < static_cast<uint32_t>(cap)) lds_keys[slot] = cand_key(pj, static_cast<int>(idx));
-      const int bin = prob_bin(pj, bin0);
-      atomicAdd(&ns.hist_mass[bin], pj);
-      atomicAdd(&ns.hist_count[bin], 1u);
-    }
-  }
-  __syncthreads();
-  const int n0 = static_cast<int>(sm.counter2);
+  block_sum2(cnt, mass, sm, buf);
+  const int n0 = static_cast<int>(cnt);
   dbg.n_candidates = n0;
-  if (n0 > cap) return false;
   if (n0 == 0) {
     token = -1;  // the reference reads probindex[-1] here
     return true;
   }
-  // ---- wave 0 walks the bins from the largest probabilities down until the mass is safely above
-  // topp; everything in those bins is selected for sorting
-  if (wave == 0) {
-    constexpr int per = kHistBins / 64;
-    float mass[per];
-    uint32_t cnt[per];
-    float lane_mass = 0.0f;
-    uint32_t lane_cnt = 0;
-#pragma unroll
-    for (int q = 0; q < per; ++q) {
-      const int bin = kHistBins - 1 - (lane * per + q);
-      mass[q] = ns.hist_mass[bin];
-      cnt[q] = ns.hist_count[bin];
-      lane_mass += mass[q];
-      lane_cnt += cnt[q];
-    }
-    float incl_m = lane_mass;
-    uint32_t incl_c = lane_cnt;
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-      const float om = __shfl_up(incl_m, d);
-      const uint32_t oc = __shfl_up(incl_c, d);
-      if (lane >= d) {
-        incl_m += om;
-        incl_c += oc;
+  // ---- B
+  const float target = topp * 1.004f + 1e-6f;
+  float tau = 0.0f;  // select everything
+  int n_sel = n0;
+  if (mass >= target && n0 > 64) {
+    float t = (1.0f / S) * 0.25f;  // the largest probability is fl(1 / S)
+    for (int step = 0; step < 24 && t > cutoff; ++step, t *= 0.25f) {
+      float c = 0.0f, m = 0.0f;
+      for (int j = tid; j < n_listed; j += kBlock) {
+        const float pj = __uint_as_float(static_cast<uint32_t>(list[j] >> 32));
+        const bool in = pj >= t;  // dropped entries hold 0
+        c += in ? 1.0f : 0.0f;
+        m += in ? pj : 0.0f;
+      }
+      block_sum2(c, m, sm, buf);
+      if (m >= target) {
+        tau = t;
+        n_sel = static_cast<int>(c);
+        break;
       }
     }
-    const float target = topp * 1.004f + 1e-6f;
-    const uint64_t hit = __ballot(incl_m >= target);
-    if (hit) {
-      const int hl = __ffsll(static_cast<long long>(hit)) - 1;
-      if (lane == hl) {
-        float run_m = incl_m - lane_mass;
-        uint32_t run_c = incl_c - lane_cnt;
-        int q_hit = per - 1;
-        uint32_t c_hit = incl_c;
-        bool got = false;
-#pragma unroll
-        for (int q = 0; q < per; ++q) {
-          run_m += mass[q];
-          run_c += cnt[q];
-          if (!got && run_m >= target) {
-            got = true;
-            q_hit = q;
-            c_hit = run_c;
-          }
+    // tighten between tau (enough mass) and 4 * tau (not enough): fewer keys to sort
+    if (tau > 0.0f && n_sel > 256) {
+      float hi = tau * 4.0f;
+      for (int step = 0; step < 3; ++step) {
+        const float mid = sqrtf(tau * hi);
+        float c = 0.0f, m = 0.0f;
+        for (int j = tid; j < n_listed; j += kBlock) {
+          const float pj = __uint_as_float(static_cast<uint32_t>(list[j] >> 32));
+          const bool in = pj >= mid;
+          c += in ? 1.0f : 0.0f;
+          m += in ? pj : 0.0f;
         }
-        sm.flag = kHistBins - 1 - (lane * per + q_hit);
-        sm.counter = c_hit;
+        block_sum2(c, m, sm, buf);
+        if (m >= target) {
+          tau = mid;
+          n_sel = static_cast<int>(c);
+        } else {
+          hi = mid;
+        }
       }
-    } else if (lane == 0) {
-      sm.flag = 0;
-      sm.counter = static_cast<uint32_t>(n0);
     }
   }
-  __syncthreads();
-  const int sel_bin = sm.flag;
-  int n_sel = static_cast<int>(sm.counter);
-  __syncthreads();
-  const uint64_t* sorted = nullptr;
-  if (n_sel < n0) {
-    // compact the selected keys: into the small buffer when they fit, else through global memory
-    // and back to the front of the LDS list
-    uint64_t* dst = (n_sel <= kSelCap) ? ns.sel : scratch;
+  // ---- C
+  for (int attempt = 0; attempt < 2; ++attempt) {
+    if (n_sel > cap) return false;
     if (tid == 0) sm.counter2 = 0u;
     __syncthreads();
-    for (int base = 0; base < n0; base += kBlock) {
+    for (int base = 0; base < n_listed; base += kBlock) {
       const int j = base + tid;
-      uint64_t key = 0;
-      bool keep = false;
-      if (j < n0) {
-        key = lds_keys[j];
-        keep = prob_bin(cand_prob(key), bin0) >= sel_bin;
-      }
+      uint64_t ent = 0ull;
+      if (j < n_listed) ent = list[j];
+      const float pj = __uint_as_float(static_cast<uint32_t>(ent >> 32));
+      const bool keep = ent != 0ull && pj >= tau;
       const uint32_t slot = wave_append_slot(keep, &sm.counter2, lane);
-      if (keep) dst[slot] = key;
+      if (keep) lds_keys[slot] = cand_key(pj, static_cast<int>(static_cast<uint32_t>(ent)));
     }
     __syncthreads();
     const int N = pow2_ceil(n_sel);
-    if (n_sel <= kSelCap) {
-      for (int i = n_sel + tid; i < N; i += kBlock) ns.sel[i] = ~0ull;
-      __syncthreads();
-      sort_keys_lds(ns.sel, N);
-      sorted = ns.sel;
-    } else {
-      // the unselected keys are still needed if the selection turns out too small: park them
-      // behind the selected ones in global memory before LDS is overwritten
-      for (int base = 0; base < n0; base += kBlock) {
-        const int j = base + tid;
-        uint64_t key = 0;
-        bool rest = false;
-        if (j < n0) {
-          key = lds_keys[j];
-          rest = prob_bin(cand_prob(key), bin0) < sel_bin;
-        }
-        const uint32_t slot = wave_append_slot(rest, &sm.counter2, lane);
-        if (rest) scratch[slot] = key;
-      }
-      __syncthreads();
-      // selected keys to the front of the LDS list, padded to a power of two with ~0 (the rest
-      // stays parked in global memory)
-      for (int i = tid; i < n_sel; i += kBlock) lds_keys[i] = scratch[i];
-      for (int i = n_sel + tid; i < N; i += kBlock) lds_keys[i] = ~0ull;
-      __syncthreads();
-      sort_keys_lds(lds_keys, N);
-      sorted = lds_keys;
+    for (int i = n_sel + tid; i < N; i += kBlock) lds_keys[i] = ~0ull;
+    __syncthreads();
+    sort_keys_lds(lds_keys, N);
+    const int pos = draw_from_sorted(lds_keys, n_sel, n0, false, 0, topp, coin, dbg, sm);
+    if (pos != -2) {
+      token = static_cast<int32_t>(static_cast<uint32_t>(lds_keys[pos]));
+      return true;
     }
-  } else {
+    tau = 0.0f;  // the pre-selection did not reach topp: take every candidate
     n_sel = n0;
-    const int N = pow2_ceil(n0);
-    for (int i = n0 + tid; i < N; i += kBlock) lds_keys[i] = ~0ull;
     __syncthreads();
-    sort_keys_lds(lds_keys, N);
-    sorted = lds_keys;
   }
-  int pos = draw_from_sorted(sorted, n_sel, n0, false, 0, topp, coin, dbg, sm);
-  if (pos == -2) {
-    // the pre-selected bins did not reach topp after all: sort every candidate
-    if (n_sel > kSelCap) {
-      for (int i = tid; i < n0; i += kBlock) lds_keys[i] = scratch[i];  // selected + parked rest
-      __syncthreads();
-    }
-    const int N = pow2_ceil(n0);
-    for (int i = n0 + tid; i < N; i += kBlock) lds_keys[i] = ~0ull;
-    __syncthreads();
-    sort_keys_lds(lds_keys, N);
-    sorted = lds_keys;
-    pos = draw_from_sorted(sorted, n0, n0, false, 0, topp, coin, dbg, sm);
-  }
-  token = static_cast<int32_t>(static_cast<uint32_t>(sorted[pos]));
-  return true;
+  return false;
 }
 
 // ---- the stochastic path: one workgroup per row -------------------------------------------------
@@ -610,7 +542,6 @@ template <int DT, bool ALIGNED>
 __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
   extern __shared__ __align__(16) uint64_t lds_keys[];
   __shared__ BlockScratch sm;
-  __shared__ NucleusScratch ns;
   constexpr int VE = VecElems<DT>::value;
   const int row = blockIdx.x;
   const int tid = threadIdx.x;
@@ -747,7 +678,7 @@ __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
     dbg.position = token;
   } else {
     bool done = false;
-    if (use_topp) done = draw_topp_listed(scratch, n_listed, S, cutoff, p.topp, coin, scratch, lds_keys, p.lds_keys, dbg, token, sm, ns);
+    if (use_topp) done = draw_topp_listed(scratch, n_listed, S, cutoff, p.topp, coin, lds_keys, p.lds_keys, dbg, token, sm);
     if (!done) {
       token = draw_general<DT>(logits, V, inv, m, S, use_topk, p.topk, p.topp, cutoff, coin, scratch, lds_keys,
                                p.lds_keys, dbg, sm);
@@ -784,22 +715,20 @@ seq_sum_kernel(const float* a, int32_t n, float s0, float threshold, float* sum_
   int base = 0;
   for (; !stopped && base + kGroup * kBlock * R <= n; base += kGroup * kBlock * R) {
     const float scale = fast_scale(st.s);
-    FastAcc cur[kGroup], next[kGroup];
+    FastAcc acc = {0.0f, 0.0f};
     uint32_t bits[kGroup][R];
     int first[kGroup];
 #pragma unroll
     for (int u = 0; u < kGroup; ++u) {
       first[u] = base + (u * kBlock + tid) * R;
-      cur[u] = {0.0f, 0.0f};
-      next[u] = {0.0f, 0.0f};
 #pragma unroll
       for (int e = 0; e < R; ++e) {
         const float v = a[first[u] + e];
         bits[u][e] = __float_as_uint(v);
-        fast_fold2(cur[u], next[u], v, scale);
+        fast_fold(acc, v, scale);
       }
     }
-    stopped = seq_sum_group<kGroup, R>(st, bits, cur, next, scale, first, n, threshold, sm);
+    stopped = seq_sum_group<kGroup, R>(st, bits, acc, scale, first, n, threshold, sm);
   }
   for (; !stopped && base < n; base += kBlock * R) {
     uint32_t bits[R];
