@@ -22,6 +22,11 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 
+# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by
+# the factors a 256 MiB device copy gives in the same runs (profiles/sample_rows_kernel_cfg2.md has
+# the commands and the raw counters): 10796 KiB * 2.00 fetched + 8378 KiB * 1.00 written.
+MEASURED_TRAFFIC_BYTES = {"cfg2": (10796 * 2.00 + 8378 * 1.00) * 1024}
+
 
 def synth_logits_device(w, count, torch, dev):
     """`count` matrices of workload `w`'s distribution generated on the device (same shape,
@@ -185,7 +190,9 @@ def main():
                                f"temperature {w.temperature}, top-p {w.topp}, per-row xorshift64* coins; "
                                f"ring of {ring_len} distinct matrices ({ring_len * step_bytes >> 20} MiB)"},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None, "kernel": "sample_rows_kernel",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES.get(w.name),
+                     "traffic_source": "profiles/sample_rows_kernel_cfg2.md" if w.name in MEASURED_TRAFFIC_BYTES else None,
+                     "kernel": "sample_rows_kernel",
                      "kernel_ms": kernel_ms, "algorithmic_bytes_per_launch": step_bytes},
         "parity": {"rows_checked": rows, "token_mismatches_vs_oracle": mismatches},
     }
