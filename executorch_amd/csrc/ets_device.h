@@ -192,7 +192,8 @@ __device__ __forceinline__ float wave_max_ignoring_nan(float v) {
 // LDS scratch shared by the workgroup-wide primitives.
 struct BlockScratch {
   uint64_t exp2tab[32];
-  ParityInc wave_total[2][kWaves];  // double-buffered, like group_total
+  ParityInc wave_total[2][64];      // per (chunk, wave) slot; double-buffered, like group_total
+  float slot_total[2][64];
   int first_flag[kWaves];
   float group_total[2][kWaves];    // same, for seq_sum_group
   float aux_total[2][kWaves];      // second value of block_sum2
@@ -367,79 +368,93 @@ __device__ void wave_resolve(float& s, int& found, const uint32_t (&bits)[R], in
   }
 }
 
-// Consumes one chunk: lane `tid` owns elements first .. first + R - 1 (global positions, in
-// lane order), given as float bit patterns in bits[] (finite, >= 0; positions >= n must hold 0).
+// Consumes U chunks: in chunk u lane `tid` owns elements first[u] .. first[u] + R - 1 (global
+// positions; chunks in increasing position, lanes in order inside a chunk), given as float bit
+// patterns in bits[u][] (finite, >= 0; positions >= n must hold 0).
 // Emulates  for each element: s += a; if (s > threshold) stop  in fp32, bit for bit.
-// Each round sums the waves' increments in order and finds the first wave that contains an event
-// (a tie, leaving the binade, crossing the threshold); the waves in front of it are committed,
-// that wave resolves its own 64 runs with wave_resolve(), and the next round restarts behind it
-// with the new ulp.  Two barriers per round, one when nothing happens.  Must be called by all
-// lanes; returns true when the threshold was crossed (st.stop_index set).
-template <int R>
-__device__ bool seq_sum_chunk(SeqSum& st, const uint32_t (&bits)[R], int first, int n, float threshold,
-                              BlockScratch& sm) {
+// The U * 16 (chunk, wave) runs are "slots" in position order.  Each round sums the slots'
+// increments in order and finds the first slot that contains an event (a tie, leaving the binade,
+// crossing the threshold); the slots in front of it are committed, its wave resolves its own 64
+// runs with wave_resolve(), and the next round restarts behind it with the new ulp.  Two barriers
+// per round, one when nothing happens.  Must be called by all lanes; returns true when the
+// threshold was crossed (st.stop_index set).
+template <int U, int R>
+__device__ bool seq_sum_rounds(SeqSum& st, const uint32_t (&bits)[U][R], const int (&first)[U], int n, float threshold,
+                               BlockScratch& sm) {
+  static_assert(U * kWaves <= 64, "one lane per slot in the cross-wave scan");
+  constexpr int kSlots = U * kWaves;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const float kBig = 67108864.0f;  // 2^26 marks a wave that must be resolved (tie inside)
-  int resume_wave = 0;             // waves below this have been consumed
+  const float kBig = 67108864.0f;  // 2^26 marks a slot that must be resolved (tie inside)
+  int resume = 0;                  // slots below this have been consumed
   while (true) {
     const float scale = fast_scale(st.s);
     const SumState ss = sum_state(st.s);
     const uint32_t buf = st.parity_buf;
     st.parity_buf ^= 1u;
-    int wstar;
+    int star;
     uint32_t S_front, S_all;
     if (scale != 0.0f) {
-      float wave_inc = 0.0f;
-      if (wave >= resume_wave) {
-        FastAcc acc = {0.0f, 0.0f};
 #pragma unroll
-        for (int e = 0; e < R; ++e) fast_fold(acc, __uint_as_float(bits[e]), scale);
-        const float inc = wave_sum_f32(acc.inc);
-        const bool tie = __ballot(acc.tie == 0.5f) != 0ull;
-        wave_inc = (tie || !(inc < kBig)) ? kBig : inc;
+      for (int u = 0; u < U; ++u) {
+        float slot_inc = 0.0f;
+        if (u * kWaves + wave >= resume) {
+          FastAcc acc = {0.0f, 0.0f};
+#pragma unroll
+          for (int e = 0; e < R; ++e) fast_fold(acc, __uint_as_float(bits[u][e]), scale);
+          const float inc = wave_sum_f32(acc.inc);
+          const bool tie = __ballot(acc.tie == 0.5f) != 0ull;
+          slot_inc = (tie || !(inc < kBig)) ? kBig : inc;
+        }
+        if (lane == 0) sm.slot_total[buf][u * kWaves + wave] = slot_inc;
       }
-      if (lane == 0) sm.group_total[buf][wave] = wave_inc;
       __syncthreads();
-      // every wave redoes the small scan over the 16 wave totals in its first 16 lanes
-      const float wt = lane < kWaves ? sm.group_total[buf][lane] : 0.0f;
+      // every wave redoes the small scan over the slot totals in its first lanes
+      const float wt = lane < kSlots ? sm.slot_total[buf][lane] : 0.0f;
       const float upto = wave_scan_inclusive_f32(wt, lane);
       const float room = static_cast<float>((1u << 24) - ss.S);
       bool event = !(upto < room);
       if (!event) event = sum_value(ss.S + static_cast<uint32_t>(upto), ss.kb) > threshold;
-      const uint64_t ballot = __ballot(event && lane < kWaves);
-      wstar = ballot ? __ffsll(static_cast<long long>(ballot)) - 1 : kWaves;
-      const float front = wstar > 0 && wstar < kWaves ? readlane_f32(upto, wstar - 1) : 0.0f;
-      const float all = readlane_f32(upto, kWaves - 1);
+      const uint64_t ballot = __ballot(event && lane < kSlots);
+      star = ballot ? __ffsll(static_cast<long long>(ballot)) - 1 : kSlots;
+      const float front = star > 0 && star < kSlots ? readlane_f32(upto, star - 1) : 0.0f;
+      const float all = readlane_f32(upto, kSlots - 1);
       S_front = ss.S + static_cast<uint32_t>(front);
       S_all = ss.S + static_cast<uint32_t>(all < room ? all : 0.0f);
     } else {
-      ParityInc mine = {0u, 0u};
-      if (wave >= resume_wave) mine = fold_run<R>(bits, st.s);
-      const ParityInc incl = wave_scan_inclusive(mine, lane);
-      if (lane == 63) sm.wave_total[buf][wave] = incl;
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        ParityInc mine = {0u, 0u};
+        if (u * kWaves + wave >= resume) mine = fold_run<R>(bits[u], st.s);
+        const ParityInc incl = wave_scan_inclusive(mine, lane);
+        if (lane == 63) sm.wave_total[buf][u * kWaves + wave] = incl;
+      }
       __syncthreads();
       ParityInc wt = {0u, 0u};
-      if (lane < kWaves) wt = sm.wave_total[buf][lane];
+      if (lane < kSlots) wt = sm.wave_total[buf][lane];
       const ParityInc upto = wave_scan_inclusive(wt, lane);
       const bool odd = ss.S & 1u;
       const uint32_t S_upto = ss.S + (odd ? upto.odd : upto.even);
       bool event = S_upto >= (1u << 24);
       if (!event) event = sum_value(S_upto, ss.kb) > threshold;
-      const uint64_t ballot = __ballot(event && lane < kWaves);
-      wstar = ballot ? __ffsll(static_cast<long long>(ballot)) - 1 : kWaves;
-      S_front = wstar > 0 && wstar < kWaves ? __shfl(S_upto, wstar - 1) : ss.S;
-      S_all = __shfl(S_upto, kWaves - 1);
+      const uint64_t ballot = __ballot(event && lane < kSlots);
+      star = ballot ? __ffsll(static_cast<long long>(ballot)) - 1 : kSlots;
+      S_front = star > 0 && star < kSlots ? __shfl(S_upto, star - 1) : ss.S;
+      S_all = __shfl(S_upto, kSlots - 1);
     }
-    if (wstar == kWaves) {
+    if (star == kSlots) {
       st.s = sum_value(S_all, ss.kb);
       return false;
     }
-    if (wave == wstar) {
+    if (wave == star % kWaves) {
+      const int ustar = star / kWaves;
       float s = sum_value(S_front, ss.kb);
       int found = -1;
-      wave_resolve<R>(s, found, bits, first, n, threshold);
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        if (u == ustar) wave_resolve<R>(s, found, bits[u], first[u], n, threshold);
+      }
       if (lane == 0) {
         sm.bc_sum = s;
         sm.bc_found = found;
@@ -452,14 +467,25 @@ __device__ bool seq_sum_chunk(SeqSum& st, const uint32_t (&bits)[R], int first, 
       st.stop_index = found;
       return true;
     }
-    resume_wave = wstar + 1;
+    resume = star + 1;
   }
+}
+
+// Single-chunk form.
+template <int R>
+__device__ __forceinline__ bool seq_sum_chunk(SeqSum& st, const uint32_t (&bits)[R], int first, int n, float threshold,
+                                              BlockScratch& sm) {
+  uint32_t b[1][R];
+#pragma unroll
+  for (int e = 0; e < R; ++e) b[0][e] = bits[e];
+  const int f[1] = {first};
+  return seq_sum_rounds<1, R>(st, b, f, n, threshold, sm);
 }
 
 // Consumes U chunks (chunk u: lane `tid` owns elements first[u] .. first[u] + R - 1, chunks in
 // increasing position) with ONE barrier when all of them stay inside the binade of s, below the
 // threshold and free of ties; `acc` must have been folded over the same elements with
-// scale = fast_scale(st.s).  Otherwise the chunks go through seq_sum_chunk one after the other.
+// scale = fast_scale(st.s).  Otherwise the chunks go through seq_sum_rounds.
 template <int U, int R>
 __device__ bool seq_sum_group(SeqSum& st, const uint32_t (&bits)[U][R], FastAcc acc, float scale,
                               const int (&first)[U], int n, float threshold, BlockScratch& sm) {
@@ -484,11 +510,7 @@ __device__ bool seq_sum_group(SeqSum& st, const uint32_t (&bits)[U][R], FastAcc 
       return false;
     }
   }
-#pragma unroll
-  for (int u = 0; u < U; ++u) {
-    if (seq_sum_chunk<R>(st, bits[u], first[u], n, threshold, sm)) return true;
-  }
-  return false;
+  return seq_sum_rounds<U, R>(st, bits, first, n, threshold, sm);
 }
 
 // Whole-array form:  s = s0; for (i < n) { s += a(i); if (s > threshold) return {s, i}; }

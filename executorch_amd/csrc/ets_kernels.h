@@ -277,7 +277,74 @@ struct ScanArgs {
   float threshold;  // kScanWalk: the coin; kScanSum: +inf
   float cutoff;     // kScanSum with listing: the reference's top-p cutoff
   uint64_t* list;   // kScanSum with listing: (exp bits << 32 | index) of possible candidates
+  const float* lut; // bf16 rows: table of expf(x - max) by logit bit pattern (see build_exp_lut)
+  int lut_base1;    //   (first live magnitude) - 1
+  int lut_top;      //   index of the "beyond" slot inside one sign half
+  int lut_half;     //   entries per sign half
 };
+
+// ---- expf by table for bf16 rows ----------------------------------------------------------------
+// A bf16 logit has 65536 possible bit patterns and e = expf(fl(fl(l * inv) - max)) is a function of
+// the pattern alone, so a row needs one exact expf per DISTINCT relevant pattern, not per entry.
+// Relevant magnitudes span a few dozen binades: below them |l * inv| is under an eighth of an ulp of
+// max, so x - max rounds to -max ("tiny" slot); above them a negative logit gives x - max < -104
+// (e == 0, "beyond" slot) and a positive one would exceed the maximum (cannot occur).  Layout per
+// sign half: [0] tiny, [1 .. R] live patterns in increasing magnitude, [R + 1] beyond.
+// Returns false (no table; the caller evaluates expf per entry) when inv or max are not positive
+// finite in the way the bounds need, or when the table would not fit in `cap` floats.
+__device__ bool build_exp_lut(float* lut, int cap, float inv, float m, const uint64_t* tab, int& base1, int& top,
+                              int& half) {
+  const float kInf = __uint_as_float(0x7f800000u);
+  if (!(inv > 0.0f && inv < kInf && m > -kInf && m < kInf)) return false;
+  const uint32_t ib = __float_as_uint(inv);
+  const int ei = static_cast<int>(ib >> 23);  // biased exponent of inv: 2^(ei-127) <= inv < 2^(ei-126)
+  if (ei == 0) return false;
+  const uint32_t mb = __float_as_uint(__builtin_fabsf(m));
+  const int em = (mb >> 23) ? static_cast<int>(mb >> 23) : 1;  // ulp(max) = 2^(em - 150)
+  // tiny: |l| < 2^(E+1-127) and inv < 2^(ei-126) give |l * inv| < 2^(E + ei - 252), to stay below
+  // ulp(max) / 8 = 2^(em - 153)
+  int e_lo = em - ei + 100;  // first live binade (biased exponent of the logit)
+  if (e_lo < 0) e_lo = 0;
+  // beyond: |l| >= 2^(E-127) and inv >= 2^(ei-127) give |l * inv| >= 2^(E + ei - 254), to reach
+  // |max| + 104 < 2^(et - 126) with et the biased exponent of (|max| + 104)
+  const int et = static_cast<int>(__float_as_uint(__builtin_fabsf(m) + 104.0f) >> 23);
+  int e_hi = et - ei + 128;  // last live binade
+  if (e_hi > 254) e_hi = 254;
+  if (e_hi < e_lo) return false;
+  const int R = (e_hi - e_lo + 1) * 128;
+  half = R + 2;
+  top = R + 1;
+  base1 = (e_lo << 7) - 1;
+  if (2 * half > cap) return false;
+  for (int idx = threadIdx.x; idx < 2 * half; idx += kBlock) {
+    const int sgn = idx >= half ? 1 : 0;
+    const int c = idx - sgn * half;
+    float e;
+    if (c == top) {
+      e = 0.0f;
+    } else {
+      float d;
+      if (c == 0) {
+        d = -m;
+      } else {
+        const uint32_t pattern = (static_cast<uint32_t>(sgn) << 15) | static_cast<uint32_t>(base1 + c);
+        const float l = __uint_as_float(pattern << 16);
+        d = l * inv - m;
+      }
+      d = __builtin_fminf(__builtin_fmaxf(d, -104.0f), 0.0f);  // positive only for patterns that cannot occur
+      e = expf_core(d, tab);
+    }
+    lut[idx] = e;
+  }
+  return true;
+}
+
+// Table slot of one bf16 pattern (16 bits: sign, 8 exponent bits, 7 mantissa bits).
+__device__ __forceinline__ int lut_slot(uint32_t mag15, uint32_t sgn, int base1, int top, int half) {
+  int c = static_cast<int>(mag15) - base1;
+  c = c < 0 ? 0 : (c > top ? top : c);
+  return static_cast<int>(sgn) * half + c;
+}
 
 constexpr int kGroup = 2;  // 16-byte vectors per lane between two barriers of the main loop
 
@@ -287,8 +354,9 @@ constexpr int kGroup = 2;  // 16-byte vectors per lane between two barriers of t
 // was crossed.  With LIST, entries whose exp could still reach the cutoff once the normaliser is
 // known (exp >= cutoff * max(1, running sum), with slack) are appended to args.list and counted
 // in sm.counter.
-template <int DT, bool ALIGNED, int MODE, bool LIST>
+template <int DT, bool ALIGNED, int MODE, bool LIST, bool LUT>
 __device__ __forceinline__ bool scan_row(const ScanArgs& a, SeqSum& st, BlockScratch& sm) {
+  static_assert(!LUT || DT == kDtypeBFloat16, "the expf table is indexed by bf16 bit patterns");
   constexpr int VE = VecElems<DT>::value;
   const int tid = threadIdx.x;
   const int V = a.V;
@@ -322,13 +390,24 @@ __device__ __forceinline__ bool scan_row(const ScanArgs& a, SeqSum& st, BlockScr
 #pragma unroll
       for (int u = 0; u < kGroup; ++u) {
         float v[VE];
-        decode_vec<DT>(raw[u], v);
+        if (LUT) {
+          const uint32_t w[4] = {raw[u].x, raw[u].y, raw[u].z, raw[u].w};
+#pragma unroll
+          for (int k = 0; k < 4; ++k) {
+            const float e_lo = a.lut[lut_slot(w[k] & 0x7fffu, (w[k] >> 15) & 1u, a.lut_base1, a.lut_top, a.lut_half)];
+            const float e_hi = a.lut[lut_slot((w[k] >> 16) & 0x7fffu, w[k] >> 31, a.lut_base1, a.lut_top, a.lut_half)];
+            v[2 * k] = MODE == kScanWalk ? e_lo / a.S : e_lo;
+            v[2 * k + 1] = MODE == kScanWalk ? e_hi / a.S : e_hi;
+          }
+        } else {
+          decode_vec<DT>(raw[u], v);
+        }
         if (more) raw[u] = vec[vbase + per_iter + u * kBlock + tid];
         first[u] = (vbase + u * kBlock + tid) * VE;
         uint32_t cmask = 0;
 #pragma unroll
         for (int e = 0; e < VE; ++e) {
-          const float val = value_of(v[e]);
+          const float val = LUT ? v[e] : value_of(v[e]);
           bits[u][e] = __float_as_uint(val);
           fast_fold(acc, val, scale);
           if (LIST && val >= cut_lo) cmask |= 1u << e;
@@ -627,13 +706,34 @@ __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
   // ---- pass 2: softmax normaliser, sequential in index order (sampler.cpp:199-203)
   const float cutoff = use_topp ? (1.0f - p.topp) / static_cast<float>(V - 1) : 0.0f;  // sampler.cpp:136
   float S = kNaN;
+  bool use_lut = false;
+  int lut_base1 = 0, lut_top = 0, lut_half = 0;
+  const float* lut = reinterpret_cast<const float*>(lds_keys);  // the key buffer is free until the draw
+  if (DT == kDtypeBFloat16 && ALIGNED && !row_nan && V >= 4 * kBlock) {
+    use_lut = build_exp_lut(reinterpret_cast<float*>(lds_keys), p.lds_keys * 2, inv, m, sm.exp2tab, lut_base1, lut_top,
+                            lut_half);
+    __syncthreads();
+  }
   if (!row_nan) {
-    ScanArgs a = {logits, V, inv, m, 0.0f, kInf, cutoff, scratch};
+    ScanArgs a = {logits, V, inv, m, 0.0f, kInf, cutoff, scratch, lut, lut_base1, lut_top, lut_half};
     SeqSum st = {0.0f, -1, 0u};
-    if (use_topp) {
-      scan_row<DT, ALIGNED, kScanSum, true>(a, st, sm);
-    } else {
-      scan_row<DT, ALIGNED, kScanSum, false>(a, st, sm);
+    bool scanned = false;
+    if constexpr (DT == kDtypeBFloat16 && ALIGNED) {
+      if (use_lut) {
+        if (use_topp) {
+          scan_row<DT, ALIGNED, kScanSum, true, true>(a, st, sm);
+        } else {
+          scan_row<DT, ALIGNED, kScanSum, false, true>(a, st, sm);
+        }
+        scanned = true;
+      }
+    }
+    if (!scanned) {
+      if (use_topp) {
+        scan_row<DT, ALIGNED, kScanSum, true, false>(a, st, sm);
+      } else {
+        scan_row<DT, ALIGNED, kScanSum, false, false>(a, st, sm);
+      }
     }
     S = st.s;
   }
@@ -670,9 +770,16 @@ __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
     token = use_mult ? V - 1 : -1;
   } else if (use_mult) {
     // ---- sampler.cpp:58-70: first index whose running sum of probabilities exceeds the coin
-    ScanArgs a = {logits, V, inv, m, S, coin, 0.0f, nullptr};
+    ScanArgs a = {logits, V, inv, m, S, coin, 0.0f, nullptr, lut, lut_base1, lut_top, lut_half};
     SeqSum walk = {0.0f, -1, 0u};
-    scan_row<DT, ALIGNED, kScanWalk, false>(a, walk, sm);
+    bool walked = false;
+    if constexpr (DT == kDtypeBFloat16 && ALIGNED) {
+      if (use_lut) {
+        scan_row<DT, ALIGNED, kScanWalk, false, true>(a, walk, sm);
+        walked = true;
+      }
+    }
+    if (!walked) scan_row<DT, ALIGNED, kScanWalk, false, false>(a, walk, sm);
     token = walk.stop_index >= 0 ? walk.stop_index : V - 1;
     dbg.cumulative = walk.s;
     dbg.position = token;
