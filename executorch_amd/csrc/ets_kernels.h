@@ -276,11 +276,14 @@ struct ScanArgs {
   float S;          // kScanWalk: normaliser
   float threshold;  // kScanWalk: the coin; kScanSum: +inf
   float cutoff;     // kScanSum with listing: the reference's top-p cutoff
-  uint64_t* list;   // kScanSum with listing: (exp bits << 32 | index) of possible candidates
+  uint64_t* list;   // kScanSum with listing: (exp bits << 32 | index) of possible candidates;
+                    //   entry j lives in lds_list[j] while j < lds_list_cap, else in list[j]
   const float* lut; // bf16 rows: table of expf(x - max) by logit bit pattern (see build_exp_lut)
   int lut_base1;    //   (first live magnitude) - 1
   int lut_top;      //   index of the "beyond" slot inside one sign half
   int lut_half;     //   entries per sign half
+  uint64_t* lds_list;
+  int lds_list_cap;
 };
 
 // ---- expf by table for bf16 rows ----------------------------------------------------------------
@@ -420,7 +423,12 @@ __device__ __forceinline__ bool scan_row(const ScanArgs& a, SeqSum& st, BlockScr
             uint32_t eb = bits[u][0];
 #pragma unroll
             for (int q = 1; q < VE; ++q) eb = (e == q) ? bits[u][q] : eb;
-            a.list[slot] = (static_cast<uint64_t>(eb) << 32) | static_cast<uint32_t>(first[u] + e);
+            const uint64_t ent = (static_cast<uint64_t>(eb) << 32) | static_cast<uint32_t>(first[u] + e);
+            if (slot < static_cast<uint32_t>(a.lds_list_cap)) {
+              a.lds_list[slot] = ent;
+            } else {
+              a.list[slot] = ent;
+            }
           }
         }
       }
@@ -441,7 +449,12 @@ __device__ __forceinline__ bool scan_row(const ScanArgs& a, SeqSum& st, BlockScr
         val = value_of(load_elem<DT>(a.logits, i));
         if (LIST && val >= cut_lo) {
           const uint32_t slot = atomicAdd(&sm.counter, 1u);
-          a.list[slot] = (static_cast<uint64_t>(__float_as_uint(val)) << 32) | static_cast<uint32_t>(i);
+          const uint64_t ent = (static_cast<uint64_t>(__float_as_uint(val)) << 32) | static_cast<uint32_t>(i);
+          if (slot < static_cast<uint32_t>(a.lds_list_cap)) {
+            a.lds_list[slot] = ent;
+          } else {
+            a.list[slot] = ent;
+          }
         }
       }
       bits[e] = __float_as_uint(val);
@@ -509,30 +522,74 @@ __device__ __forceinline__ void block_sum2(float& x, float& y, BlockScratch& sm,
   buf ^= 1u;
 }
 
-// Top-p draw from the listed possible candidates (sampler.cpp:122-171).
+// Ascending sort of n <= 64 keys at lds[0, n) by the first wave: every lane counts the keys below
+// its own (keys are distinct) and stores its key at that rank.  Ends with a workgroup barrier.
+__device__ void sort_keys_wave(uint64_t* lds, int n) {
+  if (threadIdx.x < 64) {
+    const int lane = threadIdx.x;
+    const uint64_t key = lane < n ? lds[lane] : ~0ull;
+    int rank = 0;
+    for (int j = 0; j < n; ++j) {
+      const uint64_t other = __shfl(static_cast<unsigned long long>(key), j);
+      rank += other < key ? 1 : 0;
+    }
+    if (lane < n) lds[rank] = key;  // all keys were read before the first store (one wave, in step)
+  }
+  __syncthreads();
+}
+
+// Top-p draw from the listed possible candidates (sampler.cpp:122-171).  Entry j of the list sits
+// in lds_list[j] while j < lds_list_cap and in list[j] (global memory) beyond; lds_list is the
+// upper part of the key buffer lds_keys[0, cap), starting at key index `list_base`.
 //   A. exact filter p = fl(e / S) >= cutoff (sampler.cpp:137-143); the list is rewritten in place
 //      as (p_bits << 32 | index), 0 for dropped entries;
 //   B. a probability threshold tau = p_max / 4^k is lowered until the entries above it carry
 //      safely more than topp (any-order float sums with a 0.4 % margin): the nucleus is among them;
-//   C. only those entries are sorted (bitonic, in LDS) and the reference's two CDF walks run over
-//      them; if they turn out not to reach topp after all, every candidate is sorted instead.
-// Returns false when the entries to sort do not fit in LDS (the caller takes the general path).
-__device__ bool draw_topp_listed(uint64_t* list, int n_listed, float S, float cutoff, float topp, float coin,
-                                 uint64_t* lds_keys, int cap, RowDebug& dbg, int32_t& token, BlockScratch& sm) {
+//   C. only those entries are sorted (in LDS) and the reference's two CDF walks run over them.
+// Returns false when the entries to sort do not fit in LDS or, against expectation, do not reach
+// topp (the caller takes the general path).
+__device__ bool draw_topp_listed(uint64_t* list, uint64_t* lds_list, int lds_list_cap, int list_base, int n_listed,
+                                 float S, float cutoff, float topp, float coin, uint64_t* lds_keys, int cap,
+                                 RowDebug& dbg, int32_t& token, BlockScratch& sm) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   uint32_t buf = 0u;
+  const int n_lds = n_listed < lds_list_cap ? n_listed : lds_list_cap;
+  // Calls fn(p) for the probability field of every entry (dropped entries give 0).
+  auto for_each_prob = [&](auto&& fn) {
+    for (int j = tid; j < n_lds; j += kBlock) fn(__uint_as_float(static_cast<uint32_t>(lds_list[j] >> 32)));
+    int j = n_lds + tid;
+    for (; j + 3 * kBlock < n_listed; j += 4 * kBlock) {
+      const uint64_t e0 = list[j], e1 = list[j + kBlock], e2 = list[j + 2 * kBlock], e3 = list[j + 3 * kBlock];
+      fn(__uint_as_float(static_cast<uint32_t>(e0 >> 32)));
+      fn(__uint_as_float(static_cast<uint32_t>(e1 >> 32)));
+      fn(__uint_as_float(static_cast<uint32_t>(e2 >> 32)));
+      fn(__uint_as_float(static_cast<uint32_t>(e3 >> 32)));
+    }
+    for (; j < n_listed; j += kBlock) fn(__uint_as_float(static_cast<uint32_t>(list[j] >> 32)));
+  };
   // ---- A
   float cnt = 0.0f, mass = 0.0f;
-  for (int j = tid; j < n_listed; j += kBlock) {
-    const uint64_t ent = list[j];
-    const float pj = __uint_as_float(static_cast<uint32_t>(ent >> 32)) / S;
-    const bool keep = pj >= cutoff;
-    list[j] = keep ? ((static_cast<uint64_t>(__float_as_uint(pj)) << 32) | static_cast<uint32_t>(ent)) : 0ull;
-    cnt += keep ? 1.0f : 0.0f;
-    mass += keep ? pj : 0.0f;
+  {
+    auto filter = [&](uint64_t ent) -> uint64_t {
+      const float pj = __uint_as_float(static_cast<uint32_t>(ent >> 32)) / S;
+      const bool keep = pj >= cutoff;
+      cnt += keep ? 1.0f : 0.0f;
+      mass += keep ? pj : 0.0f;
+      return keep ? ((static_cast<uint64_t>(__float_as_uint(pj)) << 32) | static_cast<uint32_t>(ent)) : 0ull;
+    };
+    for (int j = tid; j < n_lds; j += kBlock) lds_list[j] = filter(lds_list[j]);
+    int j = n_lds + tid;
+    for (; j + 3 * kBlock < n_listed; j += 4 * kBlock) {
+      const uint64_t e0 = list[j], e1 = list[j + kBlock], e2 = list[j + 2 * kBlock], e3 = list[j + 3 * kBlock];
+      list[j] = filter(e0);
+      list[j + kBlock] = filter(e1);
+      list[j + 2 * kBlock] = filter(e2);
+      list[j + 3 * kBlock] = filter(e3);
+    }
+    for (; j < n_listed; j += kBlock) list[j] = filter(list[j]);
   }
-  block_sum2(cnt, mass, sm, buf);
+  block_sum2(cnt, mass, sm, buf);  // its barrier also orders the rewrites before the reads below
   const int n0 = static_cast<int>(cnt);
   dbg.n_candidates = n0;
   if (n0 == 0) {
@@ -547,12 +604,11 @@ __device__ bool draw_topp_listed(uint64_t* list, int n_listed, float S, float cu
     float t = (1.0f / S) * 0.25f;  // the largest probability is fl(1 / S)
     for (int step = 0; step < 24 && t > cutoff; ++step, t *= 0.25f) {
       float c = 0.0f, m = 0.0f;
-      for (int j = tid; j < n_listed; j += kBlock) {
-        const float pj = __uint_as_float(static_cast<uint32_t>(list[j] >> 32));
-        const bool in = pj >= t;  // dropped entries hold 0
+      for_each_prob([&](float pj) {
+        const bool in = pj >= t;
         c += in ? 1.0f : 0.0f;
         m += in ? pj : 0.0f;
-      }
+      });
       block_sum2(c, m, sm, buf);
       if (m >= target) {
         tau = t;
@@ -566,12 +622,11 @@ __device__ bool draw_topp_listed(uint64_t* list, int n_listed, float S, float cu
       for (int step = 0; step < 3; ++step) {
         const float mid = sqrtf(tau * hi);
         float c = 0.0f, m = 0.0f;
-        for (int j = tid; j < n_listed; j += kBlock) {
-          const float pj = __uint_as_float(static_cast<uint32_t>(list[j] >> 32));
+        for_each_prob([&](float pj) {
           const bool in = pj >= mid;
           c += in ? 1.0f : 0.0f;
           m += in ? pj : 0.0f;
-        }
+        });
         block_sum2(c, m, sm, buf);
         if (m >= target) {
           tau = mid;
@@ -583,34 +638,36 @@ __device__ bool draw_topp_listed(uint64_t* list, int n_listed, float S, float cu
     }
   }
   // ---- C
-  for (int attempt = 0; attempt < 2; ++attempt) {
-    if (n_sel > cap) return false;
-    if (tid == 0) sm.counter2 = 0u;
-    __syncthreads();
-    for (int base = 0; base < n_listed; base += kBlock) {
-      const int j = base + tid;
-      uint64_t ent = 0ull;
-      if (j < n_listed) ent = list[j];
-      const float pj = __uint_as_float(static_cast<uint32_t>(ent >> 32));
-      const bool keep = ent != 0ull && pj >= tau;
-      const uint32_t slot = wave_append_slot(keep, &sm.counter2, lane);
-      if (keep) lds_keys[slot] = cand_key(pj, static_cast<int>(static_cast<uint32_t>(ent)));
-    }
-    __syncthreads();
-    const int N = pow2_ceil(n_sel);
-    for (int i = n_sel + tid; i < N; i += kBlock) lds_keys[i] = ~0ull;
-    __syncthreads();
-    sort_keys_lds(lds_keys, N);
-    const int pos = draw_from_sorted(lds_keys, n_sel, n0, false, 0, topp, coin, dbg, sm);
-    if (pos != -2) {
-      token = static_cast<int32_t>(static_cast<uint32_t>(lds_keys[pos]));
-      return true;
-    }
-    tau = 0.0f;  // the pre-selection did not reach topp: take every candidate
-    n_sel = n0;
-    __syncthreads();
+  const int N = pow2_ceil(n_sel);
+  if (N > cap) return false;
+  if (tid == 0) sm.counter2 = 0u;
+  __syncthreads();
+  // Selected entries move to lds_keys[0, n_sel).  While they fit below the list they are appended
+  // directly; otherwise the move is in place, one barrier per kBlock entries between the reads of
+  // a round and its stores (a round's stores land below the positions it read).
+  const bool in_place = N > list_base;
+  for (int base = 0; base < n_listed; base += kBlock) {
+    const int j = base + tid;
+    uint64_t ent = 0ull;
+    if (j < n_listed) ent = j < lds_list_cap ? lds_list[j] : list[j];
+    if (in_place) __syncthreads();
+    const float pj = __uint_as_float(static_cast<uint32_t>(ent >> 32));
+    const bool keep = ent != 0ull && pj >= tau;
+    const uint32_t slot = wave_append_slot(keep, &sm.counter2, lane);
+    if (keep) lds_keys[slot] = cand_key(pj, static_cast<int>(static_cast<uint32_t>(ent)));
   }
-  return false;
+  __syncthreads();
+  for (int i = n_sel + tid; i < N; i += kBlock) lds_keys[i] = ~0ull;
+  __syncthreads();
+  if (N <= 64) {
+    sort_keys_wave(lds_keys, n_sel);
+  } else {
+    sort_keys_lds(lds_keys, N);
+  }
+  const int pos = draw_from_sorted(lds_keys, n_sel, n0, false, 0, topp, coin, dbg, sm);
+  if (pos == -2) return false;  // the pre-selection did not reach topp after all
+  token = static_cast<int32_t>(static_cast<uint32_t>(lds_keys[pos]));
+  return true;
 }
 
 // ---- the stochastic path: one workgroup per row -------------------------------------------------
@@ -714,8 +771,16 @@ __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
                             lut_half);
     __syncthreads();
   }
+  // top-p candidates are listed in the key buffer above the table (and above room for a short
+  // sorted selection); what does not fit goes to the row's scratch in global memory
+  int list_base = 1024;
+  if (use_lut && lut_half > list_base) list_base = lut_half;  // 2 * lut_half floats
+  if (list_base > p.lds_keys) list_base = p.lds_keys;
+  uint64_t* lds_list = lds_keys + list_base;
+  const int lds_list_cap = p.lds_keys - list_base;
   if (!row_nan) {
-    ScanArgs a = {logits, V, inv, m, 0.0f, kInf, cutoff, scratch, lut, lut_base1, lut_top, lut_half};
+    ScanArgs a = {logits, V,        inv,       m,       0.0f,     kInf,        cutoff, scratch, lut,
+                  lut_base1, lut_top, lut_half, lds_list, lds_list_cap};
     SeqSum st = {0.0f, -1, 0u};
     bool scanned = false;
     if constexpr (DT == kDtypeBFloat16 && ALIGNED) {
@@ -770,7 +835,7 @@ __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
     token = use_mult ? V - 1 : -1;
   } else if (use_mult) {
     // ---- sampler.cpp:58-70: first index whose running sum of probabilities exceeds the coin
-    ScanArgs a = {logits, V, inv, m, S, coin, 0.0f, nullptr, lut, lut_base1, lut_top, lut_half};
+    ScanArgs a = {logits, V, inv, m, S, coin, 0.0f, nullptr, lut, lut_base1, lut_top, lut_half, nullptr, 0};
     SeqSum walk = {0.0f, -1, 0u};
     bool walked = false;
     if constexpr (DT == kDtypeBFloat16 && ALIGNED) {
@@ -785,7 +850,10 @@ __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
     dbg.position = token;
   } else {
     bool done = false;
-    if (use_topp) done = draw_topp_listed(scratch, n_listed, S, cutoff, p.topp, coin, lds_keys, p.lds_keys, dbg, token, sm);
+    if (use_topp) {
+      done = draw_topp_listed(scratch, lds_list, lds_list_cap, list_base, n_listed, S, cutoff, p.topp, coin, lds_keys,
+                              p.lds_keys, dbg, token, sm);
+    }
     if (!done) {
       token = draw_general<DT>(logits, V, inv, m, S, use_topk, p.topk, p.topp, cutoff, coin, scratch, lds_keys,
                                p.lds_keys, dbg, sm);
