@@ -102,17 +102,17 @@ ets_status launch_argmax(ets_sampler* s, const void* d_logits, int32_t batch, in
   return ETS_OK;
 }
 
-template <int DT, bool ALIGNED>
+template <int DT, bool ALIGNED, int DRAW>
 ets_status launch_rows_impl(ets_sampler* s, const ets::RowParams& p, int32_t batch, hipStream_t stream) {
   static std::once_flag once;
   static hipError_t attr_err = hipSuccess;
   const size_t lds = s->lds_bytes;
   std::call_once(once, [&] {
-    attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(&ets::sample_rows_kernel<DT, ALIGNED>),
+    attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(&ets::sample_rows_kernel<DT, ALIGNED, DRAW>),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
   });
   if (attr_err != hipSuccess) return hip_fail(s, attr_err, "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
-  hipLaunchKernelGGL((ets::sample_rows_kernel<DT, ALIGNED>), dim3(batch), dim3(ets::kBlock), lds, stream, p);
+  hipLaunchKernelGGL((ets::sample_rows_kernel<DT, ALIGNED, DRAW>), dim3(batch), dim3(ets::kBlock), lds, stream, p);
   ETS_HIP(s, hipGetLastError());
   return ETS_OK;
 }
@@ -122,7 +122,19 @@ ets_status launch_rows(ets_sampler* s, const ets::RowParams& p, int32_t batch, h
   // 128-bit loads need a 16-byte aligned base and row pitch
   const size_t esz = ets::ElemSize<DT>::value;
   const bool aligned = (reinterpret_cast<uintptr_t>(p.logits) % 16 == 0) && ((static_cast<size_t>(p.row_stride) * esz) % 16 == 0);
-  return aligned ? launch_rows_impl<DT, true>(s, p, batch, stream) : launch_rows_impl<DT, false>(s, p, batch, stream);
+  // which draw follows the softmax (sampler.cpp:238-249): one kernel instantiation each
+  const bool use_topk = p.topk > 0 && p.topk < p.vocab;
+  const bool use_mult = !use_topk && (p.topp <= 0.0f || p.topp >= 1.0f);
+  if (use_topk) {
+    return aligned ? launch_rows_impl<DT, true, ets::kDrawTopK>(s, p, batch, stream)
+                   : launch_rows_impl<DT, false, ets::kDrawTopK>(s, p, batch, stream);
+  }
+  if (use_mult) {
+    return aligned ? launch_rows_impl<DT, true, ets::kDrawMultinomial>(s, p, batch, stream)
+                   : launch_rows_impl<DT, false, ets::kDrawMultinomial>(s, p, batch, stream);
+  }
+  return aligned ? launch_rows_impl<DT, true, ets::kDrawTopP>(s, p, batch, stream)
+                 : launch_rows_impl<DT, false, ets::kDrawTopP>(s, p, batch, stream);
 }
 
 ets_status ensure_scratch(ets_sampler* s) {

@@ -273,12 +273,12 @@ struct ScanArgs {
   int V;
   float inv;
   float m;          // row maximum of x
-  float S;          // kScanWalk: normaliser
+  RowDivisor div;   // kScanWalk: the normaliser S and its reciprocal
   float threshold;  // kScanWalk: the coin; kScanSum: +inf
   float cutoff;     // kScanSum with listing: the reference's top-p cutoff
   uint64_t* list;   // kScanSum with listing: (exp bits << 32 | index) of possible candidates;
                     //   entry j lives in lds_list[j] while j < lds_list_cap, else in list[j]
-  const float* lut; // bf16 rows: table of expf(x - max) by logit bit pattern (see build_exp_lut)
+  float* lut;       // bf16 rows: table of expf(x - max) by logit bit pattern (see build_exp_lut)
   int lut_base1;    //   (first live magnitude) - 1
   int lut_top;      //   index of the "beyond" slot inside one sign half
   int lut_half;     //   entries per sign half
@@ -292,7 +292,9 @@ struct ScanArgs {
 // Relevant magnitudes span a few dozen binades: below them |l * inv| is under an eighth of an ulp of
 // max, so x - max rounds to -max ("tiny" slot); above them a negative logit gives x - max < -104
 // (e == 0, "beyond" slot) and a positive one would exceed the maximum (cannot occur).  Layout per
-// sign half: [0] tiny, [1 .. R] live patterns in increasing magnitude, [R + 1] beyond.
+// sign half: [0] tiny, [1 .. R] live patterns in increasing magnitude, [R + 1] beyond.  An entry is
+// two words: the float e and a counter (zeroed here) that the top-p scan uses as a histogram of the
+// row over the table's entries.
 // Returns false (no table; the caller evaluates expf per entry) when inv or max are not positive
 // finite in the way the bounds need, or when the table would not fit in `cap` floats.
 __device__ bool build_exp_lut(float* lut, int cap, float inv, float m, const uint64_t* tab, int& base1, int& top,
@@ -318,7 +320,7 @@ __device__ bool build_exp_lut(float* lut, int cap, float inv, float m, const uin
   half = R + 2;
   top = R + 1;
   base1 = (e_lo << 7) - 1;
-  if (2 * half > cap) return false;
+  if (4 * half > cap) return false;
   for (int idx = threadIdx.x; idx < 2 * half; idx += kBlock) {
     const int sgn = idx >= half ? 1 : 0;
     const int c = idx - sgn * half;
@@ -337,29 +339,36 @@ __device__ bool build_exp_lut(float* lut, int cap, float inv, float m, const uin
       d = __builtin_fminf(__builtin_fmaxf(d, -104.0f), 0.0f);  // positive only for patterns that cannot occur
       e = expf_core(d, tab);
     }
-    lut[idx] = e;
+    lut[2 * idx] = e;
+    lut[2 * idx + 1] = 0.0f;  // bit pattern of the integer 0
   }
   return true;
 }
 
 // Table slot of one bf16 pattern (16 bits: sign, 8 exponent bits, 7 mantissa bits).
 __device__ __forceinline__ int lut_slot(uint32_t mag15, uint32_t sgn, int base1, int top, int half) {
-  int c = static_cast<int>(mag15) - base1;
-  c = c < 0 ? 0 : (c > top ? top : c);
-  return static_cast<int>(sgn) * half + c;
+  const int c = min(max(static_cast<int>(mag15), base1), base1 + top);
+  return static_cast<int>(__umul24(sgn, static_cast<uint32_t>(half))) + c - base1;
 }
 
 constexpr int kGroup = 2;  // 16-byte vectors per lane between two barriers of the main loop
 
+// What a kScanSum pass records for the top-p draw.
+//   kListNone    nothing
+//   kListAppend  entries whose exp could still reach the cutoff once the normaliser is known
+//                (exp >= cutoff * max(1, running sum), with slack) are appended to the candidate
+//                list and counted in sm.counter
+//   kListHist    (table rows) every entry adds one to its table entry's counter
+constexpr int kListNone = 0, kListAppend = 1, kListHist = 2;
+
 // One pass over the row in index order.  The main loop handles kGroup * kBlock full vectors per
 // iteration without bounds checks (loads for the next iteration are issued before the current one
 // is processed); the remainder goes through a bounds-checked loop.  Returns true if the threshold
-// was crossed.  With LIST, entries whose exp could still reach the cutoff once the normaliser is
-// known (exp >= cutoff * max(1, running sum), with slack) are appended to args.list and counted
-// in sm.counter.
-template <int DT, bool ALIGNED, int MODE, bool LIST, bool LUT>
+// was crossed.
+template <int DT, bool ALIGNED, int MODE, int LIST, bool LUT>
 __device__ __forceinline__ bool scan_row(const ScanArgs& a, SeqSum& st, BlockScratch& sm) {
   static_assert(!LUT || DT == kDtypeBFloat16, "the expf table is indexed by bf16 bit patterns");
+  static_assert(LIST != kListHist || LUT, "the histogram lives in the expf table");
   constexpr int VE = VecElems<DT>::value;
   const int tid = threadIdx.x;
   const int V = a.V;
@@ -371,7 +380,23 @@ __device__ __forceinline__ bool scan_row(const ScanArgs& a, SeqSum& st, BlockScr
     float d = x - m;
     d = __builtin_fmaxf(d, -104.0f);  // expf is 0 below ln(2^-150); the core gives 0 at -104 too
     const float e = expf_core(d, tab);
-    return MODE == kScanWalk ? e / a.S : e;  // sampler.cpp:205-207: a true division
+    return MODE == kScanWalk ? div_row(e, a.div) : e;  // sampler.cpp:205-207: a true division
+  };
+  // table rows: e of one bf16 pattern (and the histogram update)
+  auto table_value = [&](uint32_t mag15, uint32_t sgn) -> float {
+    float* entry = a.lut + 2 * lut_slot(mag15, sgn, a.lut_base1, a.lut_top, a.lut_half);
+    if (LIST == kListHist) atomicAdd(reinterpret_cast<uint32_t*>(entry) + 1, 1u);
+    const float e = entry[0];
+    return MODE == kScanWalk ? div_row(e, a.div) : e;
+  };
+  auto append = [&](uint32_t e_bits, int index) {
+    const uint32_t slot = atomicAdd(&sm.counter, 1u);
+    const uint64_t ent = (static_cast<uint64_t>(e_bits) << 32) | static_cast<uint32_t>(index);
+    if (slot < static_cast<uint32_t>(a.lds_list_cap)) {
+      a.lds_list[slot] = ent;
+    } else {
+      a.list[slot] = ent;
+    }
   };
   if (ALIGNED) {
     const int nvec = V / VE;
@@ -385,7 +410,7 @@ __device__ __forceinline__ bool scan_row(const ScanArgs& a, SeqSum& st, BlockScr
     int vbase = 0;
     for (; vbase + per_iter <= nvec; vbase += per_iter) {
       const float scale = fast_scale(st.s);
-      const float cut_lo = LIST ? a.cutoff * __builtin_fmaxf(st.s, 1.0f) * 0.999f : 0.0f;
+      const float cut_lo = LIST == kListAppend ? a.cutoff * __builtin_fmaxf(st.s, 1.0f) * 0.999f : 0.0f;
       FastAcc acc = {0.0f, 0.0f};
       uint32_t bits[kGroup][VE];
       int first[kGroup];
@@ -397,10 +422,8 @@ __device__ __forceinline__ bool scan_row(const ScanArgs& a, SeqSum& st, BlockScr
           const uint32_t w[4] = {raw[u].x, raw[u].y, raw[u].z, raw[u].w};
 #pragma unroll
           for (int k = 0; k < 4; ++k) {
-            const float e_lo = a.lut[lut_slot(w[k] & 0x7fffu, (w[k] >> 15) & 1u, a.lut_base1, a.lut_top, a.lut_half)];
-            const float e_hi = a.lut[lut_slot((w[k] >> 16) & 0x7fffu, w[k] >> 31, a.lut_base1, a.lut_top, a.lut_half)];
-            v[2 * k] = MODE == kScanWalk ? e_lo / a.S : e_lo;
-            v[2 * k + 1] = MODE == kScanWalk ? e_hi / a.S : e_hi;
+            v[2 * k] = table_value(w[k] & 0x7fffu, (w[k] >> 15) & 1u);
+            v[2 * k + 1] = table_value((w[k] >> 16) & 0x7fffu, w[k] >> 31);
           }
         } else {
           decode_vec<DT>(raw[u], v);
@@ -413,22 +436,16 @@ __device__ __forceinline__ bool scan_row(const ScanArgs& a, SeqSum& st, BlockScr
           const float val = LUT ? v[e] : value_of(v[e]);
           bits[u][e] = __float_as_uint(val);
           fast_fold(acc, val, scale);
-          if (LIST && val >= cut_lo) cmask |= 1u << e;
+          if (LIST == kListAppend && val >= cut_lo) cmask |= 1u << e;
         }
-        if (LIST) {
+        if (LIST == kListAppend) {
           while (cmask) {
             const int e = __ffs(static_cast<int>(cmask)) - 1;
             cmask &= cmask - 1u;
-            const uint32_t slot = atomicAdd(&sm.counter, 1u);
             uint32_t eb = bits[u][0];
 #pragma unroll
             for (int q = 1; q < VE; ++q) eb = (e == q) ? bits[u][q] : eb;
-            const uint64_t ent = (static_cast<uint64_t>(eb) << 32) | static_cast<uint32_t>(first[u] + e);
-            if (slot < static_cast<uint32_t>(a.lds_list_cap)) {
-              a.lds_list[slot] = ent;
-            } else {
-              a.list[slot] = ent;
-            }
+            append(eb, first[u] + e);
           }
         }
       }
@@ -439,23 +456,21 @@ __device__ __forceinline__ bool scan_row(const ScanArgs& a, SeqSum& st, BlockScr
   // remainder (and rows whose base or pitch is not 16-byte aligned)
   for (int base = done_elems; base < V; base += kBlock * VE) {
     const int first = base + tid * VE;
-    const float cut_lo = LIST ? a.cutoff * __builtin_fmaxf(st.s, 1.0f) * 0.999f : 0.0f;
+    const float cut_lo = LIST == kListAppend ? a.cutoff * __builtin_fmaxf(st.s, 1.0f) * 0.999f : 0.0f;
     uint32_t bits[VE];
 #pragma unroll
     for (int e = 0; e < VE; ++e) {
       const int i = first + e;
       float val = 0.0f;
       if (i < V) {
-        val = value_of(load_elem<DT>(a.logits, i));
-        if (LIST && val >= cut_lo) {
-          const uint32_t slot = atomicAdd(&sm.counter, 1u);
-          const uint64_t ent = (static_cast<uint64_t>(__float_as_uint(val)) << 32) | static_cast<uint32_t>(i);
-          if (slot < static_cast<uint32_t>(a.lds_list_cap)) {
-            a.lds_list[slot] = ent;
-          } else {
-            a.list[slot] = ent;
-          }
+        const float l = load_elem<DT>(a.logits, i);
+        if (LUT) {
+          const uint32_t pattern = __float_as_uint(l) >> 16;
+          val = table_value(pattern & 0x7fffu, pattern >> 15);
+        } else {
+          val = value_of(l);
         }
+        if (LIST == kListAppend && val >= cut_lo) append(__float_as_uint(val), i);
       }
       bits[e] = __float_as_uint(val);
     }
@@ -474,6 +489,7 @@ __device__ int32_t draw_general(const char* logits, int V, float inv, float m, f
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const float cut = use_topk ? 0.0f : cutoff;
+  const RowDivisor div = row_divisor(S);
   if (tid == 0) sm.counter = 0u;
   __syncthreads();
   for (int base = 0; base < V; base += kBlock) {
@@ -482,7 +498,7 @@ __device__ int32_t draw_general(const char* logits, int V, float inv, float m, f
     bool keep = false;
     if (i < V) {
       const float x = load_elem<DT>(logits, i) * inv;
-      pi = expf_nonpositive(x - m, sm.exp2tab) / S;
+      pi = div_row(expf_nonpositive(x - m, sm.exp2tab), div);
       keep = pi >= cut;
     }
     const uint32_t slot = wave_append_slot(keep, &sm.counter, lane);
@@ -522,20 +538,67 @@ __device__ __forceinline__ void block_sum2(float& x, float& y, BlockScratch& sm,
   buf ^= 1u;
 }
 
-// Ascending sort of n <= 64 keys at lds[0, n) by the first wave: every lane counts the keys below
-// its own (keys are distinct) and stores its key at that rank.  Ends with a workgroup barrier.
-__device__ void sort_keys_wave(uint64_t* lds, int n) {
+// Sort and both CDF walks (sampler.cpp:150-170) for n <= 64 candidate keys at lds[0, n), done by
+// the first wave in registers: rank by counting, ds_permute into place, then the two scalar loops
+// with the probabilities read lane by lane.  Same contract as draw_from_sorted (returns the sorted
+// position or -2) but `token` is returned directly, since the sorted keys never go back to LDS.
+__device__ int draw_small_wave(const uint64_t* lds, int n, int n_total, float topp, float coin, RowDebug& dbg,
+                               int32_t& token, BlockScratch& sm) {
   if (threadIdx.x < 64) {
     const int lane = threadIdx.x;
     const uint64_t key = lane < n ? lds[lane] : ~0ull;
     int rank = 0;
+    const uint32_t key_hi = static_cast<uint32_t>(key >> 32), key_lo = static_cast<uint32_t>(key);
     for (int j = 0; j < n; ++j) {
-      const uint64_t other = __shfl(static_cast<unsigned long long>(key), j);
+      const uint64_t other = (static_cast<uint64_t>(readlane_u32(key_hi, j)) << 32) | readlane_u32(key_lo, j);
       rank += other < key ? 1 : 0;
     }
-    if (lane < n) lds[rank] = key;  // all keys were read before the first store (one wave, in step)
+    if (lane >= n) rank = lane;  // padding stays where it is; ranks of real keys are < n
+    const uint32_t hi = __builtin_amdgcn_ds_permute(rank * 4, static_cast<int>(key >> 32));
+    const uint32_t lo = __builtin_amdgcn_ds_permute(rank * 4, static_cast<int>(static_cast<uint32_t>(key)));
+    const float prob = __uint_as_float(0xffffffffu - hi);  // cand_prob
+    float s = 0.0f;
+    int found = -1;
+    for (int i = 0; i < n; ++i) {
+      s = s + readlane_f32(prob, i);
+      if (s > topp) {
+        found = i;
+        break;
+      }
+    }
+    int pos = -2;
+    if (found >= 0 || n == n_total) {
+      const int last_idx = found >= 0 ? found : n - 1;
+      const float r = coin * s;  // sampler.cpp:162
+      float c = 0.0f;
+      pos = last_idx;
+      for (int i = 0; i <= last_idx; ++i) {
+        c = c + readlane_f32(prob, i);
+        if (c > r) {
+          pos = i;
+          break;
+        }
+      }
+      if (lane == 0) {
+        sm.flag = last_idx;
+        sm.bc_sum = s;
+        sm.red_f[1] = r;
+        sm.counter = readlane_u32(lo, pos);
+      }
+    }
+    if (lane == 0) sm.bc_found = pos;
   }
   __syncthreads();
+  const int pos = sm.bc_found;
+  if (pos != -2) {
+    dbg.last_idx = sm.flag;
+    dbg.cumulative = sm.bc_sum;
+    dbg.r = sm.red_f[1];
+    dbg.position = pos;
+    token = static_cast<int32_t>(sm.counter);
+  }
+  __syncthreads();
+  return pos;
 }
 
 // Top-p draw from the listed possible candidates (sampler.cpp:122-171).  Entry j of the list sits
@@ -554,6 +617,7 @@ __device__ bool draw_topp_listed(uint64_t* list, uint64_t* lds_list, int lds_lis
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   uint32_t buf = 0u;
+  const RowDivisor div = row_divisor(S);
   const int n_lds = n_listed < lds_list_cap ? n_listed : lds_list_cap;
   // Calls fn(p) for the probability field of every entry (dropped entries give 0).
   auto for_each_prob = [&](auto&& fn) {
@@ -572,7 +636,7 @@ __device__ bool draw_topp_listed(uint64_t* list, uint64_t* lds_list, int lds_lis
   float cnt = 0.0f, mass = 0.0f;
   {
     auto filter = [&](uint64_t ent) -> uint64_t {
-      const float pj = __uint_as_float(static_cast<uint32_t>(ent >> 32)) / S;
+      const float pj = div_row(__uint_as_float(static_cast<uint32_t>(ent >> 32)), div);
       const bool keep = pj >= cutoff;
       cnt += keep ? 1.0f : 0.0f;
       mass += keep ? pj : 0.0f;
@@ -659,12 +723,248 @@ __device__ bool draw_topp_listed(uint64_t* list, uint64_t* lds_list, int lds_lis
   __syncthreads();
   for (int i = n_sel + tid; i < N; i += kBlock) lds_keys[i] = ~0ull;
   __syncthreads();
-  if (N <= 64) {
-    sort_keys_wave(lds_keys, n_sel);
-  } else {
-    sort_keys_lds(lds_keys, N);
-  }
+  if (n_sel <= 64) return draw_small_wave(lds_keys, n_sel, n0, topp, coin, dbg, token, sm) != -2;
+  sort_keys_lds(lds_keys, N);
   const int pos = draw_from_sorted(lds_keys, n_sel, n0, false, 0, topp, coin, dbg, sm);
+  if (pos == -2) return false;  // the pre-selection did not reach topp after all
+  token = static_cast<int32_t>(static_cast<uint32_t>(lds_keys[pos]));
+  return true;
+}
+
+// ---- top-p draw for rows scanned through the expf table ------------------------------------------
+// After a kListHist scan every table entry holds e and the number of row entries with that bit
+// pattern.  Walking the table in order of falling logit value gives, without touching the row,
+// the candidate count (p = fl(e / S) >= cutoff, exact per pattern) and a probability threshold
+// p_thr above which the entries carry safely more than topp.  One more pass over the row
+// (L2-resident) gathers exactly the entries with p >= p_thr as sort keys; they are a prefix of the
+// reference's sorted candidate array, and the two CDF walks run over them.
+
+// Table index of position q in falling-logit order: positive patterns from the largest magnitude
+// down, the positive "tiny" entry, then the negative half from "tiny" to "beyond".
+__device__ __forceinline__ int hist_entry(int q, int top, int half) { return q < half ? top - q : q; }
+
+typedef short short2v __attribute__((ext_vector_type(2)));
+
+// Order key of a bf16 pattern: larger logit <=> larger key (-0 below +0).
+__device__ __forceinline__ int pattern_order(uint32_t pattern16) {
+  const int mag = static_cast<int>(pattern16 & 0x7fffu);
+  return (pattern16 & 0x8000u) ? ~mag : mag;
+}
+
+// Returns false when the caller has to take the general path.
+template <bool ALIGNED>
+__device__ __noinline__ bool draw_topp_hist(const char* logits, int V, float inv, float m, float S, float cutoff, float topp,
+                               float coin, float* lut, int base1, int top, int half, uint64_t* lds_keys, int cap,
+                               RowDebug& dbg, int32_t& token, BlockScratch& sm) {
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const RowDivisor div = row_divisor(S);
+  const uint32_t* lut_u = reinterpret_cast<const uint32_t*>(lut);
+  const float target = topp * 1.004f + 1e-6f;
+  const int Q = 2 * half;
+  constexpr int kMaxRun = 16;  // table positions per lane; the key buffer bounds Q by 16 * kBlock
+  const int run = (Q + kBlock - 1) / kBlock;
+  if (run > kMaxRun) return false;
+  const int q0 = min(Q, tid * run), q1 = min(Q, q0 + run);
+
+  // ---- this lane's run of table positions: p and count of each, candidate mass and count
+  float pq[kMaxRun];
+  uint32_t cq[kMaxRun];
+#pragma unroll
+  for (int k = 0; k < kMaxRun; ++k) {
+    const int q = q0 + k;
+    const int idx = hist_entry(min(q, Q - 1), top, half);  // always a valid entry: no branch around the load
+    const float e = lut[2 * idx];
+    const uint32_t c = lut_u[2 * idx + 1];
+    pq[k] = q < q1 ? e : 0.0f;
+    cq[k] = q < q1 ? c : 0u;
+  }
+  float mass = 0.0f;
+  uint32_t cnt = 0u;
+  int last_cand = -1;
+#pragma unroll
+  for (int k = 0; k < kMaxRun; ++k) {
+    pq[k] = div_row(pq[k], div);
+    if (pq[k] >= cutoff && cq[k] != 0u) {  // positions past the run hold count 0
+      mass += static_cast<float>(cq[k]) * pq[k];
+      cnt += cq[k];
+      last_cand = q0 + k;
+    }
+  }
+  const float upto = wave_scan_inclusive_f32(mass, lane);
+  uint32_t cnt_w = cnt;
+  int last_w = last_cand;
+#pragma unroll
+  for (int d = 32; d > 0; d >>= 1) {
+    cnt_w += __shfl_xor(cnt_w, d);
+    last_w = max(last_w, __shfl_xor(last_w, d));
+  }
+  if (lane == 63) {
+    sm.group_total[0][wave] = upto;
+    sm.red_u[wave] = cnt_w;
+  }
+  if (lane == 0) sm.first_flag[wave] = last_w;
+  if (tid == 0) {
+    sm.bc_found = -1;
+    sm.counter2 = 0u;
+  }
+  __syncthreads();
+  float mass_before = 0.0f, mass_all = 0.0f;
+  uint32_t n0 = 0u;
+  int q_cut = -1, wave_star = -1;
+  for (int w = 0; w < kWaves; ++w) {
+    if (w == wave) mass_before = mass_all;
+    mass_all += sm.group_total[0][w];
+    n0 += sm.red_u[w];
+    q_cut = max(q_cut, sm.first_flag[w]);
+    if (wave_star < 0 && mass_all >= target) wave_star = w;
+  }
+  dbg.n_candidates = static_cast<int>(n0);
+  if (n0 == 0u) {
+    token = -1;  // the reference reads probindex[-1] here
+    return true;
+  }
+  // ---- the lane whose run takes the mass past the target fixes p_thr and how far the table
+  //      positions with p >= p_thr reach (q_ext); without such a lane every candidate is taken
+  const bool take_all = wave_star < 0 || n0 <= 64u;
+  if (!take_all && wave == wave_star) {
+    const float hi = mass_before + upto;  // any-order float sums: the margin in `target` covers them
+    const uint64_t ballot = __ballot(hi >= target);
+    const int lane_star = __ffsll(static_cast<long long>(ballot)) - 1;  // lane 63 reaches it at the latest
+    const float lo = mass_before + lane_before_f32(upto);
+    if (lane == lane_star) {
+      float running = lo;
+      int q_star = -1;
+      float p_thr = 0.0f;
+      bool reached = false;
+#pragma unroll
+      for (int k = 0; k < kMaxRun; ++k) {
+        if (!reached && pq[k] >= cutoff && cq[k] != 0u) {
+          running += static_cast<float>(cq[k]) * pq[k];
+          q_star = q0 + k;
+          p_thr = pq[k];
+          reached = running >= target;
+        }
+      }
+      int q_ext = q_star;
+      for (int q = q_star + 1; q_star >= 0 && q < Q; ++q) {
+        const int idx = hist_entry(q, top, half);
+        if (!(div_row(lut[2 * idx], div) >= p_thr)) break;
+        q_ext = q;
+      }
+      if (q_star >= 0) {
+        sm.bc_found = q_ext;
+        sm.bc_sum = p_thr;
+      }
+    }
+  }
+  __syncthreads();
+  int q_ext = sm.bc_found;
+  float p_thr = sm.bc_sum;
+  if (take_all || q_ext < 0) {
+    q_ext = q_cut;
+    p_thr = cutoff;
+  }
+  // ---- nothing behind q_ext may reach p_thr (expf need not be monotone to the last bit); count
+  //      what will be gathered
+  uint32_t n_take = 0u;
+  bool straggler = false;
+#pragma unroll
+  for (int k = 0; k < kMaxRun; ++k) {
+    const bool in = cq[k] != 0u && pq[k] >= p_thr;
+    if (in && q0 + k > q_ext) straggler = true;
+    if (in) n_take += cq[k];
+  }
+#pragma unroll
+  for (int d = 32; d > 0; d >>= 1) n_take += __shfl_xor(n_take, d);
+  const bool wave_straggler = __ballot(straggler) != 0ull;
+  if (lane == 0) {
+    sm.red_u[wave] = n_take;
+    sm.first_flag[wave] = wave_straggler ? 1 : 0;
+  }
+  __syncthreads();
+  uint32_t n_sel = 0u;
+  bool any_straggler = false;
+  for (int w = 0; w < kWaves; ++w) {
+    n_sel += sm.red_u[w];
+    any_straggler = any_straggler || sm.first_flag[w] != 0;
+  }
+  __syncthreads();  // the table is dead from here on: its memory becomes the key buffer
+  if (any_straggler || n_sel > static_cast<uint32_t>(cap) || n_sel == 0u) return false;
+
+  // ---- order key of the last table position taken
+  int k_star;
+  if (q_ext < half) {
+    const int c = top - q_ext;
+    k_star = c >= 1 ? base1 + c : 0;
+  } else {
+    const int c = q_ext - half;
+    const int mag = base1 + c;
+    k_star = c >= top ? -32768 : (mag >= 0 ? -mag - 1 : 0);
+  }
+  // ---- gather: entries with order key >= k_star and p >= p_thr
+  auto take = [&](uint32_t pattern16, int index) {
+    if (pattern_order(pattern16) < k_star) return;
+    const float x = __uint_as_float(pattern16 << 16) * inv;
+    const float pj = div_row(expf_nonpositive(x - m, sm.exp2tab), div);
+    if (pj >= p_thr) {
+      const uint32_t slot = atomicAdd(&sm.counter2, 1u);
+      if (slot < static_cast<uint32_t>(cap)) lds_keys[slot] = cand_key(pj, index);
+    }
+  };
+  int done = 0;
+  if (ALIGNED) {
+    const int nvec = V / 8;
+    const uint4* vec = reinterpret_cast<const uint4*>(logits);
+    auto best_of = [](const uint4& r) -> int {
+      const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+      short2v best = {-32768, -32768};
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const short2v h = __builtin_bit_cast(short2v, w[k]);
+        const short2v key = h ^ ((h >> 15) & static_cast<short>(0x7fff));
+        best = __builtin_elementwise_max(best, key);
+      }
+      return max(static_cast<int>(best.x), static_cast<int>(best.y));
+    };
+    auto visit = [&](const uint4& r, int j) {
+      if (best_of(r) < k_star) return;
+      const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        take(w[k] & 0xffffu, j * 8 + 2 * k);
+        take(w[k] >> 16, j * 8 + 2 * k + 1);
+      }
+    };
+    int j = tid;
+    for (; j < nvec; j += 8 * kBlock) {  // 8 loads in flight; out-of-range ones re-read vec[j]
+      uint4 r[8];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        const int jk = j + k * kBlock;
+        r[k] = vec[jk < nvec ? jk : j];
+      }
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        const int jk = j + k * kBlock;
+        if (jk < nvec) visit(r[k], jk);
+      }
+    }
+    done = nvec * 8;
+  }
+  for (int i = done + tid; i < V; i += kBlock) {
+    take(static_cast<uint32_t>(reinterpret_cast<const uint16_t*>(logits)[i]), i);
+  }
+  __syncthreads();
+  const int n_got = static_cast<int>(sm.counter2);
+  if (n_got > cap || n_got == 0) return false;
+  if (n_got <= 64) return draw_small_wave(lds_keys, n_got, static_cast<int>(n0), topp, coin, dbg, token, sm) != -2;
+  const int N = pow2_ceil(n_got);
+  for (int i = n_got + tid; i < N; i += kBlock) lds_keys[i] = ~0ull;
+  __syncthreads();
+  sort_keys_lds(lds_keys, N);
+  const int pos = draw_from_sorted(lds_keys, n_got, static_cast<int>(n0), false, 0, topp, coin, dbg, sm);
   if (pos == -2) return false;  // the pre-selection did not reach topp after all
   token = static_cast<int32_t>(static_cast<uint32_t>(lds_keys[pos]));
   return true;
@@ -674,7 +974,9 @@ __device__ bool draw_topp_listed(uint64_t* list, uint64_t* lds_list, int lds_lis
 // Pass 1 reads the row from HBM: maximum of x = logit * inv_temperature and whether any x is NaN.
 // Pass 2 re-reads it (L2 / Infinity Cache): exact expf, the sequential sum in index order, and
 // the list of possible top-p candidates.  Then the coin and the draw.
-template <int DT, bool ALIGNED>
+constexpr int kDrawTopP = 0, kDrawMultinomial = 1, kDrawTopK = 2;  // sampler.cpp:238-249, chosen by the host
+
+template <int DT, bool ALIGNED, int DRAW>
 __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
   extern __shared__ __align__(16) uint64_t lds_keys[];
   __shared__ BlockScratch sm;
@@ -693,9 +995,9 @@ __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
   if (tid < 32) sm.exp2tab[tid] = kExp2Table[tid];
   if (tid == 0) sm.counter = 0u;
 
-  const bool use_topk = p.topk > 0 && p.topk < V;
-  const bool use_mult = !use_topk && (p.topp <= 0.0f || p.topp >= 1.0f);
-  const bool use_topp = !use_topk && !use_mult;
+  constexpr bool use_topk = DRAW == kDrawTopK;
+  constexpr bool use_mult = DRAW == kDrawMultinomial;
+  constexpr bool use_topp = DRAW == kDrawTopP;
 
   // ---- pass 1: row maximum (sampler.cpp:231-233, 191-197)
   float m = -kInf;
@@ -765,39 +1067,38 @@ __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
   float S = kNaN;
   bool use_lut = false;
   int lut_base1 = 0, lut_top = 0, lut_half = 0;
-  const float* lut = reinterpret_cast<const float*>(lds_keys);  // the key buffer is free until the draw
+  float* lut = reinterpret_cast<float*>(lds_keys);  // the key buffer is free until the draw
   if (DT == kDtypeBFloat16 && ALIGNED && !row_nan && V >= 4 * kBlock) {
-    use_lut = build_exp_lut(reinterpret_cast<float*>(lds_keys), p.lds_keys * 2, inv, m, sm.exp2tab, lut_base1, lut_top,
-                            lut_half);
+    use_lut = build_exp_lut(lut, p.lds_keys * 2, inv, m, sm.exp2tab, lut_base1, lut_top, lut_half);
     __syncthreads();
   }
-  // top-p candidates are listed in the key buffer above the table (and above room for a short
-  // sorted selection); what does not fit goes to the row's scratch in global memory
+  // Rows without a table list their top-p candidates in the key buffer, above room for a short
+  // sorted selection; what does not fit goes to the row's scratch in global memory.  (Table rows
+  // count bit patterns in the table instead.)
   int list_base = 1024;
-  if (use_lut && lut_half > list_base) list_base = lut_half;  // 2 * lut_half floats
   if (list_base > p.lds_keys) list_base = p.lds_keys;
   uint64_t* lds_list = lds_keys + list_base;
   const int lds_list_cap = p.lds_keys - list_base;
   if (!row_nan) {
-    ScanArgs a = {logits, V,        inv,       m,       0.0f,     kInf,        cutoff, scratch, lut,
+    ScanArgs a = {logits, V,        inv,       m,       row_divisor(1.0f), kInf, cutoff, scratch, lut,
                   lut_base1, lut_top, lut_half, lds_list, lds_list_cap};
     SeqSum st = {0.0f, -1, 0u};
     bool scanned = false;
     if constexpr (DT == kDtypeBFloat16 && ALIGNED) {
       if (use_lut) {
         if (use_topp) {
-          scan_row<DT, ALIGNED, kScanSum, true, true>(a, st, sm);
+          scan_row<DT, ALIGNED, kScanSum, kListHist, true>(a, st, sm);
         } else {
-          scan_row<DT, ALIGNED, kScanSum, false, true>(a, st, sm);
+          scan_row<DT, ALIGNED, kScanSum, kListNone, true>(a, st, sm);
         }
         scanned = true;
       }
     }
     if (!scanned) {
       if (use_topp) {
-        scan_row<DT, ALIGNED, kScanSum, true, false>(a, st, sm);
+        scan_row<DT, ALIGNED, kScanSum, kListAppend, false>(a, st, sm);
       } else {
-        scan_row<DT, ALIGNED, kScanSum, false, false>(a, st, sm);
+        scan_row<DT, ALIGNED, kScanSum, kListNone, false>(a, st, sm);
       }
     }
     S = st.s;
@@ -820,9 +1121,17 @@ __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
 
   if (p.probs) {
     float* probs = p.probs + static_cast<int64_t>(row) * V;
-    for (int i = tid; i < V; i += kBlock) {
-      const float x = load_elem<DT>(logits, i) * inv;
-      probs[i] = expf_nonpositive(x - m, sm.exp2tab) / S;
+    if (row_nan) {
+      for (int i = tid; i < V; i += kBlock) {
+        const float x = load_elem<DT>(logits, i) * inv;
+        probs[i] = expf_nonpositive(x - m, sm.exp2tab) / S;
+      }
+    } else {
+      const RowDivisor div = row_divisor(S);
+      for (int i = tid; i < V; i += kBlock) {
+        const float x = load_elem<DT>(logits, i) * inv;
+        probs[i] = div_row(expf_nonpositive(x - m, sm.exp2tab), div);
+      }
     }
   }
 
@@ -835,22 +1144,29 @@ __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
     token = use_mult ? V - 1 : -1;
   } else if (use_mult) {
     // ---- sampler.cpp:58-70: first index whose running sum of probabilities exceeds the coin
-    ScanArgs a = {logits, V, inv, m, S, coin, 0.0f, nullptr, lut, lut_base1, lut_top, lut_half, nullptr, 0};
+    ScanArgs a = {logits, V, inv, m, row_divisor(S), coin, 0.0f, nullptr, lut, lut_base1, lut_top, lut_half, nullptr, 0};
     SeqSum walk = {0.0f, -1, 0u};
     bool walked = false;
     if constexpr (DT == kDtypeBFloat16 && ALIGNED) {
       if (use_lut) {
-        scan_row<DT, ALIGNED, kScanWalk, false, true>(a, walk, sm);
+        scan_row<DT, ALIGNED, kScanWalk, kListNone, true>(a, walk, sm);
         walked = true;
       }
     }
-    if (!walked) scan_row<DT, ALIGNED, kScanWalk, false, false>(a, walk, sm);
+    if (!walked) scan_row<DT, ALIGNED, kScanWalk, kListNone, false>(a, walk, sm);
     token = walk.stop_index >= 0 ? walk.stop_index : V - 1;
     dbg.cumulative = walk.s;
     dbg.position = token;
   } else {
-    bool done = false;
-    if (use_topp) {
+    bool done = false, tried = false;
+    if constexpr (DT == kDtypeBFloat16 && ALIGNED) {
+      if (use_topp && use_lut) {
+        done = draw_topp_hist<ALIGNED>(logits, V, inv, m, S, cutoff, p.topp, coin, lut, lut_base1, lut_top, lut_half,
+                                       lds_keys, p.lds_keys, dbg, token, sm);
+        tried = true;
+      }
+    }
+    if (use_topp && !tried) {
       done = draw_topp_listed(scratch, lds_list, lds_list_cap, list_base, n_listed, S, cutoff, p.topp, coin, lds_keys,
                               p.lds_keys, dbg, token, sm);
     }

@@ -12,6 +12,31 @@ namespace ets {
 
 constexpr uint32_t kSat = 1u << 26;  // saturation value of integer increments (> 2^24)
 
+// ---- correctly rounded float division by a row constant ----------------------------------------
+// fl(e / S) for e >= 0 and a normal S > 0, from r = double(1) / double(S) computed once per row:
+// the double product e * r is within 2^-52 (relative) of the quotient, while the quotient of two
+// 24-bit significands stays at least 2^-49 away from every rounding boundary of the NORMAL float
+// grid (a boundary has a 25-bit odd significand M, and e = M * S would need 2^24 | significand(S)),
+// so rounding the product to float rounds the quotient correctly.  On the subnormal grid exact
+// ties do occur (e = 3 * 2^-149, S = 6), so results at or below 2^-126 take the division itself.
+struct RowDivisor {
+  float S;
+  double recip;
+};
+
+ETS_HD RowDivisor row_divisor(float S) {
+  RowDivisor d;
+  d.S = S;
+  d.recip = 1.0 / static_cast<double>(S);
+  return d;
+}
+
+ETS_HD float div_row(float e, const RowDivisor& d) {
+  const float p = static_cast<float>(static_cast<double>(e) * d.recip);
+  if (p <= 1.17549435e-38f && e != 0.0f) return e / d.S;  // 2^-126 and below (also NaN-free: p >= 0)
+  return p;
+}
+
 // ---- sequential float sums as an integer scan --------------------------------------------------
 // A scalar loop `s += a[i]` (a[i] >= 0) rounds after every add.  While s stays inside one
 // binade [2^k, 2^(k+1)) every partial sum is an integer multiple of u = ulp(s): writing

@@ -176,6 +176,37 @@ int main() {
   }
   std::printf("chunks: %ld order-free, %ld ordered; scaled vs integer fold differences: %ld\n", g_fast, g_slow, g_fold_diff);
   if (g_fold_diff) ++bad;
+  // div_row against the hardware division: random quotients, exp-like numerators, and the
+  // subnormal grid where exact ties exist
+  {
+    long div_bad = 0, div_cases = 0;
+    auto same = [](float x, float y) { return __builtin_bit_cast(uint32_t, x) == __builtin_bit_cast(uint32_t, y); };
+    auto probe = [&](float e, float S) {
+      const ets::RowDivisor d = ets::row_divisor(S);
+      if (!same(ets::div_row(e, d), e / S)) {
+        if (div_bad < 10) std::printf("div_row(%a, %a) = %a, division gives %a\n", e, S, ets::div_row(e, d), e / S);
+        ++div_bad;
+      }
+      ++div_cases;
+    };
+    for (int i = 0; i < 20000000; ++i) {
+      const uint64_t r = rng();
+      float S = __builtin_bit_cast(float, 0x3f800000u + (uint32_t)(r % (24u << 23)));  // [1, 2^24)
+      float e = __builtin_bit_cast(float, (uint32_t)((r >> 32) % 0x3f800001u));        // [0, 1], denormals too
+      probe(e, S);
+    }
+    for (int i = 0; i < 2000000; ++i) {
+      const float S = (float)(1 + rng() % 4096) * std::ldexp(1.0f, (int)(rng() % 6));
+      probe(std::ldexp((float)(rng() % 100000), -149), S);              // subnormal numerators
+      probe(std::ldexp((float)(1 + rng() % 4096), -126), S);            // quotients around 2^-126
+      probe((float)std::exp(uni(-104, 0)), (float)uni(1, 200000));      // what the sampler divides
+    }
+    for (int k = 1; k < 4096; ++k) {
+      for (int q = 1; q < 64; ++q) probe(std::ldexp((float)(k * q), -149), (float)(2 * q));  // exact ties
+    }
+    std::printf("div_row: %ld cases, %ld mismatches\n", div_cases, div_bad);
+    if (div_bad) ++bad;
+  }
   std::printf("seqsum_host_check: %d cases, %d mismatches\n", cases, bad);
   return bad != 0;
 }
