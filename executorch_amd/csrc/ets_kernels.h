@@ -9,6 +9,8 @@
 // rounding as the scalar loops they replace.
 #pragma once
 
+#include <type_traits>
+
 #include "ets_device.h"
 
 namespace ets {
@@ -326,7 +328,7 @@ __device__ bool build_exp_lut(float* lut, int cap, float inv, float m, const uin
     const int c = idx - sgn * half;
     float e;
     if (c == top) {
-      e = 0.0f;
+      e = sgn ? 0.0f : 1.0f;  // the positive one cannot occur; 1 keeps e falling along the table's logit order
     } else {
       float d;
       if (c == 0) {
@@ -762,34 +764,62 @@ __device__ __noinline__ bool draw_topp_hist(const char* logits, int V, float inv
   const RowDivisor div = row_divisor(S);
   const uint32_t* lut_u = reinterpret_cast<const uint32_t*>(lut);
   const float target = topp * 1.004f + 1e-6f;
-  const int Q = 2 * half;
-  constexpr int kMaxRun = 16;  // table positions per lane; the key buffer bounds Q by 16 * kBlock
+  constexpr int kMaxRun = 16;  // table positions per lane; the key buffer bounds them by 16 * kBlock
+  // Every threshold below is at least the cutoff, and the cutoff is far above 2^-126 (1 - topp is
+  // at least 2^-24 and the vocabulary below 2^31): div_row_above is exact wherever it matters.
+  // ---- how far down the table candidates can sit: e falls along q (up to last-bit wobble of
+  //      expf, far inside the 0.1 % margin), and p >= cutoff needs e >= cutoff * S * (1 - 2^-23)
+  int Q = 2 * half;
+  {
+    const int coarse = (Q + kBlock - 1) / kBlock;
+    if (coarse > kMaxRun) return false;
+    const float e_min = cutoff * S * 0.999f;
+    const int q = tid * coarse;
+    const bool live = q < Q && lut[2 * hist_entry(min(q, Q - 1), top, half)] >= e_min;
+    const uint64_t ballot = __ballot(live);
+    if (lane == 0) sm.red_u[wave] = static_cast<uint32_t>(__popcll(ballot));
+    __syncthreads();
+    uint32_t live_lanes = 0u;
+    for (int w = 0; w < kWaves; ++w) live_lanes += sm.red_u[w];
+    __syncthreads();
+    Q = min(Q, static_cast<int>(live_lanes) * coarse);  // the first position of every later run is below e_min
+  }
   const int run = (Q + kBlock - 1) / kBlock;
-  if (run > kMaxRun) return false;
   const int q0 = min(Q, tid * run), q1 = min(Q, q0 + run);
+  if (Q == 0) {
+    dbg.n_candidates = 0;
+    token = -1;  // the reference reads probindex[-1] here
+    return true;
+  }
 
   // ---- this lane's run of table positions: p and count of each, candidate mass and count
   float pq[kMaxRun];
   uint32_t cq[kMaxRun];
 #pragma unroll
   for (int k = 0; k < kMaxRun; ++k) {
-    const int q = q0 + k;
-    const int idx = hist_entry(min(q, Q - 1), top, half);  // always a valid entry: no branch around the load
-    const float e = lut[2 * idx];
-    const uint32_t c = lut_u[2 * idx + 1];
-    pq[k] = q < q1 ? e : 0.0f;
-    cq[k] = q < q1 ? c : 0u;
+    pq[k] = 0.0f;
+    cq[k] = 0u;
+    if (k < run) {  // uniform
+      const int q = q0 + k;
+      const int idx = hist_entry(min(q, Q - 1), top, half);  // always a valid entry: no branch around the load
+      const float e = lut[2 * idx];
+      const uint32_t c = lut_u[2 * idx + 1];
+      pq[k] = q < q1 ? e : 0.0f;
+      cq[k] = q < q1 ? c : 0u;
+    }
   }
   float mass = 0.0f;
   uint32_t cnt = 0u;
   int last_cand = -1;
 #pragma unroll
   for (int k = 0; k < kMaxRun; ++k) {
-    pq[k] = div_row(pq[k], div);
-    if (pq[k] >= cutoff && cq[k] != 0u) {  // positions past the run hold count 0
-      mass += static_cast<float>(cq[k]) * pq[k];
-      cnt += cq[k];
-      last_cand = q0 + k;
+    if (k < run) {
+      pq[k] = div_row_above(pq[k], div);
+      if (pq[k] >= cutoff && cq[k] != 0u) {  // positions past the run hold count 0
+        mass += static_cast<float>(cq[k]) * pq[k];
+        cnt += cq[k];
+        last_cand = q0 + k;
+      }
     }
   }
   const float upto = wave_scan_inclusive_f32(mass, lane);
@@ -840,7 +870,7 @@ __device__ __noinline__ bool draw_topp_hist(const char* logits, int V, float inv
       bool reached = false;
 #pragma unroll
       for (int k = 0; k < kMaxRun; ++k) {
-        if (!reached && pq[k] >= cutoff && cq[k] != 0u) {
+        if (k < run && !reached && pq[k] >= cutoff && cq[k] != 0u) {
           running += static_cast<float>(cq[k]) * pq[k];
           q_star = q0 + k;
           p_thr = pq[k];
@@ -850,7 +880,7 @@ __device__ __noinline__ bool draw_topp_hist(const char* logits, int V, float inv
       int q_ext = q_star;
       for (int q = q_star + 1; q_star >= 0 && q < Q; ++q) {
         const int idx = hist_entry(q, top, half);
-        if (!(div_row(lut[2 * idx], div) >= p_thr)) break;
+        if (!(div_row_above(lut[2 * idx], div) >= p_thr)) break;
         q_ext = q;
       }
       if (q_star >= 0) {
@@ -872,9 +902,11 @@ __device__ __noinline__ bool draw_topp_hist(const char* logits, int V, float inv
   bool straggler = false;
 #pragma unroll
   for (int k = 0; k < kMaxRun; ++k) {
-    const bool in = cq[k] != 0u && pq[k] >= p_thr;
-    if (in && q0 + k > q_ext) straggler = true;
-    if (in) n_take += cq[k];
+    if (k < run) {
+      const bool in = cq[k] != 0u && pq[k] >= p_thr;
+      if (in && q0 + k > q_ext) straggler = true;
+      if (in) n_take += cq[k];
+    }
   }
 #pragma unroll
   for (int d = 32; d > 0; d >>= 1) n_take += __shfl_xor(n_take, d);
@@ -907,7 +939,7 @@ __device__ __noinline__ bool draw_topp_hist(const char* logits, int V, float inv
   auto take = [&](uint32_t pattern16, int index) {
     if (pattern_order(pattern16) < k_star) return;
     const float x = __uint_as_float(pattern16 << 16) * inv;
-    const float pj = div_row(expf_nonpositive(x - m, sm.exp2tab), div);
+    const float pj = div_row_above(expf_nonpositive(x - m, sm.exp2tab), div);
     if (pj >= p_thr) {
       const uint32_t slot = atomicAdd(&sm.counter2, 1u);
       if (slot < static_cast<uint32_t>(cap)) lds_keys[slot] = cand_key(pj, index);
@@ -917,39 +949,46 @@ __device__ __noinline__ bool draw_topp_hist(const char* logits, int V, float inv
   if (ALIGNED) {
     const int nvec = V / 8;
     const uint4* vec = reinterpret_cast<const uint4*>(logits);
-    auto best_of = [](const uint4& r) -> int {
-      const uint32_t w[4] = {r.x, r.y, r.z, r.w};
-      short2v best = {-32768, -32768};
+    // Vectors are screened by their largest order key.  For a positive threshold the patterns
+    // themselves, read as signed 16-bit numbers, decide (negative logits are negative numbers).
+    auto sweep = [&](auto positive_tag) {
+      constexpr bool kPositive = decltype(positive_tag)::value;
+      auto best_of = [](const uint4& r) -> int {
+        const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+        short2v best = {-32768, -32768};
 #pragma unroll
-      for (int k = 0; k < 4; ++k) {
-        const short2v h = __builtin_bit_cast(short2v, w[k]);
-        const short2v key = h ^ ((h >> 15) & static_cast<short>(0x7fff));
-        best = __builtin_elementwise_max(best, key);
+        for (int k = 0; k < 4; ++k) {
+          const short2v h = __builtin_bit_cast(short2v, w[k]);
+          const short2v key = kPositive ? h : h ^ ((h >> 15) & static_cast<short>(0x7fff));
+          best = __builtin_elementwise_max(best, key);
+        }
+        return max(static_cast<int>(best.x), static_cast<int>(best.y));
+      };
+      for (int j = tid; j < nvec; j += 16 * kBlock) {  // 16 loads in flight; out-of-range ones re-read vec[j]
+        uint4 r[16];
+#pragma unroll
+        for (int k = 0; k < 16; ++k) {
+          const int jk = j + k * kBlock;
+          r[k] = vec[jk < nvec ? jk : j];
+        }
+#pragma unroll
+        for (int k = 0; k < 16; ++k) {
+          const int jk = j + k * kBlock;
+          if (jk < nvec && best_of(r[k]) >= k_star) {
+            const uint32_t w[4] = {r[k].x, r[k].y, r[k].z, r[k].w};
+#pragma unroll
+            for (int h = 0; h < 4; ++h) {
+              take(w[h] & 0xffffu, jk * 8 + 2 * h);
+              take(w[h] >> 16, jk * 8 + 2 * h + 1);
+            }
+          }
+        }
       }
-      return max(static_cast<int>(best.x), static_cast<int>(best.y));
     };
-    auto visit = [&](const uint4& r, int j) {
-      if (best_of(r) < k_star) return;
-      const uint32_t w[4] = {r.x, r.y, r.z, r.w};
-#pragma unroll
-      for (int k = 0; k < 4; ++k) {
-        take(w[k] & 0xffffu, j * 8 + 2 * k);
-        take(w[k] >> 16, j * 8 + 2 * k + 1);
-      }
-    };
-    int j = tid;
-    for (; j < nvec; j += 8 * kBlock) {  // 8 loads in flight; out-of-range ones re-read vec[j]
-      uint4 r[8];
-#pragma unroll
-      for (int k = 0; k < 8; ++k) {
-        const int jk = j + k * kBlock;
-        r[k] = vec[jk < nvec ? jk : j];
-      }
-#pragma unroll
-      for (int k = 0; k < 8; ++k) {
-        const int jk = j + k * kBlock;
-        if (jk < nvec) visit(r[k], jk);
-      }
+    if (k_star > 0) {
+      sweep(std::true_type{});
+    } else {
+      sweep(std::false_type{});
     }
     done = nvec * 8;
   }

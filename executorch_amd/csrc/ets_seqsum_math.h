@@ -31,6 +31,12 @@ ETS_HD RowDivisor row_divisor(float S) {
   return d;
 }
 
+// The same quotient where only results above 2^-126 matter (comparisons against a threshold that
+// is itself above 2^-126): exact there, and at most 2^-126 whenever the true result is.
+ETS_HD float div_row_above(float e, const RowDivisor& d) {
+  return static_cast<float>(static_cast<double>(e) * d.recip);
+}
+
 ETS_HD float div_row(float e, const RowDivisor& d) {
   const float p = static_cast<float>(static_cast<double>(e) * d.recip);
   if (p <= 1.17549435e-38f && e != 0.0f) return e / d.S;  // 2^-126 and below (also NaN-free: p >= 0)

@@ -143,3 +143,72 @@ def test_total_variation_of_draws(dev):
         for _ in range(10):
             counts += np.bincount(s.sample_batch(x).cpu().numpy(), minlength=4)
         assert 0.5 * np.abs(counts / counts.sum() - np.array(target)).sum() < 0.02
+
+
+def compare_rows(oracle, dev, x, dtype, temperature, topp, seed, label):
+    """Tokens and draw internals of one batch against the oracle (stable tie order)."""
+    rows, vocab = x.shape
+    s = ea.Sampler(vocab, temperature, topp, seed, max_batch=rows)
+    states = (np.uint64(seed) + np.arange(rows, dtype=np.uint64)).astype(np.uint64)
+    ddbg = torch.zeros((rows, 8), dtype=torch.int32, device=dev)
+    got = s.sample_batch(to_device(x, dtype, dev), debug_out=ddbg).cpu().numpy()
+    want, ex = oracle.sample_rows(x, dtype, oracle.inv_temperature(temperature), topp, 0, states, mode=oracle.MODE_UPCAST,
+                                  tie=oracle.TIE_STABLE, explain=True, threads=8)
+    assert np.array_equal(got, want), (label, np.nonzero(got != want)[0][:8], got[:8], want[:8])
+    dbg = ea.debug_records(ddbg)
+    for b in range(rows):
+        e = ex[b]
+        assert f32_bits(dbg["sum"][b]) == f32_bits(e.sum), (label, b)
+        if e.branch == oracle.BRANCH_TOPP and want[b] >= 0:
+            assert dbg["n_candidates"][b] == e.n_candidates, (label, b)
+            assert dbg["last_idx"][b] == e.last_idx, (label, b)
+            assert f32_bits(dbg["cumulative"][b]) == f32_bits(e.cumulative), (label, b)
+            assert dbg["position"][b] == e.position, (label, b)
+    assert np.array_equal(s.get_rng_states(rows), states)
+
+
+@pytest.mark.parametrize("vocab", [4096, 4104, 20000, 131072])
+def test_bf16_rows_with_structure(oracle, dev, vocab):
+    """bf16 top-p rows built to stress the table path: few distinct values (the nucleus ends
+    inside a class of equal probabilities), flat rows, signed zeros and tiny magnitudes, logits
+    far enough below the maximum to underflow, and hot / cold temperatures."""
+    rng = np.random.default_rng(vocab)
+    rows = 6
+
+    def few_values(k):
+        vals = rng.standard_normal(k).astype(np.float32) * 3.0
+        return vals[rng.integers(0, k, size=(rows, vocab))]
+
+    def two_level():
+        x = np.full((rows, vocab), -2.0, dtype=np.float32) + rng.standard_normal((rows, vocab)).astype(np.float32) * 0.01
+        for b in range(rows):
+            hot = rng.choice(vocab, size=3 + 5 * b, replace=False)
+            x[b, hot] = 6.0 + rng.standard_normal(hot.size).astype(np.float32)
+        return x
+
+    def tiny():
+        x = rng.standard_normal((rows, vocab)).astype(np.float32) * 1e-30
+        x[:, ::7] = 0.0
+        x[:, 3::11] = -0.0
+        x[:, 5::13] = 1e-38
+        return x
+
+    def wide():
+        return (rng.standard_normal((rows, vocab)) * 40.0).astype(np.float32)
+
+    def negative():
+        return (-50.0 - np.abs(rng.standard_normal((rows, vocab))) * 20.0).astype(np.float32)
+
+    cases = {
+        "few16": few_values(16), "few3": few_values(3), "two_level": two_level(), "tiny": tiny(), "wide": wide(),
+        "negative": negative(), "flat": np.full((rows, vocab), 1.25, dtype=np.float32),
+        "normal": rng.standard_normal((rows, vocab)).astype(np.float32) * 2.0,
+    }
+    seed = 4242
+    for label, xf in cases.items():
+        x = W.to_storage(xf, W.DTYPE_BFLOAT16)
+        for temperature, topp in ((0.6, 0.9), (1.0, 0.5), (0.05, 0.9), (50.0, 0.999), (1.0, 0.02)):
+            if vocab > 50000 and label in ("flat", "few3") and temperature != 0.6:
+                continue  # every entry is a candidate: the full-row sort is slow, once is enough
+            compare_rows(oracle, dev, x, W.DTYPE_BFLOAT16, temperature, topp, seed, (vocab, label, temperature, topp))
+            seed += 17
