@@ -163,17 +163,6 @@ __device__ __forceinline__ float expf_nonpositive(float d, const uint64_t* tab) 
 }
 
 // ---- workgroup-wide primitives ------------------------------------------------------------------
-__device__ __forceinline__ ParityInc wave_scan_inclusive(ParityInc v, int lane) {
-#pragma unroll
-  for (int d = 1; d < 64; d <<= 1) {
-    ParityInc o;
-    o.even = __shfl_up(v.even, d);
-    o.odd = __shfl_up(v.odd, d);
-    if (lane >= d) v = compose(o, v);
-  }
-  return v;
-}
-
 __device__ __forceinline__ uint32_t wave_sum_u32(uint32_t v) {
 #pragma unroll
   for (int d = 32; d > 0; d >>= 1) v += __shfl_xor(v, d);
@@ -193,7 +182,6 @@ __device__ __forceinline__ float wave_max_ignoring_nan(float v) {
 struct BlockScratch {
   uint64_t exp2tab[32];
   ParityInc wave_total[2][64];      // per (chunk, wave) slot; double-buffered, like group_total
-  float slot_total[2][64];
   int first_flag[kWaves];
   float group_total[2][kWaves];    // same, for seq_sum_group
   float aux_total[2][kWaves];      // second value of block_sum2
@@ -257,6 +245,25 @@ __device__ __forceinline__ float wave_scan_inclusive_f32(float v, int /*lane*/) 
   v += dpp_or_zero<0x118, 0xf, 0xf>(v);
   v += dpp_or_zero<0x142, 0xa, 0xf>(v);
   v += dpp_or_zero<0x143, 0xc, 0xf>(v);
+  return v;
+}
+
+// The same scan for parity summaries (compose() is associative, not commutative: the earlier lanes
+// go on the left).  Lanes without a source read the identity {0, 0}.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ ParityInc dpp_parity_or_identity(ParityInc v) {
+  ParityInc r;
+  r.even = __builtin_amdgcn_update_dpp(0u, v.even, CTRL, ROW_MASK, 0xf, false);
+  r.odd = __builtin_amdgcn_update_dpp(0u, v.odd, CTRL, ROW_MASK, 0xf, false);
+  return r;
+}
+__device__ __forceinline__ ParityInc wave_scan_inclusive(ParityInc v, int /*lane*/) {
+  v = compose(dpp_parity_or_identity<0x111, 0xf>(v), v);
+  v = compose(dpp_parity_or_identity<0x112, 0xf>(v), v);
+  v = compose(dpp_parity_or_identity<0x114, 0xf>(v), v);
+  v = compose(dpp_parity_or_identity<0x118, 0xf>(v), v);
+  v = compose(dpp_parity_or_identity<0x142, 0xa>(v), v);
+  v = compose(dpp_parity_or_identity<0x143, 0xc>(v), v);
   return v;
 }
 
@@ -372,11 +379,11 @@ __device__ void wave_resolve(float& s, int& found, const uint32_t (&bits)[R], in
 // positions; chunks in increasing position, lanes in order inside a chunk), given as float bit
 // patterns in bits[u][] (finite, >= 0; positions >= n must hold 0).
 // Emulates  for each element: s += a; if (s > threshold) stop  in fp32, bit for bit.
-// The U * 16 (chunk, wave) runs are "slots" in position order.  Each round sums the slots'
-// increments in order and finds the first slot that contains an event (a tie, leaving the binade,
-// crossing the threshold); the slots in front of it are committed, its wave resolves its own 64
-// runs with wave_resolve(), and the next round restarts behind it with the new ulp.  Two barriers
-// per round, one when nothing happens.  Must be called by all lanes; returns true when the
+// The U * 16 (chunk, wave) runs are "slots" in position order.  Each round composes the slots'
+// parity summaries in order and finds the first slot in which the running sum leaves its binade or
+// crosses the threshold; the slots in front of it are committed, its wave resolves its own 64 runs
+// with wave_resolve(), and the next round restarts behind it with the new ulp.  Two barriers per
+// round, one when nothing happens.  Must be called by all lanes; returns true when the
 // threshold was crossed (st.stop_index set).
 template <int U, int R>
 __device__ bool seq_sum_rounds(SeqSum& st, const uint32_t (&bits)[U][R], const int (&first)[U], int n, float threshold,
@@ -395,42 +402,37 @@ __device__ bool seq_sum_rounds(SeqSum& st, const uint32_t (&bits)[U][R], const i
     st.parity_buf ^= 1u;
     int star;
     uint32_t S_front, S_all;
-    if (scale != 0.0f) {
+    // Every pending slot is summarised as a parity pair.  Without a half-ulp tie among its
+    // elements both entries are the float-summed increment; a slot with ties takes the
+    // two-hypothesis fold, so ties cost no round of their own.
 #pragma unroll
-      for (int u = 0; u < U; ++u) {
-        float slot_inc = 0.0f;
-        if (u * kWaves + wave >= resume) {
+    for (int u = 0; u < U; ++u) {
+      ParityInc slot = {0u, 0u};
+      if (u * kWaves + wave >= resume) {
+        bool by_parity = scale == 0.0f;
+        if (!by_parity) {
           FastAcc acc = {0.0f, 0.0f};
 #pragma unroll
           for (int e = 0; e < R; ++e) fast_fold(acc, __uint_as_float(bits[u][e]), scale);
-          const float inc = wave_sum_f32(acc.inc);
-          const bool tie = __ballot(acc.tie == 0.5f) != 0ull;
-          slot_inc = (tie || !(inc < kBig)) ? kBig : inc;
+          by_parity = __ballot(acc.tie == 0.5f) != 0ull;
+          if (!by_parity) {
+            const float inc = wave_sum_f32(acc.inc);
+            const uint32_t v = inc < kBig ? static_cast<uint32_t>(inc) : kSat;
+            slot.even = v;
+            slot.odd = v;
+          }
         }
-        if (lane == 0) sm.slot_total[buf][u * kWaves + wave] = slot_inc;
+        if (by_parity) {
+          const ParityInc incl = wave_scan_inclusive(fold_run<R>(bits[u], st.s), lane);
+          slot.even = readlane_u32(incl.even, 63);
+          slot.odd = readlane_u32(incl.odd, 63);
+        }
       }
-      __syncthreads();
-      // every wave redoes the small scan over the slot totals in its first lanes
-      const float wt = lane < kSlots ? sm.slot_total[buf][lane] : 0.0f;
-      const float upto = wave_scan_inclusive_f32(wt, lane);
-      const float room = static_cast<float>((1u << 24) - ss.S);
-      bool event = !(upto < room);
-      if (!event) event = sum_value(ss.S + static_cast<uint32_t>(upto), ss.kb) > threshold;
-      const uint64_t ballot = __ballot(event && lane < kSlots);
-      star = ballot ? __ffsll(static_cast<long long>(ballot)) - 1 : kSlots;
-      const float front = star > 0 && star < kSlots ? readlane_f32(upto, star - 1) : 0.0f;
-      const float all = readlane_f32(upto, kSlots - 1);
-      S_front = ss.S + static_cast<uint32_t>(front);
-      S_all = ss.S + static_cast<uint32_t>(all < room ? all : 0.0f);
-    } else {
-#pragma unroll
-      for (int u = 0; u < U; ++u) {
-        ParityInc mine = {0u, 0u};
-        if (u * kWaves + wave >= resume) mine = fold_run<R>(bits[u], st.s);
-        const ParityInc incl = wave_scan_inclusive(mine, lane);
-        if (lane == 63) sm.wave_total[buf][u * kWaves + wave] = incl;
-      }
-      __syncthreads();
+      if (lane == 0) sm.wave_total[buf][u * kWaves + wave] = slot;
+    }
+    __syncthreads();
+    {
+      // every wave redoes the small scan over the slot summaries in its first lanes
       ParityInc wt = {0u, 0u};
       if (lane < kSlots) wt = sm.wave_total[buf][lane];
       const ParityInc upto = wave_scan_inclusive(wt, lane);
@@ -440,8 +442,8 @@ __device__ bool seq_sum_rounds(SeqSum& st, const uint32_t (&bits)[U][R], const i
       if (!event) event = sum_value(S_upto, ss.kb) > threshold;
       const uint64_t ballot = __ballot(event && lane < kSlots);
       star = ballot ? __ffsll(static_cast<long long>(ballot)) - 1 : kSlots;
-      S_front = star > 0 && star < kSlots ? __shfl(S_upto, star - 1) : ss.S;
-      S_all = __shfl(S_upto, kSlots - 1);
+      S_front = star > 0 && star < kSlots ? readlane_u32(S_upto, star - 1) : ss.S;
+      S_all = readlane_u32(S_upto, kSlots - 1);
     }
     if (star == kSlots) {
       st.s = sum_value(S_all, ss.kb);

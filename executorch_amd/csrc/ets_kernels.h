@@ -265,6 +265,22 @@ __device__ int draw_from_sorted(Keys keys, int n_sorted, int n_total, bool use_t
   return pos;
 }
 
+// 32 bits filled with the storage pattern of +inf / -inf.
+template <int DT>
+struct InfPattern;
+template <>
+struct InfPattern<kDtypeFloat> {
+  static constexpr uint32_t plus = 0x7f800000u, minus = 0xff800000u;
+};
+template <>
+struct InfPattern<kDtypeHalf> {
+  static constexpr uint32_t plus = 0x7c007c00u, minus = 0xfc00fc00u;
+};
+template <>
+struct InfPattern<kDtypeBFloat16> {
+  static constexpr uint32_t plus = 0x7f807f80u, minus = 0xff80ff80u;
+};
+
 // What one pass over the row accumulates.
 //   kScanSum   e_i = expf(x_i - max), sequential sum; optionally lists top-p candidates
 //   kScanWalk  p_i = e_i / S, sequential sum until it exceeds the coin (multinomial draw)
@@ -353,6 +369,28 @@ __device__ __forceinline__ int lut_slot(uint32_t mag15, uint32_t sgn, int base1,
   return static_cast<int>(__umul24(sgn, static_cast<uint32_t>(half))) + c - base1;
 }
 
+// The same as the LDS byte address of the entry (8 bytes per entry), in three instructions: clamp,
+// sign * half + bias, shift-add.  lo = base1, hi = base1 + top, half8 = 8 * half,
+// bias = (LDS address of the table) - 8 * base1 (mod 2^32), all loop-invariant.
+typedef __attribute__((address_space(3))) float* LdsF32;
+typedef __attribute__((address_space(3))) uint32_t* LdsU32;
+struct LutAddr {
+  int lo, hi;
+  uint32_t half8, bias;
+};
+__device__ __forceinline__ LutAddr lut_addr_of(float* lut, int base1, int top, int half) {
+  const uint32_t table = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((LdsF32)lut));
+  return {base1, base1 + top, static_cast<uint32_t>(half) * 8u, table - static_cast<uint32_t>(base1) * 8u};
+}
+__device__ __forceinline__ uint32_t lut_entry_address(uint32_t mag15, uint32_t sgn, const LutAddr& t) {
+  int c;
+  uint32_t side, addr;
+  asm("v_med3_i32 %0, %1, %2, %3" : "=v"(c) : "v"(mag15), "v"(t.lo), "v"(t.hi));
+  asm("v_mad_u32_u24 %0, %1, %2, %3" : "=v"(side) : "v"(sgn), "v"(t.half8), "v"(t.bias));
+  asm("v_lshl_add_u32 %0, %1, 3, %2" : "=v"(addr) : "v"(c), "v"(side));
+  return addr;
+}
+
 constexpr int kGroup = 2;  // 16-byte vectors per lane between two barriers of the main loop
 
 // What a kScanSum pass records for the top-p draw.
@@ -360,7 +398,8 @@ constexpr int kGroup = 2;  // 16-byte vectors per lane between two barriers of t
 //   kListAppend  entries whose exp could still reach the cutoff once the normaliser is known
 //                (exp >= cutoff * max(1, running sum), with slack) are appended to the candidate
 //                list and counted in sm.counter
-//   kListHist    (table rows) every entry adds one to its table entry's counter
+//   kListHist    (table rows) entries that pass the same test add one to their table entry's
+//                counter
 constexpr int kListNone = 0, kListAppend = 1, kListHist = 2;
 
 // One pass over the row in index order.  The main loop handles kGroup * kBlock full vectors per
@@ -385,10 +424,16 @@ __device__ __forceinline__ bool scan_row(const ScanArgs& a, SeqSum& st, BlockScr
     return MODE == kScanWalk ? div_row(e, a.div) : e;  // sampler.cpp:205-207: a true division
   };
   // table rows: e of one bf16 pattern (and the histogram update)
-  auto table_value = [&](uint32_t mag15, uint32_t sgn) -> float {
-    float* entry = a.lut + 2 * lut_slot(mag15, sgn, a.lut_base1, a.lut_top, a.lut_half);
-    if (LIST == kListHist) atomicAdd(reinterpret_cast<uint32_t*>(entry) + 1, 1u);
-    const float e = entry[0];
+  const LutAddr lut_addr = lut_addr_of(a.lut, a.lut_base1, a.lut_top, a.lut_half);
+  auto table_count = [&](uint32_t entry_address, float e, float cut_lo) {
+    if (LIST == kListHist && e >= cut_lo) {
+      __hip_atomic_fetch_add((LdsU32)static_cast<uintptr_t>(entry_address + 4u), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+  };
+  auto table_value = [&](uint32_t mag15, uint32_t sgn, float cut_lo) -> float {
+    const uint32_t address = lut_entry_address(mag15, sgn, lut_addr);
+    const float e = *(LdsF32)static_cast<uintptr_t>(address);
+    table_count(address, e, cut_lo);
     return MODE == kScanWalk ? div_row(e, a.div) : e;
   };
   auto append = [&](uint32_t e_bits, int index) {
@@ -404,33 +449,49 @@ __device__ __forceinline__ bool scan_row(const ScanArgs& a, SeqSum& st, BlockScr
     const int nvec = V / VE;
     const uint4* vec = reinterpret_cast<const uint4*>(a.logits);
     constexpr int per_iter = kBlock * kGroup;
+    // The last group of a row may be partial.  Its missing vectors are replaced by logits of
+    // -inf * sign(inv): x = -inf, whose exp is 0 on every path, so they add nothing.
+    const uint32_t filler1 = inv < 0.0f ? InfPattern<DT>::plus : InfPattern<DT>::minus;
+    const uint4 filler = {filler1, filler1, filler1, filler1};
     uint4 raw[kGroup];
-    if (per_iter <= nvec) {
 #pragma unroll
-      for (int u = 0; u < kGroup; ++u) raw[u] = vec[u * kBlock + tid];
-    }
-    int vbase = 0;
-    for (; vbase + per_iter <= nvec; vbase += per_iter) {
+    for (int u = 0; u < kGroup; ++u) raw[u] = vec[min(u * kBlock + tid, nvec - 1)];
+    for (int vbase = 0; vbase < nvec; vbase += per_iter) {
+      if (vbase + per_iter > nvec) {
+#pragma unroll
+        for (int u = 0; u < kGroup; ++u) {
+          if (vbase + u * kBlock + tid >= nvec) raw[u] = filler;
+        }
+      }
       const float scale = fast_scale(st.s);
-      const float cut_lo = LIST == kListAppend ? a.cutoff * __builtin_fmaxf(st.s, 1.0f) * 0.999f : 0.0f;
+      const float cut_lo = LIST != kListNone ? a.cutoff * __builtin_fmaxf(st.s, 1.0f) * 0.999f : 0.0f;
       FastAcc acc = {0.0f, 0.0f};
       uint32_t bits[kGroup][VE];
       int first[kGroup];
-      const bool more = vbase + 2 * per_iter <= nvec;
+      const bool more = vbase + per_iter < nvec;
 #pragma unroll
       for (int u = 0; u < kGroup; ++u) {
         float v[VE];
         if (LUT) {
+          // all eight table reads are issued before the first use of one
           const uint32_t w[4] = {raw[u].x, raw[u].y, raw[u].z, raw[u].w};
+          uint32_t address[VE];
 #pragma unroll
           for (int k = 0; k < 4; ++k) {
-            v[2 * k] = table_value(w[k] & 0x7fffu, (w[k] >> 15) & 1u);
-            v[2 * k + 1] = table_value((w[k] >> 16) & 0x7fffu, w[k] >> 31);
+            address[2 * k] = lut_entry_address(w[k] & 0x7fffu, (w[k] >> 15) & 1u, lut_addr);
+            address[2 * k + 1] = lut_entry_address((w[k] >> 16) & 0x7fffu, w[k] >> 31, lut_addr);
+          }
+#pragma unroll
+          for (int e = 0; e < VE; ++e) v[e] = *(LdsF32)static_cast<uintptr_t>(address[e]);
+#pragma unroll
+          for (int e = 0; e < VE; ++e) {
+            table_count(address[e], v[e], cut_lo);
+            if (MODE == kScanWalk) v[e] = div_row(v[e], a.div);
           }
         } else {
           decode_vec<DT>(raw[u], v);
         }
-        if (more) raw[u] = vec[vbase + per_iter + u * kBlock + tid];
+        if (more) raw[u] = vec[min(vbase + per_iter + u * kBlock + tid, nvec - 1)];
         first[u] = (vbase + u * kBlock + tid) * VE;
         uint32_t cmask = 0;
 #pragma unroll
@@ -453,12 +514,12 @@ __device__ __forceinline__ bool scan_row(const ScanArgs& a, SeqSum& st, BlockScr
       }
       if (seq_sum_group<kGroup, VE>(st, bits, acc, scale, first, V, a.threshold, sm)) return true;
     }
-    done_elems = vbase * VE;
+    done_elems = nvec * VE;
   }
   // remainder (and rows whose base or pitch is not 16-byte aligned)
   for (int base = done_elems; base < V; base += kBlock * VE) {
     const int first = base + tid * VE;
-    const float cut_lo = LIST == kListAppend ? a.cutoff * __builtin_fmaxf(st.s, 1.0f) * 0.999f : 0.0f;
+    const float cut_lo = LIST != kListNone ? a.cutoff * __builtin_fmaxf(st.s, 1.0f) * 0.999f : 0.0f;
     uint32_t bits[VE];
 #pragma unroll
     for (int e = 0; e < VE; ++e) {
@@ -468,7 +529,7 @@ __device__ __forceinline__ bool scan_row(const ScanArgs& a, SeqSum& st, BlockScr
         const float l = load_elem<DT>(a.logits, i);
         if (LUT) {
           const uint32_t pattern = __float_as_uint(l) >> 16;
-          val = table_value(pattern & 0x7fffu, pattern >> 15);
+          val = table_value(pattern & 0x7fffu, pattern >> 15, cut_lo);
         } else {
           val = value_of(l);
         }
@@ -735,7 +796,8 @@ __device__ bool draw_topp_listed(uint64_t* list, uint64_t* lds_list, int lds_lis
 
 // ---- top-p draw for rows scanned through the expf table ------------------------------------------
 // After a kListHist scan every table entry holds e and the number of row entries with that bit
-// pattern.  Walking the table in order of falling logit value gives, without touching the row,
+// pattern, counted at least wherever the entry can be a candidate (the scan skips entries whose e
+// is below the cutoff times the running sum at the time, which only grows).  Walking the table in order of falling logit value gives, without touching the row,
 // the candidate count (p = fl(e / S) >= cutoff, exact per pattern) and a probability threshold
 // p_thr above which the entries carry safely more than topp.  One more pass over the row
 // (L2-resident) gathers exactly the entries with p >= p_thr as sort keys; they are a prefix of the
