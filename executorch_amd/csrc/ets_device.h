@@ -184,6 +184,8 @@ struct BlockScratch {
   ParityInc wave_total[2][64];      // per (chunk, wave) slot; double-buffered, like group_total
   int first_flag[kWaves];
   float group_total[2][kWaves];    // same, for seq_sum_group
+  float slot_sum[64];               // plain float sums per slot (seq_sum_predicted)
+  float chain_s[2];                 // running sum handed from one serial slot to the next
   float aux_total[2][kWaves];      // second value of block_sum2
   float red_f[kWaves];
   uint32_t red_u[kWaves];
@@ -375,6 +377,111 @@ __device__ void wave_resolve(float& s, int& found, const uint32_t (&bits)[R], in
   }
 }
 
+// First attempt at a group of U * 16 slots for a plain sum (no threshold): fold every slot ONCE,
+// with the ulp it is predicted to see, instead of once per binade the running sum passes through.
+//   1. plain float sums per slot give approximate running sums at the slot boundaries;
+//   2. a slot whose two boundaries lie safely inside one binade is "stable" and is folded with that
+//      binade's ulp into a parity summary; the others (a binade boundary inside or near, or sums
+//      too small for the float shortcut) are "serial";
+//   3. the slots are consumed in order from the exact running sum: a run of stable slots by
+//      composing its summaries -- after checking that the exact sum entering it has the predicted
+//      exponent and that the run does not leave the binade, which is all their validity needs --
+//      and a serial slot by wave_resolve() in its own wave, one barrier each.
+// The predictions steer only which work is done; every committed step is exact.  Returns the
+// number of slots consumed (st.s is the exact sum behind them): a failed check stops in front of
+// the offending run, and the caller continues from there with the general rounds.
+template <int U, int R>
+__device__ int seq_sum_predicted(SeqSum& st, const uint32_t (&bits)[U][R], const int (&first)[U], int n, BlockScratch& sm) {
+  static_assert(U * kWaves <= 32, "the serial-slot mask is 32 bits");
+  constexpr int kSlots = U * kWaves;
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const float kInf = __uint_as_float(0x7f800000u);
+  const float kBig = 67108864.0f;
+  // ---- 1
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    float a = 0.0f;
+#pragma unroll
+    for (int e = 0; e < R; ++e) a += __uint_as_float(bits[u][e]);
+    a = wave_sum_f32(a);
+    if (lane == 0) sm.slot_sum[u * kWaves + wave] = a;
+  }
+  __syncthreads();
+  // ---- 2 (every wave, one slot per lane)
+  const float incl = wave_scan_inclusive_f32(lane < kSlots ? sm.slot_sum[lane] : 0.0f, lane);
+  const float s_in = st.s + lane_before_f32(incl);
+  const float s_out = st.s + incl;
+  const uint32_t kb_in = __float_as_uint(s_in) >> 23, kb_out = __float_as_uint(s_out) >> 23;
+  const float edge = __uint_as_float(kb_in << 23);  // 2^(kb_in - 127) <= s_in
+  const bool serial = kb_in != kb_out || kb_in < 70u || kb_in > 250u || s_in < edge * 1.002f || s_out > edge * 1.996f;
+  const uint32_t serial_mask = static_cast<uint32_t>(__ballot(serial && lane < kSlots));
+  const uint32_t buf = st.parity_buf;
+  st.parity_buf ^= 1u;
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const int slot_index = u * kWaves + wave;
+    ParityInc slot = {0u, 0u};
+    if (!((serial_mask >> slot_index) & 1u)) {
+      const uint32_t kb = readlane_u32(kb_in, slot_index);
+      const float scale = __uint_as_float((277u - kb) << 23);  // 2^(150 - kb)
+      FastAcc acc = {0.0f, 0.0f};
+#pragma unroll
+      for (int e = 0; e < R; ++e) fast_fold(acc, __uint_as_float(bits[u][e]), scale);
+      if (__ballot(acc.tie == 0.5f) == 0ull) {
+        const float inc = wave_sum_f32(acc.inc);
+        const uint32_t v = inc < kBig ? static_cast<uint32_t>(inc) : kSat;
+        slot.even = v;
+        slot.odd = v;
+      } else {
+        const ParityInc upto = wave_scan_inclusive(fold_run<R>(bits[u], __uint_as_float(kb << 23)), lane);
+        slot.even = readlane_u32(upto.even, 63);
+        slot.odd = readlane_u32(upto.odd, 63);
+      }
+    }
+    if (lane == 0) sm.wave_total[buf][slot_index] = slot;
+  }
+  __syncthreads();
+  // ---- 3
+  ParityInc mine = {0u, 0u};
+  if (lane < kSlots) mine = sm.wave_total[buf][lane];
+  float s = st.s;
+  int pos = 0;
+  uint32_t hand = 0u;
+  while (pos < kSlots) {
+    const uint32_t ahead = serial_mask >> pos;
+    const int next_serial = ahead ? pos + __ffs(static_cast<int>(ahead)) - 1 : kSlots;
+    if (next_serial > pos) {
+      const SumState ss = sum_state(s);
+      if (static_cast<uint32_t>(ss.kb) != readlane_u32(kb_in, pos)) break;  // not the predicted binade
+      ParityInc in_run = {0u, 0u};
+      if (lane >= pos && lane < next_serial) in_run = mine;
+      const ParityInc upto = wave_scan_inclusive(in_run, lane);
+      const uint32_t total = (ss.S & 1u) ? readlane_u32(upto.odd, 63) : readlane_u32(upto.even, 63);
+      if (ss.S + total >= (1u << 24)) break;  // the run would leave the binade
+      s = sum_value(ss.S + total, ss.kb);
+      pos = next_serial;
+    }
+    if (pos == kSlots) break;
+    if (wave == pos % kWaves) {
+      const int ustar = pos / kWaves;
+      float sw = s;
+      int found = -1;
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        if (u == ustar) wave_resolve<R>(sw, found, bits[u], first[u], n, kInf);
+      }
+      if (lane == 0) sm.chain_s[hand] = sw;
+    }
+    __syncthreads();
+    s = sm.chain_s[hand];
+    hand ^= 1u;
+    ++pos;
+  }
+  st.s = s;
+  return pos;
+}
+
 // Consumes U chunks: in chunk u lane `tid` owns elements first[u] .. first[u] + R - 1 (global
 // positions; chunks in increasing position, lanes in order inside a chunk), given as float bit
 // patterns in bits[u][] (finite, >= 0; positions >= n must hold 0).
@@ -387,14 +494,14 @@ __device__ void wave_resolve(float& s, int& found, const uint32_t (&bits)[R], in
 // threshold was crossed (st.stop_index set).
 template <int U, int R>
 __device__ bool seq_sum_rounds(SeqSum& st, const uint32_t (&bits)[U][R], const int (&first)[U], int n, float threshold,
-                               BlockScratch& sm) {
+                               BlockScratch& sm, int resume = 0) {
   static_assert(U * kWaves <= 64, "one lane per slot in the cross-wave scan");
   constexpr int kSlots = U * kWaves;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const float kBig = 67108864.0f;  // 2^26 marks a slot that must be resolved (tie inside)
-  int resume = 0;                  // slots below this have been consumed
+  // slots below `resume` have been consumed
   while (true) {
     const float scale = fast_scale(st.s);
     const SumState ss = sum_state(st.s);
@@ -512,7 +619,12 @@ __device__ bool seq_sum_group(SeqSum& st, const uint32_t (&bits)[U][R], FastAcc 
       return false;
     }
   }
-  return seq_sum_rounds<U, R>(st, bits, first, n, threshold, sm);
+  int consumed = 0;
+  if (U * kWaves <= 32 && threshold == __uint_as_float(0x7f800000u)) {
+    consumed = seq_sum_predicted<U, R>(st, bits, first, n, sm);
+    if (consumed == U * kWaves) return false;
+  }
+  return seq_sum_rounds<U, R>(st, bits, first, n, threshold, sm, consumed);
 }
 
 // Whole-array form:  s = s0; for (i < n) { s += a(i); if (s > threshold) return {s, i}; }

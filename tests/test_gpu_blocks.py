@@ -105,3 +105,23 @@ def test_seq_sum_half_ulp_ties(dev):
         want = seq_sum_f32(a)
         got = gpu_seq_sum(a, 0.0, np.inf, dev)
         assert got[0].view(np.uint32) == want[0].view(np.uint32)
+
+
+def test_seq_sum_rounding_drift_defeats_prediction(dev):
+    """Addends just above half an ulp of the running sum: every add rounds UP to a whole ulp, so
+    the sequential sum runs ahead of any plain sum of the same numbers and leaves its binade tens
+    of thousands of elements before an estimate from plain sums says so.  Whatever a kernel
+    predicts from such estimates has to be caught by its exact checks."""
+    for s0, addend, n in ((1.98, 0.6 * 2.0 ** -23, 300000), (0.99, 0.55 * 2.0 ** -24, 400000), (3.97, 0.7 * 2.0 ** -22, 250000)):
+        a = np.full(n, np.float32(addend), dtype=np.float32)
+        for thr in (np.inf, s0 * 1.009):
+            want = seq_sum_f32(a, s0, thr)
+            got = gpu_seq_sum(a, s0, thr, dev)
+            assert got[0].view(np.uint32) == want[0].view(np.uint32) and got[1] == want[1], (s0, addend, n, thr, got, want)
+    # and just below half an ulp: every add is absorbed, the plain sums grow
+    a = np.full(300000, np.float32(0.49 * 2.0 ** -23), dtype=np.float32)
+    a[0] = np.float32(1.99)
+    want = seq_sum_f32(a)
+    got = gpu_seq_sum(a, 0.0, np.inf, dev)
+    assert got[0].view(np.uint32) == want[0].view(np.uint32), (got, want)
+    assert want[0] == np.float32(1.99)
