@@ -1112,28 +1112,21 @@ __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
     if (ALIGNED) {
       const int nvec = V / VE;
       const uint4* vec = reinterpret_cast<const uint4*>(logits);
-      int j = tid;
-      for (; j + 3 * kBlock < nvec; j += 4 * kBlock) {
-        const uint4 r0 = vec[j], r1 = vec[j + kBlock], r2 = vec[j + 2 * kBlock], r3 = vec[j + 3 * kBlock];
-        float v[VE];
-        decode_vec<DT>(r0, v);
+      // eight 16-byte loads in flight per lane; out-of-range ones re-read the lane's first vector
+      for (int j = tid; j < nvec; j += 8 * kBlock) {
+        uint4 r[8];
 #pragma unroll
-        for (int e = 0; e < VE; ++e) visit(v[e]);
-        decode_vec<DT>(r1, v);
+        for (int k = 0; k < 8; ++k) {
+          const int jk = j + k * kBlock;
+          r[k] = vec[jk < nvec ? jk : j];
+        }
 #pragma unroll
-        for (int e = 0; e < VE; ++e) visit(v[e]);
-        decode_vec<DT>(r2, v);
+        for (int k = 0; k < 8; ++k) {
+          float v[VE];
+          decode_vec<DT>(r[k], v);
 #pragma unroll
-        for (int e = 0; e < VE; ++e) visit(v[e]);
-        decode_vec<DT>(r3, v);
-#pragma unroll
-        for (int e = 0; e < VE; ++e) visit(v[e]);
-      }
-      for (; j < nvec; j += kBlock) {
-        float v[VE];
-        decode_vec<DT>(vec[j], v);
-#pragma unroll
-        for (int e = 0; e < VE; ++e) visit(v[e]);
+          for (int e = 0; e < VE; ++e) visit(v[e]);
+        }
       }
       for (int i = nvec * VE + tid; i < V; i += kBlock) visit(load_elem<DT>(logits, i));
     } else {
