@@ -38,6 +38,8 @@ SIGNATURES = {
     "ets_sampler_set_topp": (C.c_int32, [C.c_void_p, C.c_float]),
     "ets_sampler_sample": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int32, C.POINTER(C.c_int32)]),
     "ets_sampler_sample_batch": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int64, C.c_void_p, C.c_void_p]),
+    "ets_sampler_sample_batch_configs": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int64, C.c_void_p,
+                                         C.c_void_p, C.c_void_p, C.c_void_p]),
     "ets_sampler_sample_batch_debug": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int64, C.c_void_p,
                                                    C.c_void_p, C.c_void_p, C.c_void_p]),
     "ets_sampler_set_rng_states": (C.c_int32, [C.c_void_p, C.c_int32, C.c_int32, C.c_void_p]),

@@ -40,6 +40,12 @@ struct ets_sampler {
   uint32_t* d_counters = nullptr;  // [max_batch] argmax arrival counters (zero between launches)
   void* d_row = nullptr;           // staging for one host row (vocab * 4 bytes)
   int32_t* d_token = nullptr;      // staging for one token
+  // per-row sampling parameters of ets_sampler_sample_batch_configs(): pinned host staging, its
+  // device copy, and the event that says the last upload has left the staging buffer
+  void* h_stage = nullptr;
+  void* d_stage = nullptr;
+  hipEvent_t stage_event = nullptr;
+  bool stage_pending = false;
   std::string last_error;
 };
 
@@ -88,7 +94,7 @@ struct DeviceGuard {
 
 template <int DT>
 ets_status launch_argmax(ets_sampler* s, const void* d_logits, int32_t batch, int64_t stride, int32_t* d_tokens,
-                         hipStream_t stream) {
+                         hipStream_t stream, const int32_t* d_row_map = nullptr) {
   // Enough workgroups to fill 256 CUs several times over, but no segment under 2048 entries.
   int splits = (2048 + batch - 1) / batch;
   const int max_by_len = (s->vocab + 2047) / 2048;
@@ -97,7 +103,7 @@ ets_status launch_argmax(ets_sampler* s, const void* d_logits, int32_t batch, in
   if (splits < 1) splits = 1;
   dim3 grid(splits, batch);
   hipLaunchKernelGGL((ets::argmax_kernel<DT>), grid, dim3(ets::kArgmaxBlock), 0, stream, d_logits, stride, s->vocab,
-                     s->d_partials, s->d_counters, d_tokens);
+                     s->d_partials, s->d_counters, d_tokens, d_row_map);
   ETS_HIP(s, hipGetLastError());
   return ETS_OK;
 }
@@ -117,14 +123,21 @@ ets_status launch_rows_impl(ets_sampler* s, const ets::RowParams& p, int32_t bat
   return ETS_OK;
 }
 
+// Which draw follows the softmax (sampler.cpp:238-249).
+int draw_mode(int32_t vocab, float topp, int32_t topk) {
+  if (topk > 0 && topk < vocab) return ets::kDrawTopK;
+  if (topp <= 0.0f || topp >= 1.0f) return ets::kDrawMultinomial;
+  return ets::kDrawTopP;
+}
+
 template <int DT>
-ets_status launch_rows(ets_sampler* s, const ets::RowParams& p, int32_t batch, hipStream_t stream) {
+ets_status launch_rows(ets_sampler* s, const ets::RowParams& p, int32_t batch, hipStream_t stream, int draw) {
   // 128-bit loads need a 16-byte aligned base and row pitch
   const size_t esz = ets::ElemSize<DT>::value;
   const bool aligned = (reinterpret_cast<uintptr_t>(p.logits) % 16 == 0) && ((static_cast<size_t>(p.row_stride) * esz) % 16 == 0);
-  // which draw follows the softmax (sampler.cpp:238-249): one kernel instantiation each
-  const bool use_topk = p.topk > 0 && p.topk < p.vocab;
-  const bool use_mult = !use_topk && (p.topp <= 0.0f || p.topp >= 1.0f);
+  // one kernel instantiation per draw
+  const bool use_topk = draw == ets::kDrawTopK;
+  const bool use_mult = draw == ets::kDrawMultinomial;
   if (use_topk) {
     return aligned ? launch_rows_impl<DT, true, ets::kDrawTopK>(s, p, batch, stream)
                    : launch_rows_impl<DT, false, ets::kDrawTopK>(s, p, batch, stream);
@@ -137,6 +150,11 @@ ets_status launch_rows(ets_sampler* s, const ets::RowParams& p, int32_t batch, h
                  : launch_rows_impl<DT, false, ets::kDrawTopP>(s, p, batch, stream);
 }
 
+float inverse_temperature_ctor(float temperature) {
+  // sampler.cpp:178: static_cast<bool>(temperature) ? 1.0f / temperature : 0
+  return (temperature != 0.0f) ? 1.0f / temperature : 0.0f;
+}
+
 ets_status ensure_scratch(ets_sampler* s) {
   if (s->d_scratch) return ETS_OK;
   const size_t bytes = static_cast<size_t>(s->max_batch) * static_cast<size_t>(s->scratch_stride) * sizeof(uint64_t);
@@ -144,26 +162,43 @@ ets_status ensure_scratch(ets_sampler* s) {
   return ETS_OK;
 }
 
+ets_status argmax_device(ets_sampler* s, const void* d_logits, int32_t dtype, int32_t rows, int64_t stride,
+                         int32_t* d_tokens, hipStream_t stream, const int32_t* d_row_map) {
+  switch (dtype) {
+    case ETS_DTYPE_FLOAT:
+      return launch_argmax<ets::kDtypeFloat>(s, d_logits, rows, stride, d_tokens, stream, d_row_map);
+    case ETS_DTYPE_HALF:
+      return launch_argmax<ets::kDtypeHalf>(s, d_logits, rows, stride, d_tokens, stream, d_row_map);
+    case ETS_DTYPE_BFLOAT16:
+      return launch_argmax<ets::kDtypeBFloat16>(s, d_logits, rows, stride, d_tokens, stream, d_row_map);
+    default:
+      return launch_argmax<ets::kDtypeUInt16>(s, d_logits, rows, stride, d_tokens, stream, d_row_map);
+  }
+}
+
+const char* const kUint16Message =
+    "stochastic sampling of UInt16 logits is not supported (integer softmax of the reference degenerates to "
+    "0/1 weights); use temperature 0 or dequantise first";
+
+ets_status rows_device(ets_sampler* s, const ets::RowParams& p, int32_t dtype, int32_t rows, hipStream_t stream,
+                       int draw) {
+  switch (dtype) {
+    case ETS_DTYPE_FLOAT:
+      return launch_rows<ets::kDtypeFloat>(s, p, rows, stream, draw);
+    case ETS_DTYPE_HALF:
+      return launch_rows<ets::kDtypeHalf>(s, p, rows, stream, draw);
+    default:
+      return launch_rows<ets::kDtypeBFloat16>(s, p, rows, stream, draw);
+  }
+}
+
 ets_status sample_device(ets_sampler* s, const void* d_logits, int32_t dtype, int32_t batch, int64_t stride,
                          int32_t* d_tokens, float* d_probs, ets_row_debug* d_debug, hipStream_t stream) {
   if (s->inv_temperature == 0.0f) {
     // greedy: no coin is consumed (sampler.cpp:226-228)
-    switch (dtype) {
-      case ETS_DTYPE_FLOAT:
-        return launch_argmax<ets::kDtypeFloat>(s, d_logits, batch, stride, d_tokens, stream);
-      case ETS_DTYPE_HALF:
-        return launch_argmax<ets::kDtypeHalf>(s, d_logits, batch, stride, d_tokens, stream);
-      case ETS_DTYPE_BFLOAT16:
-        return launch_argmax<ets::kDtypeBFloat16>(s, d_logits, batch, stride, d_tokens, stream);
-      default:
-        return launch_argmax<ets::kDtypeUInt16>(s, d_logits, batch, stride, d_tokens, stream);
-    }
+    return argmax_device(s, d_logits, dtype, batch, stride, d_tokens, stream, nullptr);
   }
-  if (dtype == ETS_DTYPE_UINT16) {
-    return fail(s, ETS_NOT_SUPPORTED,
-                "stochastic sampling of UInt16 logits is not supported (integer softmax of the reference "
-                "degenerates to 0/1 weights); use temperature 0 or dequantise first");
-  }
+  if (dtype == ETS_DTYPE_UINT16) return fail(s, ETS_NOT_SUPPORTED, kUint16Message);
   ets_status st = ensure_scratch(s);
   if (st != ETS_OK) return st;
   ets::RowParams p;
@@ -180,19 +215,108 @@ ets_status sample_device(ets_sampler* s, const void* d_logits, int32_t dtype, in
   p.scratch = s->d_scratch;
   p.scratch_stride = s->scratch_stride;
   p.lds_keys = s->lds_keys;
-  switch (dtype) {
-    case ETS_DTYPE_FLOAT:
-      return launch_rows<ets::kDtypeFloat>(s, p, batch, stream);
-    case ETS_DTYPE_HALF:
-      return launch_rows<ets::kDtypeHalf>(s, p, batch, stream);
-    default:
-      return launch_rows<ets::kDtypeBFloat16>(s, p, batch, stream);
-  }
+  p.row_map = nullptr;
+  p.row_cfg = nullptr;
+  return rows_device(s, p, dtype, batch, stream, draw_mode(s->vocab, s->topp, s->topk));
 }
 
-float inverse_temperature_ctor(float temperature) {
-  // sampler.cpp:178: static_cast<bool>(temperature) ? 1.0f / temperature : 0
-  return (temperature != 0.0f) ? 1.0f / temperature : 0.0f;
+// ---- per-row parameters ------------------------------------------------------------------------
+// Staging layout for a batch of B rows: reseed u64[B] | RowConfig[B] | row maps int32[4][B]
+// (greedy, top-p, multinomial, top-k).
+struct StageLayout {
+  size_t reseed, cfg, maps, bytes;
+  explicit StageLayout(int32_t rows) {
+    reseed = 0;
+    cfg = reseed + sizeof(uint64_t) * rows;
+    maps = cfg + sizeof(ets::RowConfig) * rows;
+    maps = (maps + 15) / 16 * 16;
+    bytes = maps + sizeof(int32_t) * 4 * rows;
+  }
+};
+
+__global__ void reseed_kernel(uint64_t* rng, const uint64_t* reseed, int32_t rows) {
+  const int32_t b = blockIdx.x * blockDim.x + threadIdx.x;
+  if (b < rows && reseed[b] != 0ull) rng[b] = reseed[b];
+}
+
+ets_status ensure_stage(ets_sampler* s) {
+  if (s->h_stage) return ETS_OK;
+  const StageLayout full(s->max_batch);
+  ETS_HIP(s, hipHostMalloc(&s->h_stage, full.bytes, hipHostMallocDefault));
+  ETS_HIP(s, hipMalloc(&s->d_stage, full.bytes));
+  ETS_HIP(s, hipEventCreateWithFlags(&s->stage_event, hipEventDisableTiming));
+  return ETS_OK;
+}
+
+ets_status sample_device_configs(ets_sampler* s, const void* d_logits, int32_t dtype, int32_t batch, int64_t stride,
+                                 const ets_sampling_config* configs, int32_t* d_tokens, ets_row_debug* d_debug,
+                                 hipStream_t stream) {
+  ets_status st = ensure_stage(s);
+  if (st != ETS_OK) return st;
+  if (s->stage_pending) {
+    ETS_HIP(s, hipEventSynchronize(s->stage_event));  // the previous upload has left the staging buffer
+    s->stage_pending = false;
+  }
+  const StageLayout lay(batch);
+  char* h = static_cast<char*>(s->h_stage);
+  char* d = static_cast<char*>(s->d_stage);
+  uint64_t* h_reseed = reinterpret_cast<uint64_t*>(h + lay.reseed);
+  ets::RowConfig* h_cfg = reinterpret_cast<ets::RowConfig*>(h + lay.cfg);
+  int32_t* h_maps = reinterpret_cast<int32_t*>(h + lay.maps);
+  int32_t count[4] = {0, 0, 0, 0};  // greedy, then ets::kDrawTopP / Multinomial / TopK + 1
+  bool any_reseed = false;
+  for (int32_t b = 0; b < batch; ++b) {
+    const ets_sampling_config& c = configs[b];
+    // temperature < 0: the handle's own (SamplingConfig: "-1 temperature means implementation default")
+    const float inv = c.temperature < 0.0f ? s->inv_temperature : inverse_temperature_ctor(c.temperature);
+    h_cfg[b].inv_temperature = inv;
+    h_cfg[b].topp = c.top_p;
+    h_cfg[b].topk = c.top_k;
+    h_reseed[b] = c.seed;
+    any_reseed = any_reseed || c.seed != 0;
+    const int group = inv == 0.0f ? 0 : 1 + draw_mode(s->vocab, c.top_p, c.top_k);
+    if (group != 0 && dtype == ETS_DTYPE_UINT16) return fail(s, ETS_NOT_SUPPORTED, kUint16Message);
+    h_maps[group * batch + count[group]++] = b;
+  }
+  if (count[1] + count[2] + count[3] > 0) {
+    st = ensure_scratch(s);
+    if (st != ETS_OK) return st;
+  }
+  ETS_HIP(s, hipMemcpyAsync(d, h, lay.bytes, hipMemcpyHostToDevice, stream));
+  ETS_HIP(s, hipEventRecord(s->stage_event, stream));
+  s->stage_pending = true;
+  if (any_reseed) {
+    hipLaunchKernelGGL(reseed_kernel, dim3((batch + 255) / 256), dim3(256), 0, stream, s->d_rng,
+                       reinterpret_cast<const uint64_t*>(d + lay.reseed), batch);
+    ETS_HIP(s, hipGetLastError());
+  }
+  const int32_t* d_maps = reinterpret_cast<const int32_t*>(d + lay.maps);
+  if (count[0] > 0) {
+    st = argmax_device(s, d_logits, dtype, count[0], stride, d_tokens, stream, d_maps);
+    if (st != ETS_OK) return st;
+  }
+  ets::RowParams p;
+  p.logits = d_logits;
+  p.row_stride = stride;
+  p.vocab = s->vocab;
+  p.inv_temperature = s->inv_temperature;
+  p.topp = s->topp;
+  p.topk = s->topk;
+  p.rng = s->d_rng;
+  p.tokens = d_tokens;
+  p.probs = nullptr;
+  p.debug = reinterpret_cast<ets::RowDebug*>(d_debug);
+  p.scratch = s->d_scratch;
+  p.scratch_stride = s->scratch_stride;
+  p.lds_keys = s->lds_keys;
+  p.row_cfg = reinterpret_cast<const ets::RowConfig*>(d + lay.cfg);
+  for (int draw = 0; draw < 3; ++draw) {
+    if (count[1 + draw] == 0) continue;
+    p.row_map = d_maps + (1 + draw) * batch;
+    st = rows_device(s, p, dtype, count[1 + draw], stream, draw);
+    if (st != ETS_OK) return st;
+  }
+  return ETS_OK;
 }
 
 }  // namespace
@@ -276,6 +400,9 @@ ets_status ets_sampler_destroy(ets_sampler* s) {
     (void)hipFree(s->d_counters);
     (void)hipFree(s->d_row);
     (void)hipFree(s->d_token);
+    (void)hipFree(s->d_stage);
+    if (s->h_stage) (void)hipHostFree(s->h_stage);
+    if (s->stage_event) (void)hipEventDestroy(s->stage_event);
   }
   delete s;
   return ETS_OK;
@@ -321,6 +448,24 @@ ets_status ets_sampler_sample_batch(ets_sampler* s, const void* d_logits, int32_
                                     int64_t row_stride_elems, int32_t* d_tokens, void* hip_stream) {
   return ets_sampler_sample_batch_debug(s, d_logits, dtype, batch, row_stride_elems, d_tokens, nullptr, nullptr,
                                         hip_stream);
+}
+
+ets_status ets_sampler_sample_batch_configs(ets_sampler* s, const void* d_logits, int32_t dtype, int32_t batch,
+                                            int64_t row_stride_elems, const ets_sampling_config* configs,
+                                            int32_t* d_tokens, ets_row_debug* d_debug, void* hip_stream) {
+  if (!s) return fail(nullptr, ETS_INVALID_ARGUMENT, "ets_sampler_sample_batch_configs: null handle");
+  s->last_error.clear();
+  if (!d_logits || !d_tokens || !configs)
+    return fail(s, ETS_INVALID_ARGUMENT, "ets_sampler_sample_batch_configs: null pointer");
+  if (!dtype_ok(dtype)) return fail(s, ETS_INVALID_ARGUMENT, "ets_sampler_sample_batch_configs: unsupported dtype");
+  if (batch < 0 || batch > s->max_batch)
+    return fail(s, ETS_INVALID_ARGUMENT, "ets_sampler_sample_batch_configs: batch exceeds the handle's max_batch");
+  if (row_stride_elems < s->vocab)
+    return fail(s, ETS_INVALID_ARGUMENT, "ets_sampler_sample_batch_configs: row stride smaller than vocab_size");
+  if (batch == 0) return ETS_OK;
+  DeviceGuard g(s->device);
+  return sample_device_configs(s, d_logits, dtype, batch, row_stride_elems, configs, d_tokens, d_debug,
+                               static_cast<hipStream_t>(hip_stream));
 }
 
 ets_status ets_sampler_sample(ets_sampler* s, const void* logits, int32_t dtype, int32_t* token_out) {

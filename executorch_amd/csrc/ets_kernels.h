@@ -20,6 +20,14 @@ struct RowDebug {  // layout of ets_row_debug in include/et_sampler.h
   int32_t n_candidates, last_idx, position;
 };
 
+// Sampling parameters of one row when they differ from row to row (the batched counterpart of
+// SamplingConfig, extension/llm/runner/llm_session.h:29-34, already resolved by the host).
+struct RowConfig {
+  float inv_temperature;
+  float topp;
+  int32_t topk;
+};
+
 struct RowParams {
   const void* logits;
   int64_t row_stride;  // elements between rows
@@ -34,6 +42,8 @@ struct RowParams {
   uint64_t* scratch;  // [batch, scratch_stride] candidate keys (rows that overflow LDS)
   int64_t scratch_stride;
   int32_t lds_keys;   // power of two: keys that fit in the dynamic LDS buffer
+  const int32_t* row_map;    // workgroup -> row, or null for the identity
+  const RowConfig* row_cfg;  // [batch] per-row parameters (by row), or null for the launch-wide ones
 };
 
 // ---- argmax ---------------------------------------------------------------------------------
@@ -62,10 +72,10 @@ constexpr int kArgmaxBlock = 256;
 template <int DT>
 __global__ void __launch_bounds__(kArgmaxBlock)
 argmax_kernel(const void* logits_all, int64_t row_stride, int32_t vocab, uint64_t* partials, uint32_t* counters,
-              int32_t* tokens) {
+              int32_t* tokens, const int32_t* row_map) {
   __shared__ uint64_t red[kArgmaxBlock / 64];
   __shared__ int is_last;
-  const int row = blockIdx.y;
+  const int row = row_map ? row_map[blockIdx.y] : blockIdx.y;
   const int splits = gridDim.x;
   const int tid = threadIdx.x;
   const char* logits = static_cast<const char*>(logits_all) + static_cast<int64_t>(row) * row_stride * ElemSize<DT>::value;
@@ -1082,12 +1092,14 @@ __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
   extern __shared__ __align__(16) uint64_t lds_keys[];
   __shared__ BlockScratch sm;
   constexpr int VE = VecElems<DT>::value;
-  const int row = blockIdx.x;
+  const int row = p.row_map ? p.row_map[blockIdx.x] : blockIdx.x;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int V = p.vocab;
-  const float inv = p.inv_temperature;
+  const float inv = p.row_cfg ? p.row_cfg[row].inv_temperature : p.inv_temperature;
+  const float topp = p.row_cfg ? p.row_cfg[row].topp : p.topp;
+  const int32_t topk = p.row_cfg ? p.row_cfg[row].topk : p.topk;
   const char* logits = static_cast<const char*>(p.logits) + static_cast<int64_t>(row) * p.row_stride * ElemSize<DT>::value;
   uint64_t* scratch = p.scratch + static_cast<int64_t>(row) * p.scratch_stride;
   const float kInf = __uint_as_float(0x7f800000u);
@@ -1157,7 +1169,7 @@ __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
   }
 
   // ---- pass 2: softmax normaliser, sequential in index order (sampler.cpp:199-203)
-  const float cutoff = use_topp ? (1.0f - p.topp) / static_cast<float>(V - 1) : 0.0f;  // sampler.cpp:136
+  const float cutoff = use_topp ? (1.0f - topp) / static_cast<float>(V - 1) : 0.0f;  // sampler.cpp:136
   float S = kNaN;
   bool use_lut = false;
   int lut_base1 = 0, lut_top = 0, lut_half = 0;
@@ -1255,17 +1267,17 @@ __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
     bool done = false, tried = false;
     if constexpr (DT == kDtypeBFloat16 && ALIGNED) {
       if (use_topp && use_lut) {
-        done = draw_topp_hist<ALIGNED>(logits, V, inv, m, S, cutoff, p.topp, coin, lut, lut_base1, lut_top, lut_half,
+        done = draw_topp_hist<ALIGNED>(logits, V, inv, m, S, cutoff, topp, coin, lut, lut_base1, lut_top, lut_half,
                                        lds_keys, p.lds_keys, dbg, token, sm);
         tried = true;
       }
     }
     if (use_topp && !tried) {
-      done = draw_topp_listed(scratch, lds_list, lds_list_cap, list_base, n_listed, S, cutoff, p.topp, coin, lds_keys,
+      done = draw_topp_listed(scratch, lds_list, lds_list_cap, list_base, n_listed, S, cutoff, topp, coin, lds_keys,
                               p.lds_keys, dbg, token, sm);
     }
     if (!done) {
-      token = draw_general<DT>(logits, V, inv, m, S, use_topk, p.topk, p.topp, cutoff, coin, scratch, lds_keys,
+      token = draw_general<DT>(logits, V, inv, m, S, use_topk, topk, topp, cutoff, coin, scratch, lds_keys,
                                p.lds_keys, dbg, sm);
     }
   }

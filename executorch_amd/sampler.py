@@ -19,6 +19,11 @@ from ._capi import DTYPE_BFLOAT16, DTYPE_FLOAT, DTYPE_HALF, DTYPE_UINT16, RowDeb
 K_TOPP = 0.9  # sampler.h:29
 
 
+# layout of ets_sampling_config (include/et_sampler.h): float, float, int32, 4 bytes of padding, uint64
+SAMPLING_CONFIG_DTYPE = np.dtype({"names": ["temperature", "top_p", "top_k", "seed"], "formats": ["f4", "f4", "i4", "u8"],
+                                  "offsets": [0, 4, 8, 16], "itemsize": 24})
+
+
 class SamplerError(RuntimeError):
     """A non-Ok status from the C ABI; ``code`` holds the executorch Error value."""
 
@@ -135,6 +140,31 @@ class Sampler:
                 self._h, logits.data_ptr(), code, B, logits.stride(0), out.data_ptr(),
                 probs_out.data_ptr() if probs_out is not None else None,
                 debug_out.data_ptr() if debug_out is not None else None, stream)
+        self._check(st)
+        return out
+
+    def sample_batch_configs(self, logits: torch.Tensor, configs, out: torch.Tensor | None = None,
+                             dtype: int | None = None, debug_out: torch.Tensor | None = None) -> torch.Tensor:
+        """``sample_batch`` with one ``SamplingConfig`` per row (llm_session.h:29-34): ``configs`` is a
+        sequence of ``(temperature, top_p, top_k, seed)`` tuples or a structured array of dtype
+        ``SAMPLING_CONFIG_DTYPE``; temperature < 0 means this sampler's own, seed 0 continues the
+        row's coin stream."""
+        if not logits.is_cuda or logits.dim() != 2 or logits.stride(1) != 1:
+            raise SamplerError(_capi.INVALID_ARGUMENT, "sample_batch_configs wants a device tensor [B, vocab] with unit inner stride")
+        B, V = logits.shape
+        if V != self.vocab_size:
+            raise SamplerError(_capi.INVALID_ARGUMENT, "last dimension differs from vocab_size")
+        cfg = np.ascontiguousarray(np.asarray(configs, dtype=SAMPLING_CONFIG_DTYPE) if not isinstance(configs, np.ndarray)
+                                   else configs.astype(SAMPLING_CONFIG_DTYPE, copy=False))
+        if cfg.shape != (B,):
+            raise SamplerError(_capi.INVALID_ARGUMENT, "one config per row is required")
+        code = dtype_code(logits) if dtype is None else dtype
+        if out is None:
+            out = torch.empty(B, dtype=torch.int32, device=logits.device)
+        stream = torch.cuda.current_stream(logits.device).cuda_stream
+        st = _capi.lib().ets_sampler_sample_batch_configs(
+            self._h, logits.data_ptr(), code, B, logits.stride(0), cfg.ctypes.data, out.data_ptr(),
+            debug_out.data_ptr() if debug_out is not None else None, stream)
         self._check(st)
         return out
 

@@ -119,6 +119,30 @@ ETS_API ets_status ets_sampler_sample_batch_debug(ets_sampler* s, const void* d_
                                                  int32_t batch, int64_t row_stride_elems, int32_t* d_tokens,
                                                  float* d_probs, ets_row_debug* d_debug, void* hip_stream);
 
+/* SamplingConfig  -- extension/llm/runner/llm_session.h:29-34 (same fields, same defaults:
+ * temperature -1 = "implementation default", here the handle's temperature; top_p 1.0;
+ * top_k 0 = disabled; seed 0 = unset). */
+typedef struct ets_sampling_config {
+  float temperature;
+  float top_p;
+  int32_t top_k;
+  uint64_t seed;
+} ets_sampling_config;
+
+/* ets_sampler_sample_batch() with one SamplingConfig per row, for batches that mix requests
+ * (LLMSession::decode_one(const SamplingConfig&), llm_session.h:97-98, takes one per call; the
+ * reference's engines serve one session per call).  `configs` is a HOST array of `batch` entries,
+ * consumed before the call returns.  Row b is sampled as a reference object constructed with
+ * (vocab_size, temperature_b, top_p_b) and set_topk(top_k_b) would sample it: temperature 0 is the
+ * arg-max and consumes no coin, and the branch order is the reference's (sampler.cpp:238-249).
+ * seed_b != 0 restarts row b's coin stream at seed_b before this call's draw (the state a new
+ * object with that seed has); seed_b == 0 continues the row's stream.  `d_debug` may be null.
+ * Rows are grouped by draw and launched group by group on `hip_stream`; asynchronous. */
+ETS_API ets_status ets_sampler_sample_batch_configs(ets_sampler* s, const void* d_logits, int32_t dtype,
+                                                   int32_t batch, int64_t row_stride_elems,
+                                                   const ets_sampling_config* configs, int32_t* d_tokens,
+                                                   ets_row_debug* d_debug, void* hip_stream);
+
 /* Per-row xorshift64* states (sampler.h:82 `rng_state_`, one per row here).  HOST pointers to
  * `count` values for rows [first_row, first_row + count).  Lets a run be replayed or resumed. */
 ETS_API ets_status ets_sampler_set_rng_states(ets_sampler* s, int32_t first_row, int32_t count,

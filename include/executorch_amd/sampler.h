@@ -122,6 +122,15 @@ class Sampler {
     return status_;
   }
 
+  /// The same with one SamplingConfig per row (extension/llm/runner/llm_session.h:29-34;
+  /// ets_sampling_config has its fields): `configs` is a host array of `batch` entries.
+  ets_status sample_batch(const void* d_logits, int32_t dtype, int32_t batch, int64_t row_stride_elems,
+                          const ets_sampling_config* configs, int32_t* d_tokens, void* hip_stream = nullptr) {
+    status_ = ets_sampler_sample_batch_configs(h_, d_logits, dtype, batch, row_stride_elems, configs, d_tokens,
+                                               nullptr, hip_stream);
+    return status_;
+  }
+
   ets_status last_status() const { return status_; }
   const char* last_error() const { return ets_sampler_last_error(h_); }
   ets_sampler* handle() const { return h_; }

@@ -1,0 +1,81 @@
+"""Per-row sampling parameters (the batched counterpart of SamplingConfig, llm_session.h:29-34)
+through the C ABI: every row must come out as a reference sampler built with that row's
+parameters would sample it, whatever else shares the batch."""
+import numpy as np
+import pytest
+import torch
+
+import executorch_amd as ea
+from executorch_amd import _capi
+from executorch_amd import workloads as W
+from util import f32_bits, to_device
+
+pytestmark = pytest.mark.gpu
+
+
+def oracle_rows(oracle, x, dtype, cfgs, default_temperature, states):
+    """Row by row with the oracle; `states` is advanced in place."""
+    want = np.empty(len(cfgs), dtype=np.int32)
+    explain = []
+    for b, (t, topp, topk, seed) in enumerate(cfgs):
+        if seed:
+            states[b] = seed
+        temperature = default_temperature if t < 0 else t
+        tok, ex = oracle.sample_rows(x[b:b + 1], dtype, oracle.inv_temperature(temperature), topp, topk, states[b:b + 1],
+                                     mode=oracle.MODE_UPCAST, tie=oracle.TIE_STABLE, explain=True)
+        want[b] = tok[0]
+        explain.append(ex[0])
+    return want, explain
+
+
+@pytest.mark.parametrize("name,rows", [("cfg2", 24), ("cfg1", 9)])
+def test_mixed_batch_matches_per_row_samplers(oracle, dev, name, rows):
+    w = W.WORKLOADS[name]
+    menu = [(-1.0, 0.9, 0, 0), (0.0, 0.9, 0, 0), (0.6, 0.9, 0, 0), (1.0, 1.0, 0, 0), (0.8, 0.0, 0, 0), (0.7, 0.9, 5, 0),
+            (1.3, 0.5, 0, 12345), (0.0, 1.0, 3, 777), (0.9, 0.95, 40, 99), (0.6, 0.3, 0, 0), (2.0, 1.0, 0, 31337)]
+    cfgs = [menu[(3 * b + 1) % len(menu)] for b in range(rows)]
+    default_temperature = 0.75
+    s = ea.Sampler(w.vocab, default_temperature, 0.5, 5000, max_batch=rows)
+    states = (np.uint64(5000) + np.arange(rows, dtype=np.uint64)).astype(np.uint64)
+    for step in range(3):
+        x = W.logits(w, step, rows)
+        if step == 1:
+            cfgs = [(t, p, k, 0) for (t, p, k, _) in cfgs]  # streams continue
+        if step == 2:
+            cfgs = cfgs[1:] + cfgs[:1]  # rows change group
+        ddbg = torch.zeros((rows, 8), dtype=torch.int32, device=dev)
+        got = s.sample_batch_configs(to_device(x, w.dtype, dev), cfgs, debug_out=ddbg).cpu().numpy()
+        want, ex = oracle_rows(oracle, x, w.dtype, cfgs, default_temperature, states)
+        assert np.array_equal(got, want), (name, step, np.nonzero(got != want)[0], got, want)
+        assert np.array_equal(s.get_rng_states(rows), states), (name, step)
+        dbg = ea.debug_records(ddbg)
+        for b in range(rows):
+            if ex[b].branch in (oracle.BRANCH_TOPP, oracle.BRANCH_TOPK):
+                assert f32_bits(dbg["sum"][b]) == f32_bits(ex[b].sum)
+                assert dbg["n_candidates"][b] == ex[b].n_candidates
+                assert dbg["position"][b] == ex[b].position
+
+
+def test_uniform_configs_equal_the_plain_batch(dev):
+    w = W.WORKLOADS["cfg2"]
+    rows = 16
+    x = to_device(W.logits(w, 0, rows), w.dtype, dev)
+    a = ea.Sampler(w.vocab, w.temperature, w.topp, 42, max_batch=rows)
+    b = ea.Sampler(w.vocab, 0.123, 0.456, 42, max_batch=rows)
+    plain = a.sample_batch(x).cpu().numpy()
+    cfg = b.sample_batch_configs(x, [(w.temperature, w.topp, 0, 0)] * rows).cpu().numpy()
+    assert np.array_equal(plain, cfg)
+    assert np.array_equal(a.get_rng_states(), b.get_rng_states())
+
+
+def test_config_errors(dev):
+    s = ea.Sampler(64, 1.0, 0.9, 1, max_batch=4)
+    x = torch.zeros((4, 64), device=dev)
+    with pytest.raises(ea.SamplerError):
+        s.sample_batch_configs(x, [(1.0, 0.9, 0, 0)] * 3)
+    u16 = torch.zeros((4, 64), dtype=torch.int16, device=dev)
+    # greedy rows of UInt16 logits are fine, stochastic ones are refused
+    assert s.sample_batch_configs(u16, [(0.0, 0.9, 0, 0)] * 4, dtype=_capi.DTYPE_UINT16).cpu().tolist() == [0, 0, 0, 0]
+    with pytest.raises(ea.SamplerError) as e:
+        s.sample_batch_configs(u16, [(0.0, 0.9, 0, 0)] * 3 + [(1.0, 0.9, 0, 0)], dtype=_capi.DTYPE_UINT16)
+    assert e.value.code == _capi.NOT_SUPPORTED
