@@ -104,6 +104,61 @@ def cpu_baseline(w, seconds_budget=12.0):
     }
 
 
+def timed_us(fn, reps, torch):
+    """Mean duration of fn() in microseconds, from events on the current stream."""
+    for _ in range(3):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / reps
+
+
+def bench_logit_chain(w, logits, torch, dev):
+    """The device-side logit processors on a private copy of one batch of the workload: a chain of
+    lists (repetition penalty over a 512-token history per row, then a 16-token mask), which touches
+    a few hundred entries per row, and a chain of two whole-row processors, which has to read and
+    write every entry once whatever its length (priced against the HBM peak)."""
+    from executorch_amd.logit_processor import LogitChain
+
+    work = logits.clone()
+    g = torch.Generator(device=dev).manual_seed(7)
+    history = torch.randint(0, w.vocab, (w.batch, 512), generator=g, device=dev, dtype=torch.int32)
+    lengths = torch.full((w.batch,), 512, dtype=torch.int32, device=dev)
+    lists = LogitChain().add_repetition_penalty(1.0009765625, history, lengths).add_mask(list(range(100, 116)))
+    rows = LogitChain().add_scale(1.0).add_bias(0.0)
+    lists_us = timed_us(lambda: lists.process(work), 50, torch)
+    rows_us = timed_us(lambda: rows.process(work), 50, torch)
+    moved = 2 * w.bytes_per_step  # the batch is read once and written once
+    return {"lists_us": lists_us, "lists": "repetition penalty, 512-token history per row + mask of 16 ids",
+            "whole_rows_us": rows_us, "whole_rows": "scale + bias", "whole_rows_algorithmic_bytes": moved,
+            "whole_rows_gbs": moved / (rows_us * 1e-6) / 1e9, "whole_rows_frac_of_hbm_peak": moved / (rows_us * 1e-6) / 1e9 / HBM_PEAK_GBS}
+
+
+def bench_configs(w, s, ring, out, steps, torch):
+    """ets_sampler_sample_batch_configs on the same ring: every row with the workload's own
+    parameters (one launch, plus the upload of the per-row table), and a mix of four kinds of rows
+    (one launch per kind)."""
+    uniform = [(w.temperature, w.topp, 0, 0)] * w.batch
+    kinds = [(w.temperature, w.topp, 0, 0), (0.0, w.topp, 0, 0), (1.0, 1.0, 0, 0), (0.8, w.topp, 40, 0)]
+    mixed = [kinds[b % 4] for b in range(w.batch)]
+    state = {"i": 0}
+
+    def run(cfg):
+        def step():
+            s.sample_batch_configs(ring[state["i"] % len(ring)], cfg, out=out)
+            state["i"] += 1
+        return step
+
+    n = max(10, steps // 4)
+    return {"uniform_us": timed_us(run(uniform), n, torch), "mixed_us": timed_us(run(mixed), n, torch),
+            "mixed": "a quarter of the rows each: the workload's top-p, greedy, multinomial T=1, top-k 40 T=0.8"}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -196,6 +251,8 @@ def main():
                      "kernel_ms": kernel_ms, "algorithmic_bytes_per_launch": step_bytes},
         "parity": {"rows_checked": rows, "token_mismatches_vs_oracle": mismatches},
     }
+    line["logit_chain"] = bench_logit_chain(w, ring[0], torch, dev)
+    line["per_row_configs"] = bench_configs(w, s, ring, out, args.steps, torch)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(w)
     print(json.dumps(line))

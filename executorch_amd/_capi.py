@@ -52,6 +52,20 @@ SIGNATURES = {
     "ets_version": (C.c_char_p, []),
 }
 
+# every symbol declared in include/et_logit_processor.h
+CHAIN_SIGNATURES = {
+    "ets_logit_chain_create": (C.c_int32, [C.POINTER(C.c_void_p)]),
+    "ets_logit_chain_destroy": (C.c_int32, [C.c_void_p]),
+    "ets_logit_chain_size": (C.c_int32, [C.c_void_p]),
+    "ets_logit_chain_add_bias": (C.c_int32, [C.c_void_p, C.c_float]),
+    "ets_logit_chain_add_scale": (C.c_int32, [C.c_void_p, C.c_float]),
+    "ets_logit_chain_add_mask": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int32]),
+    "ets_logit_chain_add_token_bias": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32]),
+    "ets_logit_chain_add_repetition_penalty": (C.c_int32, [C.c_void_p, C.c_float, C.c_void_p, C.c_int64, C.c_void_p]),
+    "ets_logit_chain_process": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.POINTER(C.c_int64), C.c_void_p]),
+    "ets_logit_chain_last_error": (C.c_char_p, [C.c_void_p]),
+}
+
 # csrc/ets_test_hooks.h
 TEST_HOOKS = {
     "ets_test_expf": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p]),
@@ -69,7 +83,7 @@ def lib() -> C.CDLL:
                 f"{LIB_PATH} is missing: build it with `python -m executorch_amd.build` "
                 "(there is no CPU fallback for the sampler)")
         L = C.CDLL(LIB_PATH)
-        for table in (SIGNATURES, TEST_HOOKS):
+        for table in (SIGNATURES, CHAIN_SIGNATURES, TEST_HOOKS):
             for name, (res, args) in table.items():
                 f = getattr(L, name)
                 f.restype = res

@@ -4,6 +4,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cstdio>
 #include <cstring>
 #include <ctime>
@@ -571,3 +572,5 @@ ets_status ets_test_seq_sum(const float* d_a, int32_t n, float s0, float thresho
 }
 
 }  // extern "C"
+
+#include "ets_logit_chain.h"

@@ -8,6 +8,7 @@ import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HEADER = os.path.join(ROOT, "include", "et_sampler.h")
+CHAIN_HEADER = os.path.join(ROOT, "include", "et_logit_processor.h")
 HOOKS = os.path.join(ROOT, "executorch_amd", "csrc", "ets_test_hooks.h")
 
 
@@ -30,9 +31,10 @@ def test_library_exports_every_declared_symbol():
 
     assert os.path.exists(_capi.LIB_PATH), "build the library first: python -m executorch_amd.build"
     lib = ctypes.CDLL(_capi.LIB_PATH)
-    for name in declared(HEADER) + declared(HOOKS):
+    for name in declared(HEADER) + declared(CHAIN_HEADER) + declared(HOOKS):
         assert hasattr(lib, name), name
     assert sorted(_capi.SIGNATURES) == declared(HEADER)
+    assert sorted(_capi.CHAIN_SIGNATURES) == declared(CHAIN_HEADER)
     assert sorted(_capi.TEST_HOOKS) == declared(HOOKS)
 
 
