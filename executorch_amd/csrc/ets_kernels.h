@@ -826,16 +826,29 @@ __device__ __forceinline__ int pattern_order(uint32_t pattern16) {
 }
 
 // Returns false when the caller has to take the general path.
-template <bool ALIGNED>
+// Quotient used for comparisons: thresholds of a top-p row are far above 2^-126, those of a top-k
+// row can be anything.
+template <bool EXACT>
+__device__ __forceinline__ float row_quotient(float e, const RowDivisor& div) {
+  return EXACT ? div_row(e, div) : div_row_above(e, div);
+}
+
+// With TOPK the same walk selects by COUNT instead of mass: the entries with the `topk` largest
+// probabilities and everything tied with the last of them (sampler.cpp:87-100 sorts all entries;
+// the walks of :103-119 only read the first topk).  The caller passes cutoff = 0 and a scan that
+// counted every entry.
+template <bool ALIGNED, bool TOPK>
 __device__ __noinline__ bool draw_topp_hist(const char* logits, int V, float inv, float m, float S, float cutoff, float topp,
-                               float coin, float* lut, int base1, int top, int half, uint64_t* lds_keys, int cap,
-                               RowDebug& dbg, int32_t& token, BlockScratch& sm) {
+                               int topk, float coin, float* lut, int base1, int top, int half, uint64_t* lds_keys,
+                               int cap, RowDebug& dbg, int32_t& token, BlockScratch& sm) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const RowDivisor div = row_divisor(S);
   const uint32_t* lut_u = reinterpret_cast<const uint32_t*>(lut);
-  const float target = topp * 1.004f + 1e-6f;
+  if (TOPK && V > (1 << 24)) return false;  // counts are summed in float
+  const float target = TOPK ? static_cast<float>(topk) : topp * 1.004f + 1e-6f;
+
   constexpr int kMaxRun = 16;  // table positions per lane; the key buffer bounds them by 16 * kBlock
   // Every threshold below is at least the cutoff, and the cutoff is far above 2^-126 (1 - topp is
   // at least 2^-24 and the vocabulary below 2^31): div_row_above is exact wherever it matters.
@@ -886,9 +899,9 @@ __device__ __noinline__ bool draw_topp_hist(const char* logits, int V, float inv
 #pragma unroll
   for (int k = 0; k < kMaxRun; ++k) {
     if (k < run) {
-      pq[k] = div_row_above(pq[k], div);
+      pq[k] = row_quotient<TOPK>(pq[k], div);
       if (pq[k] >= cutoff && cq[k] != 0u) {  // positions past the run hold count 0
-        mass += static_cast<float>(cq[k]) * pq[k];
+        mass += TOPK ? static_cast<float>(cq[k]) : static_cast<float>(cq[k]) * pq[k];
         cnt += cq[k];
         last_cand = q0 + k;
       }
@@ -929,7 +942,7 @@ __device__ __noinline__ bool draw_topp_hist(const char* logits, int V, float inv
   }
   // ---- the lane whose run takes the mass past the target fixes p_thr and how far the table
   //      positions with p >= p_thr reach (q_ext); without such a lane every candidate is taken
-  const bool take_all = wave_star < 0 || n0 <= 64u;
+  const bool take_all = wave_star < 0 || (!TOPK && n0 <= 64u);
   if (!take_all && wave == wave_star) {
     const float hi = mass_before + upto;  // any-order float sums: the margin in `target` covers them
     const uint64_t ballot = __ballot(hi >= target);
@@ -943,7 +956,7 @@ __device__ __noinline__ bool draw_topp_hist(const char* logits, int V, float inv
 #pragma unroll
       for (int k = 0; k < kMaxRun; ++k) {
         if (k < run && !reached && pq[k] >= cutoff && cq[k] != 0u) {
-          running += static_cast<float>(cq[k]) * pq[k];
+          running += TOPK ? static_cast<float>(cq[k]) : static_cast<float>(cq[k]) * pq[k];
           q_star = q0 + k;
           p_thr = pq[k];
           reached = running >= target;
@@ -952,7 +965,7 @@ __device__ __noinline__ bool draw_topp_hist(const char* logits, int V, float inv
       int q_ext = q_star;
       for (int q = q_star + 1; q_star >= 0 && q < Q; ++q) {
         const int idx = hist_entry(q, top, half);
-        if (!(div_row_above(lut[2 * idx], div) >= p_thr)) break;
+        if (!(row_quotient<TOPK>(lut[2 * idx], div) >= p_thr)) break;
         q_ext = q;
       }
       if (q_star >= 0) {
@@ -1011,7 +1024,7 @@ __device__ __noinline__ bool draw_topp_hist(const char* logits, int V, float inv
   auto take = [&](uint32_t pattern16, int index) {
     if (pattern_order(pattern16) < k_star) return;
     const float x = __uint_as_float(pattern16 << 16) * inv;
-    const float pj = div_row_above(expf_nonpositive(x - m, sm.exp2tab), div);
+    const float pj = row_quotient<TOPK>(expf_nonpositive(x - m, sm.exp2tab), div);
     if (pj >= p_thr) {
       const uint32_t slot = atomicAdd(&sm.counter2, 1u);
       if (slot < static_cast<uint32_t>(cap)) lds_keys[slot] = cand_key(pj, index);
@@ -1070,12 +1083,17 @@ __device__ __noinline__ bool draw_topp_hist(const char* logits, int V, float inv
   __syncthreads();
   const int n_got = static_cast<int>(sm.counter2);
   if (n_got > cap || n_got == 0) return false;
-  if (n_got <= 64) return draw_small_wave(lds_keys, n_got, static_cast<int>(n0), topp, coin, dbg, token, sm) != -2;
+  if (TOPK) {
+    if (n_got < topk) return false;
+    dbg.n_candidates = V;  // every entry is a candidate of a top-k draw
+  } else if (n_got <= 64) {
+    return draw_small_wave(lds_keys, n_got, static_cast<int>(n0), topp, coin, dbg, token, sm) != -2;
+  }
   const int N = pow2_ceil(n_got);
   for (int i = n_got + tid; i < N; i += kBlock) lds_keys[i] = ~0ull;
   __syncthreads();
   sort_keys_lds(lds_keys, N);
-  const int pos = draw_from_sorted(lds_keys, n_got, static_cast<int>(n0), false, 0, topp, coin, dbg, sm);
+  const int pos = draw_from_sorted(lds_keys, n_got, static_cast<int>(n0), TOPK, topk, topp, coin, dbg, sm);
   if (pos == -2) return false;  // the pre-selection did not reach topp after all
   token = static_cast<int32_t>(static_cast<uint32_t>(lds_keys[pos]));
   return true;
@@ -1192,7 +1210,7 @@ __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
     bool scanned = false;
     if constexpr (DT == kDtypeBFloat16 && ALIGNED) {
       if (use_lut) {
-        if (use_topp) {
+        if (use_topp || use_topk) {  // top-k: the cutoff is 0, every entry is counted
           scan_row<DT, ALIGNED, kScanSum, kListHist, true>(a, st, sm);
         } else {
           scan_row<DT, ALIGNED, kScanSum, kListNone, true>(a, st, sm);
@@ -1267,9 +1285,13 @@ __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
     bool done = false, tried = false;
     if constexpr (DT == kDtypeBFloat16 && ALIGNED) {
       if (use_topp && use_lut) {
-        done = draw_topp_hist<ALIGNED>(logits, V, inv, m, S, cutoff, topp, coin, lut, lut_base1, lut_top, lut_half,
-                                       lds_keys, p.lds_keys, dbg, token, sm);
+        done = draw_topp_hist<ALIGNED, false>(logits, V, inv, m, S, cutoff, topp, 0, coin, lut, lut_base1, lut_top,
+                                              lut_half, lds_keys, p.lds_keys, dbg, token, sm);
         tried = true;
+      }
+      if (use_topk && use_lut) {
+        done = draw_topp_hist<ALIGNED, true>(logits, V, inv, m, S, 0.0f, topp, topk, coin, lut, lut_base1, lut_top,
+                                             lut_half, lds_keys, p.lds_keys, dbg, token, sm);
       }
     }
     if (use_topp && !tried) {

@@ -145,21 +145,22 @@ def test_total_variation_of_draws(dev):
         assert 0.5 * np.abs(counts / counts.sum() - np.array(target)).sum() < 0.02
 
 
-def compare_rows(oracle, dev, x, dtype, temperature, topp, seed, label):
+def compare_rows(oracle, dev, x, dtype, temperature, topp, seed, label, topk=0):
     """Tokens and draw internals of one batch against the oracle (stable tie order)."""
     rows, vocab = x.shape
     s = ea.Sampler(vocab, temperature, topp, seed, max_batch=rows)
+    s.set_topk(topk)
     states = (np.uint64(seed) + np.arange(rows, dtype=np.uint64)).astype(np.uint64)
     ddbg = torch.zeros((rows, 8), dtype=torch.int32, device=dev)
     got = s.sample_batch(to_device(x, dtype, dev), debug_out=ddbg).cpu().numpy()
-    want, ex = oracle.sample_rows(x, dtype, oracle.inv_temperature(temperature), topp, 0, states, mode=oracle.MODE_UPCAST,
+    want, ex = oracle.sample_rows(x, dtype, oracle.inv_temperature(temperature), topp, topk, states, mode=oracle.MODE_UPCAST,
                                   tie=oracle.TIE_STABLE, explain=True, threads=8)
     assert np.array_equal(got, want), (label, np.nonzero(got != want)[0][:8], got[:8], want[:8])
     dbg = ea.debug_records(ddbg)
     for b in range(rows):
         e = ex[b]
         assert f32_bits(dbg["sum"][b]) == f32_bits(e.sum), (label, b)
-        if e.branch == oracle.BRANCH_TOPP and want[b] >= 0:
+        if e.branch in (oracle.BRANCH_TOPP, oracle.BRANCH_TOPK) and want[b] >= 0:
             assert dbg["n_candidates"][b] == e.n_candidates, (label, b)
             assert dbg["last_idx"][b] == e.last_idx, (label, b)
             assert f32_bits(dbg["cumulative"][b]) == f32_bits(e.cumulative), (label, b)
@@ -211,4 +212,10 @@ def test_bf16_rows_with_structure(oracle, dev, vocab):
             if vocab > 50000 and label in ("flat", "few3") and temperature != 0.6:
                 continue  # every entry is a candidate: the full-row sort is slow, once is enough
             compare_rows(oracle, dev, x, W.DTYPE_BFLOAT16, temperature, topp, seed, (vocab, label, temperature, topp))
+            seed += 17
+        for topk, temperature in ((1, 1.0), (7, 0.6), (64, 1.0), (1000, 2.0), (vocab - 1, 1.0)):
+            if topk > 2000 and (vocab > 50000 or label not in ("normal", "few3")):
+                continue  # the selection outgrows LDS: the full-row sort, checked once per small vocabulary
+            compare_rows(oracle, dev, x, W.DTYPE_BFLOAT16, temperature, 0.9, seed, (vocab, label, "topk", topk, temperature),
+                         topk=topk)
             seed += 17
