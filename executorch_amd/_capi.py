@@ -15,6 +15,11 @@ OK, INTERNAL, INVALID_STATE, NOT_SUPPORTED, INVALID_ARGUMENT, MEMORY_ALLOCATION_
 DTYPE_HALF, DTYPE_FLOAT, DTYPE_BFLOAT16, DTYPE_UINT16 = 5, 6, 15, 27
 
 
+class SamplerStats(C.Structure):
+    _fields_ = [("calls", C.c_uint64), ("rows", C.c_uint64), ("aggregate_sampling_time_us", C.c_double),
+                ("last_call_us", C.c_double)]
+
+
 class RowDebug(C.Structure):
     _fields_ = [
         ("max_val", C.c_float),
@@ -42,6 +47,9 @@ SIGNATURES = {
                                          C.c_void_p, C.c_void_p, C.c_void_p]),
     "ets_sampler_sample_batch_debug": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int64, C.c_void_p,
                                                    C.c_void_p, C.c_void_p, C.c_void_p]),
+    "ets_sampler_set_timing": (C.c_int32, [C.c_void_p, C.c_int32]),
+    "ets_sampler_get_stats": (C.c_int32, [C.c_void_p, C.c_void_p]),
+    "ets_sampler_reset_stats": (C.c_int32, [C.c_void_p]),
     "ets_sampler_set_rng_states": (C.c_int32, [C.c_void_p, C.c_int32, C.c_int32, C.c_void_p]),
     "ets_sampler_get_rng_states": (C.c_int32, [C.c_void_p, C.c_int32, C.c_int32, C.c_void_p]),
     "ets_sample_from_logits": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.POINTER(C.c_int64), C.POINTER(C.c_int32)]),

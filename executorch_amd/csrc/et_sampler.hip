@@ -47,6 +47,16 @@ struct ets_sampler {
   void* d_stage = nullptr;
   hipEvent_t stage_event = nullptr;
   bool stage_pending = false;
+  // opt-in device timing (ets_sampler_set_timing): a ring of event pairs around the launches of a
+  // call, harvested when a slot is reused or the totals are read
+  bool timing = false;
+  static constexpr int kTimingSlots = 32;
+  hipEvent_t t_begin[kTimingSlots] = {};
+  hipEvent_t t_end[kTimingSlots] = {};
+  int32_t t_rows[kTimingSlots] = {};
+  bool t_busy[kTimingSlots] = {};
+  uint64_t t_next = 0;
+  ets_sampler_stats stats = {};
   std::string last_error;
 };
 
@@ -92,6 +102,45 @@ struct DeviceGuard {
     if (switched) (void)hipSetDevice(prev);
   }
 };
+
+// ---- device timing ------------------------------------------------------------------------------
+ets_status harvest_timing_slot(ets_sampler* s, int slot) {
+  if (!s->t_busy[slot]) return ETS_OK;
+  ETS_HIP(s, hipEventSynchronize(s->t_end[slot]));
+  float ms = 0.0f;
+  ETS_HIP(s, hipEventElapsedTime(&ms, s->t_begin[slot], s->t_end[slot]));
+  s->t_busy[slot] = false;
+  s->stats.calls += 1;
+  s->stats.rows += static_cast<uint64_t>(s->t_rows[slot]);
+  s->stats.last_call_us = static_cast<double>(ms) * 1e3;
+  s->stats.aggregate_sampling_time_us += s->stats.last_call_us;
+  return ETS_OK;
+}
+
+// Brackets one call's launches on `stream`; `slot` < 0 when timing is off.
+ets_status timing_begin(ets_sampler* s, hipStream_t stream, int32_t rows, int* slot) {
+  *slot = -1;
+  if (!s->timing) return ETS_OK;
+  const int k = static_cast<int>(s->t_next % ets_sampler::kTimingSlots);
+  ets_status st = harvest_timing_slot(s, k);
+  if (st != ETS_OK) return st;
+  if (!s->t_begin[k]) {
+    ETS_HIP(s, hipEventCreate(&s->t_begin[k]));
+    ETS_HIP(s, hipEventCreate(&s->t_end[k]));
+  }
+  ETS_HIP(s, hipEventRecord(s->t_begin[k], stream));
+  s->t_rows[k] = rows;
+  *slot = k;
+  return ETS_OK;
+}
+
+ets_status timing_end(ets_sampler* s, hipStream_t stream, int slot) {
+  if (slot < 0) return ETS_OK;
+  ETS_HIP(s, hipEventRecord(s->t_end[slot], stream));
+  s->t_busy[slot] = true;
+  s->t_next += 1;
+  return ETS_OK;
+}
 
 template <int DT>
 ets_status launch_argmax(ets_sampler* s, const void* d_logits, int32_t batch, int64_t stride, int32_t* d_tokens,
@@ -404,6 +453,10 @@ ets_status ets_sampler_destroy(ets_sampler* s) {
     (void)hipFree(s->d_stage);
     if (s->h_stage) (void)hipHostFree(s->h_stage);
     if (s->stage_event) (void)hipEventDestroy(s->stage_event);
+    for (int i = 0; i < ets_sampler::kTimingSlots; ++i) {
+      if (s->t_begin[i]) (void)hipEventDestroy(s->t_begin[i]);
+      if (s->t_end[i]) (void)hipEventDestroy(s->t_end[i]);
+    }
   }
   delete s;
   return ETS_OK;
@@ -441,8 +494,13 @@ ets_status ets_sampler_sample_batch_debug(ets_sampler* s, const void* d_logits, 
     return fail(s, ETS_INVALID_ARGUMENT, "ets_sampler_sample_batch: row stride smaller than vocab_size");
   if (batch == 0) return ETS_OK;
   DeviceGuard g(s->device);
-  return sample_device(s, d_logits, dtype, batch, row_stride_elems, d_tokens, d_probs, d_debug,
-                       static_cast<hipStream_t>(hip_stream));
+  hipStream_t stream = static_cast<hipStream_t>(hip_stream);
+  int slot = -1;
+  ets_status st = timing_begin(s, stream, batch, &slot);
+  if (st != ETS_OK) return st;
+  st = sample_device(s, d_logits, dtype, batch, row_stride_elems, d_tokens, d_probs, d_debug, stream);
+  if (st != ETS_OK) return st;
+  return timing_end(s, stream, slot);
 }
 
 ets_status ets_sampler_sample_batch(ets_sampler* s, const void* d_logits, int32_t dtype, int32_t batch,
@@ -465,8 +523,46 @@ ets_status ets_sampler_sample_batch_configs(ets_sampler* s, const void* d_logits
     return fail(s, ETS_INVALID_ARGUMENT, "ets_sampler_sample_batch_configs: row stride smaller than vocab_size");
   if (batch == 0) return ETS_OK;
   DeviceGuard g(s->device);
-  return sample_device_configs(s, d_logits, dtype, batch, row_stride_elems, configs, d_tokens, d_debug,
-                               static_cast<hipStream_t>(hip_stream));
+  hipStream_t stream = static_cast<hipStream_t>(hip_stream);
+  int slot = -1;
+  ets_status st = timing_begin(s, stream, batch, &slot);
+  if (st != ETS_OK) return st;
+  st = sample_device_configs(s, d_logits, dtype, batch, row_stride_elems, configs, d_tokens, d_debug, stream);
+  if (st != ETS_OK) return st;
+  return timing_end(s, stream, slot);
+}
+
+ets_status ets_sampler_set_timing(ets_sampler* s, int32_t enabled) {
+  if (!s) return fail(nullptr, ETS_INVALID_ARGUMENT, "ets_sampler_set_timing: null handle");
+  s->last_error.clear();
+  s->timing = enabled != 0;
+  return ETS_OK;
+}
+
+ets_status ets_sampler_get_stats(ets_sampler* s, ets_sampler_stats* out) {
+  if (!s) return fail(nullptr, ETS_INVALID_ARGUMENT, "ets_sampler_get_stats: null handle");
+  s->last_error.clear();
+  if (!out) return fail(s, ETS_INVALID_ARGUMENT, "ets_sampler_get_stats: null pointer");
+  DeviceGuard g(s->device);
+  // oldest first, so that last_call_us ends up as the most recent call
+  for (int i = 0; i < ets_sampler::kTimingSlots; ++i) {
+    const int slot = static_cast<int>((s->t_next + static_cast<uint64_t>(i)) % ets_sampler::kTimingSlots);
+    ets_status st = harvest_timing_slot(s, slot);
+    if (st != ETS_OK) return st;
+  }
+  *out = s->stats;
+  return ETS_OK;
+}
+
+ets_status ets_sampler_reset_stats(ets_sampler* s) {
+  if (!s) return fail(nullptr, ETS_INVALID_ARGUMENT, "ets_sampler_reset_stats: null handle");
+  s->last_error.clear();
+  DeviceGuard g(s->device);
+  ets_sampler_stats scratch;
+  ets_status st = ets_sampler_get_stats(s, &scratch);  // drains calls still in flight
+  if (st != ETS_OK) return st;
+  s->stats = ets_sampler_stats{};
+  return ETS_OK;
 }
 
 ets_status ets_sampler_sample(ets_sampler* s, const void* logits, int32_t dtype, int32_t* token_out) {

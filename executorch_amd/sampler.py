@@ -168,6 +168,19 @@ class Sampler:
         self._check(st)
         return out
 
+    # ---- sampling time in microseconds (stats.h:46-47, :62-69 keep it in whole milliseconds)
+    def set_timing(self, enabled: bool = True) -> None:
+        self._check(_capi.lib().ets_sampler_set_timing(self._h, 1 if enabled else 0))
+
+    def stats(self) -> dict:
+        st = _capi.SamplerStats()
+        self._check(_capi.lib().ets_sampler_get_stats(self._h, C.byref(st)))
+        return {"calls": st.calls, "rows": st.rows, "aggregate_sampling_time_us": st.aggregate_sampling_time_us,
+                "last_call_us": st.last_call_us}
+
+    def reset_stats(self) -> None:
+        self._check(_capi.lib().ets_sampler_reset_stats(self._h))
+
     # ---- per-row xorshift64* states (sampler.h:82)
     def set_rng_states(self, states, first_row: int = 0) -> None:
         a = np.ascontiguousarray(states, dtype=np.uint64)

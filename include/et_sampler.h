@@ -143,6 +143,26 @@ ETS_API ets_status ets_sampler_sample_batch_configs(ets_sampler* s, const void* 
                                                    const ets_sampling_config* configs, int32_t* d_tokens,
                                                    ets_row_debug* d_debug, void* hip_stream);
 
+/* Sampling time at microsecond resolution.  The reference's Stats keeps
+ * aggregate_sampling_time_ms from host clocks in whole milliseconds
+ * (extension/llm/runner/stats.h:46-47, on_sampling_begin / on_sampling_end :62-69), which reads 0
+ * for a sampler that takes tens of microseconds.  With timing enabled every
+ * ets_sampler_sample_batch*() call is bracketed by HIP events on its stream; the totals are
+ * device time of the call's launches. */
+typedef struct ets_sampler_stats {
+  uint64_t calls;                    /* timed calls that have completed                      */
+  uint64_t rows;                     /* rows sampled by them                                 */
+  double aggregate_sampling_time_us; /* Stats::aggregate_sampling_time_ms, in microseconds   */
+  double last_call_us;               /* the most recent completed call                       */
+} ets_sampler_stats;
+
+/* Off by default (two event records per call when on). */
+ETS_API ets_status ets_sampler_set_timing(ets_sampler* s, int32_t enabled);
+/* Waits for the timed calls still in flight, then copies the totals. */
+ETS_API ets_status ets_sampler_get_stats(ets_sampler* s, ets_sampler_stats* out);
+/* Stats::reset()  -- stats.h:83-110. */
+ETS_API ets_status ets_sampler_reset_stats(ets_sampler* s);
+
 /* Per-row xorshift64* states (sampler.h:82 `rng_state_`, one per row here).  HOST pointers to
  * `count` values for rows [first_row, first_row + count).  Lets a run be replayed or resumed. */
 ETS_API ets_status ets_sampler_set_rng_states(ets_sampler* s, int32_t first_row, int32_t count,
