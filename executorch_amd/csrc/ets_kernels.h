@@ -314,15 +314,18 @@ struct ScanArgs {
   int lds_list_cap;
 };
 
+constexpr int kLutCountWords = 12288;  // a table entry's counter sits 48 KiB above its e
+
 // ---- expf by table for bf16 rows ----------------------------------------------------------------
 // A bf16 logit has 65536 possible bit patterns and e = expf(fl(fl(l * inv) - max)) is a function of
 // the pattern alone, so a row needs one exact expf per DISTINCT relevant pattern, not per entry.
 // Relevant magnitudes span a few dozen binades: below them |l * inv| is under an eighth of an ulp of
 // max, so x - max rounds to -max ("tiny" slot); above them a negative logit gives x - max < -104
 // (e == 0, "beyond" slot) and a positive one would exceed the maximum (cannot occur).  Layout per
-// sign half: [0] tiny, [1 .. R] live patterns in increasing magnitude, [R + 1] beyond.  An entry is
-// two words: the float e and a counter (zeroed here) that the top-p scan uses as a histogram of the
-// row over the table's entries.
+// sign half: [0] tiny, [1 .. R] live patterns in increasing magnitude, [R + 1] beyond.  Every entry
+// also has a counter (zeroed here), kLutCountWords words above its e, that the top-p scan uses as
+// a histogram of the row over the table's entries; e and the counters are separate arrays so that
+// the look-ups of e spread over all LDS banks.
 // Returns false (no table; the caller evaluates expf per entry) when inv or max are not positive
 // finite in the way the bounds need, or when the table would not fit in `cap` floats.
 __device__ bool build_exp_lut(float* lut, int cap, float inv, float m, const uint64_t* tab, int& base1, int& top,
@@ -348,7 +351,7 @@ __device__ bool build_exp_lut(float* lut, int cap, float inv, float m, const uin
   half = R + 2;
   top = R + 1;
   base1 = (e_lo << 7) - 1;
-  if (4 * half > cap) return false;
+  if (2 * half > kLutCountWords || kLutCountWords + 2 * half > cap) return false;
   for (int idx = threadIdx.x; idx < 2 * half; idx += kBlock) {
     const int sgn = idx >= half ? 1 : 0;
     const int c = idx - sgn * half;
@@ -367,8 +370,8 @@ __device__ bool build_exp_lut(float* lut, int cap, float inv, float m, const uin
       d = __builtin_fminf(__builtin_fmaxf(d, -104.0f), 0.0f);  // positive only for patterns that cannot occur
       e = expf_core(d, tab);
     }
-    lut[2 * idx] = e;
-    lut[2 * idx + 1] = 0.0f;  // bit pattern of the integer 0
+    lut[idx] = e;
+    lut[kLutCountWords + idx] = 0.0f;  // bit pattern of the integer 0
   }
   return true;
 }
@@ -379,25 +382,25 @@ __device__ __forceinline__ int lut_slot(uint32_t mag15, uint32_t sgn, int base1,
   return static_cast<int>(__umul24(sgn, static_cast<uint32_t>(half))) + c - base1;
 }
 
-// The same as the LDS byte address of the entry (8 bytes per entry), in three instructions: clamp,
-// sign * half + bias, shift-add.  lo = base1, hi = base1 + top, half8 = 8 * half,
-// bias = (LDS address of the table) - 8 * base1 (mod 2^32), all loop-invariant.
+// The same as the LDS byte address of the entry's e (4 bytes per entry), in three instructions:
+// clamp, sign * half + bias, shift-add.  lo = base1, hi = base1 + top, half4 = 4 * half,
+// bias = (LDS address of the table) - 4 * base1 (mod 2^32), all loop-invariant.
 typedef __attribute__((address_space(3))) float* LdsF32;
 typedef __attribute__((address_space(3))) uint32_t* LdsU32;
 struct LutAddr {
   int lo, hi;
-  uint32_t half8, bias;
+  uint32_t half4, bias;
 };
 __device__ __forceinline__ LutAddr lut_addr_of(float* lut, int base1, int top, int half) {
   const uint32_t table = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((LdsF32)lut));
-  return {base1, base1 + top, static_cast<uint32_t>(half) * 8u, table - static_cast<uint32_t>(base1) * 8u};
+  return {base1, base1 + top, static_cast<uint32_t>(half) * 4u, table - static_cast<uint32_t>(base1) * 4u};
 }
 __device__ __forceinline__ uint32_t lut_entry_address(uint32_t mag15, uint32_t sgn, const LutAddr& t) {
   int c;
   uint32_t side, addr;
   asm("v_med3_i32 %0, %1, %2, %3" : "=v"(c) : "v"(mag15), "v"(t.lo), "v"(t.hi));
-  asm("v_mad_u32_u24 %0, %1, %2, %3" : "=v"(side) : "v"(sgn), "v"(t.half8), "v"(t.bias));
-  asm("v_lshl_add_u32 %0, %1, 3, %2" : "=v"(addr) : "v"(c), "v"(side));
+  asm("v_mad_u32_u24 %0, %1, %2, %3" : "=v"(side) : "v"(sgn), "v"(t.half4), "v"(t.bias));
+  asm("v_lshl_add_u32 %0, %1, 2, %2" : "=v"(addr) : "v"(c), "v"(side));
   return addr;
 }
 
@@ -437,7 +440,7 @@ __device__ __forceinline__ bool scan_row(const ScanArgs& a, SeqSum& st, BlockScr
   const LutAddr lut_addr = lut_addr_of(a.lut, a.lut_base1, a.lut_top, a.lut_half);
   auto table_count = [&](uint32_t entry_address, float e, float cut_lo) {
     if (LIST == kListHist && e >= cut_lo) {
-      __hip_atomic_fetch_add((LdsU32)static_cast<uintptr_t>(entry_address + 4u), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      __hip_atomic_fetch_add((LdsU32)static_cast<uintptr_t>(entry_address + 4u * kLutCountWords), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
   };
   auto table_value = [&](uint32_t mag15, uint32_t sgn, float cut_lo) -> float {
@@ -860,7 +863,7 @@ __device__ __noinline__ bool draw_topp_hist(const char* logits, int V, float inv
     if (coarse > kMaxRun) return false;
     const float e_min = cutoff * S * 0.999f;
     const int q = tid * coarse;
-    const bool live = q < Q && lut[2 * hist_entry(min(q, Q - 1), top, half)] >= e_min;
+    const bool live = q < Q && lut[hist_entry(min(q, Q - 1), top, half)] >= e_min;
     const uint64_t ballot = __ballot(live);
     if (lane == 0) sm.red_u[wave] = static_cast<uint32_t>(__popcll(ballot));
     __syncthreads();
@@ -887,8 +890,8 @@ __device__ __noinline__ bool draw_topp_hist(const char* logits, int V, float inv
     if (k < run) {  // uniform
       const int q = q0 + k;
       const int idx = hist_entry(min(q, Q - 1), top, half);  // always a valid entry: no branch around the load
-      const float e = lut[2 * idx];
-      const uint32_t c = lut_u[2 * idx + 1];
+      const float e = lut[idx];
+      const uint32_t c = lut_u[kLutCountWords + idx];
       pq[k] = q < q1 ? e : 0.0f;
       cq[k] = q < q1 ? c : 0u;
     }
@@ -965,7 +968,7 @@ __device__ __noinline__ bool draw_topp_hist(const char* logits, int V, float inv
       int q_ext = q_star;
       for (int q = q_star + 1; q_star >= 0 && q < Q; ++q) {
         const int idx = hist_entry(q, top, half);
-        if (!(row_quotient<TOPK>(lut[2 * idx], div) >= p_thr)) break;
+        if (!(row_quotient<TOPK>(lut[idx], div) >= p_thr)) break;
         q_ext = q;
       }
       if (q_star >= 0) {
