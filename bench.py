@@ -139,6 +139,31 @@ def bench_logit_chain(w, logits, torch, dev):
             "whole_rows_gbs": moved / (rows_us * 1e-6) / 1e9, "whole_rows_frac_of_hbm_peak": moved / (rows_us * 1e-6) / 1e9 / HBM_PEAK_GBS}
 
 
+def bench_host_buffers(w, s, logits, out, torch):
+    """What the same step costs when the boundary is handed HOST memory: one batch copied from
+    pinned host memory to the device and sampled (the PCIe-inclusive rate; never `value`), and the
+    reference-shaped single-row entry ets_sampler_sample() on a pageable host row."""
+    host = torch.empty(logits.shape, dtype=logits.dtype, pin_memory=True)
+    host.copy_(logits)
+    staged = torch.empty_like(logits)
+
+    def batch_step():
+        staged.copy_(host, non_blocking=True)
+        s.sample_batch(staged, out=out)
+
+    batch_us = timed_us(batch_step, 20, torch)
+    row = logits[0].cpu()
+    one = type(s)(w.vocab, w.temperature, w.topp, 1)
+    for _ in range(3):
+        one.sample(row)
+    t0 = time.perf_counter()
+    for _ in range(50):
+        one.sample(row)
+    row_us = (time.perf_counter() - t0) * 1e6 / 50
+    return {"batch_from_pinned_host_us": batch_us, "rows_per_s_pcie_inclusive": w.batch / (batch_us * 1e-6),
+            "single_row_host_entry_us": row_us}
+
+
 def bench_configs(w, s, ring, out, steps, torch):
     """ets_sampler_sample_batch_configs on the same ring: every row with the workload's own
     parameters (one launch, plus the upload of the per-row table), and a mix of four kinds of rows
@@ -252,6 +277,7 @@ def main():
         "parity": {"rows_checked": rows, "token_mismatches_vs_oracle": mismatches},
     }
     line["logit_chain"] = bench_logit_chain(w, ring[0], torch, dev)
+    line["host_buffers"] = bench_host_buffers(w, s, ring[0], out, torch)
     line["per_row_configs"] = bench_configs(w, s, ring, out, args.steps, torch)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(w)
