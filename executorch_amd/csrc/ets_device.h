@@ -381,8 +381,9 @@ __device__ void wave_resolve(float& s, int& found, const uint32_t (&bits)[R], in
 // with the ulp it is predicted to see, instead of once per binade the running sum passes through.
 //   1. plain float sums per slot give approximate running sums at the slot boundaries;
 //   2. a slot whose two boundaries lie safely inside one binade is "stable" and is folded with that
-//      binade's ulp into a parity summary; the others (a binade boundary inside or near, or sums
-//      too small for the float shortcut) are "serial";
+//      binade's ulp into a parity summary; the others (a binade boundary inside or within 2^-13
+//      of an end -- plain and sequential sums of a group's 16384 entries differ by random rounding,
+//      some 1e-5 of the sum -- or sums too small for the float shortcut) are "serial";
 //   3. the slots are consumed in order from the exact running sum: a run of stable slots by
 //      composing its summaries -- after checking that the exact sum entering it has the predicted
 //      exponent and that the run does not leave the binade, which is all their validity needs --
@@ -414,7 +415,7 @@ __device__ int seq_sum_predicted(SeqSum& st, const uint32_t (&bits)[U][R], const
   const float s_out = st.s + incl;
   const uint32_t kb_in = __float_as_uint(s_in) >> 23, kb_out = __float_as_uint(s_out) >> 23;
   const float edge = __uint_as_float(kb_in << 23);  // 2^(kb_in - 127) <= s_in
-  const bool serial = kb_in != kb_out || kb_in < 70u || kb_in > 250u || s_in < edge * 1.002f || s_out > edge * 1.996f;
+  const bool serial = kb_in != kb_out || kb_in < 70u || kb_in > 250u || s_in < edge * 1.0001220703125f || s_out > edge * 1.999755859375f;
   const uint32_t serial_mask = static_cast<uint32_t>(__ballot(serial && lane < kSlots));
   const uint32_t buf = st.parity_buf;
   st.parity_buf ^= 1u;
