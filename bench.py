@@ -24,8 +24,8 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by
 # the factors a 256 MiB device copy gives in the same runs (profiles/sample_rows_kernel_cfg2.md has
-# the commands and the raw counters): 9256 KiB * 2.00 fetched + 4070 KiB * 1.00 written.
-MEASURED_TRAFFIC_BYTES = {"cfg2": (9256 * 2.00 + 4070 * 1.00) * 1024}
+# the commands and the raw counters): 9225 KiB * 2.00 fetched + 3772 KiB * 1.00 written.
+MEASURED_TRAFFIC_BYTES = {"cfg2": (9225 * 2.00 + 3772 * 1.00) * 1024}
 
 
 def synth_logits_device(w, count, torch, dev):
@@ -191,6 +191,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="cfg2")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="skip the logit-chain, per-row-config and host-buffer figures (a profile of this "
+                         "command then holds the headline kernel only)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run five 256 MiB device copies: a kernel of known traffic that calibrates "
                          "FETCH_SIZE / WRITE_SIZE when this command runs under rocprofv3 --pmc")
@@ -276,9 +279,10 @@ def main():
                      "kernel_ms": kernel_ms, "algorithmic_bytes_per_launch": step_bytes},
         "parity": {"rows_checked": rows, "token_mismatches_vs_oracle": mismatches},
     }
-    line["logit_chain"] = bench_logit_chain(w, ring[0], torch, dev)
-    line["host_buffers"] = bench_host_buffers(w, s, ring[0], out, torch)
-    line["per_row_configs"] = bench_configs(w, s, ring, out, args.steps, torch)
+    if not args.no_extras:
+        line["logit_chain"] = bench_logit_chain(w, ring[0], torch, dev)
+        line["host_buffers"] = bench_host_buffers(w, s, ring[0], out, torch)
+        line["per_row_configs"] = bench_configs(w, s, ring, out, args.steps, torch)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(w)
     print(json.dumps(line))
