@@ -60,9 +60,11 @@ def synth_logits_device(w, count, torch, dev):
     return ring
 
 
-def cpu_baseline(w, seconds_budget=12.0):
+def cpu_baseline(w, gpu_tokens, seconds_budget=12.0):
     """The reference sampler on this box's host cores, on a bounded sample of the workload:
-    `sampler.cpp` itself (oracle/_ref) when it was built, else the oracle's restatement."""
+    `sampler.cpp` itself (oracle/_ref) when it was built, else the oracle's restatement.  The same
+    leg checks `gpu_tokens` (what the library returned for step 0 of the workload) against the
+    oracle: this function is the only place where bench.py touches oracle/."""
     import numpy as np
 
     from executorch_amd import workloads as W
@@ -70,6 +72,9 @@ def cpu_baseline(w, seconds_budget=12.0):
 
     rows = min(w.batch, 64)
     x = W.logits(w, 0, rows)
+    want, _ = O.sample_rows(x, w.dtype, O.inv_temperature(w.temperature), w.topp, 0, W.coin_seeds(w, rows).copy(),
+                            mode=O.MODE_UPCAST, tie=O.TIE_STABLE, threads=8)
+    mismatches = int((np.asarray(gpu_tokens)[:rows] != want).sum())
     cores = max(1, min(16, os.cpu_count() or 1))
     use_ref = O.have_ref()
 
@@ -101,6 +106,7 @@ def cpu_baseline(w, seconds_budget=12.0):
         "sample": f"{rows} rows of {w.name} step 0, each sampled {reps} times by its own Sampler, native "
                   f"{W.DTYPE_NAMES[w.dtype]} sample<T>, {cores} threads ({dt:.1f} s)",
         "rows_per_s_one_core": one_core,
+        "parity": {"rows_checked": rows, "token_mismatches_vs_oracle": mismatches},
     }
 
 
@@ -208,8 +214,6 @@ def main():
 
     import executorch_amd as ea
     from executorch_amd import workloads as W
-    from oracle import oracle as O
-
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
     w = W.WORKLOADS[args.workload]
@@ -219,7 +223,7 @@ def main():
     s = ea.Sampler(w.vocab, w.temperature, w.topp, w.coin_seed, max_batch=w.batch)
     out = torch.empty(w.batch, dtype=torch.int32, device=dev)
 
-    # parity spot check on host-generated rows before timing anything
+    # step 0 of the workload from host-generated rows: the tokens the CPU leg checks
     rows = min(w.batch, 64)
     hx = W.logits(w, 0, rows)
     if w.dtype == W.DTYPE_BFLOAT16:
@@ -228,9 +232,6 @@ def main():
         dx = torch.from_numpy(hx).to(dev)
     chk = ea.Sampler(w.vocab, w.temperature, w.topp, w.coin_seed, max_batch=rows)
     got = chk.sample_batch(dx).cpu().numpy()
-    want, _ = O.sample_rows(hx, w.dtype, O.inv_temperature(w.temperature), w.topp, 0, W.coin_seeds(w, rows).copy(),
-                            mode=O.MODE_UPCAST, tie=O.TIE_STABLE, threads=8)
-    mismatches = int((got != want).sum())
 
     if args.copy_probe:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_()
@@ -277,14 +278,13 @@ def main():
                      "traffic_source": "profiles/sample_rows_kernel_cfg2.md" if w.name in MEASURED_TRAFFIC_BYTES else None,
                      "kernel": "sample_rows_kernel",
                      "kernel_ms": kernel_ms, "algorithmic_bytes_per_launch": step_bytes},
-        "parity": {"rows_checked": rows, "token_mismatches_vs_oracle": mismatches},
     }
     if not args.no_extras:
         line["logit_chain"] = bench_logit_chain(w, ring[0], torch, dev)
         line["host_buffers"] = bench_host_buffers(w, s, ring[0], out, torch)
         line["per_row_configs"] = bench_configs(w, s, ring, out, args.steps, torch)
     if not args.no_cpu_baseline:
-        line["cpu_baseline"] = cpu_baseline(w)
+        line["cpu_baseline"] = cpu_baseline(w, got)
     print(json.dumps(line))
 
 
