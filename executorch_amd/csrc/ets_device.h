@@ -186,6 +186,7 @@ struct BlockScratch {
   float group_total[2][kWaves];    // same, for seq_sum_group
   float slot_sum[64];               // plain float sums per slot (seq_sum_predicted)
   float chain_s[2];                 // running sum handed from one serial slot to the next
+  int chain_found[2];               //   and where the threshold was crossed, if it was
   float aux_total[2][kWaves];      // second value of block_sum2
   float red_f[kWaves];
   uint32_t red_u[kWaves];
@@ -377,27 +378,33 @@ __device__ void wave_resolve(float& s, int& found, const uint32_t (&bits)[R], in
   }
 }
 
-// First attempt at a group of U * 16 slots for a plain sum (no threshold): fold every slot ONCE,
-// with the ulp it is predicted to see, instead of once per binade the running sum passes through.
+// First attempt at a group of U * 16 slots: fold every slot ONCE, with the ulp it is predicted to
+// see, instead of once per binade the running sum passes through.
 //   1. plain float sums per slot give approximate running sums at the slot boundaries;
 //   2. a slot whose two boundaries lie safely inside one binade is "stable" and is folded with that
-//      binade's ulp into a parity summary; the others (a binade boundary inside or within 2^-13
-//      of an end -- plain and sequential sums of a group's 16384 entries differ by random rounding,
-//      some 1e-5 of the sum -- or sums too small for the float shortcut) are "serial";
+//      binade's ulp into a parity summary; the others (a binade boundary or the threshold inside
+//      or within 2^-13 of an end -- plain and sequential sums of a group's 16384 entries differ by
+//      random rounding, some 1e-5 of the sum -- or sums too small for the float shortcut) are
+//      "serial";
 //   3. the slots are consumed in order from the exact running sum: a run of stable slots by
 //      composing its summaries -- after checking that the exact sum entering it has the predicted
-//      exponent and that the run does not leave the binade, which is all their validity needs --
-//      and a serial slot by wave_resolve() in its own wave, one barrier each.
+//      exponent and that the run neither leaves the binade nor crosses the threshold, which is
+//      all their validity needs -- and a serial slot by wave_resolve() in its own wave, one barrier
+//      each.
 // The predictions steer only which work is done; every committed step is exact.  Returns the
 // number of slots consumed (st.s is the exact sum behind them): a failed check stops in front of
-// the offending run, and the caller continues from there with the general rounds.
-template <int U, int R>
-__device__ int seq_sum_predicted(SeqSum& st, const uint32_t (&bits)[U][R], const int (&first)[U], int n, BlockScratch& sm) {
+// the offending run, and the caller continues from there with the general rounds.  When the
+// threshold is crossed st.stop_index is set and `stopped` is true.
+// PLAIN: the threshold is known to be +inf at compile time (a plain sum).
+template <int U, int R, bool PLAIN>
+__device__ int seq_sum_predicted(SeqSum& st, const uint32_t (&bits)[U][R], const int (&first)[U], int n, float threshold,
+                                 bool& stopped, BlockScratch& sm) {
+  if (PLAIN) threshold = __uint_as_float(0x7f800000u);
+  stopped = false;
   static_assert(U * kWaves <= 32, "the serial-slot mask is 32 bits");
   constexpr int kSlots = U * kWaves;
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
-  const float kInf = __uint_as_float(0x7f800000u);
   const float kBig = 67108864.0f;
   // ---- 1
 #pragma unroll
@@ -415,7 +422,8 @@ __device__ int seq_sum_predicted(SeqSum& st, const uint32_t (&bits)[U][R], const
   const float s_out = st.s + incl;
   const uint32_t kb_in = __float_as_uint(s_in) >> 23, kb_out = __float_as_uint(s_out) >> 23;
   const float edge = __uint_as_float(kb_in << 23);  // 2^(kb_in - 127) <= s_in
-  const bool serial = kb_in != kb_out || kb_in < 70u || kb_in > 250u || s_in < edge * 1.0001220703125f || s_out > edge * 1.999755859375f;
+  const bool serial = kb_in != kb_out || kb_in < 70u || kb_in > 250u || s_in < edge * 1.0001220703125f ||
+                      s_out > edge * 1.999755859375f || (!PLAIN && !(s_out < threshold * 0.9998779296875f));
   const uint32_t serial_mask = static_cast<uint32_t>(__ballot(serial && lane < kSlots));
   const uint32_t buf = st.parity_buf;
   st.parity_buf ^= 1u;
@@ -460,7 +468,9 @@ __device__ int seq_sum_predicted(SeqSum& st, const uint32_t (&bits)[U][R], const
       const ParityInc upto = wave_scan_inclusive(in_run, lane);
       const uint32_t total = (ss.S & 1u) ? readlane_u32(upto.odd, 63) : readlane_u32(upto.even, 63);
       if (ss.S + total >= (1u << 24)) break;  // the run would leave the binade
-      s = sum_value(ss.S + total, ss.kb);
+      const float s_run = sum_value(ss.S + total, ss.kb);
+      if (!PLAIN && s_run > threshold) break;  // the crossing lies inside the run after all
+      s = s_run;
       pos = next_serial;
     }
     if (pos == kSlots) break;
@@ -470,13 +480,23 @@ __device__ int seq_sum_predicted(SeqSum& st, const uint32_t (&bits)[U][R], const
       int found = -1;
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        if (u == ustar) wave_resolve<R>(sw, found, bits[u], first[u], n, kInf);
+        if (u == ustar) wave_resolve<R>(sw, found, bits[u], first[u], n, threshold);
       }
-      if (lane == 0) sm.chain_s[hand] = sw;
+      if (lane == 0) {
+        sm.chain_s[hand] = sw;
+        if (!PLAIN) sm.chain_found[hand] = found;
+      }
     }
     __syncthreads();
     s = sm.chain_s[hand];
+    const int found = PLAIN ? -1 : sm.chain_found[hand];
     hand ^= 1u;
+    if (found >= 0) {
+      st.s = s;
+      st.stop_index = found;
+      stopped = true;
+      return pos;
+    }
     ++pos;
   }
   st.s = s;
@@ -589,16 +609,21 @@ __device__ __forceinline__ bool seq_sum_chunk(SeqSum& st, const uint32_t (&bits)
 #pragma unroll
   for (int e = 0; e < R; ++e) b[0][e] = bits[e];
   const int f[1] = {first};
-  return seq_sum_rounds<1, R>(st, b, f, n, threshold, sm);
+  bool stopped = false;
+  const int consumed = seq_sum_predicted<1, R, false>(st, b, f, n, threshold, stopped, sm);
+  if (stopped) return true;
+  if (consumed == kWaves) return false;
+  return seq_sum_rounds<1, R>(st, b, f, n, threshold, sm, consumed);
 }
 
 // Consumes U chunks (chunk u: lane `tid` owns elements first[u] .. first[u] + R - 1, chunks in
 // increasing position) with ONE barrier when all of them stay inside the binade of s, below the
 // threshold and free of ties; `acc` must have been folded over the same elements with
 // scale = fast_scale(st.s).  Otherwise the chunks go through seq_sum_rounds.
-template <int U, int R>
+template <int U, int R, bool PLAIN = false>
 __device__ bool seq_sum_group(SeqSum& st, const uint32_t (&bits)[U][R], FastAcc acc, float scale,
                               const int (&first)[U], int n, float threshold, BlockScratch& sm) {
+  if (PLAIN) threshold = __uint_as_float(0x7f800000u);  // a plain sum: the compiler drops the comparisons
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const float kBig = 67108864.0f;  // 2^26: "take the ordered path"
@@ -621,8 +646,10 @@ __device__ bool seq_sum_group(SeqSum& st, const uint32_t (&bits)[U][R], FastAcc 
     }
   }
   int consumed = 0;
-  if (U * kWaves <= 32 && threshold == __uint_as_float(0x7f800000u)) {
-    consumed = seq_sum_predicted<U, R>(st, bits, first, n, sm);
+  if (U * kWaves <= 32) {
+    bool stopped = false;
+    consumed = seq_sum_predicted<U, R, PLAIN>(st, bits, first, n, threshold, stopped, sm);
+    if (stopped) return true;
     if (consumed == U * kWaves) return false;
   }
   return seq_sum_rounds<U, R>(st, bits, first, n, threshold, sm, consumed);

@@ -247,7 +247,7 @@ __device__ int draw_from_sorted(Keys keys, int n_sorted, int n_total, bool use_t
   if (use_topk) {
     last_idx = topk - 1;
     mass = (topk <= kSmallWalk) ? seq_sum_small(keys, topk, kInf, sm).sum
-                                : seq_sum_block<1>(sorted_prob, topk, 0.0f, kInf, sm).sum;
+                                : seq_sum_block<4>(sorted_prob, topk, 0.0f, kInf, sm).sum;
   } else {
     // a short prefix usually holds the whole nucleus
     SeqSumResult res = {0.0f, -1};
@@ -259,14 +259,14 @@ __device__ int draw_from_sorted(Keys keys, int n_sorted, int n_total, bool use_t
       res = seq_sum_small(keys, kSmallWalk, topp, sm);
       decided = res.stop_index >= 0;
     }
-    if (!decided) res = seq_sum_block<1>(sorted_prob, n_sorted, 0.0f, topp, sm);
+    if (!decided) res = seq_sum_block<4>(sorted_prob, n_sorted, 0.0f, topp, sm);
     if (res.stop_index < 0 && n_sorted < n_total) return -2;
     last_idx = res.stop_index >= 0 ? res.stop_index : n_sorted - 1;
     mass = res.sum;
   }
   const float r = coin * mass;  // sampler.cpp:109 / :162
   const SeqSumResult walk = (last_idx < kSmallWalk) ? seq_sum_small(keys, last_idx + 1, r, sm)
-                                                    : seq_sum_block<1>(sorted_prob, last_idx + 1, 0.0f, r, sm);
+                                                    : seq_sum_block<4>(sorted_prob, last_idx + 1, 0.0f, r, sm);
   const int pos = walk.stop_index >= 0 ? walk.stop_index : last_idx;
   dbg.last_idx = last_idx;
   dbg.cumulative = mass;
@@ -525,7 +525,7 @@ __device__ __forceinline__ bool scan_row(const ScanArgs& a, SeqSum& st, BlockScr
           }
         }
       }
-      if (seq_sum_group<kGroup, VE>(st, bits, acc, scale, first, V, a.threshold, sm)) return true;
+      if (seq_sum_group<kGroup, VE, MODE == kScanSum>(st, bits, acc, scale, first, V, a.threshold, sm)) return true;
     }
     done_elems = nvec * VE;
   }
