@@ -142,9 +142,52 @@ __device__ void lds_merge_stages(uint64_t* t, int T, int gbase, int k, int j_sta
   }
 }
 
-// Ascending sort of N keys (a power of two) that already sit in LDS.
+// Ascending sort of N keys (a power of two) that already sit in LDS (and are visible to the
+// workgroup).  Bitonic network; every wave owns a contiguous run of W keys, and the sub-stages
+// whose partners lie inside one run (distance < W) are done by that wave alone, back to back
+// without workgroup barriers -- LDS serves one wave's accesses in order -- so only the
+// log2(N / W) long-distance sub-stages of each merge pay a barrier.  Ends with a barrier.
 __device__ void sort_keys_lds(uint64_t* lds, int N) {
-  for (int k = 2; k <= N; k <<= 1) lds_merge_stages(lds, N, 0, k, k >> 1);
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  int waves = N / 128;  // at least two keys per lane of a participating wave
+  waves = waves < 1 ? 1 : (waves > kWaves ? kWaves : waves);
+  const int W = N / waves;
+  uint64_t* mine = lds + wave * W;
+  for (int k = 2; k <= N; k <<= 1) {
+    int j = k >> 1;
+    for (; j >= W; j >>= 1) {
+      for (int q = threadIdx.x; q < (N >> 1); q += kBlock) {
+        const int i = ((q & ~(j - 1)) << 1) | (q & (j - 1));
+        const int l = i | j;
+        const bool up = (i & k) == 0;
+        const uint64_t a = lds[i], b = lds[l];
+        if ((a > b) == up) {
+          lds[i] = b;
+          lds[l] = a;
+        }
+      }
+      __syncthreads();
+    }
+    if (wave < waves) {
+      for (; j > 0; j >>= 1) {
+        for (int q = lane; q < (W >> 1); q += 64) {
+          const int i = ((q & ~(j - 1)) << 1) | (q & (j - 1));
+          const int l = i | j;
+          const bool up = ((wave * W + i) & k) == 0;
+          const uint64_t a = mine[i], b = mine[l];
+          if ((a > b) == up) {
+            mine[i] = b;
+            mine[l] = a;
+          }
+        }
+        // other lanes of this wave read these keys next: keep the compiler from carrying values
+        // across sub-stages in registers
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+      }
+    }
+    if (k >= W) __syncthreads();  // the next merge starts with a long-distance sub-stage, or this was the last
+  }
 }
 
 // Ascending sort of keys[0, N), N a power of two, by one workgroup.  `keys` is global memory;
