@@ -170,6 +170,38 @@ def bench_host_buffers(w, s, logits, out, torch):
             "single_row_host_entry_us": row_us}
 
 
+def bench_gumbel(w, s, ring, out, torch):
+    """The Gumbel-max mode (one pass, no sequential sum) on the same ring with the library's own
+    noise: one read of the logits, priced against the HBM peak."""
+    state = {"i": 0}
+
+    def step():
+        s.gumbel_max_batch(ring[state["i"] % len(ring)], w.temperature, out=out)
+        state["i"] += 1
+
+    us = timed_us(step, 100, torch)
+    gbs = w.bytes_per_step / (us * 1e-6) / 1e9
+    return {"us_per_step": us, "rows_per_s": w.batch / (us * 1e-6), "algorithmic_bytes": w.bytes_per_step, "gbs": gbs,
+            "frac_of_hbm_peak": gbs / HBM_PEAK_GBS}
+
+
+def bench_greedy(w, ring, out, torch):
+    """Temperature 0 (arg-max, sampler.cpp:44-56) on the same ring: one read of the logits."""
+    import executorch_amd as ea
+
+    g = ea.Sampler(w.vocab, 0.0, w.topp, 1, max_batch=w.batch)
+    state = {"i": 0}
+
+    def step():
+        g.sample_batch(ring[state["i"] % len(ring)], out=out)
+        state["i"] += 1
+
+    us = timed_us(step, 100, torch)
+    gbs = w.bytes_per_step / (us * 1e-6) / 1e9
+    return {"us_per_step": us, "rows_per_s": w.batch / (us * 1e-6), "algorithmic_bytes": w.bytes_per_step, "gbs": gbs,
+            "frac_of_hbm_peak": gbs / HBM_PEAK_GBS}
+
+
 def bench_configs(w, s, ring, out, steps, torch):
     """ets_sampler_sample_batch_configs on the same ring: every row with the workload's own
     parameters (one launch, plus the upload of the per-row table), and a mix of four kinds of rows
@@ -282,6 +314,8 @@ def main():
     if not args.no_extras:
         line["logit_chain"] = bench_logit_chain(w, ring[0], torch, dev)
         line["host_buffers"] = bench_host_buffers(w, s, ring[0], out, torch)
+        line["gumbel_max"] = bench_gumbel(w, s, ring, out, torch)
+        line["greedy"] = bench_greedy(w, ring, out, torch)
         line["per_row_configs"] = bench_configs(w, s, ring, out, args.steps, torch)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(w, got)

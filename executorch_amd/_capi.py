@@ -47,6 +47,8 @@ SIGNATURES = {
                                          C.c_void_p, C.c_void_p, C.c_void_p]),
     "ets_sampler_sample_batch_debug": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int64, C.c_void_p,
                                                    C.c_void_p, C.c_void_p, C.c_void_p]),
+    "ets_sampler_gumbel_max_batch": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int64, C.c_void_p, C.c_int32,
+                                     C.c_void_p, C.c_void_p, C.c_void_p]),
     "ets_sampler_set_timing": (C.c_int32, [C.c_void_p, C.c_int32]),
     "ets_sampler_get_stats": (C.c_int32, [C.c_void_p, C.c_void_p]),
     "ets_sampler_reset_stats": (C.c_int32, [C.c_void_p]),

@@ -38,7 +38,6 @@ struct ets_sampler {
   uint64_t* d_rng = nullptr;       // [max_batch]
   uint64_t* d_scratch = nullptr;   // [max_batch, scratch_stride], allocated on first stochastic use
   uint64_t* d_partials = nullptr;  // [max_batch, kMaxSplits] argmax partial results
-  uint32_t* d_counters = nullptr;  // [max_batch] argmax arrival counters (zero between launches)
   void* d_row = nullptr;           // staging for one host row (vocab * 4 bytes)
   int32_t* d_token = nullptr;      // staging for one token
   // per-row sampling parameters of ets_sampler_sample_batch_configs(): pinned host staging, its
@@ -142,18 +141,33 @@ ets_status timing_end(ets_sampler* s, hipStream_t stream, int slot) {
   return ETS_OK;
 }
 
+// Workgroups per row of the partial kernels: enough to fill 256 CUs a few times over, but no
+// segment under 4096 entries.
+int row_splits(int32_t vocab, int32_t rows) {
+  int splits = (1024 + rows - 1) / rows;
+  const int max_by_len = (vocab + 4095) / 4096;
+  if (splits > max_by_len) splits = max_by_len;
+  if (splits > kMaxSplits) splits = kMaxSplits;
+  return splits < 1 ? 1 : splits;
+}
+
 template <int DT>
 ets_status launch_argmax(ets_sampler* s, const void* d_logits, int32_t batch, int64_t stride, int32_t* d_tokens,
                          hipStream_t stream, const int32_t* d_row_map = nullptr) {
-  // Enough workgroups to fill 256 CUs several times over, but no segment under 2048 entries.
-  int splits = (2048 + batch - 1) / batch;
-  const int max_by_len = (s->vocab + 2047) / 2048;
-  if (splits > max_by_len) splits = max_by_len;
-  if (splits > kMaxSplits) splits = kMaxSplits;
-  if (splits < 1) splits = 1;
-  dim3 grid(splits, batch);
-  hipLaunchKernelGGL((ets::argmax_kernel<DT>), grid, dim3(ets::kArgmaxBlock), 0, stream, d_logits, stride, s->vocab,
-                     s->d_partials, s->d_counters, d_tokens, d_row_map);
+  const int splits = row_splits(s->vocab, batch);
+  const size_t esz = ets::ElemSize<DT>::value;
+  const bool aligned = (reinterpret_cast<uintptr_t>(d_logits) % 16 == 0) && ((static_cast<size_t>(stride) * esz) % 16 == 0);
+  const dim3 grid(splits, batch);
+  if (aligned) {
+    hipLaunchKernelGGL((ets::argmax_partial_kernel<DT, true>), grid, dim3(ets::kArgmaxBlock), 0, stream, d_logits, stride,
+                       s->vocab, s->d_partials, d_row_map);
+  } else {
+    hipLaunchKernelGGL((ets::argmax_partial_kernel<DT, false>), grid, dim3(ets::kArgmaxBlock), 0, stream, d_logits, stride,
+                       s->vocab, s->d_partials, d_row_map);
+  }
+  ETS_HIP(s, hipGetLastError());
+  hipLaunchKernelGGL((ets::argmax_finish_kernel<DT>), dim3(batch), dim3(64), 0, stream, d_logits, stride, s->d_partials,
+                     splits, d_tokens, d_row_map);
   ETS_HIP(s, hipGetLastError());
   return ETS_OK;
 }
@@ -414,10 +428,6 @@ ets_status ets_sampler_create(int32_t vocab_size, float temperature, float topp,
   if (e != hipSuccess) return bail(e, "hipMalloc(rng states)");
   e = hipMalloc(reinterpret_cast<void**>(&s->d_partials), sizeof(uint64_t) * max_batch * kMaxSplits);
   if (e != hipSuccess) return bail(e, "hipMalloc(argmax partials)");
-  e = hipMalloc(reinterpret_cast<void**>(&s->d_counters), sizeof(uint32_t) * max_batch);
-  if (e != hipSuccess) return bail(e, "hipMalloc(argmax counters)");
-  e = hipMemset(s->d_counters, 0, sizeof(uint32_t) * max_batch);
-  if (e != hipSuccess) return bail(e, "hipMemset(argmax counters)");
   e = hipMalloc(&s->d_row, static_cast<size_t>(vocab_size) * 4);
   if (e != hipSuccess) return bail(e, "hipMalloc(row staging)");
   e = hipMalloc(reinterpret_cast<void**>(&s->d_token), sizeof(int32_t));
@@ -447,7 +457,6 @@ ets_status ets_sampler_destroy(ets_sampler* s) {
     (void)hipFree(s->d_rng);
     (void)hipFree(s->d_scratch);
     (void)hipFree(s->d_partials);
-    (void)hipFree(s->d_counters);
     (void)hipFree(s->d_row);
     (void)hipFree(s->d_token);
     (void)hipFree(s->d_stage);
@@ -529,6 +538,74 @@ ets_status ets_sampler_sample_batch_configs(ets_sampler* s, const void* d_logits
   if (st != ETS_OK) return st;
   st = sample_device_configs(s, d_logits, dtype, batch, row_stride_elems, configs, d_tokens, d_debug, stream);
   if (st != ETS_OK) return st;
+  return timing_end(s, stream, slot);
+}
+
+ets_status ets_sampler_gumbel_max_batch(ets_sampler* s, const void* d_logits, int32_t dtype, int32_t batch,
+                                        int64_t row_stride_elems, const float* temperatures, int32_t n_temperatures,
+                                        const float* d_noise, int32_t* d_tokens, void* hip_stream) {
+  if (!s) return fail(nullptr, ETS_INVALID_ARGUMENT, "ets_sampler_gumbel_max_batch: null handle");
+  s->last_error.clear();
+  if (!d_logits || !d_tokens || !temperatures)
+    return fail(s, ETS_INVALID_ARGUMENT, "ets_sampler_gumbel_max_batch: null pointer");
+  if (dtype != ETS_DTYPE_FLOAT && dtype != ETS_DTYPE_HALF && dtype != ETS_DTYPE_BFLOAT16)
+    return fail(s, ETS_INVALID_ARGUMENT, "ets_sampler_gumbel_max_batch: element type must be Float, Half or BFloat16");
+  if (batch < 0 || batch > s->max_batch)
+    return fail(s, ETS_INVALID_ARGUMENT, "ets_sampler_gumbel_max_batch: batch exceeds the handle's max_batch");
+  if (row_stride_elems < s->vocab)
+    return fail(s, ETS_INVALID_ARGUMENT, "ets_sampler_gumbel_max_batch: row stride smaller than vocab_size");
+  if (n_temperatures != 1 && n_temperatures != batch)
+    return fail(s, ETS_INVALID_ARGUMENT, "ets_sampler_gumbel_max_batch: one temperature, or one per row");
+  if (batch == 0) return ETS_OK;
+  DeviceGuard g(s->device);
+  hipStream_t stream = static_cast<hipStream_t>(hip_stream);
+  // one temperature travels as a kernel argument; one per row goes through the pinned staging
+  // buffer (waiting, if need be, until the previous upload has left it)
+  ets_status st = ETS_OK;
+  const float* d_row_temperatures = nullptr;
+  if (n_temperatures > 1) {
+    st = ensure_stage(s);
+    if (st != ETS_OK) return st;
+    if (s->stage_pending) {
+      ETS_HIP(s, hipEventSynchronize(s->stage_event));
+      s->stage_pending = false;
+    }
+    std::memcpy(s->h_stage, temperatures, sizeof(float) * n_temperatures);
+    ETS_HIP(s, hipMemcpyAsync(s->d_stage, s->h_stage, sizeof(float) * n_temperatures, hipMemcpyHostToDevice, stream));
+    ETS_HIP(s, hipEventRecord(s->stage_event, stream));
+    s->stage_pending = true;
+    d_row_temperatures = static_cast<const float*>(s->d_stage);
+  }
+  const float temperature = temperatures[0];
+  int slot = -1;
+  st = timing_begin(s, stream, batch, &slot);
+  if (st != ETS_OK) return st;
+  // the draw is bound by instruction issue, not by bytes: more, smaller segments than the arg-max
+  int splits = (2048 + batch - 1) / batch;
+  const int max_by_len = (s->vocab + 1023) / 1024;
+  if (splits > max_by_len) splits = max_by_len;
+  if (splits > kMaxSplits) splits = kMaxSplits;
+  if (splits < 1) splits = 1;
+  const dim3 grid(splits, batch);
+  switch (dtype) {
+    case ETS_DTYPE_FLOAT:
+      hipLaunchKernelGGL((ets::gumbel_partial_kernel<ets::kDtypeFloat>), grid, dim3(ets::kArgmaxBlock), 0, stream, d_logits,
+                         row_stride_elems, s->vocab, temperature, d_row_temperatures, d_noise, s->d_rng, s->d_partials);
+      break;
+    case ETS_DTYPE_HALF:
+      hipLaunchKernelGGL((ets::gumbel_partial_kernel<ets::kDtypeHalf>), grid, dim3(ets::kArgmaxBlock), 0, stream, d_logits,
+                         row_stride_elems, s->vocab, temperature, d_row_temperatures, d_noise, s->d_rng, s->d_partials);
+      break;
+    default:
+      hipLaunchKernelGGL((ets::gumbel_partial_kernel<ets::kDtypeBFloat16>), grid, dim3(ets::kArgmaxBlock), 0, stream,
+                         d_logits, row_stride_elems, s->vocab, temperature, d_row_temperatures, d_noise, s->d_rng,
+                         s->d_partials);
+      break;
+  }
+  ETS_HIP(s, hipGetLastError());
+  hipLaunchKernelGGL(ets::gumbel_finish_kernel, dim3(batch), dim3(64), 0, stream, s->d_partials, splits,
+                     d_noise ? 0 : 1, s->d_rng, d_tokens);
+  ETS_HIP(s, hipGetLastError());
   return timing_end(s, stream, slot);
 }
 

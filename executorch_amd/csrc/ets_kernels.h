@@ -1,6 +1,6 @@
 // gfx950 kernels of the token sampler.
 //
-//   argmax_kernel        temperature == 0 (Sampler::sample_argmax, sampler.cpp:44-56)
+//   argmax_*_kernel      temperature == 0 (Sampler::sample_argmax, sampler.cpp:44-56)
 //   sample_rows_kernel   temperature != 0: scale, softmax, coin, top-k / multinomial / top-p
 //                        (sampler.cpp:58-171, 189-251), one workgroup per row
 //
@@ -66,60 +66,160 @@ __device__ __forceinline__ uint64_t wave_max_u64(uint64_t v) {
 
 constexpr int kArgmaxBlock = 256;
 
-// grid = (splits, batch).  Each workgroup scans one segment of a row; the workgroup that
-// finishes a row last combines the partial results.  counters[] must be zero on entry and is
-// left zero.
-template <int DT>
-__global__ void __launch_bounds__(kArgmaxBlock)
-argmax_kernel(const void* logits_all, int64_t row_stride, int32_t vocab, uint64_t* partials, uint32_t* counters,
-              int32_t* tokens, const int32_t* row_map) {
+// The arg-max and the Gumbel-max draw are two launches each: a partial kernel, grid = (splits,
+// rows), in which every workgroup reduces one segment of a row to one 64-bit (key, ~index)
+// maximum, and a finish kernel, one wave per row, that combines the row's partial results.  The
+// kernel boundary orders the two; a single kernel with a device-scope fence per workgroup costs
+// several times more on a part whose L2 is split over 8 dies.
+__device__ __forceinline__ uint64_t pack_best(uint32_t key, int index) {
+  // ties go to the lower index: larger (0xffffffff - index)
+  return (static_cast<uint64_t>(key) << 32) | (0xffffffffu - static_cast<uint32_t>(index));
+}
+
+__device__ __forceinline__ void store_block_best(uint64_t best, uint64_t* slot) {
   __shared__ uint64_t red[kArgmaxBlock / 64];
-  __shared__ int is_last;
+  best = wave_max_u64(best);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = best;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < kArgmaxBlock / 64; ++w) best = red[w] > best ? red[w] : best;
+    *slot = best;
+  }
+}
+
+// ALIGNED: the row's base and pitch are multiples of 16 bytes (128-bit loads).
+template <int DT, bool ALIGNED>
+__global__ void __launch_bounds__(kArgmaxBlock)
+argmax_partial_kernel(const void* logits_all, int64_t row_stride, int32_t vocab, uint64_t* partials,
+                      const int32_t* row_map) {
+  constexpr int VE = VecElems<DT>::value;
   const int row = row_map ? row_map[blockIdx.y] : blockIdx.y;
   const int splits = gridDim.x;
   const int tid = threadIdx.x;
   const char* logits = static_cast<const char*>(logits_all) + static_cast<int64_t>(row) * row_stride * ElemSize<DT>::value;
+  uint64_t best = 0;
+  auto visit = [&](float value, uint32_t raw16, int index) {
+    const uint32_t key = DT == kDtypeUInt16 ? raw16 + 1u : order_key(value);
+    const uint64_t packed = pack_best(key, index);
+    best = packed > best ? packed : best;
+  };
+  int scalar_lo = 0, scalar_hi = vocab;  // entries left to the scalar loop
+  if (ALIGNED && DT != kDtypeUInt16) {
+    const int nvec = vocab / VE;
+    const int seg = (nvec + splits - 1) / splits;
+    const int lo = blockIdx.x * seg, hi = min(nvec, lo + seg);
+    const uint4* vec = reinterpret_cast<const uint4*>(logits);
+    for (int j = lo + tid; j < hi; j += 4 * kArgmaxBlock) {  // four loads in flight; extra ones re-read vec[j]
+      uint4 r[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const int jk = j + k * kArgmaxBlock;
+        r[k] = vec[jk < hi ? jk : j];
+      }
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const int jk = j + k * kArgmaxBlock;
+        if (jk < hi) {
+          float v[VE];
+          decode_vec<DT>(r[k], v);
+#pragma unroll
+          for (int e = 0; e < VE; ++e) visit(v[e], 0u, jk * VE + e);
+        }
+      }
+    }
+    // the last workgroup of the row also takes the entries behind the last full vector
+    scalar_lo = blockIdx.x == splits - 1 ? nvec * VE : vocab;
+  } else {
+    const int seg = (vocab + splits - 1) / splits;
+    scalar_lo = blockIdx.x * seg;
+    scalar_hi = min(vocab, scalar_lo + seg);
+  }
+  for (int i = scalar_lo + tid; i < scalar_hi; i += kArgmaxBlock) {
+    if (DT == kDtypeUInt16) {
+      visit(0.0f, static_cast<uint32_t>(static_cast<const uint16_t*>(static_cast<const void*>(logits))[i]), i);
+    } else {
+      visit(load_elem<DT>(logits, i), 0u, i);
+    }
+  }
+  store_block_best(best, &partials[static_cast<int64_t>(blockIdx.y) * splits + blockIdx.x]);
+}
+
+// grid = (rows), 64 lanes: lane l reads the row's l-th partial result (splits <= 64).
+template <int DT>
+__global__ void __launch_bounds__(64)
+argmax_finish_kernel(const void* logits_all, int64_t row_stride, const uint64_t* partials, int32_t splits,
+                     int32_t* tokens, const int32_t* row_map) {
+  const int row = row_map ? row_map[blockIdx.x] : blockIdx.x;
+  const int lane = threadIdx.x;
+  uint64_t b = lane < splits ? partials[static_cast<int64_t>(blockIdx.x) * splits + lane] : 0ull;
+  b = wave_max_u64(b);
+  if (lane != 0) return;
+  int32_t token = static_cast<int32_t>(0xffffffffu - static_cast<uint32_t>(b));
+  if (DT != kDtypeUInt16) {
+    // `x > NaN` is never true: a NaN in slot 0 stays the maximum (sampler.cpp:47-50)
+    const char* logits = static_cast<const char*>(logits_all) + static_cast<int64_t>(row) * row_stride * ElemSize<DT>::value;
+    const float x0 = load_elem<DT>(logits, 0);
+    if (x0 != x0) token = 0;
+  }
+  tokens[row] = token;
+}
+
+// ---- Gumbel-max draw -------------------------------------------------------------------------
+// argmax_i(logit_i / T + g_i), g_i = -log(-log(u_i + 1e-20) + 1e-20), the in-graph sampler of
+// examples/models/qwen3_5_moe/sampler.py:52-60: one pass over the row, no sequential dependency.
+// u comes from `noise` ([batch, vocab] fp32, e.g. torch.rand_like(logits)) or, when that is
+// null, from a counter-based generator keyed by the row's coin state and the entry's index; the
+// finish kernel then advances the row's xorshift64* state by one step.
+__device__ __forceinline__ float uniform_of(uint64_t state, uint32_t index) {
+  // splitmix64 finaliser over (state, index); 24 random bits -> [0, 1)
+  uint64_t z = state + (static_cast<uint64_t>(index) + 1ull) * 0x9E3779B97F4A7C15ull;
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  z ^= z >> 31;
+  return static_cast<float>(static_cast<uint32_t>(z >> 40)) * (1.0f / 16777216.0f);
+}
+
+__device__ __forceinline__ float gumbel_of(float u) { return -logf(-logf(u + 1e-20f) + 1e-20f); }
+
+template <int DT>
+__global__ void __launch_bounds__(kArgmaxBlock)
+gumbel_partial_kernel(const void* logits_all, int64_t row_stride, int32_t vocab, float temperature,
+                      const float* row_temperatures, const float* noise, const uint64_t* rng, uint64_t* partials) {
+  const int row = blockIdx.y;
+  const int splits = gridDim.x;
+  const int tid = threadIdx.x;
+  const char* logits = static_cast<const char*>(logits_all) + static_cast<int64_t>(row) * row_stride * ElemSize<DT>::value;
+  // logits / temperature.clamp(min=1e-6)  (sampler.py:50)
+  const RowDivisor div = row_divisor(__builtin_fmaxf(row_temperatures ? row_temperatures[row] : temperature, 1e-6f));
+  const uint64_t state = rng[row];
+  const float* u_row = noise ? noise + static_cast<int64_t>(row) * vocab : nullptr;
   const int seg = (vocab + splits - 1) / splits;
   const int lo = blockIdx.x * seg;
   const int hi = min(vocab, lo + seg);
   uint64_t best = 0;
   for (int i = lo + tid; i < hi; i += kArgmaxBlock) {
-    uint32_t key;
-    if (DT == kDtypeUInt16) {
-      key = static_cast<uint32_t>(static_cast<const uint16_t*>(static_cast<const void*>(logits))[i]) + 1u;
-    } else {
-      key = order_key(load_elem<DT>(logits, i));
-    }
-    // ties go to the lower index: larger (0xffffffff - i)
-    const uint64_t packed = (static_cast<uint64_t>(key) << 32) | (0xffffffffu - static_cast<uint32_t>(i));
+    const float x = div_row_signed(load_elem<DT>(logits, i), div);
+    const float u = u_row ? u_row[i] : uniform_of(state, static_cast<uint32_t>(i));
+    const uint64_t packed = pack_best(order_key(x + gumbel_of(u)), i);
     best = packed > best ? packed : best;
   }
-  best = wave_max_u64(best);
-  if ((tid & 63) == 0) red[tid >> 6] = best;
-  __syncthreads();
-  if (tid == 0) {
-    for (int w = 1; w < kArgmaxBlock / 64; ++w) best = red[w] > best ? red[w] : best;
-    partials[static_cast<int64_t>(row) * splits + blockIdx.x] = best;
-    __threadfence();
-    const uint32_t done = atomicAdd(&counters[row], 1u);
-    is_last = (done == static_cast<uint32_t>(splits - 1));
-  }
-  __syncthreads();
-  if (is_last && tid == 0) {
-    __threadfence();
-    uint64_t b = 0;
-    for (int sp = 0; sp < splits; ++sp) {
-      const uint64_t v = __atomic_load_n(&partials[static_cast<int64_t>(row) * splits + sp], __ATOMIC_RELAXED);
-      b = v > b ? v : b;
-    }
-    int32_t token = static_cast<int32_t>(0xffffffffu - static_cast<uint32_t>(b));
-    if (DT != kDtypeUInt16) {
-      // `x > NaN` is never true: a NaN in slot 0 stays the maximum (sampler.cpp:47-50)
-      const float x0 = load_elem<DT>(logits, 0);
-      if (x0 != x0) token = 0;
-    }
-    tokens[row] = token;
-    counters[row] = 0u;
+  store_block_best(best, &partials[static_cast<int64_t>(row) * splits + blockIdx.x]);
+}
+
+__global__ void __launch_bounds__(64)
+gumbel_finish_kernel(const uint64_t* partials, int32_t splits, int32_t advance_rng, uint64_t* rng, int32_t* tokens) {
+  const int row = blockIdx.x;
+  const int lane = threadIdx.x;
+  uint64_t b = lane < splits ? partials[static_cast<int64_t>(row) * splits + lane] : 0ull;
+  b = wave_max_u64(b);
+  if (lane != 0) return;
+  tokens[row] = static_cast<int32_t>(0xffffffffu - static_cast<uint32_t>(b));
+  if (advance_rng) {  // one step of the row's stream per call (sampler.cpp:210-214)
+    uint64_t rs = rng[row];
+    rs ^= rs >> 12;
+    rs ^= rs << 25;
+    rs ^= rs >> 27;
+    rng[row] = rs;
   }
 }
 

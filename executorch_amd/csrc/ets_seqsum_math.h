@@ -43,6 +43,13 @@ ETS_HD float div_row(float e, const RowDivisor& d) {
   return p;
 }
 
+// The same for a numerator of either sign (logits divided by a temperature).
+ETS_HD float div_row_signed(float x, const RowDivisor& d) {
+  const float q = static_cast<float>(static_cast<double>(x) * d.recip);
+  if (__builtin_fabsf(q) <= 1.17549435e-38f && x != 0.0f) return x / d.S;
+  return q;
+}
+
 // ---- sequential float sums as an integer scan --------------------------------------------------
 // A scalar loop `s += a[i]` (a[i] >= 0) rounds after every add.  While s stays inside one
 // binade [2^k, 2^(k+1)) every partial sum is an integer multiple of u = ulp(s): writing

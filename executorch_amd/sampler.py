@@ -168,6 +168,30 @@ class Sampler:
         self._check(st)
         return out
 
+    def gumbel_max_batch(self, logits: torch.Tensor, temperature, noise: torch.Tensor | None = None,
+                         out: torch.Tensor | None = None, dtype: int | None = None) -> torch.Tensor:
+        """The in-graph Gumbel-max sampler (examples/models/qwen3_5_moe/sampler.py:17-60):
+        ``argmax(logits / T.clamp(min=1e-6) + gumbel)``.  ``temperature`` is a float or one per row;
+        ``noise`` is a device fp32 ``[B, vocab]`` tensor of uniforms (``torch.rand_like(logits)`` in the
+        reference) or None for the library's own generator."""
+        if not logits.is_cuda or logits.dim() != 2 or logits.stride(1) != 1:
+            raise SamplerError(_capi.INVALID_ARGUMENT, "gumbel_max_batch wants a device tensor [B, vocab] with unit inner stride")
+        B, V = logits.shape
+        if V != self.vocab_size:
+            raise SamplerError(_capi.INVALID_ARGUMENT, "last dimension differs from vocab_size")
+        t = np.ascontiguousarray(np.atleast_1d(np.asarray(temperature, dtype=np.float32)))
+        if noise is not None and not (noise.is_cuda and noise.dtype == torch.float32 and noise.shape == (B, V)
+                                      and noise.is_contiguous()):
+            raise SamplerError(_capi.INVALID_ARGUMENT, "noise must be a contiguous device fp32 tensor [B, vocab]")
+        code = dtype_code(logits) if dtype is None else dtype
+        if out is None:
+            out = torch.empty(B, dtype=torch.int32, device=logits.device)
+        stream = torch.cuda.current_stream(logits.device).cuda_stream
+        self._check(_capi.lib().ets_sampler_gumbel_max_batch(
+            self._h, logits.data_ptr(), code, B, logits.stride(0), t.ctypes.data, t.size,
+            noise.data_ptr() if noise is not None else None, out.data_ptr(), stream))
+        return out
+
     # ---- sampling time in microseconds (stats.h:46-47, :62-69 keep it in whole milliseconds)
     def set_timing(self, enabled: bool = True) -> None:
         self._check(_capi.lib().ets_sampler_set_timing(self._h, 1 if enabled else 0))

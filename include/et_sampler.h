@@ -143,6 +143,24 @@ ETS_API ets_status ets_sampler_sample_batch_configs(ets_sampler* s, const void* 
                                                    const ets_sampling_config* configs, int32_t* d_tokens,
                                                    ets_row_debug* d_debug, void* hip_stream);
 
+/* The in-graph Gumbel-max sampler, sample(logits, temperature) of
+ * examples/models/qwen3_5_moe/sampler.py:17-60 (the same draw as backends/mlx/llm/sampling.py:39-44
+ * asks of its backend): token = argmax_i(logits_i / max(T, 1e-6) + g_i) with
+ * g_i = -log(-log(u_i + 1e-20) + 1e-20) in fp32, lowest index on ties.  It draws from
+ * softmax(logits / T) like the Sampler above but is NOT the same arithmetic: one pass over the
+ * row, no softmax sum, so its tokens differ from ets_sampler_sample_batch() for the same seed.
+ *   `temperatures`  HOST: one value (a 0-D temperature) or `batch` values (1-D, one per row);
+ *   `d_noise`       DEVICE fp32 [batch, vocab_size] of uniforms in [0, 1) -- what
+ *                   torch.rand_like(logits) is in the reference -- or NULL: then u_i comes from
+ *                   a counter-based generator keyed by row b's coin state and i, and the state
+ *                   advances by one xorshift64* step per call;
+ *   element types   Float (the reference's contract), Half, BFloat16 (converted to fp32).
+ * Asynchronous on `hip_stream`. */
+ETS_API ets_status ets_sampler_gumbel_max_batch(ets_sampler* s, const void* d_logits, int32_t dtype, int32_t batch,
+                                               int64_t row_stride_elems, const float* temperatures,
+                                               int32_t n_temperatures, const float* d_noise, int32_t* d_tokens,
+                                               void* hip_stream);
+
 /* Sampling time at microsecond resolution.  The reference's Stats keeps
  * aggregate_sampling_time_ms from host clocks in whole milliseconds
  * (extension/llm/runner/stats.h:46-47, on_sampling_begin / on_sampling_end :62-69), which reads 0
