@@ -979,6 +979,68 @@ __device__ __forceinline__ float row_quotient(float e, const RowDivisor& div) {
   return EXACT ? div_row(e, div) : div_row_above(e, div);
 }
 
+// Third pass of the histogram draw: entries with order key >= k_star and p >= p_thr go to the key
+// buffer.  Plain functions, not closures: a closure the compiler leaves out of line reads every
+// captured value through memory.
+struct GatherArgs {
+  float inv, m, p_thr;
+  int k_star, cap;
+  RowDivisor div;
+  uint64_t* lds_keys;
+  BlockScratch* sm;
+};
+
+template <bool EXACT>
+__device__ __forceinline__ void gather_take(uint32_t pattern16, int index, const GatherArgs& a) {
+  if (pattern_order(pattern16) < a.k_star) return;
+  const float x = __uint_as_float(pattern16 << 16) * a.inv;
+  const float pj = row_quotient<EXACT>(expf_nonpositive(x - a.m, a.sm->exp2tab), a.div);
+  if (pj >= a.p_thr) {
+    const uint32_t slot = atomicAdd(&a.sm->counter2, 1u);
+    if (slot < static_cast<uint32_t>(a.cap)) a.lds_keys[slot] = cand_key(pj, index);
+  }
+}
+
+// Vectors are screened by their largest order key.  For a positive threshold the patterns
+// themselves, read as signed 16-bit numbers, decide (negative logits are negative numbers).
+template <bool POSITIVE>
+__device__ __forceinline__ int best_order_key(const uint4& r) {
+  const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+  short2v best = {-32768, -32768};
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const short2v h = __builtin_bit_cast(short2v, w[k]);
+    const short2v key = POSITIVE ? h : h ^ ((h >> 15) & static_cast<short>(0x7fff));
+    best = __builtin_elementwise_max(best, key);
+  }
+  return max(static_cast<int>(best.x), static_cast<int>(best.y));
+}
+
+template <bool POSITIVE, bool EXACT>
+__device__ __forceinline__ void gather_sweep(const uint4* vec, int nvec, const GatherArgs& a) {
+  const int tid = threadIdx.x;
+  for (int j = tid; j < nvec; j += 16 * kBlock) {  // 16 loads in flight; out-of-range ones re-read vec[j]
+    uint4 r[16];
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+      const int jk = j + k * kBlock;
+      r[k] = vec[jk < nvec ? jk : j];
+    }
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+      const int jk = j + k * kBlock;
+      if (jk < nvec && best_order_key<POSITIVE>(r[k]) >= a.k_star) {
+        const uint32_t w[4] = {r[k].x, r[k].y, r[k].z, r[k].w};
+#pragma unroll
+        for (int h = 0; h < 4; ++h) {
+          gather_take<EXACT>(w[h] & 0xffffu, jk * 8 + 2 * h, a);
+          gather_take<EXACT>(w[h] >> 16, jk * 8 + 2 * h + 1, a);
+        }
+      }
+    }
+  }
+}
+
 // With TOPK the same walk selects by COUNT instead of mass: the entries with the `topk` largest
 // probabilities and everything tied with the last of them (sampler.cpp:87-100 sorts all entries;
 // the walks of :103-119 only read the first topk).  The caller passes cutoff = 0 and a scan that
@@ -1167,64 +1229,20 @@ __device__ __noinline__ bool draw_topp_hist(const char* logits, int V, float inv
     k_star = c >= top ? -32768 : (mag >= 0 ? -mag - 1 : 0);
   }
   // ---- gather: entries with order key >= k_star and p >= p_thr
-  auto take = [&](uint32_t pattern16, int index) {
-    if (pattern_order(pattern16) < k_star) return;
-    const float x = __uint_as_float(pattern16 << 16) * inv;
-    const float pj = row_quotient<TOPK>(expf_nonpositive(x - m, sm.exp2tab), div);
-    if (pj >= p_thr) {
-      const uint32_t slot = atomicAdd(&sm.counter2, 1u);
-      if (slot < static_cast<uint32_t>(cap)) lds_keys[slot] = cand_key(pj, index);
-    }
-  };
+  const GatherArgs ga = {inv, m, p_thr, k_star, cap, div, lds_keys, &sm};
   int done = 0;
   if (ALIGNED) {
     const int nvec = V / 8;
     const uint4* vec = reinterpret_cast<const uint4*>(logits);
-    // Vectors are screened by their largest order key.  For a positive threshold the patterns
-    // themselves, read as signed 16-bit numbers, decide (negative logits are negative numbers).
-    auto sweep = [&](auto positive_tag) {
-      constexpr bool kPositive = decltype(positive_tag)::value;
-      auto best_of = [](const uint4& r) -> int {
-        const uint32_t w[4] = {r.x, r.y, r.z, r.w};
-        short2v best = {-32768, -32768};
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-          const short2v h = __builtin_bit_cast(short2v, w[k]);
-          const short2v key = kPositive ? h : h ^ ((h >> 15) & static_cast<short>(0x7fff));
-          best = __builtin_elementwise_max(best, key);
-        }
-        return max(static_cast<int>(best.x), static_cast<int>(best.y));
-      };
-      for (int j = tid; j < nvec; j += 16 * kBlock) {  // 16 loads in flight; out-of-range ones re-read vec[j]
-        uint4 r[16];
-#pragma unroll
-        for (int k = 0; k < 16; ++k) {
-          const int jk = j + k * kBlock;
-          r[k] = vec[jk < nvec ? jk : j];
-        }
-#pragma unroll
-        for (int k = 0; k < 16; ++k) {
-          const int jk = j + k * kBlock;
-          if (jk < nvec && best_of(r[k]) >= k_star) {
-            const uint32_t w[4] = {r[k].x, r[k].y, r[k].z, r[k].w};
-#pragma unroll
-            for (int h = 0; h < 4; ++h) {
-              take(w[h] & 0xffffu, jk * 8 + 2 * h);
-              take(w[h] >> 16, jk * 8 + 2 * h + 1);
-            }
-          }
-        }
-      }
-    };
     if (k_star > 0) {
-      sweep(std::true_type{});
+      gather_sweep<true, TOPK>(vec, nvec, ga);
     } else {
-      sweep(std::false_type{});
+      gather_sweep<false, TOPK>(vec, nvec, ga);
     }
     done = nvec * 8;
   }
   for (int i = done + tid; i < V; i += kBlock) {
-    take(static_cast<uint32_t>(reinterpret_cast<const uint16_t*>(logits)[i]), i);
+    gather_take<TOPK>(static_cast<uint32_t>(reinterpret_cast<const uint16_t*>(logits)[i]), i, ga);
   }
   __syncthreads();
   const int n_got = static_cast<int>(sm.counter2);
