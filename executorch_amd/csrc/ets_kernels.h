@@ -455,6 +455,7 @@ struct ScanArgs {
   int lut_half;     //   entries per sign half
   uint64_t* lds_list;
   int lds_list_cap;
+  float list_floor;  // kListAppend with FLOOR (top-k rows): entries with exp below this are not listed
 };
 
 constexpr int kLutCountWords = 12288;  // a table entry's counter sits 48 KiB above its e
@@ -558,11 +559,19 @@ constexpr int kGroup = 2;  // 16-byte vectors per lane between two barriers of t
 //                counter
 constexpr int kListNone = 0, kListAppend = 1, kListHist = 2;
 
+// Smallest exp a listing pass records while the running sum is s.
+template <int LIST, bool FLOOR>
+__device__ __forceinline__ float list_cut(const ScanArgs& a, float s) {
+  if (LIST == kListNone) return 0.0f;
+  if (FLOOR) return a.list_floor;  // top-k rows: the cutoff is 0
+  return a.cutoff * __builtin_fmaxf(s, 1.0f) * 0.999f;
+}
+
 // One pass over the row in index order.  The main loop handles kGroup * kBlock full vectors per
 // iteration without bounds checks (loads for the next iteration are issued before the current one
 // is processed); the remainder goes through a bounds-checked loop.  Returns true if the threshold
 // was crossed.
-template <int DT, bool ALIGNED, int MODE, int LIST, bool LUT>
+template <int DT, bool ALIGNED, int MODE, int LIST, bool LUT, bool FLOOR = false>
 __device__ __forceinline__ bool scan_row(const ScanArgs& a, SeqSum& st, BlockScratch& sm) {
   static_assert(!LUT || DT == kDtypeBFloat16, "the expf table is indexed by bf16 bit patterns");
   static_assert(LIST != kListHist || LUT, "the histogram lives in the expf table");
@@ -620,7 +629,7 @@ __device__ __forceinline__ bool scan_row(const ScanArgs& a, SeqSum& st, BlockScr
         }
       }
       const float scale = fast_scale(st.s);
-      const float cut_lo = LIST != kListNone ? a.cutoff * __builtin_fmaxf(st.s, 1.0f) * 0.999f : 0.0f;
+      const float cut_lo = list_cut<LIST, FLOOR>(a, st.s);
       FastAcc acc = {0.0f, 0.0f};
       uint32_t bits[kGroup][VE];
       int first[kGroup];
@@ -675,7 +684,7 @@ __device__ __forceinline__ bool scan_row(const ScanArgs& a, SeqSum& st, BlockScr
   // remainder (and rows whose base or pitch is not 16-byte aligned)
   for (int base = done_elems; base < V; base += kBlock * VE) {
     const int first = base + tid * VE;
-    const float cut_lo = LIST != kListNone ? a.cutoff * __builtin_fmaxf(st.s, 1.0f) * 0.999f : 0.0f;
+    const float cut_lo = list_cut<LIST, FLOOR>(a, st.s);
     uint32_t bits[VE];
 #pragma unroll
     for (int e = 0; e < VE; ++e) {
@@ -1263,6 +1272,41 @@ __device__ __noinline__ bool draw_topp_hist(const char* logits, int V, float inv
   return true;
 }
 
+// Top-k draw of a row whose scan listed every entry with exp >= list_floor (at least topk of them
+// by construction): sorts the listed entries and walks the first topk (sampler.cpp:87-119).
+// Entries that were not listed have a smaller exp than every listed one; they could only tie with
+// the topk-th probability where the division loses resolution, which the check against the
+// floor's own quotient rules out.  Returns false when the caller has to take the general path.
+// The list sits `list_base` keys above the start of the key buffer; the sort keys are written from
+// the start of the buffer, so that the sort and the walks run on the buffer itself like every
+// other caller's.
+constexpr int kTopkListMax = 256;
+__device__ __noinline__ bool draw_topk_listed(uint64_t* lds_keys, int cap, int list_base, int n_listed, float S,
+                                              float list_floor, int topk, float topp, float coin, int V, RowDebug& dbg,
+                                              int32_t& token, BlockScratch& sm) {
+  const int tid = threadIdx.x;
+  if (n_listed < topk || n_listed > cap - list_base || list_base != kBlock) return false;
+  const int N = pow2_ceil(n_listed);
+  if (N > cap) return false;
+  const RowDivisor div = row_divisor(S);
+  // key i replaces list entry i - kBlock: the slot a lane writes is the one it read one step earlier
+  for (int i = tid; i < N; i += kBlock) {
+    uint64_t key = ~0ull;
+    if (i < n_listed) {
+      const uint64_t ent = lds_keys[list_base + i];
+      key = cand_key(div_row(__uint_as_float(static_cast<uint32_t>(ent >> 32)), div), static_cast<int>(static_cast<uint32_t>(ent)));
+    }
+    lds_keys[i] = key;
+  }
+  __syncthreads();
+  sort_keys_lds(lds_keys, N);
+  if (!(cand_prob(lds_keys[topk - 1]) > div_row(list_floor, div))) return false;
+  dbg.n_candidates = V;  // every entry is a candidate of a top-k draw
+  const int pos = draw_from_sorted(lds_keys, n_listed, n_listed, true, topk, topp, coin, dbg, sm);
+  token = static_cast<int32_t>(static_cast<uint32_t>(lds_keys[pos]));
+  return true;
+}
+
 // ---- the stochastic path: one workgroup per row -------------------------------------------------
 // Pass 1 reads the row from HBM: maximum of x = logit * inv_temperature and whether any x is NaN.
 // Pass 2 re-reads it (L2 / Infinity Cache): exact expf, the sequential sum in index order, and
@@ -1327,6 +1371,7 @@ __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
       for (int i = tid; i < V; i += kBlock) visit(load_elem<DT>(logits, i));
     }
   }
+  const float lane_max = m;  // of the entries this lane read
   bool row_nan;
   {
     m = wave_max_ignoring_nan(m);
@@ -1367,9 +1412,26 @@ __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
   if (list_base > p.lds_keys) list_base = p.lds_keys;
   uint64_t* lds_list = lds_keys + list_base;
   const int lds_list_cap = p.lds_keys - list_base;
+  // Top-k rows without a table list the entries that can be among the k largest.  At least k
+  // entries are >= the k-th largest of the lanes' maxima, so everything clearly below the exp of
+  // that value is out.
+  // (fp32 and fp16 rows only: bf16 rows outside the table's range keep the full-row sort)
+  float list_floor = 0.0f;
+  bool topk_listed = false;
+  if (use_topk && DT != kDtypeBFloat16 && !row_nan && topk >= 1 && topk <= kTopkListMax && p.lds_keys >= 2 * kBlock) {
+    lds_keys[tid] = (static_cast<uint64_t>(~order_key(lane_max)) << 32) | static_cast<uint32_t>(tid);
+    __syncthreads();
+    sort_keys_lds(lds_keys, kBlock);
+    const uint32_t kth = ~static_cast<uint32_t>(lds_keys[topk - 1] >> 32);  // never NaN or -0: order_key inverts
+    const float t = __uint_as_float((kth & 0x80000000u) ? (kth & 0x7fffffffu) : ~kth);
+    __syncthreads();
+    list_floor = expf_nonpositive(t - m, sm.exp2tab) * 0.998f;
+    topk_listed = list_floor > 0.0f;
+    if (!topk_listed) list_floor = kInf;  // nothing is listed; the general path sorts the row
+  }
   if (!row_nan) {
     ScanArgs a = {logits, V,        inv,       m,       row_divisor(1.0f), kInf, cutoff, scratch, lut,
-                  lut_base1, lut_top, lut_half, lds_list, lds_list_cap};
+                  lut_base1, lut_top, lut_half, lds_list, lds_list_cap, list_floor};
     SeqSum st = {0.0f, -1, 0u};
     bool scanned = false;
     if constexpr (DT == kDtypeBFloat16 && ALIGNED) {
@@ -1383,7 +1445,9 @@ __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
       }
     }
     if (!scanned) {
-      if (use_topp) {
+      if (use_topk && DT != kDtypeBFloat16 && topk_listed) {
+        scan_row<DT, ALIGNED, kScanSum, kListAppend, false, true>(a, st, sm);
+      } else if (use_topp) {
         scan_row<DT, ALIGNED, kScanSum, kListAppend, false>(a, st, sm);
       } else {
         scan_row<DT, ALIGNED, kScanSum, kListNone, false>(a, st, sm);
@@ -1432,7 +1496,7 @@ __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
     token = use_mult ? V - 1 : -1;
   } else if (use_mult) {
     // ---- sampler.cpp:58-70: first index whose running sum of probabilities exceeds the coin
-    ScanArgs a = {logits, V, inv, m, row_divisor(S), coin, 0.0f, nullptr, lut, lut_base1, lut_top, lut_half, nullptr, 0};
+    ScanArgs a = {logits, V, inv, m, row_divisor(S), coin, 0.0f, nullptr, lut, lut_base1, lut_top, lut_half, nullptr, 0, 0.0f};
     SeqSum walk = {0.0f, -1, 0u};
     bool walked = false;
     if constexpr (DT == kDtypeBFloat16 && ALIGNED) {
@@ -1457,6 +1521,9 @@ __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
         done = draw_topp_hist<ALIGNED, true>(logits, V, inv, m, S, 0.0f, topp, topk, coin, lut, lut_base1, lut_top,
                                              lut_half, lds_keys, p.lds_keys, dbg, token, sm);
       }
+    }
+    if (use_topk && DT != kDtypeBFloat16 && topk_listed) {
+      done = draw_topk_listed(lds_keys, p.lds_keys, list_base, n_listed, S, list_floor, topk, topp, coin, V, dbg, token, sm);
     }
     if (use_topp && !tried) {
       done = draw_topp_listed(scratch, lds_list, lds_list_cap, list_base, n_listed, S, cutoff, topp, coin, lds_keys,

@@ -219,3 +219,51 @@ def test_bf16_rows_with_structure(oracle, dev, vocab):
             compare_rows(oracle, dev, x, W.DTYPE_BFLOAT16, temperature, 0.9, seed, (vocab, label, "topk", topk, temperature),
                          topk=topk)
             seed += 17
+
+
+@pytest.mark.parametrize("dtype_name", ["float", "half"])
+@pytest.mark.parametrize("vocab", [4100, 32000, 128256])
+def test_topk_rows_with_structure(oracle, dev, dtype_name, vocab):
+    """Top-k on fp32 / fp16 rows: the listed selection (k up to 256) and the full-row sort beyond
+    it, on rows that stress the selection threshold -- sorted rows (every lane's maximum sits in
+    one end of the row), classes of equal logits around the k-th place, a k-th place far enough
+    below the maximum for its probability to underflow, -inf entries, flat rows."""
+    dtype = {"float": W.DTYPE_FLOAT, "half": W.DTYPE_HALF}[dtype_name]
+    rng = np.random.default_rng(vocab + 7)
+    rows = 4
+    normal = rng.standard_normal((rows, vocab)).astype(np.float32) * 2.0
+
+    def few_values(k):
+        vals = rng.standard_normal(k).astype(np.float32) * 3.0
+        return vals[rng.integers(0, k, size=(rows, vocab))]
+
+    def cliff():
+        x = np.full((rows, vocab), -150.0, dtype=np.float32) + rng.standard_normal((rows, vocab)).astype(np.float32)
+        for b in range(rows):
+            hot = rng.choice(vocab, size=3 + 9 * b, replace=False)
+            x[b, hot] = 5.0 + rng.standard_normal(hot.size).astype(np.float32)
+        return x
+
+    def with_neg_inf():
+        x = normal.copy()
+        x[:, ::3] = -np.inf
+        x[0, :] = -np.inf
+        x[0, 17:17 + 50] = 1.0
+        return x
+
+    cases = {
+        "normal": normal, "ascending": np.sort(normal, axis=1), "descending": -np.sort(-normal, axis=1),
+        "few16": few_values(16), "few200": few_values(200), "cliff": cliff(), "neg_inf": with_neg_inf(),
+        "flat": np.full((rows, vocab), 0.75, dtype=np.float32),
+    }
+    seed = 9090
+    for label, xf in cases.items():
+        x = W.to_storage(xf, dtype)
+        for topk, temperature in ((1, 1.0), (2, 0.6), (40, 0.6), (64, 1.0), (256, 1.3), (257, 1.0), (1000, 2.0)):
+            if topk > 256 and (vocab > 50000 or label not in ("normal", "few16")):
+                continue  # beyond the listed selection: the full-row sort, checked on the small vocabularies
+            if vocab > 50000 and label in ("flat", "few16", "cliff", "neg_inf") and topk not in (2, 40):
+                continue  # rows that fall back to the full-row sort: slow, twice is enough
+            compare_rows(oracle, dev, x, dtype, temperature, 0.9, seed, (vocab, dtype_name, label, "topk", topk, temperature),
+                         topk=topk)
+            seed += 13
