@@ -223,6 +223,11 @@ gumbel_finish_kernel(const uint64_t* partials, int32_t splits, int32_t advance_r
   }
 }
 
+// Sort keys in LDS are addressed as LDS, never through a generic pointer: a helper that is left
+// out of line would otherwise use flat loads and stores for them unless the compiler happens to
+// see the same buffer at every call site.
+typedef __attribute__((address_space(3))) uint64_t* LdsKeys;
+
 // ---- sorting candidate keys -----------------------------------------------------------------
 // Bitonic merge sub-stages j = j_start, j_start/2, ..., 1 of merge size k on a tile of T keys
 // held in LDS whose first key has global position gbase.
@@ -247,13 +252,13 @@ __device__ void lds_merge_stages(uint64_t* t, int T, int gbase, int k, int j_sta
 // whose partners lie inside one run (distance < W) are done by that wave alone, back to back
 // without workgroup barriers -- LDS serves one wave's accesses in order -- so only the
 // log2(N / W) long-distance sub-stages of each merge pay a barrier.  Ends with a barrier.
-__device__ void sort_keys_lds(uint64_t* lds, int N) {
+__device__ void sort_keys_lds(LdsKeys lds, int N) {
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   int waves = N / 128;  // at least two keys per lane of a participating wave
   waves = waves < 1 ? 1 : (waves > kWaves ? kWaves : waves);
   const int W = N / waves;
-  uint64_t* mine = lds + wave * W;
+  LdsKeys mine = lds + wave * W;
   for (int k = 2; k <= N; k <<= 1) {
     int j = k >> 1;
     for (; j >= W; j >>= 1) {
@@ -952,8 +957,8 @@ __device__ bool draw_topp_listed(uint64_t* list, uint64_t* lds_list, int lds_lis
   for (int i = n_sel + tid; i < N; i += kBlock) lds_keys[i] = ~0ull;
   __syncthreads();
   if (n_sel <= 64) return draw_small_wave(lds_keys, n_sel, n0, topp, coin, dbg, token, sm) != -2;
-  sort_keys_lds(lds_keys, N);
-  const int pos = draw_from_sorted(lds_keys, n_sel, n0, false, 0, topp, coin, dbg, sm);
+  sort_keys_lds((LdsKeys)lds_keys, N);
+  const int pos = draw_from_sorted((LdsKeys)lds_keys, n_sel, n0, false, 0, topp, coin, dbg, sm);
   if (pos == -2) return false;  // the pre-selection did not reach topp after all
   token = static_cast<int32_t>(static_cast<uint32_t>(lds_keys[pos]));
   return true;
@@ -1265,8 +1270,8 @@ __device__ __noinline__ bool draw_topp_hist(const char* logits, int V, float inv
   const int N = pow2_ceil(n_got);
   for (int i = n_got + tid; i < N; i += kBlock) lds_keys[i] = ~0ull;
   __syncthreads();
-  sort_keys_lds(lds_keys, N);
-  const int pos = draw_from_sorted(lds_keys, n_got, static_cast<int>(n0), TOPK, topk, topp, coin, dbg, sm);
+  sort_keys_lds((LdsKeys)lds_keys, N);
+  const int pos = draw_from_sorted((LdsKeys)lds_keys, n_got, static_cast<int>(n0), TOPK, topk, topp, coin, dbg, sm);
   if (pos == -2) return false;  // the pre-selection did not reach topp after all
   token = static_cast<int32_t>(static_cast<uint32_t>(lds_keys[pos]));
   return true;
@@ -1299,10 +1304,10 @@ __device__ __noinline__ bool draw_topk_listed(uint64_t* lds_keys, int cap, int l
     lds_keys[i] = key;
   }
   __syncthreads();
-  sort_keys_lds(lds_keys, N);
+  sort_keys_lds((LdsKeys)lds_keys, N);
   if (!(cand_prob(lds_keys[topk - 1]) > div_row(list_floor, div))) return false;
   dbg.n_candidates = V;  // every entry is a candidate of a top-k draw
-  const int pos = draw_from_sorted(lds_keys, n_listed, n_listed, true, topk, topp, coin, dbg, sm);
+  const int pos = draw_from_sorted((LdsKeys)lds_keys, n_listed, n_listed, true, topk, topp, coin, dbg, sm);
   token = static_cast<int32_t>(static_cast<uint32_t>(lds_keys[pos]));
   return true;
 }
@@ -1415,13 +1420,12 @@ __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
   // Top-k rows without a table list the entries that can be among the k largest.  At least k
   // entries are >= the k-th largest of the lanes' maxima, so everything clearly below the exp of
   // that value is out.
-  // (fp32 and fp16 rows only: bf16 rows outside the table's range keep the full-row sort)
   float list_floor = 0.0f;
   bool topk_listed = false;
-  if (use_topk && DT != kDtypeBFloat16 && !row_nan && topk >= 1 && topk <= kTopkListMax && p.lds_keys >= 2 * kBlock) {
+  if (use_topk && !use_lut && !row_nan && topk >= 1 && topk <= kTopkListMax && p.lds_keys >= 2 * kBlock) {
     lds_keys[tid] = (static_cast<uint64_t>(~order_key(lane_max)) << 32) | static_cast<uint32_t>(tid);
     __syncthreads();
-    sort_keys_lds(lds_keys, kBlock);
+    sort_keys_lds((LdsKeys)lds_keys, kBlock);
     const uint32_t kth = ~static_cast<uint32_t>(lds_keys[topk - 1] >> 32);  // never NaN or -0: order_key inverts
     const float t = __uint_as_float((kth & 0x80000000u) ? (kth & 0x7fffffffu) : ~kth);
     __syncthreads();
@@ -1445,7 +1449,7 @@ __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
       }
     }
     if (!scanned) {
-      if (use_topk && DT != kDtypeBFloat16 && topk_listed) {
+      if (use_topk && topk_listed) {
         scan_row<DT, ALIGNED, kScanSum, kListAppend, false, true>(a, st, sm);
       } else if (use_topp) {
         scan_row<DT, ALIGNED, kScanSum, kListAppend, false>(a, st, sm);
@@ -1522,7 +1526,7 @@ __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
                                              lut_half, lds_keys, p.lds_keys, dbg, token, sm);
       }
     }
-    if (use_topk && DT != kDtypeBFloat16 && topk_listed) {
+    if (use_topk && topk_listed) {
       done = draw_topk_listed(lds_keys, p.lds_keys, list_base, n_listed, S, list_floor, topk, topp, coin, V, dbg, token, sm);
     }
     if (use_topp && !tried) {
