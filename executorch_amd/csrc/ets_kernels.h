@@ -1277,6 +1277,43 @@ __device__ __noinline__ bool draw_topp_hist(const char* logits, int V, float inv
   return true;
 }
 
+// A lower bound of the k-th largest of the workgroup's kBlock values (one per lane, never NaN),
+// exact in the upper 20 bits of the float order: wave 0 holds all values in registers and fixes
+// the bound one bit at a time by counting the values at or above the trial.  `buf` is LDS for
+// kBlock words.  Ends with a barrier.
+__device__ __forceinline__ float kth_largest_lane_value(float v, int k, uint32_t* buf, BlockScratch& sm) {
+  static_assert(kBlock == 1024, "sixteen values per lane of the selecting wave");
+  const int tid = threadIdx.x;
+  buf[tid] = order_key(v);
+  __syncthreads();
+  if (tid < 64) {
+    const uint4* rows = reinterpret_cast<const uint4*>(buf);
+    uint32_t key[16];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint4 r = rows[j * 64 + tid];
+      key[4 * j] = r.x;
+      key[4 * j + 1] = r.y;
+      key[4 * j + 2] = r.z;
+      key[4 * j + 3] = r.w;
+    }
+    uint32_t bound = 0u;
+    for (int bit = 31; bit >= 12; --bit) {
+      const uint32_t trial = bound | (1u << bit);
+      int count = 0;
+#pragma unroll
+      for (int j = 0; j < 16; ++j) count += __popcll(__ballot(key[j] >= trial));
+      if (count >= k) bound = trial;
+    }
+    // back from the order key to the float (order_key maps NaN to 0, which no value here has)
+    if (tid == 0) sm.bc_sum = __uint_as_float((bound & 0x80000000u) ? (bound & 0x7fffffffu) : ~bound);
+  }
+  __syncthreads();
+  const float t = sm.bc_sum;
+  __syncthreads();
+  return t;
+}
+
 // Top-k draw of a row whose scan listed every entry with exp >= list_floor (at least topk of them
 // by construction): sorts the listed entries and walks the first topk (sampler.cpp:87-119).
 // Entries that were not listed have a smaller exp than every listed one; they could only tie with
@@ -1290,11 +1327,12 @@ __device__ __noinline__ bool draw_topk_listed(uint64_t* lds_keys, int cap, int l
                                               float list_floor, int topk, float topp, float coin, int V, RowDebug& dbg,
                                               int32_t& token, BlockScratch& sm) {
   const int tid = threadIdx.x;
-  if (n_listed < topk || n_listed > cap - list_base || list_base != kBlock) return false;
+  if (n_listed < topk || n_listed > cap - list_base) return false;
   const int N = pow2_ceil(n_listed);
-  if (N > cap) return false;
+  if (N > cap || (list_base != kBlock && list_base < N)) return false;
   const RowDivisor div = row_divisor(S);
-  // key i replaces list entry i - kBlock: the slot a lane writes is the one it read one step earlier
+  // with the list kBlock keys up, key i replaces list entry i - kBlock: the slot a lane writes is
+  // the one it read one step earlier; a list further up is clear of the keys
   for (int i = tid; i < N; i += kBlock) {
     uint64_t key = ~0ull;
     if (i < n_listed) {
@@ -1403,6 +1441,17 @@ __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
   // ---- pass 2: softmax normaliser, sequential in index order (sampler.cpp:199-203)
   const float cutoff = use_topp ? (1.0f - topp) / static_cast<float>(V - 1) : 0.0f;  // sampler.cpp:136
   float S = kNaN;
+  // Top-k rows (k up to kTopkListMax) list the entries that can be among the k largest.  At least k
+  // entries are >= the k-th largest of the lanes' maxima, so everything clearly below the exp of
+  // that value is out.
+  float list_floor = 0.0f;
+  bool topk_listed = false;
+  if (use_topk && !row_nan && topk >= 1 && topk <= kTopkListMax && p.lds_keys >= 2 * kBlock) {
+    const float t = kth_largest_lane_value(lane_max, topk, reinterpret_cast<uint32_t*>(lds_keys), sm);
+    list_floor = expf_nonpositive(t - m, sm.exp2tab) * 0.998f;
+    topk_listed = list_floor > 0.0f;
+    if (!topk_listed) list_floor = kInf;  // nothing is listed; the draw sorts the row
+  }
   bool use_lut = false;
   int lut_base1 = 0, lut_top = 0, lut_half = 0;
   float* lut = reinterpret_cast<float*>(lds_keys);  // the key buffer is free until the draw
@@ -1410,29 +1459,13 @@ __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
     use_lut = build_exp_lut(lut, p.lds_keys * 2, inv, m, sm.exp2tab, lut_base1, lut_top, lut_half);
     __syncthreads();
   }
-  // Rows without a table list their top-p candidates in the key buffer, above room for a short
-  // sorted selection; what does not fit goes to the row's scratch in global memory.  (Table rows
-  // count bit patterns in the table instead.)
-  int list_base = 1024;
+  // Candidate lists live in the key buffer: above room for a short sorted selection, or above
+  // the table and its counters; what does not fit goes to the row's scratch in global memory.
+  // (Top-p rows with a table count bit patterns in the table instead.)
+  int list_base = use_lut ? kLutCountWords : kBlock;  // 2 * kLutCountWords words of table = kLutCountWords keys
   if (list_base > p.lds_keys) list_base = p.lds_keys;
   uint64_t* lds_list = lds_keys + list_base;
   const int lds_list_cap = p.lds_keys - list_base;
-  // Top-k rows without a table list the entries that can be among the k largest.  At least k
-  // entries are >= the k-th largest of the lanes' maxima, so everything clearly below the exp of
-  // that value is out.
-  float list_floor = 0.0f;
-  bool topk_listed = false;
-  if (use_topk && !use_lut && !row_nan && topk >= 1 && topk <= kTopkListMax && p.lds_keys >= 2 * kBlock) {
-    lds_keys[tid] = (static_cast<uint64_t>(~order_key(lane_max)) << 32) | static_cast<uint32_t>(tid);
-    __syncthreads();
-    sort_keys_lds((LdsKeys)lds_keys, kBlock);
-    const uint32_t kth = ~static_cast<uint32_t>(lds_keys[topk - 1] >> 32);  // never NaN or -0: order_key inverts
-    const float t = __uint_as_float((kth & 0x80000000u) ? (kth & 0x7fffffffu) : ~kth);
-    __syncthreads();
-    list_floor = expf_nonpositive(t - m, sm.exp2tab) * 0.998f;
-    topk_listed = list_floor > 0.0f;
-    if (!topk_listed) list_floor = kInf;  // nothing is listed; the general path sorts the row
-  }
   if (!row_nan) {
     ScanArgs a = {logits, V,        inv,       m,       row_divisor(1.0f), kInf, cutoff, scratch, lut,
                   lut_base1, lut_top, lut_half, lds_list, lds_list_cap, list_floor};
@@ -1440,7 +1473,9 @@ __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
     bool scanned = false;
     if constexpr (DT == kDtypeBFloat16 && ALIGNED) {
       if (use_lut) {
-        if (use_topp || use_topk) {  // top-k: the cutoff is 0, every entry is counted
+        if (use_topk && topk_listed) {
+          scan_row<DT, ALIGNED, kScanSum, kListAppend, true, true>(a, st, sm);
+        } else if (use_topp || use_topk) {  // top-k beyond the listed sizes: the cutoff is 0, every entry is counted
           scan_row<DT, ALIGNED, kScanSum, kListHist, true>(a, st, sm);
         } else {
           scan_row<DT, ALIGNED, kScanSum, kListNone, true>(a, st, sm);
@@ -1521,7 +1556,7 @@ __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
                                               lut_half, lds_keys, p.lds_keys, dbg, token, sm);
         tried = true;
       }
-      if (use_topk && use_lut) {
+      if (use_topk && use_lut && !topk_listed) {
         done = draw_topp_hist<ALIGNED, true>(logits, V, inv, m, S, 0.0f, topp, topk, coin, lut, lut_base1, lut_top,
                                              lut_half, lds_keys, p.lds_keys, dbg, token, sm);
       }
