@@ -34,7 +34,7 @@ struct ets_sampler {
   int device = 0;
   int lds_keys = 0;            // keys that fit in the dynamic LDS sort buffer (power of two)
   size_t lds_bytes = 0;
-  int64_t scratch_stride = 0;  // keys per row of candidate scratch (power of two >= vocab)
+  int64_t scratch_stride = 0;  // keys per row of candidate scratch (twice the vocabulary, rounded up)
   uint64_t* d_rng = nullptr;       // [max_batch]
   uint64_t* d_scratch = nullptr;   // [max_batch, scratch_stride], allocated on first stochastic use
   uint64_t* d_partials = nullptr;  // [max_batch, kMaxSplits] argmax partial results
@@ -415,14 +415,15 @@ ets_status ets_sampler_create(int32_t vocab_size, float temperature, float topp,
   // the row kernel's static LDS (reduction scratch, selection buffer, histogram) stays under 16 KiB
   int keys = 1;
   while (static_cast<size_t>(keys) * 2 * sizeof(uint64_t) + 16384 <= static_cast<size_t>(lds_limit)) keys *= 2;
-  if (keys < 64) {
+  // the radix sort of large candidate sets keeps a 48 KiB table in the key buffer
+  if (keys < 8192) {
     ets_sampler_destroy(s);
     return fail(nullptr, ETS_INTERNAL, "ets_sampler_create: device reports too little LDS per workgroup");
   }
   s->lds_keys = keys;
   s->lds_bytes = static_cast<size_t>(keys) * sizeof(uint64_t);
-  s->scratch_stride = 2;
-  while (s->scratch_stride < vocab_size) s->scratch_stride *= 2;
+  // two buffers of a row's sort keys (the radix sort of large candidate sets moves between them)
+  s->scratch_stride = 2 * ((static_cast<int64_t>(vocab_size) + 63) / 64 * 64);
 
   e = hipMalloc(reinterpret_cast<void**>(&s->d_rng), sizeof(uint64_t) * max_batch);
   if (e != hipSuccess) return bail(e, "hipMalloc(rng states)");

@@ -229,24 +229,6 @@ gumbel_finish_kernel(const uint64_t* partials, int32_t splits, int32_t advance_r
 typedef __attribute__((address_space(3))) uint64_t* LdsKeys;
 
 // ---- sorting candidate keys -----------------------------------------------------------------
-// Bitonic merge sub-stages j = j_start, j_start/2, ..., 1 of merge size k on a tile of T keys
-// held in LDS whose first key has global position gbase.
-__device__ void lds_merge_stages(uint64_t* t, int T, int gbase, int k, int j_start) {
-  for (int j = j_start; j > 0; j >>= 1) {
-    for (int q = threadIdx.x; q < (T >> 1); q += kBlock) {
-      const int i = ((q & ~(j - 1)) << 1) | (q & (j - 1));
-      const int l = i | j;
-      const bool up = ((gbase + i) & k) == 0;
-      const uint64_t a = t[i], b = t[l];
-      if ((a > b) == up) {
-        t[i] = b;
-        t[l] = a;
-      }
-    }
-    __syncthreads();
-  }
-}
-
 // Ascending sort of N keys (a power of two) that already sit in LDS (and are visible to the
 // workgroup).  Bitonic network; every wave owns a contiguous run of W keys, and the sub-stages
 // whose partners lie inside one run (distance < W) are done by that wave alone, back to back
@@ -292,42 +274,6 @@ __device__ void sort_keys_lds(LdsKeys lds, int N) {
       }
     }
     if (k >= W) __syncthreads();  // the next merge starts with a long-distance sub-stage, or this was the last
-  }
-}
-
-// Ascending sort of keys[0, N), N a power of two, by one workgroup.  `keys` is global memory;
-// `lds` holds T keys (T a power of two).  N <= T leaves the sorted keys in LDS as well.
-__device__ void sort_keys_block(uint64_t* keys, int N, uint64_t* lds, int T) {
-  const int tid = threadIdx.x;
-  if (T > N) T = N;
-  for (int base = 0; base < N; base += T) {
-    for (int i = tid; i < T; i += kBlock) lds[i] = keys[base + i];
-    __syncthreads();
-    for (int k = 2; k <= T; k <<= 1) lds_merge_stages(lds, T, base, k, k >> 1);
-    for (int i = tid; i < T; i += kBlock) keys[base + i] = lds[i];
-    __syncthreads();
-  }
-  for (int k = T << 1; k <= N; k <<= 1) {
-    for (int j = k >> 1; j >= T; j >>= 1) {
-      for (int q = tid; q < (N >> 1); q += kBlock) {
-        const int i = ((q & ~(j - 1)) << 1) | (q & (j - 1));
-        const int l = i | j;
-        const bool up = (i & k) == 0;
-        const uint64_t a = keys[i], b = keys[l];
-        if ((a > b) == up) {
-          keys[i] = b;
-          keys[l] = a;
-        }
-      }
-      __syncthreads();
-    }
-    for (int base = 0; base < N; base += T) {
-      for (int i = tid; i < T; i += kBlock) lds[i] = keys[base + i];
-      __syncthreads();
-      lds_merge_stages(lds, T, base, k, T >> 1);
-      for (int i = tid; i < T; i += kBlock) keys[base + i] = lds[i];
-      __syncthreads();
-    }
   }
 }
 
@@ -712,40 +658,174 @@ __device__ __forceinline__ bool scan_row(const ScanArgs& a, SeqSum& st, BlockScr
   return false;
 }
 
+// Stable radix sort of n entries by their upper 32 bits, least significant byte first, by one
+// workgroup; `a` holds the entries, `b` is a second buffer of n entries (both global memory), `table`
+// is LDS for 3 * kWaves * 256 words.  Every wave owns a contiguous chunk of the input: it counts its
+// chunk's digits into its own row of the table, the rows become write positions (digit-major, then
+// wave), and the wave moves its chunk 64 entries at a time -- lanes with equal digits find each
+// other through a 64-bit word per digit in which each sets its bit, and take consecutive positions
+// in lane order -- so equal digits keep their input
+// order and the scatter needs no synchronisation between waves.  A byte that is the same in every
+// entry costs only its counting pass.  Returns the buffer that holds the sorted entries.
+__device__ uint64_t* radix_sort_block(uint64_t* a, uint64_t* b, int n, LdsU32 table, BlockScratch& sm) {
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int chunk = (((n + kWaves - 1) / kWaves) + 63) & ~63;
+  const int c0 = min(n, wave * chunk), c1 = min(n, c0 + chunk);
+  LdsU32 mine = table + wave * 256;
+  LdsKeys board = (LdsKeys)(table + kWaves * 256) + wave * 256;
+  for (int d = lane; d < 256; d += 64) board[d] = 0ull;  // left clear by every use
+  for (int shift = 32; shift < 64; shift += 8) {
+    // ---- count
+    for (int d = lane; d < 256; d += 64) mine[d] = 0u;
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    for (int base = c0; base < c1; base += 64 * 8) {  // eight loads in flight
+      uint64_t entry[8];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        const int i = base + k * 64 + lane;
+        entry[k] = a[i < c1 ? i : c0];
+      }
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        if (base + k * 64 + lane < c1) {
+          const uint32_t digit = static_cast<uint32_t>(entry[k] >> shift) & 255u;
+          __hip_atomic_fetch_add(&mine[digit], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+        }
+      }
+    }
+    __syncthreads();
+    // ---- positions: exclusive prefix over (digit, wave); lane t holds digit t / 4, waves 4 * (t % 4) ...
+    const int digit0 = tid >> 2, wave0 = (tid & 3) * 4;
+    uint32_t c[4];
+    uint32_t sum = 0u;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      c[k] = table[(wave0 + k) * 256 + digit0];
+      sum += c[k];
+    }
+    // digits are spread over groups of four lanes: a digit's total is the sum over its group
+    uint32_t digit_total = sum + __shfl_xor(sum, 1);
+    digit_total += __shfl_xor(digit_total, 2);
+    const bool one_digit = __ballot(digit_total == static_cast<uint32_t>(n)) != 0ull;
+    const float upto = wave_scan_inclusive_f32(static_cast<float>(sum), lane);  // exact: n is below 2^24
+    if (lane == 63) sm.red_f[wave] = upto;
+    if (lane == 0) sm.red_u[wave] = one_digit ? 1u : 0u;
+    __syncthreads();
+    float before = 0.0f;
+    uint32_t any_one = 0u;
+    for (int w = 0; w < kWaves; ++w) {
+      if (w < wave) before += sm.red_f[w];
+      any_one |= sm.red_u[w];
+    }
+    uint32_t start = static_cast<uint32_t>(before + upto) - sum;
+    if (!any_one) {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        table[(wave0 + k) * 256 + digit0] = start;
+        start += c[k];
+      }
+    }
+    __syncthreads();
+    if (any_one) continue;  // every entry has the same byte here
+    // ---- move
+    for (int base4 = c0; base4 < c1; base4 += 64 * 4) {  // four loads in flight
+      uint64_t entry4[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const int i = base4 + k * 64 + lane;
+        entry4[k] = a[i < c1 ? i : c0];
+      }
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+      const int base = base4 + k * 64;
+      if (base >= c1) break;
+      const int i = base + lane;
+      const bool valid = i < c1;
+      const uint64_t entry = entry4[k];
+      const uint32_t digit = static_cast<uint32_t>(entry >> shift) & 255u;
+      // the lanes with this digit: every lane sets its bit in the digit's word, then reads the word
+      if (valid) __hip_atomic_fetch_or(&board[digit], 1ull << lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+      const uint64_t peers = valid ? board[digit] : 0ull;
+      const uint32_t rank = static_cast<uint32_t>(__popcll(peers & ((1ull << lane) - 1ull)));
+      uint32_t position = 0u;
+      if (valid) {
+        position = mine[digit];
+        b[position + rank] = entry;
+      }
+      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");  // every peer has read the position
+      if (valid && rank == 0u) {
+        mine[digit] = position + static_cast<uint32_t>(__popcll(peers));
+        board[digit] = 0ull;
+      }
+      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+      }
+    }
+    __syncthreads();
+    uint64_t* t = a;
+    a = b;
+    b = t;
+  }
+  return a;
+}
+
 // General path: every candidate (top-p: p >= cutoff; top-k: the whole row, sampler.cpp:87-100)
-// goes to global memory as a sort key and the full list is sorted.  Used by top-k and by top-p
-// rows whose candidates do not fit in LDS.
+// becomes a sort key and the full list is sorted: in LDS when it fits (bitonic network), otherwise
+// by the radix sort above over the whole row in index order, with keys that sort last in place of
+// the entries that are no candidates (a candidate's probability is positive in top-p, and in top-k
+// every entry is one, so no candidate ties with them).  Used by large top-k and by top-p rows
+// whose candidates do not fit in LDS.  `scratch` holds `scratch_cap` entries.
 template <int DT>
 __device__ int32_t draw_general(const char* logits, int V, float inv, float m, float S, bool use_topk,
                                              int topk, float topp, float cutoff, float coin, uint64_t* scratch,
-                                             uint64_t* lds_keys, int cap, RowDebug& dbg, BlockScratch& sm) {
+                                             int64_t scratch_cap, uint64_t* lds_keys, int cap, RowDebug& dbg,
+                                             BlockScratch& sm) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const float cut = use_topk ? 0.0f : cutoff;
   const RowDivisor div = row_divisor(S);
   if (tid == 0) sm.counter = 0u;
   __syncthreads();
+  uint32_t kept = 0u;
   for (int base = 0; base < V; base += kBlock) {
     const int i = base + tid;
-    float pi = 0.0f;
-    bool keep = false;
     if (i < V) {
       const float x = load_elem<DT>(logits, i) * inv;
-      pi = div_row(expf_nonpositive(x - m, sm.exp2tab), div);
-      keep = pi >= cut;
+      const float pi = div_row(expf_nonpositive(x - m, sm.exp2tab), div);
+      const bool keep = pi >= cut;
+      scratch[i] = keep ? cand_key(pi, i) : ~0ull;
+      kept += keep ? 1u : 0u;
     }
-    const uint32_t slot = wave_append_slot(keep, &sm.counter, lane);
-    if (keep) scratch[slot] = cand_key(pi, i);
   }
+  kept = wave_sum_u32(kept);
+  if (lane == 0 && kept != 0u) atomicAdd(&sm.counter, kept);
   __syncthreads();
   const int n0 = static_cast<int>(sm.counter);
   dbg.n_candidates = n0;
   if (n0 == 0) return -1;  // the reference reads probindex[-1] here
   const int N = pow2_ceil(n0);
-  for (int i = n0 + tid; i < N; i += kBlock) scratch[i] = ~0ull;
-  __syncthreads();
-  sort_keys_block(scratch, N, lds_keys, cap);
-  const uint64_t* keys = (N <= cap) ? lds_keys : scratch;
+  const uint64_t* keys;
+  if (N <= cap) {
+    __syncthreads();
+    if (tid == 0) sm.counter = 0u;
+    __syncthreads();
+    for (int base = 0; base < V; base += kBlock) {
+      const int i = base + tid;
+      const uint64_t key = i < V ? scratch[i] : ~0ull;
+      const bool keep = key != ~0ull;
+      const uint32_t slot = wave_append_slot(keep, &sm.counter, lane);
+      if (keep) lds_keys[slot] = key;
+    }
+    for (int i = n0 + tid; i < N; i += kBlock) lds_keys[i] = ~0ull;
+    __syncthreads();
+    sort_keys_lds((LdsKeys)lds_keys, N);
+    keys = lds_keys;
+  } else {
+    // the host sizes the scratch for two buffers of V entries and the key buffer for the sort's table
+    keys = radix_sort_block(scratch, scratch + scratch_cap / 2, V, (LdsU32)lds_keys, sm);
+  }
   const int pos = draw_from_sorted(keys, n0, n0, use_topk, topk, topp, coin, dbg, sm);
   return static_cast<int32_t>(static_cast<uint32_t>(keys[pos]));
 }
@@ -1569,8 +1649,8 @@ __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
                               p.lds_keys, dbg, token, sm);
     }
     if (!done) {
-      token = draw_general<DT>(logits, V, inv, m, S, use_topk, topk, topp, cutoff, coin, scratch, lds_keys,
-                               p.lds_keys, dbg, sm);
+      token = draw_general<DT>(logits, V, inv, m, S, use_topk, topk, topp, cutoff, coin, scratch, p.scratch_stride,
+                               lds_keys, p.lds_keys, dbg, sm);
     }
   }
   if (tid == 0) {
