@@ -22,8 +22,11 @@ def run_case(oracle, dev, w, rows, steps, topk=0, probs=False, topp=None, temper
     topp = w.topp if topp is None else topp
     temperature = w.temperature if temperature is None else temperature
     s = ea.Sampler(w.vocab, temperature, topp, w.coin_seed, max_batch=rows)
+    # a second sampler without debug records: the kernel may then take short cuts that the records rule out
+    plain = ea.Sampler(w.vocab, temperature, topp, w.coin_seed, max_batch=rows)
     if topk:
         s.set_topk(topk)
+        plain.set_topk(topk)
     states = W.coin_seeds(w, rows).copy()
     inv = oracle.inv_temperature(temperature)
     tie_rows = total = 0
@@ -39,6 +42,8 @@ def run_case(oracle, dev, w, rows, steps, topk=0, probs=False, topp=None, temper
         ref, _ = oracle.sample_rows(x, w.dtype, inv, topp, topk, lib_states, mode=oracle.MODE_UPCAST,
                                     tie=oracle.TIE_LIBSTDCXX, threads=8)
         assert np.array_equal(got, want), (w.name, st, np.nonzero(got != want)[0][:8])
+        got_plain = plain.sample_batch(dx).cpu().numpy()
+        assert np.array_equal(got_plain, want), (w.name, st, "no debug records", np.nonzero(got_plain != want)[0][:8])
         dbg = ea.debug_records(ddbg)
         for b in range(rows):
             e = ex[b]
@@ -166,6 +171,11 @@ def compare_rows(oracle, dev, x, dtype, temperature, topp, seed, label, topk=0):
             assert f32_bits(dbg["cumulative"][b]) == f32_bits(e.cumulative), (label, b)
             assert dbg["position"][b] == e.position, (label, b)
     assert np.array_equal(s.get_rng_states(rows), states)
+    # without debug records the kernel may take short cuts that the records rule out
+    plain = ea.Sampler(vocab, temperature, topp, seed, max_batch=rows)
+    plain.set_topk(topk)
+    got_plain = plain.sample_batch(to_device(x, dtype, dev)).cpu().numpy()
+    assert np.array_equal(got_plain, want), (label, "no debug records", np.nonzero(got_plain != want)[0][:8])
 
 
 @pytest.mark.parametrize("vocab", [4096, 4104, 20000, 131072])
