@@ -24,8 +24,8 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by
 # the factors a 256 MiB device copy gives in the same runs (profiles/sample_rows_kernel_cfg2.md has
-# the commands and the raw counters): 9225 KiB * 2.00 fetched + 3772 KiB * 1.00 written.
-MEASURED_TRAFFIC_BYTES = {"cfg2": (9225 * 2.00 + 3772 * 1.00) * 1024}
+# the commands and the raw counters): 9221 KiB * 2.00 fetched + 3780 KiB * 1.00 written.
+MEASURED_TRAFFIC_BYTES = {"cfg2": (9221 * 2.00 + 3780 * 1.00) * 1024}
 
 
 def synth_logits_device(w, count, torch, dev):
@@ -222,6 +222,39 @@ def bench_configs(w, s, ring, out, steps, torch):
             "mixed": "a quarter of the rows each: the workload's top-p, greedy, multinomial T=1, top-k 40 T=0.8"}
 
 
+def bench_draw_modes(w, logits, out, torch):
+    """The other element types and draws on the headline's shape and rows: the same matrix as
+    fp16 / fp32, each with the workload's top-p, the multinomial draw (top-p 1) and top-k 40
+    (microseconds per batch, one launch each)."""
+    import executorch_amd as ea
+
+    res = {}
+    for name, tdt in (("bf16", torch.bfloat16), ("fp16", torch.float16), ("fp32", torch.float32)):
+        x = logits.to(tdt).contiguous()
+        for mode, topp, topk in (("top_p", w.topp, 0), ("multinomial", 1.0, 0), ("top_k_40", w.topp, 40)):
+            s = ea.Sampler(w.vocab, w.temperature, topp, w.coin_seed, max_batch=w.batch)
+            s.set_topk(topk)
+            res[f"{name}_{mode}_us"] = timed_us(lambda: s.sample_batch(x, out=out), 30, torch)
+    return res
+
+
+def bench_flat_rows(torch, dev):
+    """Near-flat rows, where every entry is a top-p candidate and the draw sorts the whole row
+    (cfg3's rows: vocab 151936, fp16, N(0, 0.5), T=1, top-p 0.95), 64 rows per batch."""
+    import executorch_amd as ea
+    from executorch_amd import workloads as W
+
+    w = W.WORKLOADS["cfg3"]
+    rows = 64
+    g = torch.Generator(device=dev)
+    g.manual_seed(7)
+    x = (torch.randn((rows, w.vocab), generator=g, device=dev, dtype=torch.float32) * 0.5).to(torch.float16)
+    s = ea.Sampler(w.vocab, w.temperature, w.topp, w.coin_seed, max_batch=rows)
+    out = torch.empty(rows, dtype=torch.int32, device=dev)
+    us = timed_us(lambda: s.sample_batch(x, out=out), 5, torch)
+    return {"us_per_batch": us, "rows": rows, "rows_per_s": rows / (us * 1e-6)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -317,6 +350,8 @@ def main():
         line["gumbel_max"] = bench_gumbel(w, s, ring, out, torch)
         line["greedy"] = bench_greedy(w, ring, out, torch)
         line["per_row_configs"] = bench_configs(w, s, ring, out, args.steps, torch)
+        line["draw_modes"] = bench_draw_modes(w, ring[0], out, torch)
+        line["flat_rows"] = bench_flat_rows(torch, dev)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(w, got)
     print(json.dumps(line))
