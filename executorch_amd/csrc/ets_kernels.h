@@ -855,8 +855,11 @@ __device__ __forceinline__ void block_sum2(float& x, float& y, BlockScratch& sm,
 // the first wave in registers: rank by counting, ds_permute into place, then the two scalar loops
 // with the probabilities read lane by lane.  Same contract as draw_from_sorted (returns the sorted
 // position or -2) but `token` is returned directly, since the sorted keys never go back to LDS.
-__device__ int draw_small_wave(const uint64_t* lds, int n, int n_total, float topp, float coin, RowDebug& dbg,
-                               int32_t& token, BlockScratch& sm) {
+// With topk > 0 (n >= topk) the walks are top-k's (sampler.cpp:103-119): the mass of the first topk
+// keys, no threshold.  `p_floor`: entries that are not among the keys may have probabilities up to
+// p_floor; the last key walked must have a larger one for the prefix to be the reference's (else -2).
+__device__ int draw_small_wave(LdsKeys lds, int n, int n_total, float topp, float coin, RowDebug& dbg,
+                               int32_t& token, BlockScratch& sm, int topk = 0, float p_floor = -1.0f) {
   if (threadIdx.x < 64) {
     const int lane = threadIdx.x;
     const uint64_t key = lane < n ? lds[lane] : ~0ull;
@@ -872,15 +875,20 @@ __device__ int draw_small_wave(const uint64_t* lds, int n, int n_total, float to
     const float prob = __uint_as_float(0xffffffffu - hi);  // cand_prob
     float s = 0.0f;
     int found = -1;
-    for (int i = 0; i < n; ++i) {
-      s = s + readlane_f32(prob, i);
-      if (s > topp) {
-        found = i;
-        break;
+    if (topk > 0) {
+      for (int i = 0; i < topk; ++i) s = s + readlane_f32(prob, i);
+      found = topk - 1;
+    } else {
+      for (int i = 0; i < n; ++i) {
+        s = s + readlane_f32(prob, i);
+        if (s > topp) {
+          found = i;
+          break;
+        }
       }
     }
     int pos = -2;
-    if (found >= 0 || n == n_total) {
+    if ((found >= 0 || n == n_total) && readlane_f32(prob, found >= 0 ? found : n - 1) > p_floor) {
       const int last_idx = found >= 0 ? found : n - 1;
       const float r = coin * s;  // sampler.cpp:162
       float c = 0.0f;
@@ -1036,7 +1044,7 @@ __device__ bool draw_topp_listed(uint64_t* list, uint64_t* lds_list, int lds_lis
   __syncthreads();
   for (int i = n_sel + tid; i < N; i += kBlock) lds_keys[i] = ~0ull;
   __syncthreads();
-  if (n_sel <= 64) return draw_small_wave(lds_keys, n_sel, n0, topp, coin, dbg, token, sm) != -2;
+  if (n_sel <= 64) return draw_small_wave((LdsKeys)lds_keys, n_sel, n0, topp, coin, dbg, token, sm) != -2;
   sort_keys_lds((LdsKeys)lds_keys, N);
   const int pos = draw_from_sorted((LdsKeys)lds_keys, n_sel, n0, false, 0, topp, coin, dbg, sm);
   if (pos == -2) return false;  // the pre-selection did not reach topp after all
@@ -1345,7 +1353,7 @@ __device__ __noinline__ bool draw_topp_hist(const char* logits, int V, float inv
     if (n_got < topk) return false;
     dbg.n_candidates = V;  // every entry is a candidate of a top-k draw
   } else if (n_got <= 64) {
-    return draw_small_wave(lds_keys, n_got, static_cast<int>(n0), topp, coin, dbg, token, sm) != -2;
+    return draw_small_wave((LdsKeys)lds_keys, n_got, static_cast<int>(n0), topp, coin, dbg, token, sm) != -2;
   }
   const int N = pow2_ceil(n_got);
   for (int i = n_got + tid; i < N; i += kBlock) lds_keys[i] = ~0ull;
@@ -1422,9 +1430,13 @@ __device__ __noinline__ bool draw_topk_listed(uint64_t* lds_keys, int cap, int l
     lds_keys[i] = key;
   }
   __syncthreads();
+  dbg.n_candidates = V;  // every entry is a candidate of a top-k draw
+  if (n_listed <= 64) {
+    return draw_small_wave((LdsKeys)lds_keys, n_listed, n_listed, topp, coin, dbg, token, sm, topk,
+                           div_row(list_floor, div)) != -2;
+  }
   sort_keys_lds((LdsKeys)lds_keys, N);
   if (!(cand_prob(lds_keys[topk - 1]) > div_row(list_floor, div))) return false;
-  dbg.n_candidates = V;  // every entry is a candidate of a top-k draw
   const int pos = draw_from_sorted((LdsKeys)lds_keys, n_listed, n_listed, true, topk, topp, coin, dbg, sm);
   token = static_cast<int32_t>(static_cast<uint32_t>(lds_keys[pos]));
   return true;
