@@ -1366,40 +1366,47 @@ __device__ __noinline__ bool draw_topp_hist(const char* logits, int V, float inv
 }
 
 // A lower bound of the k-th largest of the workgroup's kBlock values (one per lane, never NaN),
-// exact in the upper 20 bits of the float order: wave 0 holds all values in registers and fixes
-// the bound one bit at a time by counting the values at or above the trial.  `buf` is LDS for
-// kBlock words.  Ends with a barrier.
+// exact in the upper 20 bits of the float order.  Every wave holds all values in registers; the
+// bound is fixed four bits at a time: wave w counts the values at or above the bound with w in the
+// next four bits, and the largest w that still leaves k values wins.  `buf` is LDS for kBlock
+// words.  Ends with a barrier.
 __device__ __forceinline__ float kth_largest_lane_value(float v, int k, uint32_t* buf, BlockScratch& sm) {
-  static_assert(kBlock == 1024, "sixteen values per lane of the selecting wave");
+  static_assert(kBlock == 1024 && kWaves == 16, "sixteen values per lane, sixteen trials per step");
   const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
   buf[tid] = order_key(v);
   __syncthreads();
-  if (tid < 64) {
-    const uint4* rows = reinterpret_cast<const uint4*>(buf);
-    uint32_t key[16];
+  const uint4* rows = reinterpret_cast<const uint4*>(buf);
+  uint32_t key[16];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const uint4 r = rows[j * 64 + tid];
-      key[4 * j] = r.x;
-      key[4 * j + 1] = r.y;
-      key[4 * j + 2] = r.z;
-      key[4 * j + 3] = r.w;
-    }
-    uint32_t bound = 0u;
-    for (int bit = 31; bit >= 12; --bit) {
-      const uint32_t trial = bound | (1u << bit);
-      int count = 0;
+  for (int j = 0; j < 4; ++j) {
+    const uint4 r = rows[j * 64 + lane];
+    key[4 * j] = r.x;
+    key[4 * j + 1] = r.y;
+    key[4 * j + 2] = r.z;
+    key[4 * j + 3] = r.w;
+  }
+  uint32_t bound = 0u;
+  uint32_t hand = 0u;
+  for (int shift = 28; shift >= 12; shift -= 4) {
+    const uint32_t trial = bound | (static_cast<uint32_t>(wave) << shift);
+    int count = 0;
 #pragma unroll
-      for (int j = 0; j < 16; ++j) count += __popcll(__ballot(key[j] >= trial));
-      if (count >= k) bound = trial;
+    for (int j = 0; j < 16; ++j) count += __popcll(__ballot(key[j] >= trial));
+    if (lane == 0) sm.aux_total[hand][wave] = static_cast<float>(count);  // at most kBlock: exact
+    __syncthreads();
+    uint32_t best = 0u;  // trial 0 is the bound itself: at least k values reach it
+#pragma unroll
+    for (int w = 1; w < kWaves; ++w) {
+      if (sm.aux_total[hand][w] >= static_cast<float>(k)) best = static_cast<uint32_t>(w);  // counts fall with w
     }
-    // back from the order key to the float (order_key maps NaN to 0, which no value here has)
-    if (tid == 0) sm.bc_sum = __uint_as_float((bound & 0x80000000u) ? (bound & 0x7fffffffu) : ~bound);
+    bound |= best << shift;
+    hand ^= 1u;
   }
   __syncthreads();
-  const float t = sm.bc_sum;
-  __syncthreads();
-  return t;
+  // back from the order key to the float (order_key maps NaN to 0, which no value here has)
+  return __uint_as_float((bound & 0x80000000u) ? (bound & 0x7fffffffu) : ~bound);
 }
 
 // Top-k draw of a row whose scan listed every entry with exp >= list_floor (at least topk of them
