@@ -550,7 +550,7 @@ __device__ __forceinline__ bool scan_row(const ScanArgs& a, SeqSum& st, BlockScr
     const uint32_t address = lut_entry_address(mag15, sgn, lut_addr);
     const float e = *(LdsF32)static_cast<uintptr_t>(address);
     table_count(address, e, cut_lo);
-    return MODE == kScanWalk ? div_row(e, a.div) : e;
+    return e;  // a walk's table already holds the probabilities
   };
   auto append = [&](uint32_t e_bits, int index) {
     const uint32_t slot = atomicAdd(&sm.counter, 1u);
@@ -601,8 +601,7 @@ __device__ __forceinline__ bool scan_row(const ScanArgs& a, SeqSum& st, BlockScr
           for (int e = 0; e < VE; ++e) v[e] = *(LdsF32)static_cast<uintptr_t>(address[e]);
 #pragma unroll
           for (int e = 0; e < VE; ++e) {
-            table_count(address[e], v[e], cut_lo);
-            if (MODE == kScanWalk) v[e] = div_row(v[e], a.div);
+            table_count(address[e], v[e], cut_lo);  // (a walk's table already holds the probabilities)
           }
         } else {
           decode_vec<DT>(raw[u], v);
@@ -1639,6 +1638,10 @@ __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
     bool walked = false;
     if constexpr (DT == kDtypeBFloat16 && ALIGNED) {
       if (use_lut) {
+        // one division per bit pattern instead of one per entry: the table becomes p = fl(e / S)
+        const RowDivisor div = row_divisor(S);
+        for (int idx = tid; idx < 2 * lut_half; idx += kBlock) lut[idx] = div_row(lut[idx], div);
+        __syncthreads();
         scan_row<DT, ALIGNED, kScanWalk, kListNone, true>(a, walk, sm);
         walked = true;
       }
