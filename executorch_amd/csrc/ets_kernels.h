@@ -388,7 +388,8 @@ struct InfPattern<kDtypeBFloat16> {
 // What one pass over the row accumulates.
 //   kScanSum   e_i = expf(x_i - max), sequential sum; optionally lists top-p candidates
 //   kScanWalk  p_i = e_i / S, sequential sum until it exceeds the coin (multinomial draw)
-constexpr int kScanSum = 0, kScanWalk = 1;
+//   kScanWalkCached  the same walk over a row of fp32 e_i that a kScanSum pass kept (keep_e)
+constexpr int kScanSum = 0, kScanWalk = 1, kScanWalkCached = 2;
 
 struct ScanArgs {
   const char* logits;
@@ -407,6 +408,7 @@ struct ScanArgs {
   uint64_t* lds_list;
   int lds_list_cap;
   float list_floor;  // kListAppend with FLOOR (top-k rows): entries with exp below this are not listed
+  float* keep_e;     // kScanSum without a table: where to keep every e_i (global memory, V floats), or null
 };
 
 constexpr int kLutCountWords = 12288;  // a table entry's counter sits 48 KiB above its e
@@ -533,6 +535,7 @@ __device__ __forceinline__ bool scan_row(const ScanArgs& a, SeqSum& st, BlockScr
   const uint64_t* tab = sm.exp2tab;
   int done_elems = 0;
   auto value_of = [&](float l) -> float {
+    if (MODE == kScanWalkCached) return div_row(l, a.div);  // l is e_i
     const float x = l * inv;
     float d = x - m;
     d = __builtin_fmaxf(d, -104.0f);  // expf is 0 below ln(2^-150); the core gives 0 at -104 too
@@ -567,7 +570,7 @@ __device__ __forceinline__ bool scan_row(const ScanArgs& a, SeqSum& st, BlockScr
     constexpr int per_iter = kBlock * kGroup;
     // The last group of a row may be partial.  Its missing vectors are replaced by logits of
     // -inf * sign(inv): x = -inf, whose exp is 0 on every path, so they add nothing.
-    const uint32_t filler1 = inv < 0.0f ? InfPattern<DT>::plus : InfPattern<DT>::minus;
+    const uint32_t filler1 = MODE == kScanWalkCached ? 0u : (inv < 0.0f ? InfPattern<DT>::plus : InfPattern<DT>::minus);
     const uint4 filler = {filler1, filler1, filler1, filler1};
     uint4 raw[kGroup];
 #pragma unroll
@@ -626,6 +629,11 @@ __device__ __forceinline__ bool scan_row(const ScanArgs& a, SeqSum& st, BlockScr
             append(eb, first[u] + e);
           }
         }
+        if (!LUT && MODE == kScanSum && a.keep_e != nullptr && vbase + u * kBlock + tid < nvec) {
+          uint4* kept = reinterpret_cast<uint4*>(a.keep_e + first[u]);
+#pragma unroll
+          for (int q = 0; q < VE / 4; ++q) kept[q] = {bits[u][4 * q], bits[u][4 * q + 1], bits[u][4 * q + 2], bits[u][4 * q + 3]};
+        }
       }
       if (seq_sum_group<kGroup, VE, MODE == kScanSum>(st, bits, acc, scale, first, V, a.threshold, sm)) return true;
     }
@@ -649,6 +657,7 @@ __device__ __forceinline__ bool scan_row(const ScanArgs& a, SeqSum& st, BlockScr
           val = value_of(l);
         }
         if (LIST == kListAppend && val >= cut_lo) append(__float_as_uint(val), i);
+        if (!LUT && MODE == kScanSum && a.keep_e != nullptr) a.keep_e[i] = val;
       }
       bits[e] = __float_as_uint(val);
     }
@@ -1566,7 +1575,8 @@ __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
   const int lds_list_cap = p.lds_keys - list_base;
   if (!row_nan) {
     ScanArgs a = {logits, V,        inv,       m,       row_divisor(1.0f), kInf, cutoff, scratch, lut,
-                  lut_base1, lut_top, lut_half, lds_list, lds_list_cap, list_floor};
+                  lut_base1, lut_top, lut_half, lds_list, lds_list_cap, list_floor,
+                  (use_mult && !use_lut) ? reinterpret_cast<float*>(scratch) : nullptr};
     SeqSum st = {0.0f, -1, 0u};
     bool scanned = false;
     if constexpr (DT == kDtypeBFloat16 && ALIGNED) {
@@ -1633,7 +1643,7 @@ __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
     token = use_mult ? V - 1 : -1;
   } else if (use_mult) {
     // ---- sampler.cpp:58-70: first index whose running sum of probabilities exceeds the coin
-    ScanArgs a = {logits, V, inv, m, row_divisor(S), coin, 0.0f, nullptr, lut, lut_base1, lut_top, lut_half, nullptr, 0, 0.0f};
+    ScanArgs a = {logits, V, inv, m, row_divisor(S), coin, 0.0f, nullptr, lut, lut_base1, lut_top, lut_half, nullptr, 0, 0.0f, nullptr};
     SeqSum walk = {0.0f, -1, 0u};
     bool walked = false;
     if constexpr (DT == kDtypeBFloat16 && ALIGNED) {
@@ -1646,7 +1656,11 @@ __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
         walked = true;
       }
     }
-    if (!walked) scan_row<DT, ALIGNED, kScanWalk, kListNone, false>(a, walk, sm);
+    if (!walked) {
+      // pass 2 kept every e_i in the row's scratch: the walk divides them instead of redoing expf
+      a.logits = reinterpret_cast<const char*>(scratch);
+      scan_row<kDtypeFloat, true, kScanWalkCached, kListNone, false>(a, walk, sm);
+    }
     token = walk.stop_index >= 0 ? walk.stop_index : V - 1;
     dbg.cumulative = walk.s;
     dbg.position = token;
