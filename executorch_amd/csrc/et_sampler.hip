@@ -394,6 +394,8 @@ ets_status ets_sampler_create(int32_t vocab_size, float temperature, float topp,
   if (!out) return fail(nullptr, ETS_INVALID_ARGUMENT, "ets_sampler_create: out is null");
   *out = nullptr;
   if (vocab_size < 1) return fail(nullptr, ETS_INVALID_ARGUMENT, "ets_sampler_create: vocab_size must be >= 1");
+  // counts of a row's entries are carried in floats in places (exact below 2^24)
+  if (vocab_size >= (1 << 24)) return fail(nullptr, ETS_NOT_SUPPORTED, "ets_sampler_create: vocab_size must be below 16777216");
   if (max_batch < 1) return fail(nullptr, ETS_INVALID_ARGUMENT, "ets_sampler_create: max_batch must be >= 1");
   ets_sampler* s = new (std::nothrow) ets_sampler();
   if (!s) return fail(nullptr, ETS_MEMORY_ALLOCATION_FAILED, "ets_sampler_create: out of host memory");

@@ -76,7 +76,8 @@ typedef struct {
  * rng_seed)  -- sampler.cpp:173-181.  No clamping of temperature (a negative value gives a
  * negative inverse, as there).  `max_batch` (>= 1) is the largest batch later passed to
  * ets_sampler_sample_batch(); row b starts with xorshift64* state rng_seed + b, so row 0 is
- * the reference object's own stream.  The handle lives on the current HIP device. */
+ * the reference object's own stream.  The handle lives on the current HIP device.
+ * vocab_size must be below 2^24 (ETS_NOT_SUPPORTED otherwise). */
 ETS_API ets_status ets_sampler_create(int32_t vocab_size, float temperature, float topp, uint64_t rng_seed,
                                       int32_t max_batch, ets_sampler** out);
 

@@ -111,6 +111,8 @@ def test_errors_are_statuses_not_aborts(dev):
     s.set_temperature(0.0)
     assert list(s.sample_batch(u16).cpu().numpy()) == [0, 0]  # greedy over quantised logits is supported
     assert L.ets_sampler_sample_batch(s._h, x.data_ptr(), _capi.DTYPE_FLOAT, 0, 100, x.data_ptr(), None) == _capi.OK
+    h = C.c_void_p()
+    assert L.ets_sampler_create(1 << 24, 1.0, 0.9, 1, 1, C.byref(h)) == _capi.NOT_SUPPORTED  # counts are kept in floats
 
 
 def test_runs_on_a_side_stream(oracle, dev):
