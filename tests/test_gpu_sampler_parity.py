@@ -277,3 +277,46 @@ def test_topk_rows_with_structure(oracle, dev, dtype_name, vocab):
             compare_rows(oracle, dev, x, dtype, temperature, 0.9, seed, (vocab, dtype_name, label, "topk", topk, temperature),
                          topk=topk)
             seed += 13
+
+
+@pytest.mark.parametrize("name", ["cfg3", "cfg4", "cfg5"])
+def test_full_batches(oracle, dev, name):
+    """The workloads' full batch sizes (256, 512 and 1024 rows): more rows than the GPU has
+    compute units, so workgroups queue behind one another.  Rows of the workload's distribution
+    are generated on the device; the whole batch must give the tokens of its two halves sampled
+    separately (a row depends on its own logits and coin stream alone), every token must lie in
+    the vocabulary, and a spread of rows is compared with the oracle bit for bit."""
+    w = W.WORKLOADS[name]
+    rows = w.batch
+    g = torch.Generator(device=dev)
+    g.manual_seed(1000 + rows)
+    tdt = {W.DTYPE_FLOAT: torch.float32, W.DTYPE_HALF: torch.float16, W.DTYPE_BFLOAT16: torch.bfloat16}[w.dtype]
+    sigma = {"cfg3": 0.5, "cfg4": 1.5, "cfg5": 1.0}[name]
+    x = torch.randn((rows, w.vocab), generator=g, device=dev, dtype=torch.float32) * sigma
+    if name == "cfg5":  # odd rows peaked, as in the workload
+        hot = torch.randint(0, w.vocab, (rows // 2,), generator=g, device=dev)
+        x[torch.arange(1, rows, 2, device=dev), hot] += 12.0
+    x = x.to(tdt).contiguous()
+    seed = 4000 + rows
+    a = ea.Sampler(w.vocab, w.temperature, w.topp, seed, max_batch=rows)
+    seeds = a.get_rng_states()
+    whole = a.sample_batch(x).cpu().numpy()
+    assert whole.min() >= 0 and whole.max() < w.vocab
+    halves = np.empty(rows, dtype=np.int32)
+    half = rows // 2
+    for lo, hi in ((0, half), (half, rows)):
+        c = ea.Sampler(w.vocab, w.temperature, w.topp, 0, max_batch=hi - lo)
+        c.set_rng_states(seeds[lo:hi])
+        halves[lo:hi] = c.sample_batch(x[lo:hi]).cpu().numpy()
+    assert np.array_equal(whole, halves)
+    picked = np.linspace(0, rows - 1, 6).astype(np.int64)
+    if name == "cfg5":  # four peaked (odd) rows and two flat ones
+        picked = np.array([1, rows // 3 | 1, 2 * rows // 3 | 1, rows - 1, 0, rows - 2], dtype=np.int64)
+    sub = x[torch.from_numpy(picked).to(dev)]
+    if w.dtype == W.DTYPE_BFLOAT16:
+        host = sub.view(torch.int16).cpu().numpy().view(np.uint16)
+    else:
+        host = sub.cpu().numpy()
+    want, _ = oracle.sample_rows(np.ascontiguousarray(host), w.dtype, oracle.inv_temperature(w.temperature), w.topp, 0,
+                                 seeds[picked].copy(), mode=oracle.MODE_UPCAST, tie=oracle.TIE_STABLE, threads=8)
+    assert np.array_equal(whole[picked], want), (name, picked, whole[picked], want)
