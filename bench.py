@@ -238,6 +238,26 @@ def bench_draw_modes(w, logits, out, torch):
     return res
 
 
+def bench_batch_sweep(w, torch, dev):
+    """The headline's rows at other batch sizes: one workgroup per row, so a batch of 64 occupies a
+    quarter of the 256 CUs and larger batches run several rows per CU one after another."""
+    import executorch_amd as ea
+
+    res = {}
+    g = torch.Generator(device=dev)
+    g.manual_seed(11)
+    for rows in (1, 8, 64, 256, 1024):
+        x = torch.randn((rows, w.vocab), generator=g, device=dev, dtype=torch.float32)
+        ids = torch.randint(0, w.vocab, (rows, 20), generator=g, device=dev)
+        x.scatter_add_(1, ids, torch.full(ids.shape, 8.0, device=dev))
+        x = x.to(torch.bfloat16).contiguous()
+        s = ea.Sampler(w.vocab, w.temperature, w.topp, w.coin_seed, max_batch=rows)
+        out = torch.empty(rows, dtype=torch.int32, device=dev)
+        us = timed_us(lambda: s.sample_batch(x, out=out), 30, torch)
+        res[f"B{rows}"] = {"us_per_batch": us, "rows_per_s": rows / (us * 1e-6)}
+    return res
+
+
 def bench_flat_rows(torch, dev):
     """Near-flat rows, where every entry is a top-p candidate and the draw sorts the whole row
     (cfg3's rows: vocab 151936, fp16, N(0, 0.5), T=1, top-p 0.95), 64 rows per batch."""
@@ -352,6 +372,8 @@ def main():
         line["per_row_configs"] = bench_configs(w, s, ring, out, args.steps, torch)
         line["draw_modes"] = bench_draw_modes(w, ring[0], out, torch)
         line["flat_rows"] = bench_flat_rows(torch, dev)
+        if w.dtype == W.DTYPE_BFLOAT16 and w.kind == "peaked":
+            line["batch_sweep"] = bench_batch_sweep(w, torch, dev)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(w, got)
     print(json.dumps(line))
