@@ -303,22 +303,30 @@ __device__ __forceinline__ uint32_t wave_append_slot(bool keep, uint32_t* counte
   return slot0 + static_cast<uint32_t>(__popcll(mask & ((1ull << lane) - 1ull)));
 }
 
-// Single-lane form of the CDF walk for short lists (the nucleus of a peaked row is a handful of
-// entries; a workgroup-wide scan would spend its time in barriers).
+// The CDF walk for short lists (n <= 192; the nucleus of a peaked row is a handful of entries, and
+// a workgroup-wide scan would spend its time in barriers): the first wave loads the probabilities
+// into registers, three per lane, and adds them one by one from there.
 template <typename Keys>
 __device__ SeqSumResult seq_sum_small(Keys keys, int n, float threshold, BlockScratch& sm) {
-  if (threadIdx.x == 0) {
+  if (threadIdx.x < 64) {
+    const int lane = threadIdx.x;
+    float p[3];
+#pragma unroll
+    for (int k = 0; k < 3; ++k) p[k] = (lane + 64 * k < n) ? cand_prob(keys[lane + 64 * k]) : 0.0f;
     float s = 0.0f;
     int found = -1;
-    for (int i = 0; i < n; ++i) {
-      s = s + cand_prob(keys[i]);
-      if (s > threshold) {
-        found = i;
-        break;
+#pragma unroll
+    for (int k = 0; k < 3; ++k) {
+      const int hi = min(n - 64 * k, 64);
+      for (int i = 0; i < hi && found < 0; ++i) {
+        s = s + readlane_f32(p[k], i);
+        if (s > threshold) found = 64 * k + i;
       }
     }
-    sm.bc_sum = s;
-    sm.bc_found = found;
+    if (lane == 0) {
+      sm.bc_sum = s;
+      sm.bc_found = found;
+    }
   }
   __syncthreads();
   const SeqSumResult r = {sm.bc_sum, sm.bc_found};
