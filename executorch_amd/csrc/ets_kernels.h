@@ -1645,10 +1645,12 @@ __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
   RowDebug dbg = {m, S, coin, 0.0f, 0.0f, 0, 0, 0};
   int32_t token = -1;
   if (row_nan) {
-    // Every probability is NaN.  The multinomial walk never fires and returns the last index;
-    // top-p keeps no candidate and top-k's comparisons are all false, which the reference does
-    // not define: report -1.
-    token = use_mult ? V - 1 : -1;
+    // Every probability is NaN.  The multinomial walk never fires and returns the last index
+    // (sampler.cpp:58-70); top-p keeps no candidate, where the reference reads probindex[-1]:
+    // report -1; top-k's comparisons are all false, so every entry ties with every other: in
+    // index order the first topk are entries 0 .. topk-1, their mass is NaN, the walk never fires
+    // and the fallback is the last of them (sampler.cpp:103-119).
+    token = use_mult ? V - 1 : (use_topk ? topk - 1 : -1);
   } else if (use_mult) {
     // ---- sampler.cpp:58-70: first index whose running sum of probabilities exceeds the coin
     ScanArgs a = {logits, V, inv, m, row_divisor(S), coin, 0.0f, nullptr, lut, lut_base1, lut_top, lut_half, nullptr, 0, 0.0f, nullptr};

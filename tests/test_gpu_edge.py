@@ -36,7 +36,8 @@ def test_masked_rows(oracle, dev):
 
 def test_nan_and_all_masked_rows(oracle, dev):
     """Rows the reference turns into all-NaN probabilities: multinomial returns the last index;
-    top-p keeps no candidate, which the reference leaves undefined and both sides report as -1."""
+    top-p keeps no candidate, which the reference leaves undefined and both sides report as -1;
+    top-k falls back to its last entry in index order."""
     V = 500
     f = np.random.default_rng(2).standard_normal((3, V)).astype(np.float32)
     f[0, 7] = np.nan
@@ -49,6 +50,13 @@ def test_nan_and_all_masked_rows(oracle, dev):
         assert list(got) == [want] * 3
         assert np.array_equal(got, oracle_tokens(oracle, f, W.DTYPE_FLOAT, 1.0, topp, 0, seeds))
         assert not np.array_equal(s.get_rng_states(), seeds)  # the coin is still drawn
+    # top-k: all comparisons are false, every entry ties; in index order the walk falls back to entry topk - 1
+    for topk in (1, 40, V - 1):
+        s = ea.Sampler(V, 1.0, 0.9, 9, max_batch=3)
+        s.set_topk(topk)
+        got = s.sample_batch(torch.from_numpy(f).to(dev)).cpu().numpy()
+        assert list(got) == [topk - 1] * 3
+        assert np.array_equal(got, oracle_tokens(oracle, f, W.DTYPE_FLOAT, 1.0, 0.9, topk, seeds))
 
 
 def test_seed_zero_and_negative_temperature(oracle, dev):
