@@ -56,6 +56,8 @@ def main():
     ap.add_argument("--cases", type=int, default=2000)
     ap.add_argument("--seed", type=int, default=1)
     ap.add_argument("--max-vocab", type=int, default=300000)
+    ap.add_argument("--configs", action="store_true",
+                    help="give every row its own (temperature, top-p, top-k, seed) through sample_batch_configs")
     args = ap.parse_args()
 
     import torch
@@ -86,7 +88,7 @@ def main():
         vocab = min(vocab, args.max_vocab)
         dtype = int(rng.choice(dtypes))
         kind = str(rng.choice(kinds))
-        rows = int(rng.integers(1, 5))
+        rows = int(rng.integers(1, 9 if args.configs else 5))
         temperature = float(rng.choice([0.05, 0.3, 0.6, 0.8, 1.0, 1.5, 7.0, 50.0, -1.0, 0.0]))
         topp = float(rng.choice([0.0, 0.02, 0.5, 0.8, 0.9, 0.95, 0.999, 1.0]))
         topk = int(rng.choice([0, 0, 0, 1, 2, 40, 64, 65, 256, 257, 1000, vocab - 1, vocab, vocab + 5]))
@@ -101,18 +103,39 @@ def main():
         dx = to_device(padded, dtype, dev)[:, :vocab]  # row pitch vocab + pad elements
         states = (np.uint64(seed) + np.arange(rows, dtype=np.uint64)).astype(np.uint64)
         try:
-            s = ea.Sampler(vocab, temperature, topp, seed, max_batch=rows)
-            s.set_topk(topk)
-            ddbg = torch.zeros((rows, 8), dtype=torch.int32, device=dev)
-            got = s.sample_batch(dx, debug_out=ddbg).cpu().numpy()
-            after = s.get_rng_states(rows)
-            plain = ea.Sampler(vocab, temperature, topp, seed, max_batch=rows)
-            plain.set_topk(topk)
-            got_plain = plain.sample_batch(dx).cpu().numpy()
-            # the constructor does not clamp: a negative temperature gives a negative inverse (sampler.cpp:173-181)
-            want, _ = O.sample_rows(np.ascontiguousarray(x), dtype, O.inv_temperature(temperature), topp, topk, states, mode=O.MODE_UPCAST,
-                                    tie=O.TIE_STABLE, threads=4)
-            ok = np.array_equal(got, want) and np.array_equal(got_plain, want) and np.array_equal(after, states)
+            if args.configs:
+                cfgs = []
+                want = np.empty(rows, dtype=np.int32)
+                for b in range(rows):
+                    t_b = float(rng.choice([0.05, 0.6, 1.0, 7.0, 0.0, -1.0]))  # -1: the sampler's own
+                    p_b = float(rng.choice([0.0, 0.5, 0.9, 0.999, 1.0]))
+                    k_b = int(rng.choice([0, 0, 1, 40, 257, vocab - 1, vocab + 1]))
+                    seed_b = int(rng.choice([0, int(rng.integers(1, 2**31))]))  # 0: continue the row's stream
+                    cfgs.append((t_b, p_b, k_b, seed_b))
+                    st_b = np.array([seed_b if seed_b else states[b]], dtype=np.uint64)
+                    t_eff = max(temperature, 0.0) if t_b < 0 else t_b
+                    want[b] = O.sample_rows(np.ascontiguousarray(x[b:b + 1]), dtype, O.inv_temperature(t_eff), p_b, k_b, st_b,
+                                            mode=O.MODE_UPCAST, tie=O.TIE_STABLE)[0][0]
+                    states[b] = st_b[0]
+                label["configs"] = cfgs
+                s = ea.Sampler(vocab, max(temperature, 0.0), topp, seed, max_batch=rows)
+                got = s.sample_batch_configs(dx, cfgs).cpu().numpy()
+                after = s.get_rng_states(rows)
+                got_plain = got
+                ok = np.array_equal(got, want) and np.array_equal(after, states)
+            else:
+                s = ea.Sampler(vocab, temperature, topp, seed, max_batch=rows)
+                s.set_topk(topk)
+                ddbg = torch.zeros((rows, 8), dtype=torch.int32, device=dev)
+                got = s.sample_batch(dx, debug_out=ddbg).cpu().numpy()
+                after = s.get_rng_states(rows)
+                plain = ea.Sampler(vocab, temperature, topp, seed, max_batch=rows)
+                plain.set_topk(topk)
+                got_plain = plain.sample_batch(dx).cpu().numpy()
+                # the constructor does not clamp: a negative temperature gives a negative inverse (sampler.cpp:173-181)
+                want, _ = O.sample_rows(np.ascontiguousarray(x), dtype, O.inv_temperature(temperature), topp, topk, states,
+                                        mode=O.MODE_UPCAST, tie=O.TIE_STABLE, threads=4)
+                ok = np.array_equal(got, want) and np.array_equal(got_plain, want) and np.array_equal(after, states)
         except Exception as e:  # an error status is a failure here: every case is a legal call
             ok = False
             label["error"] = repr(e)[:300]
