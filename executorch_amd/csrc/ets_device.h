@@ -276,6 +276,12 @@ __device__ __forceinline__ float readlane_f32(float v, int l) {
 }
 __device__ __forceinline__ uint32_t readlane_u32(uint32_t v, int l) { return __builtin_amdgcn_readlane(v, l); }
 
+// A value that is the same in every lane, moved to a scalar register: what is computed from it
+// (exponent, mantissa, branches) then runs on the scalar unit.
+__device__ __forceinline__ float uniform_f32(float v) {
+  return __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(v)));
+}
+
 // Sum over the 64 lanes, in every lane.
 __device__ __forceinline__ float wave_sum_f32(float v) { return readlane_f32(wave_scan_inclusive_f32(v, 0), 63); }
 
@@ -309,11 +315,41 @@ __device__ __forceinline__ ParityInc fold_run(const uint32_t (&bits)[R], float s
 // the scan restarts behind it with the new ulp.  Tiny running sums use the two-hypothesis parity
 // summaries instead (integer arithmetic, any magnitude).
 template <int R>
-__device__ void wave_resolve(float& s, int& found, const uint32_t (&bits)[R], int first, int n, float threshold) {
+__device__ void wave_resolve(float& s, int& found, const uint32_t (&bits)[R], int first, int n, float threshold,
+                             int consumed = 0) {  // lanes below `consumed` have been consumed
   const int lane = threadIdx.x & 63;
-  int consumed = 0;  // lanes below this have been consumed
   found = -1;
-  while (true) {
+  s = uniform_f32(s);
+  if (s == 0.0f && consumed == 0) {
+    // The start of a row: while the running sum is of the order of its addends it leaves a binade
+    // or meets a half-ulp tie every few elements (about ln(k) times in the first k), and every
+    // such event costs the loop below a round.  The first lanes add their elements natively, one
+    // lane after the other.
+    constexpr int kNativeLanes = 8;
+#pragma unroll 1
+    for (int l = 0; l < kNativeLanes; ++l) {
+      float sl = s;
+      int fl = -1;
+      if (lane == l) {
+#pragma unroll
+        for (int e = 0; e < R; ++e) {
+          const int i = first + e;
+          if (i < n && fl < 0) {
+            sl = sl + __uint_as_float(bits[e]);
+            if (sl > threshold) fl = i;
+          }
+        }
+      }
+      s = readlane_f32(sl, l);
+      fl = static_cast<int>(readlane_u32(static_cast<uint32_t>(fl), l));
+      if (fl >= 0) {
+        found = fl;
+        return;
+      }
+    }
+    consumed = kNativeLanes;
+  }
+  while (consumed < 64) {
     const float scale = fast_scale(s);
     const SumState ss = sum_state(s);
     uint64_t ballot;
@@ -378,6 +414,46 @@ __device__ void wave_resolve(float& s, int& found, const uint32_t (&bits)[R], in
   }
 }
 
+// One wavefront consumes its 64 runs of a plain sum (no threshold) from prefix sums prepared in
+// advance: incl_a / incl_b are the inclusive scans of the lanes' increments rne(a / ulp) for the
+// binades with biased exponents kb_a (the one s is expected to be in) and kb_b > kb_a (the one the
+// slot is expected to end in); the caller has checked that no element ties under either ulp and
+// that the last entry of incl_b is below 2^24 (so every entry of it is exact).  If s is in binade
+// kb_a, the first lane whose prefix under A reaches the end of the binade adds its elements
+// natively; if that lands in binade kb_b and the increments of the lanes behind it stay inside, s
+// is the sum after the slot and 64 is returned.  Otherwise s is the exact sum in front of the
+// returned lane (0 .. 63), and the caller continues there with wave_resolve().
+template <int R>
+__device__ __forceinline__ int resolve_prepared(float& s, const uint32_t (&bits)[R], float incl_a, float incl_b,
+                                                uint32_t kb_a, uint32_t kb_b) {
+  const int lane = threadIdx.x & 63;
+  s = uniform_f32(s);
+  const SumState ss = sum_state(s);
+  if (static_cast<uint32_t>(ss.kb) != kb_a) return 0;
+  const float room = static_cast<float>((1u << 24) - ss.S);
+  const uint64_t ballot = __ballot(!(incl_a < room));
+  if (!ballot) {
+    s = sum_value(ss.S + static_cast<uint32_t>(readlane_f32(incl_a, 63)), ss.kb);
+    return 64;
+  }
+  const int j = __ffsll(static_cast<long long>(ballot)) - 1;
+  const float excl_a = lane_before_f32(incl_a);  // exact in lane j: every prefix in front of it is below `room`
+  float sj = 0.0f;
+  if (lane == j) {
+    sj = sum_value(ss.S + static_cast<uint32_t>(excl_a), ss.kb);
+#pragma unroll
+    for (int e = 0; e < R; ++e) sj = sj + __uint_as_float(bits[e]);
+  }
+  s = readlane_f32(sj, j);
+  const SumState s2 = sum_state(s);
+  if (static_cast<uint32_t>(s2.kb) != kb_b) return j + 1;
+  const float rest = readlane_f32(incl_b, 63) - readlane_f32(incl_b, j);
+  const uint32_t S_end = s2.S + static_cast<uint32_t>(rest);
+  if (S_end >= (1u << 24)) return j + 1;
+  s = sum_value(S_end, s2.kb);
+  return 64;
+}
+
 // First attempt at a group of U * 16 slots: fold every slot ONCE, with the ulp it is predicted to
 // see, instead of once per binade the running sum passes through.
 //   1. plain float sums per slot give approximate running sums at the slot boundaries;
@@ -427,10 +503,40 @@ __device__ int seq_sum_predicted(SeqSum& st, const uint32_t (&bits)[U][R], const
   const uint32_t serial_mask = static_cast<uint32_t>(__ballot(serial && lane < kSlots));
   const uint32_t buf = st.parity_buf;
   st.parity_buf ^= 1u;
+  // A serial slot of a plain sum is prepared by its wave while the others fold theirs: prefix sums
+  // of the lanes' increments with the ulp of the binade it is predicted to be entered in (A) and of
+  // the one it is predicted to be left in (B).  With them, and no tie under either ulp, the slot
+  // costs step 3 one comparison, the crossing lane's native adds and one subtraction instead of
+  // two folds (see resolve_prepared).
+  float prep_a[U], prep_b[U];
+  uint32_t prep_kb_a[U], prep_kb_b[U];
+  bool prepared[U];
 #pragma unroll
   for (int u = 0; u < U; ++u) {
     const int slot_index = u * kWaves + wave;
     ParityInc slot = {0u, 0u};
+    prepared[u] = false;
+    prep_a[u] = prep_b[u] = 0.0f;
+    prep_kb_a[u] = prep_kb_b[u] = 0u;
+    if (PLAIN && ((serial_mask >> slot_index) & 1u)) {
+      const uint32_t kba = readlane_u32(kb_in, slot_index);
+      const uint32_t kbo = readlane_u32(kb_out, slot_index);
+      const uint32_t kbb = kbo > kba ? kbo : kba + 1u;
+      if (kba >= 70u && kbb <= 250u) {
+        const float scale_a = __uint_as_float((277u - kba) << 23), scale_b = __uint_as_float((277u - kbb) << 23);
+        FastAcc fa = {0.0f, 0.0f}, fb = {0.0f, 0.0f};
+#pragma unroll
+        for (int e = 0; e < R; ++e) {
+          fast_fold(fa, __uint_as_float(bits[u][e]), scale_a);
+          fast_fold(fb, __uint_as_float(bits[u][e]), scale_b);
+        }
+        prep_a[u] = wave_scan_inclusive_f32(fa.inc, lane);
+        prep_b[u] = wave_scan_inclusive_f32(fb.inc, lane);
+        prep_kb_a[u] = kba;
+        prep_kb_b[u] = kbb;
+        prepared[u] = __ballot(fa.tie == 0.5f || fb.tie == 0.5f) == 0ull && readlane_f32(prep_b[u], 63) < 16777216.0f;
+      }
+    }
     if (!((serial_mask >> slot_index) & 1u)) {
       const uint32_t kb = readlane_u32(kb_in, slot_index);
       const float scale = __uint_as_float((277u - kb) << 23);  // 2^(150 - kb)
@@ -454,7 +560,19 @@ __device__ int seq_sum_predicted(SeqSum& st, const uint32_t (&bits)[U][R], const
   // ---- 3
   ParityInc mine = {0u, 0u};
   if (lane < kSlots) mine = sm.wave_total[buf][lane];
-  float s = st.s;
+  // Without a tie in any stable slot (the usual case) a run's total is a difference of two plain
+  // prefix sums (at most 32 summaries of at most 2^26 each: no overflow); serial slots hold 0.
+  const bool no_ties = __ballot(mine.even != mine.odd) == 0ull;
+  uint32_t plain_upto = mine.even;
+  if (no_ties) {
+    plain_upto += __builtin_amdgcn_update_dpp(0u, plain_upto, 0x111, 0xf, 0xf, false);
+    plain_upto += __builtin_amdgcn_update_dpp(0u, plain_upto, 0x112, 0xf, 0xf, false);
+    plain_upto += __builtin_amdgcn_update_dpp(0u, plain_upto, 0x114, 0xf, 0xf, false);
+    plain_upto += __builtin_amdgcn_update_dpp(0u, plain_upto, 0x118, 0xf, 0xf, false);
+    plain_upto += __builtin_amdgcn_update_dpp(0u, plain_upto, 0x142, 0xa, 0xf, false);
+    plain_upto += __builtin_amdgcn_update_dpp(0u, plain_upto, 0x143, 0xc, 0xf, false);
+  }
+  float s = uniform_f32(st.s);
   int pos = 0;
   uint32_t hand = 0u;
   while (pos < kSlots) {
@@ -463,10 +581,15 @@ __device__ int seq_sum_predicted(SeqSum& st, const uint32_t (&bits)[U][R], const
     if (next_serial > pos) {
       const SumState ss = sum_state(s);
       if (static_cast<uint32_t>(ss.kb) != readlane_u32(kb_in, pos)) break;  // not the predicted binade
-      ParityInc in_run = {0u, 0u};
-      if (lane >= pos && lane < next_serial) in_run = mine;
-      const ParityInc upto = wave_scan_inclusive(in_run, lane);
-      const uint32_t total = (ss.S & 1u) ? readlane_u32(upto.odd, 63) : readlane_u32(upto.even, 63);
+      uint32_t total;
+      if (no_ties) {
+        total = readlane_u32(plain_upto, next_serial - 1) - (pos ? readlane_u32(plain_upto, pos - 1) : 0u);
+      } else {
+        ParityInc in_run = {0u, 0u};
+        if (lane >= pos && lane < next_serial) in_run = mine;
+        const ParityInc upto = wave_scan_inclusive(in_run, lane);
+        total = (ss.S & 1u) ? readlane_u32(upto.odd, 63) : readlane_u32(upto.even, 63);
+      }
       if (ss.S + total >= (1u << 24)) break;  // the run would leave the binade
       const float s_run = sum_value(ss.S + total, ss.kb);
       if (!PLAIN && s_run > threshold) break;  // the crossing lies inside the run after all
@@ -480,7 +603,11 @@ __device__ int seq_sum_predicted(SeqSum& st, const uint32_t (&bits)[U][R], const
       int found = -1;
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        if (u == ustar) wave_resolve<R>(sw, found, bits[u], first[u], n, threshold);
+        if (u == ustar) {
+          int from = 0;
+          if (PLAIN && prepared[u]) from = resolve_prepared<R>(sw, bits[u], prep_a[u], prep_b[u], prep_kb_a[u], prep_kb_b[u]);
+          if (from < 64) wave_resolve<R>(sw, found, bits[u], first[u], n, threshold, from);
+        }
       }
       if (lane == 0) {
         sm.chain_s[hand] = sw;
@@ -488,7 +615,7 @@ __device__ int seq_sum_predicted(SeqSum& st, const uint32_t (&bits)[U][R], const
       }
     }
     __syncthreads();
-    s = sm.chain_s[hand];
+    s = uniform_f32(sm.chain_s[hand]);
     const int found = PLAIN ? -1 : sm.chain_found[hand];
     hand ^= 1u;
     if (found >= 0) {

@@ -1505,7 +1505,65 @@ __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
       m = __builtin_fmaxf(m, x);  // ignores NaN, like `if (x > max)`
       any_nan = any_nan || (x != x);
     };
-    if (ALIGNED) {
+    bool vectors_done = false;
+    if constexpr (ALIGNED && (DT == kDtypeBFloat16 || DT == kDtypeHalf)) {
+      // 16-bit rows with a positive finite 1/temperature: fl(l * inv) does not decrease as l grows,
+      // so the maximum of x is the x of the largest logit, and that one is found on the raw bit
+      // patterns, two per instruction.  As signed 16-bit integers the non-negative patterns order
+      // like their values and every negative one is below them; among negative patterns the
+      // smallest integer is the value nearest to zero.  NaN patterns lie above +inf's in signed
+      // order (positive NaN) or above -inf's in unsigned order (negative NaN).
+      if (inv > 0.0f && inv < kInf) {
+        typedef short Short2 __attribute__((ext_vector_type(2)));
+        typedef unsigned short UShort2 __attribute__((ext_vector_type(2)));
+        union Word {
+          uint32_t u;
+          Short2 s;
+          UShort2 us;
+        };
+        Word hi_s, lo_s, hi_u;
+        hi_s.u = 0x80008000u;
+        lo_s.u = 0x7fff7fffu;
+        hi_u.u = 0u;
+        const int nvec = V / VE;
+        const uint4* vec = reinterpret_cast<const uint4*>(logits);
+        for (int j = tid; j < nvec; j += 8 * kBlock) {
+          uint4 r[8];
+#pragma unroll
+          for (int k = 0; k < 8; ++k) {
+            const int jk = j + k * kBlock;
+            r[k] = vec[jk < nvec ? jk : j];
+          }
+#pragma unroll
+          for (int k = 0; k < 8; ++k) {
+            const uint32_t w[4] = {r[k].x, r[k].y, r[k].z, r[k].w};
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              Word x;
+              x.u = w[q];
+              hi_s.s = __builtin_elementwise_max(hi_s.s, x.s);
+              lo_s.s = __builtin_elementwise_min(lo_s.s, x.s);
+              hi_u.us = __builtin_elementwise_max(hi_u.us, x.us);
+            }
+          }
+        }
+        const int top = max(static_cast<int>(hi_s.s.x), static_cast<int>(hi_s.s.y));
+        const int low = min(static_cast<int>(lo_s.s.x), static_cast<int>(lo_s.s.y));
+        const uint32_t utop = max(static_cast<uint32_t>(hi_u.us.x), static_cast<uint32_t>(hi_u.us.y));
+        constexpr uint32_t kInf16 = DT == kDtypeBFloat16 ? 0x7f80u : 0x7c00u;
+        const bool nan_seen = top > static_cast<int>(kInf16) || utop > (0x8000u | kInf16);
+        if (!nan_seen && tid < nvec) {  // (a lane with a NaN redoes its entries below, value by value)
+          const uint32_t pattern = static_cast<uint32_t>(top >= 0 ? top : low) & 0xffffu;
+          const float l = DT == kDtypeBFloat16 ? __uint_as_float(pattern << 16) : half_bits_to_float(pattern);
+          m = l * inv;
+        }
+        vectors_done = !nan_seen;
+      }
+    }
+    if (ALIGNED && vectors_done) {
+      const int nvec = V / VE;
+      for (int i = nvec * VE + tid; i < V; i += kBlock) visit(load_elem<DT>(logits, i));
+    } else if (ALIGNED) {
       const int nvec = V / VE;
       const uint4* vec = reinterpret_cast<const uint4*>(logits);
       // eight 16-byte loads in flight per lane; out-of-range ones re-read the lane's first vector
