@@ -279,6 +279,40 @@ def test_topk_rows_with_structure(oracle, dev, dtype_name, vocab):
             seed += 13
 
 
+@pytest.mark.parametrize("dtype_name", ["bfloat16", "float"])
+def test_running_sum_jumps_at_chosen_places(oracle, dev, dtype_name):
+    """Rows whose running sum leaves its binade at chosen places of the kernel's layout (a wave
+    holds 512 consecutive entries, eight per lane; 16 384 entries pass between two barriers): large
+    entries in the first and the last lane of a wave's run, on both sides of a run's and of a
+    group's boundary, several in one run (a second jump behind the first), in consecutive runs,
+    among the row's first 64 entries and as its very first entry; one and several binades per
+    jump.  The normaliser (bit for bit), the candidates and the token must be the oracle's, for
+    the nucleus draw and for the multinomial walk."""
+    dtype = {"bfloat16": W.DTYPE_BFLOAT16, "float": W.DTYPE_FLOAT}[dtype_name]
+    vocab = 70000
+    rng = np.random.default_rng(vocab + dtype)
+    places = [
+        [0], [1, 7, 8, 63, 64], [511], [512], [510, 511, 512, 513], [504, 1016, 1528],  # lanes 63 of three runs
+        [8192 - 1, 8192], [16384 - 1, 16384, 16385], [3 * 512 + 8 * 17 + 3, 3 * 512 + 8 * 40, 3 * 512 + 8 * 41 + 7],
+        [20000, 20001, 20002, 20003], [5 * 512, 6 * 512, 7 * 512, 8 * 512], [vocab - 1], [vocab - 513, vocab - 2],
+        list(range(30000, 30000 + 512, 37)),
+    ]
+    rows = len(places) * 2
+    base = (rng.standard_normal((rows, vocab)) * 0.3 - 9.0).astype(np.float32)
+    for b in range(rows):
+        at = places[b % len(places)]
+        # sizes: the first half of the rows roughly doubles the sum at every place, the second half
+        # multiplies it by up to a few thousand
+        grow = 0.7 if b < len(places) else 2.5
+        for k, i in enumerate(at):
+            base[b, i] = -3.0 + grow * k + rng.standard_normal() * 0.05
+    x = W.to_storage(base, dtype)
+    seed = 97
+    for temperature, topp in ((1.0, 0.9), (0.6, 0.9), (1.0, 1.0), (1.7, 0.5)):
+        compare_rows(oracle, dev, x, dtype, temperature, topp, seed, (dtype_name, temperature, topp))
+        seed += 31
+
+
 @pytest.mark.parametrize("name", ["cfg3", "cfg4", "cfg5"])
 def test_full_batches(oracle, dev, name):
     """The workloads' full batch sizes (256, 512 and 1024 rows): more rows than the GPU has
