@@ -1144,16 +1144,27 @@ __device__ __forceinline__ void gather_sweep(const uint4* vec, int nvec, const G
       const int jk = j + k * kBlock;
       r[k] = vec[jk < nvec ? jk : j];
     }
+    // screen first, take afterwards: the screening code stays compact (the rare take, with its
+    // expf, exists once and reads its vector again)
+    uint32_t hits = 0u;
 #pragma unroll
     for (int k = 0; k < 16; ++k) {
       const int jk = j + k * kBlock;
-      if (jk < nvec && best_order_key<POSITIVE>(r[k]) >= a.k_star) {
-        const uint32_t w[4] = {r[k].x, r[k].y, r[k].z, r[k].w};
-#pragma unroll
-        for (int h = 0; h < 4; ++h) {
-          gather_take<EXACT>(w[h] & 0xffffu, jk * 8 + 2 * h, a);
-          gather_take<EXACT>(w[h] >> 16, jk * 8 + 2 * h + 1, a);
-        }
+      if (jk < nvec && best_order_key<POSITIVE>(r[k]) >= a.k_star) hits |= 1u << k;
+    }
+    while (hits) {
+      const int k = __ffs(static_cast<int>(hits)) - 1;
+      hits &= hits - 1u;
+      const int jk = j + k * kBlock;
+      const uint4 v = vec[jk];
+      const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll 1
+      for (int h = 0; h < 8; ++h) {
+        uint32_t word = w[0];
+        word = (h >> 1) == 1 ? w[1] : word;
+        word = (h >> 1) == 2 ? w[2] : word;
+        word = (h >> 1) == 3 ? w[3] : word;
+        gather_take<EXACT>((word >> ((h & 1) * 16)) & 0xffffu, jk * 8 + h, a);
       }
     }
   }
