@@ -163,19 +163,45 @@ __device__ __forceinline__ float expf_nonpositive(float d, const uint64_t* tab) 
 }
 
 // ---- workgroup-wide primitives ------------------------------------------------------------------
+// Reductions over the 64 lanes, result in every lane.  Six DPP steps (a VALU operand taken from
+// another lane: shifts inside each row of 16, then two row broadcasts) leave the total in lane 63;
+// a butterfly of shuffles would cost six round trips through the LDS crossbar.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ uint32_t dpp_u32_or(uint32_t fallback, uint32_t v) {
+  // lanes without a source under CTRL (or masked off) read `fallback`
+  return __builtin_amdgcn_update_dpp(fallback, v, CTRL, ROW_MASK, 0xf, false);
+}
 __device__ __forceinline__ uint32_t wave_sum_u32(uint32_t v) {
-#pragma unroll
-  for (int d = 32; d > 0; d >>= 1) v += __shfl_xor(v, d);
-  return v;
+  v += dpp_u32_or<0x111, 0xf>(0u, v);
+  v += dpp_u32_or<0x112, 0xf>(0u, v);
+  v += dpp_u32_or<0x114, 0xf>(0u, v);
+  v += dpp_u32_or<0x118, 0xf>(0u, v);
+  v += dpp_u32_or<0x142, 0xa>(0u, v);
+  v += dpp_u32_or<0x143, 0xc>(0u, v);
+  return __builtin_amdgcn_readlane(v, 63);
+}
+__device__ __forceinline__ int wave_max_i32(int v) {
+#define ETS_MAX_STEP(CTRL, MASK)                                                                      \
+  {                                                                                                   \
+    const int o = static_cast<int>(dpp_u32_or<CTRL, MASK>(static_cast<uint32_t>(v), static_cast<uint32_t>(v))); \
+    v = o > v ? o : v;                                                                                \
+  }
+  ETS_MAX_STEP(0x111, 0xf) ETS_MAX_STEP(0x112, 0xf) ETS_MAX_STEP(0x114, 0xf) ETS_MAX_STEP(0x118, 0xf)
+  ETS_MAX_STEP(0x142, 0xa) ETS_MAX_STEP(0x143, 0xc)
+#undef ETS_MAX_STEP
+  return static_cast<int>(__builtin_amdgcn_readlane(static_cast<uint32_t>(v), 63));
 }
 
 __device__ __forceinline__ float wave_max_ignoring_nan(float v) {
-#pragma unroll
-  for (int d = 32; d > 0; d >>= 1) {
-    const float o = __shfl_xor(v, d);
-    v = (o > v) ? o : v;
+#define ETS_MAX_STEP(CTRL, MASK)                                                                      \
+  {                                                                                                   \
+    const float o = __uint_as_float(dpp_u32_or<CTRL, MASK>(__float_as_uint(v), __float_as_uint(v)));    \
+    v = (o > v) ? o : v;                                                                              \
   }
-  return v;
+  ETS_MAX_STEP(0x111, 0xf) ETS_MAX_STEP(0x112, 0xf) ETS_MAX_STEP(0x114, 0xf) ETS_MAX_STEP(0x118, 0xf)
+  ETS_MAX_STEP(0x142, 0xa) ETS_MAX_STEP(0x143, 0xc)
+#undef ETS_MAX_STEP
+  return __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(v), 63));
 }
 
 // LDS scratch shared by the workgroup-wide primitives.

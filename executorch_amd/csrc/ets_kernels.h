@@ -1245,13 +1245,8 @@ __device__ __noinline__ bool draw_topp_hist(const char* logits, int V, float inv
     }
   }
   const float upto = wave_scan_inclusive_f32(mass, lane);
-  uint32_t cnt_w = cnt;
-  int last_w = last_cand;
-#pragma unroll
-  for (int d = 32; d > 0; d >>= 1) {
-    cnt_w += __shfl_xor(cnt_w, d);
-    last_w = max(last_w, __shfl_xor(last_w, d));
-  }
+  const uint32_t cnt_w = wave_sum_u32(cnt);
+  const int last_w = wave_max_i32(last_cand);
   if (lane == 63) {
     sm.group_total[0][wave] = upto;
     sm.red_u[wave] = cnt_w;
@@ -1330,8 +1325,7 @@ __device__ __noinline__ bool draw_topp_hist(const char* logits, int V, float inv
       if (in) n_take += cq[k];
     }
   }
-#pragma unroll
-  for (int d = 32; d > 0; d >>= 1) n_take += __shfl_xor(n_take, d);
+  n_take = wave_sum_u32(n_take);
   const bool wave_straggler = __ballot(straggler) != 0ull;
   if (lane == 0) {
     sm.red_u[wave] = n_take;
