@@ -209,7 +209,8 @@ struct BlockScratch {
   uint64_t exp2tab[32];
   ParityInc wave_total[2][64];      // per (chunk, wave) slot; double-buffered, like group_total
   int first_flag[kWaves];
-  float group_total[2][kWaves];    // same, for seq_sum_group
+  float group_total[2][kWaves];    // same, for block_sum2
+  float slot_total[2][2 * kWaves];  // same, for seq_sum_group: one entry per (chunk, wave) slot
   float slot_sum[64];               // plain float sums per slot (seq_sum_predicted)
   float chain_s[2];                 // running sum handed from one serial slot to the next
   int chain_found[2];               //   and where the threshold was crossed, if it was
@@ -771,32 +772,119 @@ __device__ __forceinline__ bool seq_sum_chunk(SeqSum& st, const uint32_t (&bits)
 
 // Consumes U chunks (chunk u: lane `tid` owns elements first[u] .. first[u] + R - 1, chunks in
 // increasing position) with ONE barrier when all of them stay inside the binade of s, below the
-// threshold and free of ties; `acc` must have been folded over the same elements with
-// scale = fast_scale(st.s).  Otherwise the chunks go through seq_sum_rounds.
+// threshold and free of ties; `acc[u]` must have been folded over chunk u's elements with
+// scale = fast_scale(st.s).
+// A plain sum that leaves the binade in exactly one place of the group, again without ties, takes
+// three barriers: the slots' increments under the old ulp are exact, so their prefix sums name
+// the slot the sum leaves the binade in and the exact sum entering it; that slot's wave finds the
+// lane the same way from its lanes' increments and lets it add its elements natively; every wave
+// then folds what lies behind that lane with the ulp of the new sum, and the totals are added after
+// checking that they hold no tie and stay inside the new binade.  Everything else (ties, a second
+// change of binade, sums too small for float increments, threshold walks) goes through the
+// predicted pass and the general rounds, from the sum the group was entered with.
 template <int U, int R, bool PLAIN = false>
-__device__ bool seq_sum_group(SeqSum& st, const uint32_t (&bits)[U][R], FastAcc acc, float scale,
+__device__ bool seq_sum_group(SeqSum& st, const uint32_t (&bits)[U][R], const FastAcc (&acc)[U], float scale,
                               const int (&first)[U], int n, float threshold, BlockScratch& sm) {
+  static_assert(U <= 2, "slot_total holds two chunks");
   if (PLAIN) threshold = __uint_as_float(0x7f800000u);  // a plain sum: the compiler drops the comparisons
+  constexpr int kSlots = U * kWaves;
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const float kBig = 67108864.0f;  // 2^26: "take the ordered path"
-  float inc = wave_sum_f32(acc.inc);
-  const bool any_tie = __ballot(acc.tie == 0.5f) != 0ull;
-  if (any_tie || scale == 0.0f || !(inc < kBig)) inc = kBig;
+  bool tie = false;
+#pragma unroll
+  for (int u = 0; u < U; ++u) tie = tie || acc[u].tie == 0.5f;
+  const bool ordered = __ballot(tie) != 0ull || scale == 0.0f;
+  float inc[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    inc[u] = wave_sum_f32(acc[u].inc);
+    if (ordered || !(inc[u] < kBig)) inc[u] = kBig;
+  }
   const uint32_t buf = st.parity_buf;
   st.parity_buf ^= 1u;
-  if (lane == 0) sm.group_total[buf][wave] = inc;
-  __syncthreads();
-  float total = 0.0f;
+  if (lane == 0) {
 #pragma unroll
-  for (int w = 0; w < kWaves; ++w) total += sm.group_total[buf][w];
-  const SumState ss = sum_state(st.s);
-  if (total < static_cast<float>((1u << 24) - ss.S)) {  // stays inside the binade
-    const float s_new = sum_value(ss.S + static_cast<uint32_t>(total), ss.kb);
+    for (int u = 0; u < U; ++u) sm.slot_total[buf][u * kWaves + wave] = inc[u];
+  }
+  __syncthreads();
+  const float mine = lane < kSlots ? sm.slot_total[buf][lane] : 0.0f;
+  const float upto = wave_scan_inclusive_f32(mine, lane);  // exact wherever it is below 2^24
+  const float s_in = uniform_f32(st.s);
+  const SumState ss = sum_state(s_in);
+  const float room = static_cast<float>((1u << 24) - ss.S);
+  const uint64_t leaves = __ballot(lane < kSlots && !(upto < room));
+  if (!leaves) {  // stays inside the binade
+    const float s_new = sum_value(ss.S + static_cast<uint32_t>(readlane_f32(upto, kSlots - 1)), ss.kb);
     if (!(s_new > threshold)) {
       st.s = s_new;
       return false;
     }
+  }
+  if (PLAIN && leaves && __ballot(mine >= kBig) == 0ull) {
+    const int c = __ffsll(static_cast<long long>(leaves)) - 1;  // the slot the sum leaves the binade in
+    const uint32_t S_c = ss.S + static_cast<uint32_t>(readlane_f32(lane_before_f32(upto), c));
+    int j = 64;  // (in the slot's wave) the lane that added natively
+    if (wave == c % kWaves) {
+      float own = 0.0f;
+#pragma unroll
+      for (int u = 0; u < U; ++u) own = (u == c / kWaves) ? acc[u].inc : own;
+      const float lanes_upto = wave_scan_inclusive_f32(own, lane);
+      const float room_c = static_cast<float>((1u << 24) - S_c);
+      const uint64_t over = __ballot(!(lanes_upto < room_c));  // not empty: the slot's total is not below room_c
+      j = __ffsll(static_cast<long long>(over)) - 1;
+      const float before = lane_before_f32(lanes_upto);
+      float sj = 0.0f;
+      if (lane == j) {
+        sj = sum_value(S_c + static_cast<uint32_t>(before), ss.kb);
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          if (u == c / kWaves) {
+#pragma unroll
+            for (int e = 0; e < R; ++e) sj = sj + __uint_as_float(bits[u][e]);  // (entries past n hold 0)
+          }
+        }
+      }
+      if (lane == 0) {
+        sm.bc_sum = readlane_f32(sj, over ? j : 0);
+        sm.bc_found = over ? 1 : 0;  // (always 1: the slot's total, the last of these prefix sums, is not below room_c)
+      }
+    }
+    __syncthreads();
+    const float s_mid = uniform_f32(sm.bc_sum);  // the exact sum behind lane j of slot c
+    const SumState sb = sum_state(s_mid);
+    const bool usable = sm.bc_found != 0 && sb.kb >= 64 && sb.kb < 250;
+    if (usable) {
+      const float scale_b = __uint_as_float(static_cast<uint32_t>(277 - sb.kb) << 23);  // 2^(150 - kb)
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int slot = u * kWaves + wave;
+        float v = 0.0f;
+        if (slot >= c) {  // wave-uniform
+          FastAcc fb = {0.0f, 0.0f};
+          if (slot > c || lane > j) {
+#pragma unroll
+            for (int e = 0; e < R; ++e) fast_fold(fb, __uint_as_float(bits[u][e]), scale_b);
+          }
+          v = wave_sum_f32(fb.inc);
+          if (__ballot(fb.tie == 0.5f) != 0ull || !(v < kBig)) v = kBig;
+        }
+        if (lane == 0) sm.slot_total[buf ^ 1u][slot] = v;
+      }
+    }
+    __syncthreads();
+    if (usable) {
+      const float behind = lane < kSlots ? sm.slot_total[buf ^ 1u][lane] : 0.0f;
+      if (__ballot(behind >= kBig) == 0ull) {
+        const float total = wave_sum_f32(behind);
+        if (total < static_cast<float>((1u << 24) - sb.S)) {
+          st.s = sum_value(sb.S + static_cast<uint32_t>(total), sb.kb);
+          st.parity_buf ^= 1u;  // the next group writes the half that was read before the last two barriers
+          return false;
+        }
+      }
+    }
+    __syncthreads();  // the ordered paths below reuse bc_sum
   }
   int consumed = 0;
   if (U * kWaves <= 32) {

@@ -592,7 +592,9 @@ __device__ __forceinline__ bool scan_row(const ScanArgs& a, SeqSum& st, BlockScr
       }
       const float scale = fast_scale(st.s);
       const float cut_lo = list_cut<LIST, FLOOR>(a, st.s);
-      FastAcc acc = {0.0f, 0.0f};
+      FastAcc acc[kGroup];
+#pragma unroll
+      for (int u = 0; u < kGroup; ++u) acc[u] = {0.0f, 0.0f};
       uint32_t bits[kGroup][VE];
       int first[kGroup];
       const bool more = vbase + per_iter < nvec;
@@ -624,7 +626,7 @@ __device__ __forceinline__ bool scan_row(const ScanArgs& a, SeqSum& st, BlockScr
         for (int e = 0; e < VE; ++e) {
           const float val = LUT ? v[e] : value_of(v[e]);
           bits[u][e] = __float_as_uint(val);
-          fast_fold(acc, val, scale);
+          fast_fold(acc[u], val, scale);
           if (LIST == kListAppend && val >= cut_lo) cmask |= 1u << e;
         }
         if (LIST == kListAppend) {
@@ -1793,7 +1795,9 @@ seq_sum_kernel(const float* a, int32_t n, float s0, float threshold, float* sum_
   int base = 0;
   for (; !stopped && base + kGroup * kBlock * R <= n; base += kGroup * kBlock * R) {
     const float scale = fast_scale(st.s);
-    FastAcc acc = {0.0f, 0.0f};
+    FastAcc acc[kGroup];
+#pragma unroll
+    for (int u = 0; u < kGroup; ++u) acc[u] = {0.0f, 0.0f};
     uint32_t bits[kGroup][R];
     int first[kGroup];
 #pragma unroll
@@ -1803,7 +1807,7 @@ seq_sum_kernel(const float* a, int32_t n, float s0, float threshold, float* sum_
       for (int e = 0; e < R; ++e) {
         const float v = a[first[u] + e];
         bits[u][e] = __float_as_uint(v);
-        fast_fold(acc, v, scale);
+        fast_fold(acc[u], v, scale);
       }
     }
     stopped = seq_sum_group<kGroup, R>(st, bits, acc, scale, first, n, threshold, sm);
