@@ -180,6 +180,16 @@ __device__ __forceinline__ uint32_t wave_sum_u32(uint32_t v) {
   v += dpp_u32_or<0x143, 0xc>(0u, v);
   return __builtin_amdgcn_readlane(v, 63);
 }
+// Inclusive prefix sums of a 32-bit value over the 64 lanes (wraps like the type).
+__device__ __forceinline__ uint32_t wave_scan_inclusive_u32(uint32_t v) {
+  v += dpp_u32_or<0x111, 0xf>(0u, v);
+  v += dpp_u32_or<0x112, 0xf>(0u, v);
+  v += dpp_u32_or<0x114, 0xf>(0u, v);
+  v += dpp_u32_or<0x118, 0xf>(0u, v);
+  v += dpp_u32_or<0x142, 0xa>(0u, v);
+  v += dpp_u32_or<0x143, 0xc>(0u, v);
+  return v;
+}
 __device__ __forceinline__ int wave_max_i32(int v) {
 #define ETS_MAX_STEP(CTRL, MASK)                                                                      \
   {                                                                                                   \
@@ -211,6 +221,8 @@ struct BlockScratch {
   int first_flag[kWaves];
   float group_total[2][kWaves];    // same, for block_sum2
   float slot_total[2][2 * kWaves];  // same, for seq_sum_group: one entry per (chunk, wave) slot
+  uint32_t slot_tie[2][2 * kWaves];  //   whether the slot holds a half-ulp tie
+  uint32_t tie_fix[2 * kWaves];     //   what a slot's ties add to its increments (see seq_sum_group)
   float slot_sum[64];               // plain float sums per slot (seq_sum_predicted)
   float chain_s[2];                 // running sum handed from one serial slot to the next
   int chain_found[2];               //   and where the threshold was crossed, if it was
@@ -791,10 +803,15 @@ __device__ bool seq_sum_group(SeqSum& st, const uint32_t (&bits)[U][R], const Fa
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const float kBig = 67108864.0f;  // 2^26: "take the ordered path"
-  bool tie = false;
+  bool slot_has_tie[U];
+  bool wave_has_tie = false;
 #pragma unroll
-  for (int u = 0; u < U; ++u) tie = tie || acc[u].tie == 0.5f;
-  const bool ordered = __ballot(tie) != 0ull || scale == 0.0f;
+  for (int u = 0; u < U; ++u) {
+    slot_has_tie[u] = __ballot(acc[u].tie == 0.5f) != 0ull;
+    wave_has_tie = wave_has_tie || slot_has_tie[u];
+  }
+  // (a threshold walk leaves every tie to the ordered paths; a plain sum corrects for them below)
+  const bool ordered = scale == 0.0f || (!PLAIN && wave_has_tie);
   float inc[U];
 #pragma unroll
   for (int u = 0; u < U; ++u) {
@@ -805,30 +822,121 @@ __device__ bool seq_sum_group(SeqSum& st, const uint32_t (&bits)[U][R], const Fa
   st.parity_buf ^= 1u;
   if (lane == 0) {
 #pragma unroll
-    for (int u = 0; u < U; ++u) sm.slot_total[buf][u * kWaves + wave] = inc[u];
+    for (int u = 0; u < U; ++u) {
+      sm.slot_total[buf][u * kWaves + wave] = inc[u];
+      if (PLAIN) sm.slot_tie[buf][u * kWaves + wave] = slot_has_tie[u] ? 1u : 0u;
+    }
   }
   __syncthreads();
   const float mine = lane < kSlots ? sm.slot_total[buf][lane] : 0.0f;
-  const float upto = wave_scan_inclusive_f32(mine, lane);  // exact wherever it is below 2^24
+  float upto = wave_scan_inclusive_f32(mine, lane);  // exact wherever it is below 2^24
   const float s_in = uniform_f32(st.s);
   const SumState ss = sum_state(s_in);
   const float room = static_cast<float>((1u << 24) - ss.S);
+  const bool any_big = __ballot(mine >= kBig) != 0ull;
+  uint32_t tie_slots = 0u;
+  if (PLAIN) tie_slots = static_cast<uint32_t>(__ballot(lane < kSlots && sm.slot_tie[buf][lane] != 0u));
+  float lane_fix[U];  // what this lane's ties add to its increments of chunk u (0 without ties)
+#pragma unroll
+  for (int u = 0; u < U; ++u) lane_fix[u] = 0.0f;
+  const bool with_ties = PLAIN && tie_slots != 0u && !any_big;
+  if (with_ties) {
+    // ---- half-ulp ties in a plain sum.  The totals above count rint(t) for a tie t = n0 + 1/2, the
+    // even one of its neighbours; the sequential sum adds n0 or n0 + 1, whichever makes the running
+    // integer even: the same when the integer in front of the tie is even, the other neighbour
+    // (+1 for even n0, -1 for odd n0) when it is odd.  Write a_i for the parity of the PROVISIONAL
+    // integer in front of the i-th tie of the group (entering integer plus the counted increments
+    // of everything before it) and x_i for the parity of the true one.  Every earlier correction is
+    // odd exactly when its own x is, so x_i = a_i ^ x_1 ^ .. ^ x_(i-1), hence x_1 ^ .. ^ x_i = a_i
+    // and x_i = a_i ^ a_(i-1): a tie needs the provisional parity in front of itself and in front
+    // of the tie before it, nothing else.  A wave works out the ties of its slots, for both values
+    // the a of the last tie of an earlier slot can have; after one more barrier everybody chains
+    // the slots.  (All of this is exact up to the place where the sum leaves the binade, which is all
+    // that is used of it.)
+    int d0[U], d1[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      d0[u] = 0;
+      d1[u] = 0;
+      if (slot_has_tie[u]) {  // wave-uniform
+        const int slot = u * kWaves + wave;
+        const uint32_t entering = ss.S + static_cast<uint32_t>(readlane_f32(lane_before_f32(upto), slot));
+        const uint32_t own = static_cast<uint32_t>(__builtin_fminf(acc[u].inc, kBig));
+        uint32_t parity = (entering + wave_scan_inclusive_u32(own) - own) & 1u;  // in front of the lane's first element
+        uint32_t has = 0u, a_first = 0u, a_last = 0u, odd_first = 0u;
+        int rest = 0;  // corrections of the lane's ties after its first
+#pragma unroll
+        for (int e = 0; e < R; ++e) {
+          const float t = __uint_as_float(bits[u][e]) * scale;
+          const float r = __builtin_rintf(t);
+          if (__builtin_fabsf(t - r) == 0.5f) {  // (then t < 2^23)
+            const uint32_t odd = static_cast<uint32_t>(__builtin_floorf(t)) & 1u;
+            if (has) {
+              rest += (parity ^ a_last) ? 1 - 2 * static_cast<int>(odd) : 0;
+            } else {
+              has = 1u;
+              a_first = parity;
+              odd_first = odd;
+            }
+            a_last = parity;
+          }
+          parity ^= r < 16777216.0f ? (static_cast<uint32_t>(r) & 1u) : 0u;
+        }
+        const uint64_t has_mask = __ballot(has != 0u);
+        const uint64_t last_mask = __ballot(has != 0u && a_last != 0u);
+        if (has) {
+          const uint64_t below = has_mask & ((1ull << lane) - 1ull);
+          const int step = 1 - 2 * static_cast<int>(odd_first);
+          if (below) {
+            const uint32_t before = static_cast<uint32_t>(last_mask >> (63 - __clzll(static_cast<long long>(below)))) & 1u;
+            d0[u] = d1[u] = rest + ((a_first ^ before) ? step : 0);
+          } else {  // the slot's first tie: its predecessor is in an earlier slot, or there is none (a = 0)
+            d0[u] = rest + (a_first ? step : 0);
+            d1[u] = rest + (a_first ? 0 : step);
+          }
+        }
+        const uint32_t D0 = wave_sum_u32(static_cast<uint32_t>(d0[u])) + 1024u;  // |D| <= 512
+        const uint32_t D1 = wave_sum_u32(static_cast<uint32_t>(d1[u])) + 1024u;
+        const uint32_t slot_last = static_cast<uint32_t>(last_mask >> (63 - __clzll(static_cast<long long>(has_mask)))) & 1u;
+        if (lane == 0) sm.tie_fix[slot] = (D0 & 0xfffu) | ((D1 & 0xfffu) << 12) | (slot_last << 24);
+      }
+    }
+    __syncthreads();
+    const uint32_t my_fix = (lane < kSlots && ((tie_slots >> lane) & 1u)) ? sm.tie_fix[lane] : 0u;
+    uint32_t before = 0u;  // a of the last tie so far
+    int shift = 0;         // what the ties up to this lane's slot add
+    uint32_t pending = tie_slots;
+    while (pending) {  // uniform
+      const int t = __ffs(static_cast<int>(pending)) - 1;
+      pending &= pending - 1u;
+      const uint32_t f = readlane_u32(my_fix, t);
+      const int D = static_cast<int>((before ? (f >> 12) : f) & 0xfffu) - 1024;
+      if (lane >= t) shift += D;
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        if (t == u * kWaves + wave) lane_fix[u] = static_cast<float>(before ? d1[u] : d0[u]);
+      }
+      before = (f >> 24) & 1u;
+    }
+    upto += static_cast<float>(shift);
+  }
+  const bool countable = !any_big && (tie_slots == 0u || with_ties);  // `upto` holds the true prefix sums
   const uint64_t leaves = __ballot(lane < kSlots && !(upto < room));
-  if (!leaves) {  // stays inside the binade
+  if (countable && !leaves) {  // stays inside the binade
     const float s_new = sum_value(ss.S + static_cast<uint32_t>(readlane_f32(upto, kSlots - 1)), ss.kb);
     if (!(s_new > threshold)) {
       st.s = s_new;
       return false;
     }
   }
-  if (PLAIN && leaves && __ballot(mine >= kBig) == 0ull) {
+  if (PLAIN && countable && leaves) {
     const int c = __ffsll(static_cast<long long>(leaves)) - 1;  // the slot the sum leaves the binade in
     const uint32_t S_c = ss.S + static_cast<uint32_t>(readlane_f32(lane_before_f32(upto), c));
     int j = 64;  // (in the slot's wave) the lane that added natively
     if (wave == c % kWaves) {
       float own = 0.0f;
 #pragma unroll
-      for (int u = 0; u < U; ++u) own = (u == c / kWaves) ? acc[u].inc : own;
+      for (int u = 0; u < U; ++u) own = (u == c / kWaves) ? acc[u].inc + lane_fix[u] : own;
       const float lanes_upto = wave_scan_inclusive_f32(own, lane);
       const float room_c = static_cast<float>((1u << 24) - S_c);
       const uint64_t over = __ballot(!(lanes_upto < room_c));  // not empty: the slot's total is not below room_c

@@ -7,7 +7,7 @@ Every case draws a vocabulary size (1 .. 300 000, biased to small and to sizes a
 vectorisation and LDS limits), an element type, a row pitch (aligned or not), a temperature, top-p,
 top-k and a row structure (normal, peaked, few distinct values, flat, wide range, tiny magnitudes,
 masked with -inf, sorted), samples a few rows on the device with and without debug records and
-compares tokens and coin states with the oracle (test infrastructure, never the thing measured) in
+compares tokens, coin states and the softmax normaliser (bit for bit) with the oracle (test infrastructure, never the thing measured) in
 the arithmetic the HIP sampler implements.  Prints one JSON line; exits non-zero on a mismatch and
 names the case.  Not collected by pytest.
 """
@@ -133,9 +133,16 @@ def main():
                 plain.set_topk(topk)
                 got_plain = plain.sample_batch(dx).cpu().numpy()
                 # the constructor does not clamp: a negative temperature gives a negative inverse (sampler.cpp:173-181)
-                want, _ = O.sample_rows(np.ascontiguousarray(x), dtype, O.inv_temperature(temperature), topp, topk, states,
-                                        mode=O.MODE_UPCAST, tie=O.TIE_STABLE, threads=4)
+                want, ex = O.sample_rows(np.ascontiguousarray(x), dtype, O.inv_temperature(temperature), topp, topk, states,
+                                         mode=O.MODE_UPCAST, tie=O.TIE_STABLE, threads=4, explain=True)
                 ok = np.array_equal(got, want) and np.array_equal(got_plain, want) and np.array_equal(after, states)
+                if temperature != 0.0:  # the softmax normaliser, bit for bit (the arg-max computes none)
+                    sums = ea.debug_records(ddbg)["sum"]
+                    for b in range(rows):
+                        a, w_ = np.float32(sums[b]), np.float32(ex[b].sum)
+                        if not (a.view(np.uint32) == w_.view(np.uint32) or (np.isnan(a) and np.isnan(w_))):
+                            ok = False
+                            label["sum"] = [b, float(a), float(w_)]
         except Exception as e:  # an error status is a failure here: every case is a legal call
             ok = False
             label["error"] = repr(e)[:300]
