@@ -25,7 +25,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by
 # the factors a 256 MiB device copy gives in the same runs (profiles/sample_rows_kernel_cfg2.md has
 # the commands and the raw counters): 9221 KiB * 2.00 fetched + 3780 KiB * 1.00 written.
-MEASURED_TRAFFIC_BYTES = {"cfg2": (8913 * 2.00 + 3742 * 1.00) * 1024}
+MEASURED_TRAFFIC_BYTES = {"cfg2": (8940 * 2.00 + 3817 * 1.00) * 1024}
 
 
 def synth_logits_device(w, count, torch, dev):
