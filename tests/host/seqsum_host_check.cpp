@@ -198,7 +198,7 @@ int main() {
     for (int i = 0; i < 2000000; ++i) {
       const float S = (float)(1 + rng() % 4096) * std::ldexp(1.0f, (int)(rng() % 6));
       probe(std::ldexp((float)(rng() % 100000), -149), S);              // subnormal numerators
-      probe(std::ldexp((float)(1 + rng() % 4096), -126), S);            // quotients around 2^-126
+      probe(std::ldexp((float)(1 + rng() % 4096), -126), S);            // quotients near 2^-126
       probe((float)std::exp(uni(-104, 0)), (float)uni(1, 200000));      // what the sampler divides
     }
     for (int k = 1; k < 4096; ++k) {
