@@ -353,8 +353,10 @@ __device__ __forceinline__ ParityInc fold_run(const uint32_t (&bits)[R], float s
 // the binade of s or crosses the threshold.  The first event lane adds its elements natively and
 // the scan restarts behind it with the new ulp.  Tiny running sums use the two-hypothesis parity
 // summaries instead (integer arithmetic, any magnitude).
+// (The ordered paths are forced inline: left out of line they take the group's entries by
+// reference, which puts that array -- written for every entry of the row -- into private memory.)
 template <int R>
-__device__ void wave_resolve(float& s, int& found, const uint32_t (&bits)[R], int first, int n, float threshold,
+__device__ __forceinline__ void wave_resolve(float& s, int& found, const uint32_t (&bits)[R], int first, int n, float threshold,
                              int consumed = 0) {  // lanes below `consumed` have been consumed
   const int lane = threadIdx.x & 63;
   found = -1;
@@ -512,7 +514,7 @@ __device__ __forceinline__ int resolve_prepared(float& s, const uint32_t (&bits)
 // threshold is crossed st.stop_index is set and `stopped` is true.
 // PLAIN: the threshold is known to be +inf at compile time (a plain sum).
 template <int U, int R, bool PLAIN>
-__device__ int seq_sum_predicted(SeqSum& st, const uint32_t (&bits)[U][R], const int (&first)[U], int n, float threshold,
+__device__ __forceinline__ int seq_sum_predicted(SeqSum& st, const uint32_t (&bits)[U][R], const int (&first)[U], int n, float threshold,
                                  bool& stopped, BlockScratch& sm) {
   if (PLAIN) threshold = __uint_as_float(0x7f800000u);
   stopped = false;
@@ -680,7 +682,7 @@ __device__ int seq_sum_predicted(SeqSum& st, const uint32_t (&bits)[U][R], const
 // round, one when nothing happens.  Must be called by all lanes; returns true when the
 // threshold was crossed (st.stop_index set).
 template <int U, int R>
-__device__ bool seq_sum_rounds(SeqSum& st, const uint32_t (&bits)[U][R], const int (&first)[U], int n, float threshold,
+__device__ __forceinline__ bool seq_sum_rounds(SeqSum& st, const uint32_t (&bits)[U][R], const int (&first)[U], int n, float threshold,
                                BlockScratch& sm, int resume = 0) {
   static_assert(U * kWaves <= 64, "one lane per slot in the cross-wave scan");
   constexpr int kSlots = U * kWaves;
@@ -795,7 +797,7 @@ __device__ __forceinline__ bool seq_sum_chunk(SeqSum& st, const uint32_t (&bits)
 // change of binade, sums too small for float increments, threshold walks) goes through the
 // predicted pass and the general rounds, from the sum the group was entered with.
 template <int U, int R, bool PLAIN = false>
-__device__ bool seq_sum_group(SeqSum& st, const uint32_t (&bits)[U][R], const FastAcc (&acc)[U], float scale,
+__device__ __forceinline__ bool seq_sum_group(SeqSum& st, const uint32_t (&bits)[U][R], const FastAcc (&acc)[U], float scale,
                               const int (&first)[U], int n, float threshold, BlockScratch& sm) {
   static_assert(U <= 2, "slot_total holds two chunks");
   if (PLAIN) threshold = __uint_as_float(0x7f800000u);  // a plain sum: the compiler drops the comparisons
