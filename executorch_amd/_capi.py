@@ -41,6 +41,7 @@ SIGNATURES = {
     "ets_sampler_set_temperature": (C.c_int32, [C.c_void_p, C.c_float]),
     "ets_sampler_set_topk": (C.c_int32, [C.c_void_p, C.c_int32]),
     "ets_sampler_set_topp": (C.c_int32, [C.c_void_p, C.c_float]),
+    "ets_sampler_set_row_split": (C.c_int32, [C.c_void_p, C.c_int32]),
     "ets_sampler_sample": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int32, C.POINTER(C.c_int32)]),
     "ets_sampler_sample_batch": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int64, C.c_void_p, C.c_void_p]),
     "ets_sampler_sample_batch_configs": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int64, C.c_void_p,
@@ -80,6 +81,7 @@ CHAIN_SIGNATURES = {
 TEST_HOOKS = {
     "ets_test_expf": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p]),
     "ets_test_seq_sum": (C.c_int32, [C.c_void_p, C.c_int32, C.c_float, C.c_float, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "ets_test_split_timers": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int32]),
 }
 
 _lib = None

@@ -36,8 +36,8 @@ def hipcc() -> str:
     return exe
 
 
-def build_library(verbose: bool = True) -> str:
-    cmd = [hipcc(), *HIPCC_FLAGS, os.path.join(CSRC, "et_sampler.hip"), "-o", LIB]
+def build_library(verbose: bool = True, extra_flags: list[str] | None = None, out: str = LIB) -> str:
+    cmd = [hipcc(), *HIPCC_FLAGS, *(extra_flags or []), os.path.join(CSRC, "et_sampler.hip"), "-o", out]
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.check_call(cmd)

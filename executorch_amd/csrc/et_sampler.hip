@@ -5,6 +5,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <atomic>
 #include <cstdio>
 #include <cstring>
 #include <ctime>
@@ -12,7 +13,10 @@
 #include <new>
 #include <string>
 
+#include <cstdlib>
+
 #include "ets_kernels.h"
+#include "ets_split.h"
 #include "ets_test_hooks.h"
 
 namespace {
@@ -40,6 +44,12 @@ struct ets_sampler {
   uint64_t* d_partials = nullptr;  // [max_batch, kMaxSplits] argmax partial results
   void* d_row = nullptr;           // staging for one host row (vocab * 4 bytes)
   int32_t* d_token = nullptr;      // staging for one token
+  // work buffers of the path that spreads a row over several workgroups (ets_split.h): one
+  // allocation, made on first use
+  int split_mode = 0;  // ETS_ROW_SPLIT_AUTO
+  int num_cus = 0;
+  void* d_split = nullptr;
+  ets::SplitParams split = {};
   // per-row sampling parameters of ets_sampler_sample_batch_configs(): pinned host staging, its
   // device copy, and the event that says the last upload has left the staging buffer
   void* h_stage = nullptr;
@@ -172,16 +182,23 @@ ets_status launch_argmax(ets_sampler* s, const void* d_logits, int32_t batch, in
   return ETS_OK;
 }
 
+// Raises a kernel's dynamic-LDS limit to `bytes` on the handle's device.  The limit is kept per
+// kernel and device, so it is set again only when a handle asks for more than was set before.
+constexpr int kMaxDevices = 64;
+ets_status allow_dynamic_lds(ets_sampler* s, const void* kernel, size_t bytes, std::atomic<size_t>* set_bytes) {
+  const int dev = s->device >= 0 && s->device < kMaxDevices ? s->device : 0;
+  if (set_bytes[dev].load(std::memory_order_acquire) >= bytes) return ETS_OK;
+  ETS_HIP(s, hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(bytes)));
+  set_bytes[dev].store(bytes, std::memory_order_release);
+  return ETS_OK;
+}
+
 template <int DT, bool ALIGNED, int DRAW>
 ets_status launch_rows_impl(ets_sampler* s, const ets::RowParams& p, int32_t batch, hipStream_t stream) {
-  static std::once_flag once;
-  static hipError_t attr_err = hipSuccess;
+  static std::atomic<size_t> set_bytes[kMaxDevices];
   const size_t lds = s->lds_bytes;
-  std::call_once(once, [&] {
-    attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(&ets::sample_rows_kernel<DT, ALIGNED, DRAW>),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
-  });
-  if (attr_err != hipSuccess) return hip_fail(s, attr_err, "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
+  ets_status st = allow_dynamic_lds(s, reinterpret_cast<const void*>(&ets::sample_rows_kernel<DT, ALIGNED, DRAW>), lds, set_bytes);
+  if (st != ETS_OK) return st;
   hipLaunchKernelGGL((ets::sample_rows_kernel<DT, ALIGNED, DRAW>), dim3(batch), dim3(ets::kBlock), lds, stream, p);
   ETS_HIP(s, hipGetLastError());
   return ETS_OK;
@@ -244,8 +261,122 @@ const char* const kUint16Message =
     "stochastic sampling of UInt16 logits is not supported (integer softmax of the reference degenerates to "
     "0/1 weights); use temperature 0 or dequantise first";
 
+
+// ---- rows spread over several workgroups (ets_split.h) -------------------------------------------
+size_t round_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+// Workgroups per row of pass 2: about one per CU over the batch, sixteen slots each at least.
+int pass2_workgroups(const ets_sampler* s, int32_t rows, int32_t ns) {
+  static const int forced = [] {
+    const char* e = std::getenv("ETS_SPLIT_WORKGROUPS");
+    return e ? std::atoi(e) : 0;
+  }();
+  int g = forced > 0 ? forced : ((s->num_cus > 0 ? s->num_cus : 256) + rows - 1) / rows;
+  const int by_len = (ns + 15) / 16;
+  if (g > by_len) g = by_len;
+  if (g > ets::kMaxRowWorkgroups) g = ets::kMaxRowWorkgroups;
+  return g < 1 ? 1 : g;
+}
+
+// Candidates one workgroup of pass 2 can list when `g` of them share a row: all of its entries,
+// up to kListRegion.
+int32_t list_region(int32_t ns, int g) {
+  const int per_wg = ((ns + g - 1) / g + 15) / 16 * 16;
+  const int64_t entries = static_cast<int64_t>(per_wg) * ets::kSlot;
+  return static_cast<int32_t>(entries < ets::kListRegion ? entries : ets::kListRegion);
+}
+
+ets_status ensure_split(ets_sampler* s) {
+  if (s->d_split) return ETS_OK;
+  ets::SplitParams& sp = s->split;
+  const size_t rows = static_cast<size_t>(s->max_batch);
+  sp.ns = (s->vocab + ets::kSlot - 1) / ets::kSlot;
+  sp.ns_stride = static_cast<int32_t>(round_up(static_cast<size_t>(sp.ns), 4));
+  sp.prep_cap = ets::kPrepCap;
+  // the candidate lists of the largest launch: rows x workgroups per row x region
+  size_t list_entries = 0, row_wgs = 0;
+  for (int32_t r = 1; r <= s->max_batch; ++r) {
+    const int g = pass2_workgroups(s, r, sp.ns);
+    const size_t need = static_cast<size_t>(r) * g * list_region(sp.ns, g);
+    if (need > list_entries) list_entries = need;
+    if (static_cast<size_t>(r) * g > row_wgs) row_wgs = static_cast<size_t>(r) * g;
+  }
+  size_t at = 0;
+  auto take = [&](size_t bytes) {
+    const size_t here = at;
+    at = round_up(at + bytes, 256);
+    return here;
+  };
+  const size_t o_max = take(rows * sp.ns_stride * sizeof(float));
+  const size_t o_sum = take(rows * sp.ns_stride * sizeof(float));
+  const size_t o_rec = take(rows * sp.ns_stride * sizeof(ets::SlotRec));
+  const size_t o_prep = take(rows * sp.prep_cap * sizeof(ets::PrepSlot));
+  const size_t o_state = take(rows * sizeof(ets::RowState));
+  const size_t o_count = take(rows * ets::kMaxRowWorkgroups * sizeof(uint32_t));
+  const size_t o_timers = take(rows * 12 * sizeof(uint64_t));
+  const size_t o_hist = take(row_wgs * ets::kHistBuckets * sizeof(uint32_t));
+  const size_t o_list = take(list_entries * sizeof(uint64_t));
+  ETS_HIP(s, hipMalloc(&s->d_split, at));
+  char* base = static_cast<char*>(s->d_split);
+  sp.slot_max = reinterpret_cast<float*>(base + o_max);
+  sp.slot_sum = reinterpret_cast<float*>(base + o_sum);
+  sp.slot_rec = reinterpret_cast<ets::SlotRec*>(base + o_rec);
+  sp.prep = reinterpret_cast<ets::PrepSlot*>(base + o_prep);
+  sp.row_state = reinterpret_cast<ets::RowState*>(base + o_state);
+  sp.list_count = reinterpret_cast<uint32_t*>(base + o_count);
+  sp.hist = reinterpret_cast<uint32_t*>(base + o_hist);
+  sp.list = reinterpret_cast<uint64_t*>(base + o_list);
+  sp.timers = std::getenv("ETS_SPLIT_TIMERS") ? reinterpret_cast<uint64_t*>(base + o_timers) : nullptr;
+  return ETS_OK;
+}
+
+// Whether a launch of `rows` rows with draw `draw` takes the three-launch path.
+bool use_split(const ets_sampler* s, const void* d_logits, int64_t stride, int32_t dtype, int draw) {
+  if (s->split_mode == ETS_ROW_SPLIT_OFF || draw != ets::kDrawTopP) return false;
+  const size_t esz = dtype_size(dtype);
+  const bool aligned = (reinterpret_cast<uintptr_t>(d_logits) % 16 == 0) && ((static_cast<size_t>(stride) * esz) % 16 == 0);
+  if (!aligned || (s->vocab + ets::kSlot - 1) / ets::kSlot > ets::kMaxSlots) return false;
+  return s->split_mode == ETS_ROW_SPLIT_ON || s->vocab >= 8192;
+}
+
+template <int DT>
+ets_status launch_split(ets_sampler* s, const ets::RowParams& p, int32_t rows, hipStream_t stream) {
+  ets_status st = ensure_split(s);
+  if (st != ETS_OK) return st;
+  ets::SplitParams sp = s->split;
+  sp.row = p;
+  sp.row_wgs = pass2_workgroups(s, rows, sp.ns);
+  sp.list_region = list_region(sp.ns, sp.row_wgs);
+  const int per_block = (ets::kPass1Block / 64) * ets::kPass1SlotsPerWave;
+  hipLaunchKernelGGL((ets::split_pass1_kernel<DT>), dim3((sp.ns + per_block - 1) / per_block, rows), dim3(ets::kPass1Block), 0,
+                     stream, sp);
+  ETS_HIP(s, hipGetLastError());
+  const size_t lut_bytes = DT == ets::kDtypeBFloat16 ? sizeof(float) * ets::kLutCountWords : 0;
+  static std::atomic<size_t> set_bytes2[kMaxDevices];
+  st = allow_dynamic_lds(s, reinterpret_cast<const void*>(&ets::split_pass2_kernel<DT, true>), lut_bytes, set_bytes2);
+  if (st != ETS_OK) return st;
+  hipLaunchKernelGGL((ets::split_pass2_kernel<DT, true>), dim3(sp.row_wgs, rows), dim3(ets::kBlock), lut_bytes, stream, sp);
+  ETS_HIP(s, hipGetLastError());
+  static std::atomic<size_t> set_bytes[kMaxDevices];
+  st = allow_dynamic_lds(s, reinterpret_cast<const void*>(&ets::split_finish_kernel<DT>), s->lds_bytes, set_bytes);
+  if (st != ETS_OK) return st;
+  hipLaunchKernelGGL((ets::split_finish_kernel<DT>), dim3(rows), dim3(ets::kBlock), s->lds_bytes, stream, sp);
+  ETS_HIP(s, hipGetLastError());
+  return ETS_OK;
+}
+
 ets_status rows_device(ets_sampler* s, const ets::RowParams& p, int32_t dtype, int32_t rows, hipStream_t stream,
                        int draw) {
+  if (use_split(s, p.logits, p.row_stride, dtype, draw)) {
+    switch (dtype) {
+      case ETS_DTYPE_FLOAT:
+        return launch_split<ets::kDtypeFloat>(s, p, rows, stream);
+      case ETS_DTYPE_HALF:
+        return launch_split<ets::kDtypeHalf>(s, p, rows, stream);
+      default:
+        return launch_split<ets::kDtypeBFloat16>(s, p, rows, stream);
+    }
+  }
   switch (dtype) {
     case ETS_DTYPE_FLOAT:
       return launch_rows<ets::kDtypeFloat>(s, p, rows, stream, draw);
@@ -404,6 +535,10 @@ ets_status ets_sampler_create(int32_t vocab_size, float temperature, float topp,
   s->topp = topp;
   s->topk = 0;
   s->max_batch = max_batch;
+  if (const char* e = std::getenv("ETS_ROW_SPLIT")) {  // default of ets_sampler_set_row_split()
+    const int mode = std::atoi(e);
+    if (mode == ETS_ROW_SPLIT_ON || mode == ETS_ROW_SPLIT_OFF) s->split_mode = mode;
+  }
   auto bail = [&](hipError_t e, const char* what) {
     ets_status st = hip_fail(nullptr, e, what);
     ets_sampler_destroy(s);
@@ -414,6 +549,8 @@ ets_status ets_sampler_create(int32_t vocab_size, float temperature, float topp,
   int lds_limit = 0;
   e = hipDeviceGetAttribute(&lds_limit, hipDeviceAttributeMaxSharedMemoryPerBlock, s->device);
   if (e != hipSuccess) return bail(e, "hipDeviceGetAttribute(MaxSharedMemoryPerBlock)");
+  e = hipDeviceGetAttribute(&s->num_cus, hipDeviceAttributeMultiprocessorCount, s->device);
+  if (e != hipSuccess) return bail(e, "hipDeviceGetAttribute(MultiprocessorCount)");
   // the row kernel's static LDS (reduction scratch, selection buffer, histogram) stays under 16 KiB
   int keys = 1;
   while (static_cast<size_t>(keys) * 2 * sizeof(uint64_t) + 16384 <= static_cast<size_t>(lds_limit)) keys *= 2;
@@ -459,6 +596,7 @@ ets_status ets_sampler_destroy(ets_sampler* s) {
     DeviceGuard g(s->device);
     (void)hipFree(s->d_rng);
     (void)hipFree(s->d_scratch);
+    (void)hipFree(s->d_split);
     (void)hipFree(s->d_partials);
     (void)hipFree(s->d_row);
     (void)hipFree(s->d_token);
@@ -484,6 +622,14 @@ ets_status ets_sampler_set_temperature(ets_sampler* s, float temperature) {
 ets_status ets_sampler_set_topk(ets_sampler* s, int32_t topk) {
   if (!s) return fail(nullptr, ETS_INVALID_ARGUMENT, "ets_sampler_set_topk: null handle");
   s->topk = topk;
+  return ETS_OK;
+}
+
+ets_status ets_sampler_set_row_split(ets_sampler* s, int32_t mode) {
+  if (!s) return fail(nullptr, ETS_INVALID_ARGUMENT, "ets_sampler_set_row_split: null handle");
+  if (mode != ETS_ROW_SPLIT_AUTO && mode != ETS_ROW_SPLIT_ON && mode != ETS_ROW_SPLIT_OFF)
+    return fail(s, ETS_INVALID_ARGUMENT, "ets_sampler_set_row_split: unknown mode");
+  s->split_mode = mode;
   return ETS_OK;
 }
 
@@ -744,6 +890,15 @@ ets_status ets_test_seq_sum(const float* d_a, int32_t n, float s0, float thresho
   hipLaunchKernelGGL(ets::seq_sum_kernel, dim3(1), dim3(ets::kBlock), 0, static_cast<hipStream_t>(hip_stream), d_a, n,
                      s0, threshold, d_sum, d_stop);
   ETS_HIP(nullptr, hipGetLastError());
+  return ETS_OK;
+}
+
+ets_status ets_test_split_timers(ets_sampler* s, uint64_t* out, int32_t rows) {
+  if (!s || !out || rows < 0 || rows > s->max_batch) return fail(s, ETS_INVALID_ARGUMENT, "ets_test_split_timers: bad arguments");
+  if (!s->d_split || !s->split.timers)
+    return fail(s, ETS_INVALID_STATE, "ets_test_split_timers: set ETS_SPLIT_TIMERS before the handle's first stochastic call");
+  DeviceGuard g(s->device);
+  ETS_HIP(s, hipMemcpy(out, s->split.timers, sizeof(uint64_t) * 12 * rows, hipMemcpyDeviceToHost));
   return ETS_OK;
 }
 

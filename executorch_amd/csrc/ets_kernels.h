@@ -433,6 +433,8 @@ constexpr int kLutCountWords = 12288;  // a table entry's counter sits 48 KiB ab
 // the look-ups of e spread over all LDS banks.
 // Returns false (no table; the caller evaluates expf per entry) when inv or max are not positive
 // finite in the way the bounds need, or when the table would not fit in `cap` floats.
+// COUNTERS = false builds the table alone (`cap` then only has to hold its 2 * half floats).
+template <bool COUNTERS = true>
 __device__ bool build_exp_lut(float* lut, int cap, float inv, float m, const uint64_t* tab, int& base1, int& top,
                               int& half) {
   const float kInf = __uint_as_float(0x7f800000u);
@@ -456,7 +458,7 @@ __device__ bool build_exp_lut(float* lut, int cap, float inv, float m, const uin
   half = R + 2;
   top = R + 1;
   base1 = (e_lo << 7) - 1;
-  if (2 * half > kLutCountWords || kLutCountWords + 2 * half > cap) return false;
+  if (2 * half > kLutCountWords || (COUNTERS ? kLutCountWords + 2 * half : 2 * half) > cap) return false;
   for (int idx = threadIdx.x; idx < 2 * half; idx += kBlock) {
     const int sgn = idx >= half ? 1 : 0;
     const int c = idx - sgn * half;
@@ -476,7 +478,7 @@ __device__ bool build_exp_lut(float* lut, int cap, float inv, float m, const uin
       e = expf_core(d, tab);
     }
     lut[idx] = e;
-    lut[kLutCountWords + idx] = 0.0f;  // bit pattern of the integer 0
+    if (COUNTERS) lut[kLutCountWords + idx] = 0.0f;  // bit pattern of the integer 0
   }
   return true;
 }

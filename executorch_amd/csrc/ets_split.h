@@ -1,0 +1,978 @@
+// The stochastic path with every row spread over several workgroups: three launches.
+//
+//   split_pass1_kernel   (HBM read) per slot of 512 entries: the maximum of x = logit * inv_temperature
+//                        and an approximate sum of exp(x - slot maximum)
+//   split_pass2_kernel   (re-read, L2 / Infinity Cache) exact e = expf(x - row maximum) per entry; from
+//                        the approximate running sums every slot learns the binade the sequential
+//                        softmax sum will be in when it reaches the slot and folds its entries ONCE,
+//                        with that binade's ulp, into a parity summary (ets_seqsum_math.h); slots that
+//                        cannot be placed inside one binade keep their entries and prefix sums under
+//                        the two candidate ulps instead; top-p candidates are listed
+//   split_finish_kernel  one workgroup per row: composes the summaries in index order from the exact
+//                        running sum, checks every prediction exactly, resolves the few slots in which
+//                        the sum changes binade entry by entry, then draws the coin and the token
+//
+// Passes 1 and 2 hold no step that depends on another slot, so any number of workgroups share a
+// row; what is inherently ordered (sampler.cpp:199-203 adds the entries one after the other) is
+// reduced to one wave walking a few hundred 16-byte records.  Predictions only select the work:
+// every value that reaches the result has been verified against the exact running sum.
+#pragma once
+
+#include "ets_kernels.h"
+
+namespace ets {
+
+constexpr int kSlot = 512;        // entries per slot: 64 lanes x 8 consecutive entries
+constexpr int kMaxSlots = 2048;   // rows of up to 1048576 entries take this path
+constexpr int kPass1Block = 256;  // lanes per workgroup of pass 1
+constexpr int kPass1SlotsPerWave = 4;
+constexpr int kPrepCap = 40;      // prepared slots per row (a row of the usual kind needs 10 to 20)
+
+constexpr uint32_t kSlotStable = 0u;  // even / odd hold the slot's parity summary for binade `kb`
+constexpr uint32_t kSlotZero = 1u;    // every entry is 0: adds nothing whatever the running sum
+constexpr uint32_t kSlotSerial = 2u;  // to be resolved in order (prepared data at index `prep`, if any)
+constexpr uint32_t kSlotDual = 3u;    // no entry ties under the ulp of binade kb or of kb + 1: `even` is the slot's
+                                      //   increment for a sum that passes it inside binade kb, `odd` inside kb + 1
+constexpr uint32_t kSlotExact = 4u;   // slot 0 only: `even` holds the bits of the exact sum behind the slot
+
+struct SlotRec {
+  uint32_t meta;  // bits 0-7: biased exponent the summary was folded for; bits 8-10: kind
+  uint32_t even, odd;
+  uint32_t prep;  // index of the slot's PrepSlot, or 0xffffffff
+};
+
+// What pass 2 keeps of a slot that is resolved in order: its entries and the inclusive prefix sums
+// over the lanes of the increments rne(e / ulp) of each lane's 8 entries, under the ulp of the
+// binade the running sum is expected to enter the slot in (a) and of the one it is expected to
+// leave it in (b), with the lanes in which an entry sits on a half-ulp tie (their increment
+// depends on the order of the adds).  A lane's increment is capped at 2^25 (far beyond what any
+// binade has room for), so the sums are exact integers wherever they matter and never wrap.
+struct PrepSlot {
+  float e[kSlot];
+  uint32_t pre_a[64];
+  uint32_t pre_b[64];
+  uint32_t kb_a, kb_b;
+  uint32_t tie_a_lo, tie_a_hi, tie_b_lo, tie_b_hi;
+  uint32_t usable;  // both binades are in the range of the float shortcut
+  uint32_t pad;
+};
+static_assert(sizeof(PrepSlot) % 16 == 0, "prepared slots are copied as 16-byte vectors");
+
+struct RowState {
+  uint32_t prep_count;  // slots that pass 2 set aside to be resolved in order (may exceed the capacity)
+  float m;              // row maximum of x (NaN when x[0] is NaN, like the reference's loop)
+  uint32_t nan;         // some expf(x - m) is NaN
+  float a_total;        // approximate softmax sum, in units of exp(-m)
+};
+
+constexpr int kMaxRowWorkgroups = 64;  // workgroups of pass 2 per row
+constexpr int kListRegion = 16384;     // candidates one workgroup of pass 2 can list
+
+// Histogram of a row's candidates by the size of exp: 64 buckets per binade, from 1 downwards.
+// Bucket b holds exp bit patterns in (0x3F800000 - (b + 1) * 2^17, 0x3F800000 - b * 2^17]; the last
+// bucket also takes everything below.
+constexpr int kHistBuckets = 2048;
+__device__ __forceinline__ uint32_t hist_bucket(uint32_t e_bits) {
+  const uint32_t b = (0x3F800000u - e_bits) >> 17;  // (exp <= 1)
+  return b < static_cast<uint32_t>(kHistBuckets - 1) ? b : static_cast<uint32_t>(kHistBuckets - 1);
+}
+// Every exp in buckets 0 .. b - 1 is above hist_edge(b); every one in buckets b .. is at most that.
+__device__ __forceinline__ float hist_edge(int b) {
+  return b >= kHistBuckets ? 0.0f : __uint_as_float(0x3F800000u - (static_cast<uint32_t>(b) << 17));
+}
+
+struct SplitParams {
+  RowParams row;        // what the one-workgroup kernel takes
+  float* slot_max;      // [rows, ns_stride]
+  float* slot_sum;      // [rows, ns_stride]
+  SlotRec* slot_rec;    // [rows, ns_stride]
+  PrepSlot* prep;       // [rows, prep_cap]
+  RowState* row_state;  // [rows]
+  uint64_t* list;       // [rows, row_wgs, list_region] (exp bits << 32 | index) of possible top-p
+                        //   candidates: every workgroup of pass 2 fills its own region
+  uint32_t* list_count; // [rows, kMaxRowWorkgroups] candidates each workgroup found (may exceed its region)
+  uint32_t* hist;       // [rows, row_wgs, kHistBuckets] the same candidates by size
+  uint64_t* timers;     // phase clocks (profiling), or null
+  int32_t list_region;  // entries per region
+  int32_t row_wgs;      // workgroups of pass 2 per row
+  int32_t ns;           // slots per row
+  int32_t ns_stride;
+  int32_t prep_cap;
+};
+
+// Relative distance between the exact sequential sum after i entries and the approximate sum of
+// pass 1: every add rounds by at most half an ulp of a running sum that never decreases, so the
+// sequential sum is within i * 2^-24 of the mathematical one; pass 1's exponentials and float
+// additions are within 1e-4 of it.
+__device__ __forceinline__ float split_eps(int entries) {
+  return static_cast<float>(entries) * (1.02f / 16777216.0f) + 2e-4f;
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+constexpr float kLog2e = 1.44269504088896340736f;
+
+// The 8 entries of lane `lane` of slot `s` as floats; positions past the row read as `fill`.
+template <int DT>
+__device__ __forceinline__ void load_slot_lane(const char* logits, int s, int lane, int V, float fill, float* out) {
+  constexpr int VE = VecElems<DT>::value;
+  const int first = s * kSlot + lane * 8;
+#pragma unroll
+  for (int q = 0; q < 8 / VE; ++q) load_run<DT, true>(logits, first + q * VE, V, fill, out + q * VE);
+}
+
+// ---- pass 1 ---------------------------------------------------------------------------------------
+template <int DT>
+__global__ void __launch_bounds__(kPass1Block) split_pass1_kernel(SplitParams p) {
+  const int row = p.row.row_map ? p.row.row_map[blockIdx.y] : blockIdx.y;
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int V = p.row.vocab;
+  const float inv = p.row.row_cfg ? p.row.row_cfg[row].inv_temperature : p.row.inv_temperature;
+  const char* logits = static_cast<const char*>(p.row.logits) + static_cast<int64_t>(row) * p.row.row_stride * ElemSize<DT>::value;
+  const float kInf = __uint_as_float(0x7f800000u);
+  const float fill = inv < 0.0f ? kInf : -kInf;  // x = -inf: adds nothing
+  const int slot0 = (blockIdx.x * (kPass1Block / 64) + wave) * kPass1SlotsPerWave;
+  float v[kPass1SlotsPerWave][8];
+#pragma unroll
+  for (int k = 0; k < kPass1SlotsPerWave; ++k) {
+    if (slot0 + k < p.ns) load_slot_lane<DT>(logits, slot0 + k, lane, V, fill, v[k]);
+  }
+#pragma unroll
+  for (int k = 0; k < kPass1SlotsPerWave; ++k) {
+    const int s = slot0 + k;
+    if (s >= p.ns) break;
+    float lmax = -kInf;
+    bool nan = false;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      v[k][e] = v[k][e] * inv;
+      lmax = __builtin_fmaxf(lmax, v[k][e]);  // ignores NaN
+      nan = nan || (v[k][e] != v[k][e]);
+    }
+    const float M = wave_max_ignoring_nan(lmax);
+    const bool any_nan = __ballot(nan) != 0ull;
+    float sum = 0.0f;
+    if (M > -kInf) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float t = fast_exp2((v[k][e] - M) * kLog2e);
+        sum += (v[k][e] == v[k][e]) ? t : 0.0f;
+      }
+    }
+    sum = wave_sum_f32(sum);
+    if (lane == 0) {
+      const int64_t at = static_cast<int64_t>(row) * p.ns_stride + s;
+      p.slot_max[at] = any_nan ? __uint_as_float(0x7fc00000u) : M;
+      p.slot_sum[at] = sum;
+    }
+  }
+}
+
+// ---- pass 2 ---------------------------------------------------------------------------------------
+// LDS of pass 2 beyond the expf table.
+struct Pass2Shared {
+  BlockScratch sm;
+  float upto[kMaxSlots + 1];  // approximate running sum in front of every slot, in units of exp(-m)
+  uint32_t cls[kMaxSlots];    // per slot: kb_lo | kb_hi << 8 | kind << 16 | prepared-slot index << 19
+  uint32_t hist[kHistBuckets];
+  uint32_t list_count;        // candidates this workgroup has listed
+};
+
+// One wave, one slot: e[] are the lane's 8 entries; `cls` is the slot's entry of Pass2Shared::cls.
+template <bool TOPP>
+__device__ __forceinline__ void split_fold_slot(const SplitParams& p, int row, int s, const float (&e)[8], uint32_t cls,
+                                                float cut_lo, int V, uint64_t* region, Pass2Shared& sh) {
+  const int lane = threadIdx.x & 63;
+  const int64_t rec_at = static_cast<int64_t>(row) * p.ns_stride + s;
+  // ---- candidates of the top-p draw (sampler.cpp:137-143), by a cut that is safely below the
+  //      reference's once the exact normaliser is known
+  if (TOPP) {
+    uint32_t cmask = 0u;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) cmask |= (e[k] >= cut_lo && s * kSlot + lane * 8 + k < V) ? (1u << k) : 0u;
+    if (__ballot(cmask != 0u) != 0ull) {
+      const uint32_t mine = static_cast<uint32_t>(__popc(cmask));
+      const uint32_t incl = wave_scan_inclusive_u32(mine);
+      const uint32_t total = readlane_u32(incl, 63);
+      uint32_t base = 0u;
+      if (lane == 0) base = atomicAdd(&sh.list_count, total);
+      base = readlane_u32(base, 0);
+      uint32_t at = base + incl - mine;
+      const int first = s * kSlot + lane * 8;
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        if ((cmask >> k) & 1u) {
+          const uint32_t eb = __float_as_uint(e[k]);
+          atomicAdd(&sh.hist[hist_bucket(eb)], 1u);
+          if (at < static_cast<uint32_t>(p.list_region)) region[at] = (static_cast<uint64_t>(eb) << 32) | static_cast<uint32_t>(first + k);
+          ++at;
+        }
+      }
+    }
+  }
+  uint32_t bits[8];
+#pragma unroll
+  for (int k = 0; k < 8; ++k) bits[k] = __float_as_uint(e[k]);
+  // ---- the row's first slot is entered with the sum 0: worked out here, entry by entry
+  if (s == 0) {
+    float sum = 0.0f;
+    int found = -1;
+    wave_resolve<8>(sum, found, bits, lane * 8, V, __uint_as_float(0x7f800000u));
+    if (lane == 0) p.slot_rec[rec_at] = {kSlotExact << 8, __float_as_uint(sum), 0u, 0xffffffffu};
+    return;
+  }
+  // ---- every entry 0: no effect on any running sum
+  bool nonzero = false;
+#pragma unroll
+  for (int k = 0; k < 8; ++k) nonzero = nonzero || e[k] != 0.0f;
+  if (__ballot(nonzero) == 0ull) {
+    if (lane == 0) p.slot_rec[rec_at] = {kSlotZero << 8, 0u, 0u, 0xffffffffu};
+    return;
+  }
+  const uint32_t kb_lo = cls & 255u, kb_hi = (cls >> 8) & 255u;
+  const uint32_t kind = (cls >> 16) & 7u;
+  if (kind == kSlotStable) {
+    // ---- the sum stays in binade kb_lo throughout the slot
+    const float scale = __uint_as_float((277u - kb_lo) << 23);  // 2^(150 - kb)
+    FastAcc acc = {0.0f, 0.0f};
+#pragma unroll
+    for (int k = 0; k < 8; ++k) fast_fold(acc, e[k], scale);
+    ParityInc slot;
+    if (__ballot(acc.tie == 0.5f) == 0ull) {
+      const float inc = wave_sum_f32(acc.inc);
+      const uint32_t v = inc < 67108864.0f ? static_cast<uint32_t>(inc) : kSat;
+      slot.even = v;
+      slot.odd = v;
+    } else {
+      const ParityInc upto = wave_scan_inclusive(fold_run<8>(bits, __uint_as_float(kb_lo << 23)), lane);
+      slot.even = readlane_u32(upto.even, 63);
+      slot.odd = readlane_u32(upto.odd, 63);
+    }
+    if (lane == 0) p.slot_rec[rec_at] = {kb_lo | (kSlotStable << 8), slot.even, slot.odd, 0xffffffffu};
+    return;
+  }
+  if (kind == kSlotDual) {
+    // ---- the sum passes the slot inside binade kb_lo or inside kb_lo + 1
+    const float scale_a = __uint_as_float((277u - kb_lo) << 23), scale_b = __uint_as_float((276u - kb_lo) << 23);
+    FastAcc fa = {0.0f, 0.0f}, fb = {0.0f, 0.0f};
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      fast_fold(fa, e[k], scale_a);
+      fast_fold(fb, e[k], scale_b);
+    }
+    const bool ties = __ballot(fa.tie == 0.5f || fb.tie == 0.5f) != 0ull;
+    const float inc_a = wave_sum_f32(fa.inc), inc_b = wave_sum_f32(fb.inc);
+    if (lane == 0) {
+      if (ties) {  // (rare) the finish kernel works the slot out from the logits
+        p.slot_rec[rec_at] = {kb_lo | (kSlotSerial << 8), 0u, 0u, 0xffffffffu};
+      } else {
+        p.slot_rec[rec_at] = {kb_lo | (kSlotDual << 8), inc_a < 67108864.0f ? static_cast<uint32_t>(inc_a) : kSat,
+                              inc_b < 67108864.0f ? static_cast<uint32_t>(inc_b) : kSat, 0xffffffffu};
+      }
+    }
+    return;
+  }
+  // ---- to be resolved in order: keep the entries and the lanes' increments under both candidate ulps
+  const uint32_t idx = cls >> 19;
+  const uint32_t kb_a = kb_lo, kb_b = kb_hi > kb_lo ? kb_hi : kb_lo + 1u;
+  if (idx < static_cast<uint32_t>(p.prep_cap)) {
+    PrepSlot& ps = p.prep[static_cast<int64_t>(row) * p.prep_cap + idx];
+    float4* pe = reinterpret_cast<float4*>(ps.e + lane * 8);
+    pe[0] = {e[0], e[1], e[2], e[3]};
+    pe[1] = {e[4], e[5], e[6], e[7]};
+    const bool usable = kb_a >= 70u && kb_b <= 250u;
+    FastAcc fa = {0.0f, 0.0f}, fb = {0.0f, 0.0f};
+    if (usable) {
+      const float scale_a = __uint_as_float((277u - kb_a) << 23), scale_b = __uint_as_float((277u - kb_b) << 23);
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        fast_fold(fa, e[k], scale_a);
+        fast_fold(fb, e[k], scale_b);
+      }
+    }
+    const float kCap = 33554432.0f;  // 2^25
+    ps.pre_a[lane] = wave_scan_inclusive_u32(static_cast<uint32_t>(__builtin_fminf(fa.inc, kCap)));
+    ps.pre_b[lane] = wave_scan_inclusive_u32(static_cast<uint32_t>(__builtin_fminf(fb.inc, kCap)));
+    const uint64_t tie_a = __ballot(fa.tie == 0.5f), tie_b = __ballot(fb.tie == 0.5f);
+    if (lane == 0) {
+      ps.kb_a = kb_a;
+      ps.kb_b = kb_b;
+      ps.tie_a_lo = static_cast<uint32_t>(tie_a);
+      ps.tie_a_hi = static_cast<uint32_t>(tie_a >> 32);
+      ps.tie_b_lo = static_cast<uint32_t>(tie_b);
+      ps.tie_b_hi = static_cast<uint32_t>(tie_b >> 32);
+      ps.usable = usable ? 1u : 0u;
+      ps.pad = 0u;
+    }
+  }
+  if (lane == 0) {
+    p.slot_rec[rec_at] = {kb_a | (kSlotSerial << 8), 0u, 0u,
+                          idx < static_cast<uint32_t>(p.prep_cap) ? idx : 0xffffffffu};
+  }
+}
+
+// grid = (workgroups per row, rows); dynamic LDS: the expf table of bf16 rows (kLutCountWords floats).
+#ifndef ETS_PASS2_WAVES_PER_EU
+#define ETS_PASS2_WAVES_PER_EU 4
+#endif
+template <int DT, bool TOPP>
+__global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_kernel(SplitParams p) {
+  extern __shared__ __align__(16) float lut_mem[];
+  __shared__ Pass2Shared sh;
+  BlockScratch& sm = sh.sm;
+  const int row = p.row.row_map ? p.row.row_map[blockIdx.y] : blockIdx.y;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int V = p.row.vocab;
+  const int ns = p.ns;
+  const float inv = p.row.row_cfg ? p.row.row_cfg[row].inv_temperature : p.row.inv_temperature;
+  const float topp = p.row.row_cfg ? p.row.row_cfg[row].topp : p.row.topp;
+  const char* logits = static_cast<const char*>(p.row.logits) + static_cast<int64_t>(row) * p.row.row_stride * ElemSize<DT>::value;
+  const float* slot_max = p.slot_max + static_cast<int64_t>(row) * p.ns_stride;
+  const float* slot_sum = p.slot_sum + static_cast<int64_t>(row) * p.ns_stride;
+  const float kInf = __uint_as_float(0x7f800000u);
+  const float fill = inv < 0.0f ? kInf : -kInf;
+  uint64_t c0 = 0, c1 = 0, c2 = 0, c3 = 0;
+  if (p.timers) c0 = wall_clock64();
+  if (tid < 32) sm.exp2tab[tid] = kExp2Table[tid];
+  if (tid == 0) sh.list_count = 0u;
+  if (TOPP) {
+    for (int b = tid; b < kHistBuckets; b += kBlock) sh.hist[b] = 0u;
+  }
+
+  // ---- this workgroup's slots: wave w takes s_begin + w, s_begin + w + 16, ...; the first one's
+  //      entries are requested before anything else
+  const int per_wg = (((ns + static_cast<int>(gridDim.x) - 1) / static_cast<int>(gridDim.x)) + kWaves - 1) / kWaves * kWaves;
+  const int s_begin = blockIdx.x * per_wg;
+  const int s_end = min(ns, s_begin + per_wg);
+  float l[8];
+  int s_mine = s_begin + wave;
+  if (s_mine < s_end) load_slot_lane<DT>(logits, s_mine, lane, V, fill, l);
+
+  // ---- row maximum (sampler.cpp:191-197) from the slots' maxima
+  float m = -kInf;
+  bool any_nan = false;
+  float first_max = 0.0f, first_sum = 0.0f;  // the scan below starts with the same slots
+  for (int s = tid; s < ns; s += kBlock) {
+    const float v = slot_max[s];
+    if (s == tid) {
+      first_max = v;
+      first_sum = slot_sum[s];
+    }
+    any_nan = any_nan || (v != v);
+    m = __builtin_fmaxf(m, v);
+  }
+  m = wave_max_ignoring_nan(m);
+  const uint64_t nan_ballot = __ballot(any_nan);
+  if (lane == 0) {
+    sm.red_f[wave] = m;
+    sm.red_u[wave] = nan_ballot ? 1u : 0u;
+  }
+  __syncthreads();
+  m = sm.red_f[0];
+  uint32_t nan_any = sm.red_u[0];
+  for (int w = 1; w < kWaves; ++w) {
+    m = (sm.red_f[w] > m) ? sm.red_f[w] : m;
+    nan_any |= sm.red_u[w];
+  }
+  const float x0 = load_elem<DT>(logits, 0) * inv;
+  if (x0 != x0) m = x0;  // max_val starts at x[0]; nothing compares greater than NaN
+  const bool row_nan = nan_any != 0u || !(m > -kInf && m < kInf);
+  if (row_nan) {  // one NaN addend poisons the sum: the finish kernel needs nothing else
+    if (blockIdx.x == 0 && tid == 0) p.row_state[row] = {0u, m, 1u, 0.0f};
+    return;
+  }
+  __syncthreads();
+  if (p.timers) c1 = wall_clock64();
+
+  // ---- approximate running sums in front of every slot; from them, the binades the sequential
+  //      sum can be in at the two ends of each slot.  A slot that cannot be placed inside one
+  //      binade (or one of two neighbours) is resolved in order by the finish kernel and gets a
+  //      prepared-slot index.
+  float carry = 0.0f;
+  uint32_t serial_before = 0u;
+  for (int base = 0; base < ns; base += kBlock) {
+    const int s = base + tid;
+    float a = 0.0f;
+    if (s < ns) {
+      const float sum = base == 0 ? first_sum : slot_sum[s];
+      const float smax = base == 0 ? first_max : slot_max[s];
+      a = sum > 0.0f ? sum * fast_exp2((smax - m) * kLog2e) : 0.0f;
+    }
+    const float incl = wave_scan_inclusive_f32(a, lane);
+    if (lane == 63) sm.group_total[0][wave] = incl;
+    __syncthreads();
+    float before = carry, all = carry;
+    for (int w = 0; w < kWaves; ++w) {
+      if (w == wave) before = all;
+      all += sm.group_total[0][w];
+    }
+    const float a_out = before + incl;
+    const float a_in = before + lane_before_f32(incl);
+    if (s < ns) sh.upto[s + 1] = a_out;
+    carry = all;
+    const float lo = a_in * (1.0f - split_eps(s * kSlot));
+    const float hi = a_out * (1.0f + split_eps((s + 1) * kSlot));
+    const uint32_t kb_lo = __float_as_uint(lo > 0.0f ? lo : 0.0f) >> 23, kb_hi = __float_as_uint(hi) >> 23;
+    // inside one binade for certain; or inside one of two neighbours, the sums themselves
+    // pointing at no change inside the slot (kept as one increment per binade); or in order
+    uint32_t kind = kSlotSerial;
+    if (lo > 0.0f && kb_lo >= 70u && kb_hi <= 250u) {
+      if (kb_lo == kb_hi) {
+        kind = kSlotStable;
+      } else if (kb_hi == kb_lo + 1u && (__float_as_uint(a_in) >> 23) == (__float_as_uint(a_out) >> 23)) {
+        kind = kSlotDual;
+      }
+    }
+    const bool serial = s < ns && s > 0 && kind == kSlotSerial;  // (slot 0 is worked out in this kernel)
+    const uint64_t serial_ballot = __ballot(serial);
+    if (lane == 0) sm.red_u[wave] = static_cast<uint32_t>(__popcll(serial_ballot));
+    __syncthreads();
+    uint32_t rank = serial_before;
+    uint32_t chunk_total = 0u;
+    for (int w = 0; w < kWaves; ++w) {
+      if (w < wave) rank += sm.red_u[w];
+      chunk_total += sm.red_u[w];
+    }
+    rank += static_cast<uint32_t>(__popcll(serial_ballot & ((1ull << lane) - 1ull)));
+    if (s < ns) sh.cls[s] = (kb_lo & 255u) | ((kb_hi > 255u ? 255u : kb_hi) << 8) | (kind << 16) | (rank << 19);
+    serial_before += chunk_total;
+  }
+  const float a_total = carry;
+  if (blockIdx.x == 0 && tid == 0) p.row_state[row] = {serial_before, m, 0u, a_total};
+  if (p.timers) c2 = wall_clock64();
+
+  // ---- bf16 rows: expf by bit pattern
+  bool use_lut = false;
+  int lut_base1 = 0, lut_top = 0, lut_half = 0;
+  if constexpr (DT == kDtypeBFloat16) {
+    use_lut = build_exp_lut<false>(lut_mem, kLutCountWords, inv, m, sm.exp2tab, lut_base1, lut_top, lut_half);
+  }
+  __syncthreads();
+  if (p.timers) c3 = wall_clock64();
+  const LutAddr lut_addr = lut_addr_of(lut_mem, lut_base1, lut_top, lut_half);
+
+  const float cutoff = TOPP ? (1.0f - topp) / static_cast<float>(V - 1) : 0.0f;  // sampler.cpp:136
+  const float cut_lo = cutoff * a_total * (1.0f - split_eps(V)) * 0.999f;
+  uint64_t* region = p.list + (static_cast<int64_t>(row) * p.row_wgs + blockIdx.x) * p.list_region;
+
+  // ---- the slots, no barriers.  Two buffers take turns, so that the entries of the slot after this
+  //      one are on their way while this one is worked on (a copy from one buffer to the other
+  //      would have to wait for them).
+  const uint64_t* tab = sm.exp2tab;
+  auto work = [&](int s, const float (&in)[8]) {
+    float e[8];
+    bool done = false;
+    if constexpr (DT == kDtypeBFloat16) {
+      if (use_lut) {
+        uint32_t address[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+          const uint32_t fb = __float_as_uint(in[k]);
+          address[k] = lut_entry_address((fb >> 16) & 0x7fffu, fb >> 31, lut_addr);
+        }
+#pragma unroll
+        for (int k = 0; k < 8; ++k) e[k] = *(LdsF32)static_cast<uintptr_t>(address[k]);
+        done = true;
+      }
+    }
+    if (!done) {
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        const float d = __builtin_fmaxf(in[k] * inv - m, -104.0f);  // expf is 0 below ln(2^-150); the core gives 0 at -104 too
+        e[k] = expf_core(d, tab);
+      }
+    }
+    split_fold_slot<TOPP>(p, row, s, e, sh.cls[s], cut_lo, V, region, sh);
+  };
+  float l2[8];
+  while (s_mine < s_end) {
+    if (s_mine + kWaves < s_end) load_slot_lane<DT>(logits, s_mine + kWaves, lane, V, fill, l2);
+    work(s_mine, l);
+    s_mine += kWaves;
+    if (s_mine >= s_end) break;
+    if (s_mine + kWaves < s_end) load_slot_lane<DT>(logits, s_mine + kWaves, lane, V, fill, l);
+    work(s_mine, l2);
+    s_mine += kWaves;
+  }
+  if (TOPP) {
+    __syncthreads();
+    if (tid == 0) p.list_count[static_cast<int64_t>(row) * kMaxRowWorkgroups + blockIdx.x] = sh.list_count;
+    uint32_t* hist_out = p.hist + (static_cast<int64_t>(row) * p.row_wgs + blockIdx.x) * kHistBuckets;
+    for (int b = tid; b < kHistBuckets; b += kBlock) hist_out[b] = sh.hist[b];
+  }
+  if (p.timers && blockIdx.x == 0 && tid == 0) {
+    uint64_t* t = p.timers + static_cast<int64_t>(gridDim.y) * 8 + static_cast<int64_t>(blockIdx.y) * 4;
+    t[0] = c1 - c0;
+    t[1] = c2 - c1;
+    t[2] = c3 - c2;
+    t[3] = wall_clock64() - c3;
+  }
+}
+
+// ---- finish ---------------------------------------------------------------------------------------
+// One wave works a slot out from what pass 2 prepared: `bits` are the lane's 8 entries, pre_a /
+// pre_b the inclusive prefix sums over the lanes of their increments under the ulp of binade kb_a /
+// kb_b, tie_a / tie_b the lanes that hold a half-ulp tie under either.  While the running sum is in
+// one of the two binades, differences of prefix sums commit every lane in front of the first one
+// that holds a tie or behind which the sum would leave the binade; that lane adds its entries
+// natively, and the walk goes on behind it (with the other binade's sums if the sum has moved
+// there).  A sum in any other binade hands the remaining lanes to wave_resolve().  Returns with s
+// the exact sum behind the slot.
+__device__ __forceinline__ void resolve_lanes(float& s, const uint32_t (&bits)[8], uint32_t pre_a, uint32_t pre_b,
+                                              uint64_t tie_a, uint64_t tie_b, uint32_t kb_a, uint32_t kb_b, int first, int V,
+                                              uint32_t* inner = nullptr) {
+  const int lane = threadIdx.x & 63;
+  int cur = 0;
+  while (cur < 64) {
+    if (inner) ++*inner;
+    s = uniform_f32(s);
+    const SumState ss = sum_state(s);
+    const uint32_t K = static_cast<uint32_t>(ss.kb);
+    if (K != kb_a && K != kb_b) {
+      int found = -1;
+      wave_resolve<8>(s, found, bits, first, V, __uint_as_float(0x7f800000u), cur);
+      return;
+    }
+    const uint32_t pre = K == kb_a ? pre_a : pre_b;
+    const uint64_t tie = K == kb_a ? tie_a : tie_b;
+    const uint32_t done_before = cur > 0 ? readlane_u32(pre, cur - 1) : 0u;
+    const uint32_t room = (1u << 24) - ss.S;
+    const uint64_t over = __ballot(lane >= cur && pre - done_before >= room);
+    const uint64_t events = (tie & (~0ull << cur)) | over;
+    const int j = events ? __ffsll(static_cast<long long>(events)) - 1 : 64;
+    uint32_t S_j = ss.S;
+    if (j > cur) S_j += readlane_u32(pre, j - 1) - done_before;
+    if (j == 64) {
+      s = sum_value(S_j, ss.kb);
+      return;
+    }
+    float sj = 0.0f;
+    if (lane == j) {
+      sj = sum_value(S_j, ss.kb);
+#pragma unroll
+      for (int k = 0; k < 8; ++k) sj = sj + __uint_as_float(bits[k]);  // (entries past the row hold 0)
+    }
+    s = readlane_f32(sj, j);
+    cur = j + 1;
+  }
+}
+
+// The sequential softmax sum of one row (sampler.cpp:199-203) from the slot records, by ONE wave.
+// `recs` (ns records) and `prep` (the first `n_prep` prepared slots) are in LDS.  Sixty-four
+// records at a time, one per lane.  Under the binade K of the exact running sum a record is
+// "plain" when its increment is known whatever the sum's parity: a zero slot, a stable slot folded
+// for K without a tie, a dual slot folded for K or K - 1.  One prefix sum over the plain increments
+// (redone only when K changes) gives, for every run of plain records, the exact sum behind each of
+// them; a run is committed up to the first record that is not plain or behind which the sum
+// would leave binade K.  That record is then worked out exactly -- a stable slot with a tie takes
+// the increment for the sum's parity; a slot pass 2 prepared goes through resolve_lanes(); anything
+// else is redone entry by entry from the logits -- and the walk goes on behind it.  Every step
+// advances by at least one record.
+template <int DT>
+__device__ __forceinline__ float split_chain(const SlotRec* recs, int ns, const PrepSlot* prep, uint32_t n_prep,
+                                             const char* logits, int V, float inv, float m, const uint64_t* tab,
+                                             uint64_t* stats = nullptr) {
+  const int lane = threadIdx.x & 63;
+  const float kInf = __uint_as_float(0x7f800000u);
+  const float fill = inv < 0.0f ? kInf : -kInf;
+  float s = 0.0f;
+  uint64_t c_start = 0;
+  uint32_t n_iter = 0, n_generic = 0, n_prep_used = 0, n_tie = 0, n_inner = 0;
+  uint64_t c_prep = 0;
+  if (stats) c_start = wall_clock64();
+  for (int base = 0; base < ns; base += 64) {
+    SlotRec r = {kSlotZero << 8, 0u, 0u, 0xffffffffu};
+    if (base + lane < ns) r = recs[base + lane];
+    const uint32_t kind = (r.meta >> 8) & 7u, kb = r.meta & 255u;
+    int cur = 0;
+    if (base == 0 && readlane_u32(kind, 0) == kSlotExact) {  // pass 2 worked the first slot out
+      s = __uint_as_float(readlane_u32(r.even, 0));
+      cur = 1;
+    }
+    int K_scan = -1;
+    uint32_t incl = 0u;
+    uint64_t plain_mask = 0ull;
+    while (cur < 64) {
+      s = uniform_f32(s);
+      const SumState ss = sum_state(s);
+      const uint32_t K = static_cast<uint32_t>(ss.kb);
+      if (ss.kb != K_scan) {
+        const bool plain = kind == kSlotZero || (kind == kSlotStable && kb == K && r.even == r.odd) ||
+                           (kind == kSlotDual && (kb == K || kb + 1u == K));
+        const uint32_t inc = kind == kSlotZero ? 0u : ((kind == kSlotDual && kb != K) ? r.odd : r.even);
+        incl = wave_scan_inclusive_u32(plain ? inc : 0u);  // 64 values of at most 2^26 each
+        plain_mask = __ballot(plain);
+        K_scan = ss.kb;
+      }
+      const uint64_t from_cur = ~0ull << cur;
+      const uint64_t not_plain = ~plain_mask & from_cur;
+      const int jn = not_plain ? __ffsll(static_cast<long long>(not_plain)) - 1 : 64;
+      const uint32_t before = cur > 0 ? readlane_u32(incl, cur - 1) : 0u;
+      const uint32_t S_upto = ss.S + (incl - before);
+      const uint64_t over = __ballot(lane >= cur && lane < jn && S_upto >= (1u << 24));
+      const int jo = over ? __ffsll(static_cast<long long>(over)) - 1 : 64;
+      const int j = jn < jo ? jn : jo;
+      if (j > cur) s = sum_value(readlane_u32(S_upto, j - 1), ss.kb);
+      if (j == 64) break;
+      // ---- record base + j, exactly
+      const int slot = base + j;
+      const uint32_t kind_j = readlane_u32(kind, j), kb_j = readlane_u32(kb, j);
+      bool resolved = false;
+      if (j == jn && kind_j == kSlotStable && kb_j == K) {  // a tie inside: the increment follows the parity
+        const SumState sj = sum_state(s);
+        const uint32_t inc = (sj.S & 1u) ? readlane_u32(r.odd, j) : readlane_u32(r.even, j);
+        if (sj.S + inc < (1u << 24)) {
+          s = sum_value(sj.S + inc, sj.kb);
+          resolved = true;
+          ++n_tie;
+        }
+      }
+      if (!resolved) {
+        const uint32_t pi = readlane_u32(r.prep, j);
+        uint32_t bits[8];
+        if (j == jn && kind_j == kSlotSerial && pi < n_prep) {
+          const PrepSlot& ps = prep[pi];
+          const float4 e0 = *reinterpret_cast<const float4*>(ps.e + lane * 8);
+          const float4 e1 = *reinterpret_cast<const float4*>(ps.e + lane * 8 + 4);
+          bits[0] = __float_as_uint(e0.x); bits[1] = __float_as_uint(e0.y); bits[2] = __float_as_uint(e0.z); bits[3] = __float_as_uint(e0.w);
+          bits[4] = __float_as_uint(e1.x); bits[5] = __float_as_uint(e1.y); bits[6] = __float_as_uint(e1.z); bits[7] = __float_as_uint(e1.w);
+          if (ps.usable) {
+            const uint64_t tie_a = (static_cast<uint64_t>(ps.tie_a_hi) << 32) | ps.tie_a_lo;
+            const uint64_t tie_b = (static_cast<uint64_t>(ps.tie_b_hi) << 32) | ps.tie_b_lo;
+            const uint64_t cb = stats ? wall_clock64() : 0;
+            resolve_lanes(s, bits, ps.pre_a[lane], ps.pre_b[lane], tie_a, tie_b, ps.kb_a, ps.kb_b, slot * kSlot + lane * 8, V,
+                          stats ? &n_inner : nullptr);
+            if (stats) c_prep += wall_clock64() - cb;
+            ++n_prep_used;
+          } else {
+            int found = -1;
+            wave_resolve<8>(s, found, bits, slot * kSlot + lane * 8, V, kInf);
+            ++n_generic;
+          }
+        } else {
+          float l[8];
+          load_slot_lane<DT>(logits, slot, lane, V, fill, l);
+#pragma unroll
+          for (int k = 0; k < 8; ++k) bits[k] = __float_as_uint(expf_core(__builtin_fmaxf(l[k] * inv - m, -104.0f), tab));
+          int found = -1;
+          wave_resolve<8>(s, found, bits, slot * kSlot + lane * 8, V, kInf);
+          ++n_generic;
+        }
+      }
+      cur = j + 1;
+      ++n_iter;
+    }
+    if (stats && base == 0 && lane == 0) stats[5] = wall_clock64() - c_start;
+  }
+  if (stats && lane == 0) {
+    stats[4] = 0;
+    stats[6] = static_cast<uint64_t>(n_iter) | (static_cast<uint64_t>(n_generic) << 32);
+    stats[7] = static_cast<uint64_t>(n_prep_used) | (static_cast<uint64_t>(n_tie) << 16) | (static_cast<uint64_t>(n_inner) << 32) |
+               (c_prep << 48);
+  }
+  return uniform_f32(s);
+}
+
+// What the histogram says before the normaliser is known:
+//   b_sel      the candidates in buckets 0 .. b_sel safely carry more than topp of the mass
+//              whatever the exact normaliser turns out to be (-1: no such bucket);
+//   n_sel      how many they are;
+//   b_band     candidates in buckets below b_band reach the cutoff for certain;
+//   n_certain  how many they are.
+struct HistPlan {
+  int b_sel, n_sel, b_band, n_certain;
+};
+
+// Shared by the phases of the finish kernel.
+constexpr int kBandCap = 4096;
+struct FinishShared {
+  uint32_t count[kMaxRowWorkgroups];  // candidates per workgroup of pass 2
+  uint32_t offset[kMaxRowWorkgroups + 1];
+  uint32_t hist[kHistBuckets];        // the row's candidates by size
+  uint64_t sel[64];                   // the candidates of the largest buckets (exp bits << 32 | index)
+  uint32_t band[kBandCap];            // exp bits of the candidates that may or may not reach the cutoff
+  uint32_t sel_count, band_count;
+  uint32_t overflow;
+  HistPlan plan;
+};
+
+// By the whole workgroup, two buckets per lane; `plan_out` is LDS.  Ends with a barrier.
+__device__ __forceinline__ HistPlan split_plan(const uint32_t* hist, float a_total, float topp, float cutoff, int V,
+                                               HistPlan* plan_out, BlockScratch& sm) {
+  static_assert(kHistBuckets == 2 * kBlock, "two buckets per lane");
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const float target = (topp * 1.004f + 1e-6f) * a_total * (1.0f + split_eps(V));
+  const float cut_hi = cutoff * a_total * (1.0f + split_eps(V)) * 1.001f;
+  const int b_band = (cut_hi <= 1.0f && cut_hi > 0.0f) ? static_cast<int>(hist_bucket(__float_as_uint(cut_hi))) : 0;
+  const int b0 = 2 * tid;
+  const uint32_t c0 = hist[b0], c1 = hist[b0 + 1];
+  const float m0 = static_cast<float>(c0) * hist_edge(b0 + 1), m1 = static_cast<float>(c1) * hist_edge(b0 + 2);
+  const uint32_t certain = (b0 < b_band ? c0 : 0u) + (b0 + 1 < b_band ? c1 : 0u);
+  const uint32_t inclC = wave_scan_inclusive_u32(c0 + c1);
+  const float inclM = wave_scan_inclusive_f32(m0 + m1, lane);
+  const uint32_t certain_w = wave_sum_u32(certain);
+  if (lane == 63) {
+    sm.red_u[wave] = inclC;
+    sm.red_f[wave] = inclM;
+  }
+  if (lane == 0) sm.first_flag[wave] = static_cast<int>(certain_w);
+  if (tid == 0) *plan_out = {-1, 0, b_band, 0};
+  __syncthreads();
+  uint32_t cnt_before = 0u;
+  float mass_before = 0.0f;
+  int n_certain = 0;
+  for (int w = 0; w < kWaves; ++w) {
+    if (w < wave) {
+      cnt_before += sm.red_u[w];
+      mass_before += sm.red_f[w];
+    }
+    n_certain += sm.first_flag[w];
+  }
+  // the lane in which the mass reaches the target (at most one: `below` is what lies in front of it)
+  const float upto = mass_before + inclM;
+  const float below = upto - (m0 + m1);
+  if (upto >= target && !(below >= target)) {
+    const bool first = below + m0 >= target;
+    plan_out->b_sel = first ? b0 : b0 + 1;
+    plan_out->n_sel = static_cast<int>(cnt_before + inclC - (first ? c1 : 0u));
+  }
+  if (tid == 0) plan_out->n_certain = n_certain;
+  __syncthreads();
+  return *plan_out;
+}
+
+// grid = rows; dynamic LDS: the key buffer of the draw (p.row.lds_keys keys), which holds the
+// slot records and the prepared slots while the sum is composed.
+template <int DT>
+__global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
+  extern __shared__ __align__(16) uint64_t lds_keys[];
+  __shared__ BlockScratch sm;
+  __shared__ FinishShared fs;
+  const int row = p.row.row_map ? p.row.row_map[blockIdx.x] : blockIdx.x;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int V = p.row.vocab;
+  const int ns = p.ns;
+  const float inv = p.row.row_cfg ? p.row.row_cfg[row].inv_temperature : p.row.inv_temperature;
+  const float topp = p.row.row_cfg ? p.row.row_cfg[row].topp : p.row.topp;
+  const char* logits = static_cast<const char*>(p.row.logits) + static_cast<int64_t>(row) * p.row.row_stride * ElemSize<DT>::value;
+  const float kNaN = __uint_as_float(0x7fc00000u);
+  const RowState rs = p.row_state[row];
+  const float m = rs.m;
+  const bool row_nan = rs.nan != 0u;
+  const float cutoff = (1.0f - topp) / static_cast<float>(V - 1);  // sampler.cpp:136
+  uint64_t t0 = 0, t1 = 0, t2 = 0;
+  if (p.timers) t0 = wall_clock64();
+  if (tid < 32) sm.exp2tab[tid] = kExp2Table[tid];
+
+  float S = kNaN;
+  int n_listed = 0;
+  HistPlan plan = {-1, 0, 0, 0};
+  bool lists_ok = false;
+  if (!row_nan) {
+    // ---- how many candidates the workgroups of pass 2 listed; their histograms, added up
+    if (tid < 64) {
+      const uint32_t c = tid < p.row_wgs ? p.list_count[static_cast<int64_t>(row) * kMaxRowWorkgroups + tid] : 0u;
+      const uint32_t incl = wave_scan_inclusive_u32(c);
+      fs.count[tid] = c;
+      fs.offset[tid + 1] = incl;
+      if (tid == 0) fs.offset[0] = 0u;
+      const uint64_t over = __ballot(c > static_cast<uint32_t>(p.list_region));
+      if (tid == 0) {
+        fs.overflow = over ? 1u : 0u;
+        fs.sel_count = 0u;
+        fs.band_count = 0u;
+      }
+    }
+    {
+      // (four workgroups' counts are requested at a time: a loop of one load each would wait for each)
+      const uint32_t* hist_in = p.hist + static_cast<int64_t>(row) * p.row_wgs * kHistBuckets;
+      uint32_t c[kHistBuckets / kBlock];
+#pragma unroll
+      for (int q = 0; q < kHistBuckets / kBlock; ++q) c[q] = 0u;
+      for (int g = 0; g < p.row_wgs; g += 4) {
+        uint32_t v[4][kHistBuckets / kBlock];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          const int gk = g + k < p.row_wgs ? g + k : g;
+#pragma unroll
+          for (int q = 0; q < kHistBuckets / kBlock; ++q) v[k][q] = hist_in[gk * kHistBuckets + q * kBlock + tid];
+        }
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+#pragma unroll
+          for (int q = 0; q < kHistBuckets / kBlock; ++q) c[q] += g + k < p.row_wgs ? v[k][q] : 0u;
+        }
+      }
+#pragma unroll
+      for (int q = 0; q < kHistBuckets / kBlock; ++q) fs.hist[q * kBlock + tid] = c[q];
+    }
+    // ---- LDS: the records, then as many prepared slots as fit (one that does not is redone from
+    //      the logits when its turn comes)
+    const size_t lds_bytes = static_cast<size_t>(p.row.lds_keys) * sizeof(uint64_t);
+    const size_t rec_bytes = (static_cast<size_t>(ns) * sizeof(SlotRec) + 15) / 16 * 16;
+    uint32_t n_prep = rs.prep_count < static_cast<uint32_t>(p.prep_cap) ? rs.prep_count : static_cast<uint32_t>(p.prep_cap);
+    const uint32_t fit = static_cast<uint32_t>((lds_bytes - rec_bytes) / sizeof(PrepSlot));
+    n_prep = n_prep < fit ? n_prep : fit;
+    uint4* lds_vec = reinterpret_cast<uint4*>(lds_keys);
+    const uint4* rec_src = reinterpret_cast<const uint4*>(p.slot_rec + static_cast<int64_t>(row) * p.ns_stride);
+    for (int i = tid; i < ns; i += kBlock) lds_vec[i] = rec_src[i];
+    const uint4* prep_src = reinterpret_cast<const uint4*>(p.prep + static_cast<int64_t>(row) * p.prep_cap);
+    uint4* prep_dst = lds_vec + rec_bytes / 16;
+    const int prep_vecs = static_cast<int>(n_prep * (sizeof(PrepSlot) / 16));
+    for (int i = tid; i < prep_vecs; i += kBlock) prep_dst[i] = prep_src[i];
+    __syncthreads();
+    n_listed = static_cast<int>(fs.offset[p.row_wgs]);
+    lists_ok = fs.overflow == 0u;
+    plan = split_plan(fs.hist, rs.a_total, topp, cutoff, V, &fs.plan, sm);
+    if (p.timers) t1 = wall_clock64();
+    if (wave == 0) {
+      const float sum = split_chain<DT>(reinterpret_cast<const SlotRec*>(lds_keys), ns,
+                                        reinterpret_cast<const PrepSlot*>(prep_dst), n_prep, logits, V, inv, m, sm.exp2tab,
+                                        p.timers ? p.timers + static_cast<int64_t>(row) * 8 : nullptr);
+      if (lane == 0) sm.bc_sum = sum;
+    } else if (lists_ok && plan.b_sel >= 0 && plan.n_sel <= 64) {
+      // ---- the other waves, meanwhile: one pass over the listed candidates picks out those of the
+      //      largest buckets and those that may or may not reach the cutoff
+      for (int g = 0; g < p.row_wgs; ++g) {
+        const uint64_t* src = p.list + (static_cast<int64_t>(row) * p.row_wgs + g) * p.list_region;
+        const int c = static_cast<int>(fs.count[g]);
+        for (int j = (wave - 1) * 64 + lane; j < c; j += (kWaves - 1) * 64) {
+          const uint64_t ent = src[j];
+          const int b = static_cast<int>(hist_bucket(static_cast<uint32_t>(ent >> 32)));
+          if (b <= plan.b_sel) {
+            const uint32_t at = atomicAdd(&fs.sel_count, 1u);
+            if (at < 64u) fs.sel[at] = ent;
+          }
+          if (b >= plan.b_band) {
+            const uint32_t at = atomicAdd(&fs.band_count, 1u);
+            if (at < static_cast<uint32_t>(kBandCap)) fs.band[at] = static_cast<uint32_t>(ent >> 32);
+          }
+        }
+      }
+    }
+    __syncthreads();
+    S = sm.bc_sum;
+    if (p.timers) t2 = wall_clock64();
+  }
+
+  // ---- one coin per call (sampler.cpp:237, 210-220)
+  if (tid == 0) {
+    uint64_t st = p.row.rng[row];
+    st ^= st >> 12;
+    st ^= st << 25;
+    st ^= st >> 27;
+    p.row.rng[row] = st;
+    const uint32_t u = static_cast<uint32_t>((st * 0x2545F4914F6CDD1Dull) >> 32);
+    sm.red_f[0] = static_cast<float>(u >> 8) / 16777216.0f;
+  }
+  __syncthreads();  // (the records and prepared slots are dead from here on: the buffer becomes the key buffer)
+  const float coin = sm.red_f[0];
+  __syncthreads();
+
+  if (p.row.probs) {
+    float* probs = p.row.probs + static_cast<int64_t>(row) * V;
+    if (row_nan) {
+      for (int i = tid; i < V; i += kBlock) {
+        const float x = load_elem<DT>(logits, i) * inv;
+        probs[i] = expf_nonpositive(x - m, sm.exp2tab) / S;
+      }
+    } else {
+      const RowDivisor div = row_divisor(S);
+      for (int i = tid; i < V; i += kBlock) {
+        const float x = load_elem<DT>(logits, i) * inv;
+        probs[i] = div_row(expf_nonpositive(x - m, sm.exp2tab), div);
+      }
+    }
+  }
+
+  RowDebug dbg = {m, S, coin, 0.0f, 0.0f, 0, 0, 0};
+  int32_t token = -1;  // a NaN row keeps no candidate, where the reference reads probindex[-1]
+  int path = 0;
+  if (!row_nan) {
+    bool done = false;
+    const RowDivisor div = row_divisor(S);
+    if (lists_ok && n_listed == 0) {
+      done = true;  // no candidate (the reference reads probindex[-1] here)
+    } else if (lists_ok && plan.b_sel >= 0 && plan.n_sel >= 1 && plan.n_sel <= 64 &&
+               fs.sel_count == static_cast<uint32_t>(plan.n_sel) && fs.band_count <= static_cast<uint32_t>(kBandCap) &&
+               fs.band_count + static_cast<uint32_t>(plan.n_certain) == static_cast<uint32_t>(n_listed)) {
+      // ---- exact candidate count (sampler.cpp:137-143): the certain ones, plus those of the band
+      //      whose probability reaches the cutoff
+      const int n_band = static_cast<int>(fs.band_count);
+      uint32_t cnt = 0u;
+      for (int j = tid; j < n_band; j += kBlock) cnt += div_row(__uint_as_float(fs.band[j]), div) >= cutoff ? 1u : 0u;
+      cnt = wave_sum_u32(cnt);
+      if (lane == 0) sm.red_u[wave] = cnt;
+      // ---- the short selection: every selected entry must be a candidate
+      const int n_sel = plan.n_sel;
+      if (tid < 64) {
+        bool is_in = true;
+        uint64_t key = ~0ull;
+        if (tid < n_sel) {
+          const uint64_t ent = fs.sel[tid];
+          const float pj = div_row(__uint_as_float(static_cast<uint32_t>(ent >> 32)), div);
+          is_in = pj >= cutoff;
+          key = cand_key(pj, static_cast<int>(static_cast<uint32_t>(ent)));
+        }
+        lds_keys[tid] = key;
+        const uint64_t out = __ballot(!is_in);
+        if (tid == 0) sm.flag = out ? 0 : 1;
+      }
+      __syncthreads();
+      uint32_t n0 = static_cast<uint32_t>(plan.n_certain);
+      for (int w = 0; w < kWaves; ++w) n0 += sm.red_u[w];
+      const bool ok = sm.flag != 0;
+      __syncthreads();
+      if (n0 == 0u) {
+        dbg.n_candidates = 0;
+        done = true;
+      } else if (ok) {
+        // entries outside the selection have exp up to the edge of the next bucket
+        const float p_floor = (n_sel == static_cast<int>(n0)) ? -1.0f : div_row(hist_edge(plan.b_sel + 1), div);
+        dbg.n_candidates = static_cast<int>(n0);
+        done = draw_small_wave((LdsKeys)lds_keys, n_sel, static_cast<int>(n0), topp, coin, dbg, token, sm, 0, p_floor) != -2;
+        path = 1;
+      }
+    }
+    if (!done && lists_ok && n_listed <= p.row.lds_keys - kBlock) {
+      // ---- a longer nucleus: the whole list goes to LDS, selection by probability, sort, walks
+      for (int g = wave; g < p.row_wgs; g += kWaves) {
+        const uint64_t* src = p.list + (static_cast<int64_t>(row) * p.row_wgs + g) * p.list_region;
+        uint64_t* dst = lds_keys + kBlock + fs.offset[g];
+        const int c = static_cast<int>(fs.count[g]);
+        for (int j = lane; j < c; j += 64) dst[j] = src[j];
+      }
+      __syncthreads();
+      done = draw_topp_listed(nullptr, lds_keys + kBlock, p.row.lds_keys - kBlock, kBlock, n_listed, S, cutoff, topp, coin,
+                              lds_keys, p.row.lds_keys, dbg, token, sm);
+      path = 2;
+    }
+    if (!done) {
+      uint64_t* scratch = p.row.scratch + static_cast<int64_t>(row) * p.row.scratch_stride;
+      token = draw_general<DT>(logits, V, inv, m, S, false, 0, topp, cutoff, coin, scratch, p.row.scratch_stride, lds_keys,
+                               p.row.lds_keys, dbg, sm);
+      path = 3;
+    }
+  }
+  if (tid == 0) {
+    p.row.tokens[row] = token;
+    if (p.row.debug) p.row.debug[row] = dbg;
+    if (p.timers) {
+      uint64_t* t = p.timers + static_cast<int64_t>(row) * 8;
+      t[0] = t1 - t0;
+      t[1] = t2 - t1;
+      t[2] = wall_clock64() - t2;
+      t[3] = static_cast<uint64_t>(n_listed) | (static_cast<uint64_t>(rs.prep_count) << 32);
+      t[4] = static_cast<uint64_t>(path) | (static_cast<uint64_t>(plan.n_sel) << 8) | (static_cast<uint64_t>(fs.band_count) << 32);
+    }
+  }
+}
+
+}  // namespace ets

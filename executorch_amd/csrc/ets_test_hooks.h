@@ -18,6 +18,12 @@ ETS_API ets_status ets_test_expf(const float* d_x, float* d_y, int64_t n, void* 
 ETS_API ets_status ets_test_seq_sum(const float* d_a, int32_t n, float s0, float threshold, float* d_sum,
                                     int32_t* d_stop, void* hip_stream);
 
+/* Phase clocks of the finish kernel of the several-workgroups-per-row path, four 64-bit words per
+ * row (staging, ordered sum, draw, in ticks of the 100 MHz wall clock; then the candidate and
+ * prepared-slot counts), filled when ETS_SPLIT_TIMERS was set before the handle's first stochastic
+ * call.  HOST pointer. */
+ETS_API ets_status ets_test_split_timers(ets_sampler* s, uint64_t* out, int32_t rows);
+
 #ifdef __cplusplus
 }
 #endif

@@ -100,6 +100,10 @@ class Sampler:
     def set_topp(self, topp: float) -> None:
         self._check(_capi.lib().ets_sampler_set_topp(self._h, topp))
 
+    def set_row_split(self, mode: int) -> None:
+        """0 = automatic, 1 = several workgroups per row wherever that path applies, 2 = never."""
+        self._check(_capi.lib().ets_sampler_set_row_split(self._h, mode))
+
     # ---- sampler.cpp:222-251
     def sample(self, logits, dtype: int | None = None) -> int:
         """One row of ``vocab_size`` logits in host memory (numpy array or CPU tensor)."""

@@ -99,6 +99,18 @@ ETS_API ets_status ets_sampler_set_topk(ets_sampler* s, int32_t topk);
  * handle can serve requests with different nucleus sizes. */
 ETS_API ets_status ets_sampler_set_topp(ets_sampler* s, float topp);
 
+/* No counterpart (the reference is one scalar loop).  How the stochastic path uses the GPU:
+ *   ETS_ROW_SPLIT_AUTO  rows of 8192 entries and more take three launches in which many
+ *                       workgroups share a row (16-byte aligned rows, top-p draw); smaller ones,
+ *                       other draws and unaligned rows take one launch, one workgroup per row;
+ *   ETS_ROW_SPLIT_ON    the three launches wherever they apply, whatever the vocabulary size;
+ *   ETS_ROW_SPLIT_OFF   always one workgroup per row.
+ * The tokens, coin states and debug records are the same on every setting. */
+#define ETS_ROW_SPLIT_AUTO 0
+#define ETS_ROW_SPLIT_ON 1
+#define ETS_ROW_SPLIT_OFF 2
+ETS_API ets_status ets_sampler_set_row_split(ets_sampler* s, int32_t mode);
+
 /* Sampler::sample<T>(T* logits)  -- sampler.cpp:222-251, instantiations :253-258.
  * `logits` is a HOST pointer to vocab_size elements of `dtype`; the row is copied to the
  * device, sampled there and the token copied back (synchronous).  Consumes row 0's coin. */

@@ -1,0 +1,112 @@
+"""The path that spreads a row over several workgroups (three launches: slot maxima and approximate
+sums; exact exponentials folded per slot under the predicted binade; one workgroup per row that
+composes, verifies and draws) against the CPU oracle and against the one-workgroup-per-row kernel.
+Bit-exact: tokens, coin states, the sequential softmax sum, the nucleus mass and positions."""
+import numpy as np
+import pytest
+import torch
+
+import executorch_amd as ea
+from executorch_amd import workloads as W
+import test_gpu_sampler_parity as parity
+from util import f32_bits, to_device
+
+pytestmark = pytest.mark.gpu
+
+SPLIT_ON, SPLIT_OFF = 1, 2
+
+
+@pytest.fixture
+def forced_split(monkeypatch):
+    monkeypatch.setenv("ETS_ROW_SPLIT", "1")  # the default of ets_sampler_set_row_split() for new handles
+
+
+@pytest.mark.parametrize("name,rows,steps", [("cfg1", 1, 20), ("cfg2", 64, 2), ("cfg3", 4, 1), ("cfg5", 8, 1)])
+def test_workloads_bit_exact_when_split(oracle, dev, forced_split, name, rows, steps):
+    parity.run_case(oracle, dev, W.WORKLOADS[name], rows, steps, probs=(name == "cfg2"))
+
+
+def test_small_and_ragged_vocabularies_when_split(oracle, dev, forced_split):
+    parity.test_small_and_ragged_vocabularies(oracle, dev)
+
+
+@pytest.mark.parametrize("topp,temperature", [(0.5, 0.3), (0.99, 1.0), (0.05, 1.0), (0.9, 0.05), (0.9, 5.0)])
+def test_parameter_sweep_when_split(oracle, dev, forced_split, topp, temperature):
+    for name, rows in (("cfg1", 2), ("cfg2", 8)):
+        parity.run_case(oracle, dev, W.WORKLOADS[name], rows, 1, topp=topp, temperature=temperature)
+
+
+def sample_both(x, dtype, dev, V, temperature, topp, seed):
+    rows = x.shape[0]
+    res = []
+    for mode in (SPLIT_ON, SPLIT_OFF):
+        s = ea.Sampler(V, temperature, topp, seed, max_batch=rows)
+        s.set_row_split(mode)
+        dbg = torch.zeros((rows, 8), dtype=torch.int32, device=dev)
+        tok = s.sample_batch(to_device(x, dtype, dev), debug_out=dbg).cpu().numpy()
+        res.append((tok, ea.debug_records(dbg).copy(), s.get_rng_states(rows)))
+    return res
+
+
+def assert_same(a, b):
+    assert np.array_equal(a[0], b[0])
+    assert np.array_equal(a[2], b[2])
+    for field in ("max_val", "sum", "coin", "cumulative", "r"):
+        assert np.array_equal(f32_bits(a[1][field]), f32_bits(b[1][field])), field
+    for field in ("n_candidates", "last_idx", "position"):
+        assert np.array_equal(a[1][field], b[1][field]), field
+
+
+@pytest.mark.parametrize("dtype", [W.DTYPE_FLOAT, W.DTYPE_HALF, W.DTYPE_BFLOAT16])
+def test_masked_and_degenerate_rows_match_the_one_workgroup_kernel(oracle, dev, dtype):
+    """Rows with whole slots of -inf (token masks), a leading masked stretch (the sum stays 0 for
+    thousands of entries), one surviving entry, NaN and +inf entries, equal logits (every entry ties),
+    and a vocabulary that ends inside a slot."""
+    rng = np.random.default_rng(5)
+    V = 20000 + 37
+    base = (rng.standard_normal((9, V)) * 1.5).astype(np.float32)
+    base[0, :6000] = -np.inf
+    base[1, 3000:15000] = -np.inf
+    base[2, :] = -np.inf
+    base[2, 12345] = 0.5
+    base[3, 777] = np.nan
+    base[4, 778] = np.inf
+    base[5, :] = 0.25
+    base[6, ::2] = -np.inf
+    base[7, :] = -np.inf
+    base[8, :512] = 30.0  # the sum leaves many binades inside the first slots
+    x = W.to_storage(base, dtype)
+    for topp in (0.9, 0.3):
+        on, off = sample_both(x, dtype, dev, V, 0.7, topp, 77)
+        assert_same(on, off)
+        states = (np.uint64(77) + np.arange(9, dtype=np.uint64)).astype(np.uint64)
+        want, _ = oracle.sample_rows(x, dtype, oracle.inv_temperature(0.7), topp, 0, states, mode=oracle.MODE_UPCAST,
+                                     tie=oracle.TIE_STABLE)
+        assert np.array_equal(on[0], want)
+        assert np.array_equal(on[2], states)
+
+
+def test_row_pitch_and_row_map_when_split(oracle, dev):
+    """Rows at a pitch larger than the vocabulary (16-byte aligned, so the split path applies), and
+    per-row parameters, which reach the kernels through a row map."""
+    rng = np.random.default_rng(8)
+    V, B, pitch = 50000, 6, 50048
+    x = (rng.standard_normal((B, V)) * 2.0).astype(np.float32)
+    buf = torch.zeros((B, pitch), dtype=torch.float32, device=dev)
+    buf[:, :V] = torch.from_numpy(x).to(dev)
+    s = ea.Sampler(V, 0.8, 0.9, 300, max_batch=B)
+    s.set_row_split(SPLIT_ON)
+    got = s.sample_batch(buf[:, :V]).cpu().numpy()
+    states = (np.uint64(300) + np.arange(B, dtype=np.uint64)).astype(np.uint64)
+    want, _ = oracle.sample_rows(x, W.DTYPE_FLOAT, oracle.inv_temperature(0.8), 0.9, 0, states, mode=oracle.MODE_UPCAST,
+                                 tie=oracle.TIE_STABLE)
+    assert np.array_equal(got, want)
+    # per-row parameters: top-p rows of different temperatures mixed with greedy and multinomial rows
+    cfgs = [(0.8, 0.9, 0, 0), (0.0, 0.9, 0, 0), (0.5, 0.7, 0, 0), (1.0, 1.0, 0, 0), (1.3, 0.95, 0, 0), (0.8, 0.9, 5, 0)]
+    s2 = ea.Sampler(V, 0.8, 0.9, 400, max_batch=B)
+    s2.set_row_split(SPLIT_ON)
+    got2 = s2.sample_batch_configs(buf[:, :V], cfgs).cpu().numpy()
+    for b, (t, p, k, _) in enumerate(cfgs):
+        o = oracle.Sampler(V, t, p, 400 + b, mode=oracle.MODE_UPCAST, tie=oracle.TIE_STABLE)
+        o.set_topk(k)
+        assert got2[b] == o.sample(x[b].copy(), W.DTYPE_FLOAT), b
