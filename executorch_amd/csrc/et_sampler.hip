@@ -46,9 +46,11 @@ struct ets_sampler {
   int32_t* d_token = nullptr;      // staging for one token
   // work buffers of the path that spreads a row over several workgroups (ets_split.h): one
   // allocation, made on first use
+  size_t split_row_wgs = 0;  // (row, workgroup) pairs of the largest launch
   int split_mode = 0;  // ETS_ROW_SPLIT_AUTO
   int num_cus = 0;
   void* d_split = nullptr;
+  void* d_phist = nullptr;  // pattern histograms of 16-bit rows, allocated on their first use
   ets::SplitParams split = {};
   // per-row sampling parameters of ets_sampler_sample_batch_configs(): pinned host staging, its
   // device copy, and the event that says the last upload has left the staging buffer
@@ -327,6 +329,19 @@ ets_status ensure_split(ets_sampler* s) {
   sp.hist = reinterpret_cast<uint32_t*>(base + o_hist);
   sp.list = reinterpret_cast<uint64_t*>(base + o_list);
   sp.timers = std::getenv("ETS_SPLIT_TIMERS") ? reinterpret_cast<uint64_t*>(base + o_timers) : nullptr;
+  s->split_row_wgs = row_wgs;
+  return ETS_OK;
+}
+
+// Words of packed 16-bit counters per (row, workgroup) of the pattern histogram: what fits in
+// pass 2's LDS next to the expf table.
+constexpr int kPhistWordsHalf = 24576, kPhistWordsBFloat16 = 8192;
+
+ets_status ensure_phist(ets_sampler* s) {
+  if (s->d_phist) return ETS_OK;
+  const size_t bytes = round_up(s->split_row_wgs * kPhistWordsHalf * sizeof(uint32_t), 256);
+  ETS_HIP(s, hipMalloc(&s->d_phist, bytes));
+  s->split.phist = static_cast<uint32_t*>(s->d_phist);
   return ETS_OK;
 }
 
@@ -343,15 +358,21 @@ template <int DT>
 ets_status launch_split(ets_sampler* s, const ets::RowParams& p, int32_t rows, hipStream_t stream) {
   ets_status st = ensure_split(s);
   if (st != ETS_OK) return st;
+  constexpr bool k16 = DT == ets::kDtypeBFloat16 || DT == ets::kDtypeHalf;
+  if (k16) {
+    st = ensure_phist(s);
+    if (st != ETS_OK) return st;
+  }
   ets::SplitParams sp = s->split;
   sp.row = p;
+  sp.phist_words = DT == ets::kDtypeBFloat16 ? kPhistWordsBFloat16 : (DT == ets::kDtypeHalf ? kPhistWordsHalf : 0);
   sp.row_wgs = pass2_workgroups(s, rows, sp.ns);
   sp.list_region = list_region(sp.ns, sp.row_wgs);
   const int per_block = (ets::kPass1Block / 64) * ets::kPass1SlotsPerWave;
   hipLaunchKernelGGL((ets::split_pass1_kernel<DT>), dim3((sp.ns + per_block - 1) / per_block, rows), dim3(ets::kPass1Block), 0,
                      stream, sp);
   ETS_HIP(s, hipGetLastError());
-  const size_t lut_bytes = DT == ets::kDtypeBFloat16 ? sizeof(float) * ets::kLutCountWords : 0;
+  const size_t lut_bytes = (DT == ets::kDtypeBFloat16 ? sizeof(float) * ets::kLutCountWords : 0) + sizeof(uint32_t) * sp.phist_words;
   static std::atomic<size_t> set_bytes2[kMaxDevices];
   st = allow_dynamic_lds(s, reinterpret_cast<const void*>(&ets::split_pass2_kernel<DT, true>), lut_bytes, set_bytes2);
   if (st != ETS_OK) return st;
@@ -597,6 +618,7 @@ ets_status ets_sampler_destroy(ets_sampler* s) {
     (void)hipFree(s->d_rng);
     (void)hipFree(s->d_scratch);
     (void)hipFree(s->d_split);
+    (void)hipFree(s->d_phist);
     (void)hipFree(s->d_partials);
     (void)hipFree(s->d_row);
     (void)hipFree(s->d_token);

@@ -63,6 +63,10 @@ struct RowState {
   float m;              // row maximum of x (NaN when x[0] is NaN, like the reference's loop)
   uint32_t nan;         // some expf(x - m) is NaN
   float a_total;        // approximate softmax sum, in units of exp(-m)
+  int32_t key_cut;      // 16-bit rows: order key of the first bin of the pattern histogram,
+  int32_t n_bins;       //   how many bins it has (0: no pattern histogram)
+  int32_t mag_min;      //   and the KeyMap's first magnitude with a key of its own
+  uint32_t pad;
 };
 
 constexpr int kMaxRowWorkgroups = 64;  // workgroups of pass 2 per row
@@ -81,6 +85,42 @@ __device__ __forceinline__ float hist_edge(int b) {
   return b >= kHistBuckets ? 0.0f : __uint_as_float(0x3F800000u - (static_cast<uint32_t>(b) << 17));
 }
 
+// Order key of a 16-bit float pattern (fp16 or bf16): a larger value has a larger key.  Magnitudes
+// below `mag_min` are so small that x = logit * inv_temperature vanishes against the row maximum
+// (|x| under an eighth of its ulp), so all of them give the same exp as a logit of 0: they share one
+// key per sign, which keeps the range of keys of a row short.  -0 sits just below +0.
+struct KeyMap {
+  int mag_min;  // first magnitude pattern with a key of its own
+  int key_cut;  // key of the pattern histogram's first bin
+  int n_bins;   // 0: no pattern histogram
+};
+__device__ __forceinline__ int pattern_key(uint32_t pattern16, int mag_min) {
+  const int mag = static_cast<int>(pattern16 & 0x7fffu);
+  const int cm = mag < mag_min ? 0 : mag - mag_min + 1;
+  return (pattern16 & 0x8000u) ? 0x7fff - cm : 0x8000 + cm;
+}
+// A pattern with that key (the zero of its sign for the shared keys).
+__device__ __forceinline__ uint32_t key_pattern(int key, int mag_min) {
+  const int cm = key >= 0x8000 ? key - 0x8000 : 0x7fff - key;
+  const uint32_t mag = cm == 0 ? 0u : static_cast<uint32_t>(cm - 1 + mag_min);
+  return (key >= 0x8000 ? 0u : 0x8000u) | (mag & 0x7fffu);
+}
+template <int DT>
+__device__ __forceinline__ float pattern_value(uint32_t pattern16) {
+  return DT == kDtypeBFloat16 ? __uint_as_float(pattern16 << 16) : half_bits_to_float(pattern16);
+}
+// The 16-bit pattern of a value that was converted from one (exactly).
+template <int DT>
+__device__ __forceinline__ uint32_t value_pattern(float v) {
+  if (DT == kDtypeBFloat16) return __float_as_uint(v) >> 16;
+  union {
+    _Float16 f;
+    uint16_t u;
+  } cvt;
+  cvt.f = static_cast<_Float16>(v);
+  return cvt.u;
+}
+
 struct SplitParams {
   RowParams row;        // what the one-workgroup kernel takes
   float* slot_max;      // [rows, ns_stride]
@@ -92,6 +132,9 @@ struct SplitParams {
                         //   candidates: every workgroup of pass 2 fills its own region
   uint32_t* list_count; // [rows, kMaxRowWorkgroups] candidates each workgroup found (may exceed its region)
   uint32_t* hist;       // [rows, row_wgs, kHistBuckets] the same candidates by size
+  uint32_t* phist;      // [rows, row_wgs, phist_words] 16-bit rows: entries per bit pattern, two 16-bit
+                        //   counters per word, from order key RowState::key_cut upwards
+  int32_t phist_words;  // words per (row, workgroup) region; 0 disables the pattern histogram
   uint64_t* timers;     // phase clocks (profiling), or null
   int32_t list_region;  // entries per region
   int32_t row_wgs;      // workgroups of pass 2 per row
@@ -180,9 +223,10 @@ struct Pass2Shared {
 };
 
 // One wave, one slot: e[] are the lane's 8 entries; `cls` is the slot's entry of Pass2Shared::cls.
-template <bool TOPP>
-__device__ __forceinline__ void split_fold_slot(const SplitParams& p, int row, int s, const float (&e)[8], uint32_t cls,
-                                                float cut_lo, int V, uint64_t* region, Pass2Shared& sh) {
+template <bool TOPP, int DT>
+__device__ __forceinline__ void split_fold_slot(const SplitParams& p, int row, int s, const float (&e)[8],
+                                                const float (&logit)[8], uint32_t cls, float cut_lo, int V, uint64_t* region,
+                                                Pass2Shared& sh, const KeyMap& km, uint32_t* ph) {
   const int lane = threadIdx.x & 63;
   const int64_t rec_at = static_cast<int64_t>(row) * p.ns_stride + s;
   // ---- candidates of the top-p draw (sampler.cpp:137-143), by a cut that is safely below the
@@ -205,6 +249,12 @@ __device__ __forceinline__ void split_fold_slot(const SplitParams& p, int row, i
         if ((cmask >> k) & 1u) {
           const uint32_t eb = __float_as_uint(e[k]);
           atomicAdd(&sh.hist[hist_bucket(eb)], 1u);
+          if constexpr (DT == kDtypeBFloat16 || DT == kDtypeHalf) {
+            // 16-bit rows: the same candidates per bit pattern (one outside the range of bins is
+            // missed there, which the totals give away)
+            const int bin = pattern_key(value_pattern<DT>(logit[k]), km.mag_min) - km.key_cut;
+            if (bin >= 0 && bin < km.n_bins) atomicAdd(&ph[bin >> 1], 1u << ((bin & 1) << 4));
+          }
           if (at < static_cast<uint32_t>(p.list_region)) region[at] = (static_cast<uint64_t>(eb) << 32) | static_cast<uint32_t>(first + k);
           ++at;
         }
@@ -321,6 +371,7 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
   extern __shared__ __align__(16) float lut_mem[];
   __shared__ Pass2Shared sh;
   BlockScratch& sm = sh.sm;
+  const int lrow = blockIdx.y;  // row of this launch: indexes the buffers whose layout depends on the launch
   const int row = p.row.row_map ? p.row.row_map[blockIdx.y] : blockIdx.y;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -338,8 +389,14 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
   if (p.timers) c0 = wall_clock64();
   if (tid < 32) sm.exp2tab[tid] = kExp2Table[tid];
   if (tid == 0) sh.list_count = 0u;
+  // 16-bit rows: entries per bit pattern, behind the expf table
+  constexpr bool kPatterns = TOPP && (DT == kDtypeBFloat16 || DT == kDtypeHalf);
+  uint32_t* ph = reinterpret_cast<uint32_t*>(lut_mem + (DT == kDtypeBFloat16 ? kLutCountWords : 0));
   if (TOPP) {
     for (int b = tid; b < kHistBuckets; b += kBlock) sh.hist[b] = 0u;
+    if (kPatterns) {
+      for (int b = tid; b < p.phist_words; b += kBlock) ph[b] = 0u;
+    }
   }
 
   // ---- this workgroup's slots: wave w takes s_begin + w, s_begin + w + 16, ...; the first one's
@@ -381,7 +438,7 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
   if (x0 != x0) m = x0;  // max_val starts at x[0]; nothing compares greater than NaN
   const bool row_nan = nan_any != 0u || !(m > -kInf && m < kInf);
   if (row_nan) {  // one NaN addend poisons the sum: the finish kernel needs nothing else
-    if (blockIdx.x == 0 && tid == 0) p.row_state[row] = {0u, m, 1u, 0.0f};
+    if (blockIdx.x == 0 && tid == 0) p.row_state[row] = {0u, m, 1u, 0.0f, 0, 0, 0, 0u};
     return;
   }
   __syncthreads();
@@ -441,7 +498,7 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
     serial_before += chunk_total;
   }
   const float a_total = carry;
-  if (blockIdx.x == 0 && tid == 0) p.row_state[row] = {serial_before, m, 0u, a_total};
+  if (blockIdx.x == 0 && tid == 0) p.row_state[row] = {serial_before, m, 0u, a_total, 0, 0, 0, 0u};
   if (p.timers) c2 = wall_clock64();
 
   // ---- bf16 rows: expf by bit pattern
@@ -456,7 +513,35 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
 
   const float cutoff = TOPP ? (1.0f - topp) / static_cast<float>(V - 1) : 0.0f;  // sampler.cpp:136
   const float cut_lo = cutoff * a_total * (1.0f - split_eps(V)) * 0.999f;
-  uint64_t* region = p.list + (static_cast<int64_t>(row) * p.row_wgs + blockIdx.x) * p.list_region;
+  uint64_t* region = p.list + (static_cast<int64_t>(lrow) * p.row_wgs + blockIdx.x) * p.list_region;
+  // ---- the pattern histogram's range of order keys: from safely below the smallest logit whose exp
+  //      can reach cut_lo up to the row's largest logit (every workgroup of the row arrives at the
+  //      same two numbers).  Too many bins for the LDS set aside: no pattern histogram.
+  KeyMap km = {0, 0, 0};
+  if (kPatterns && p.phist_words > 0 && inv > 0.0f && inv < kInf && cut_lo > 0.0f && (__float_as_uint(inv) >> 23) != 0u) {
+    // magnitudes below 2^(em - ei - 27) vanish against m (em, ei: biased exponents of |m| and inv)
+    const uint32_t mb = __float_as_uint(__builtin_fabsf(m));
+    const int em = (mb >> 23) ? static_cast<int>(mb >> 23) : 1;
+    const int et = em - static_cast<int>(__float_as_uint(inv) >> 23) - 27 + 127;
+    if (et >= 1) km.mag_min = static_cast<int>(value_pattern<DT>(__uint_as_float(static_cast<uint32_t>(et > 254 ? 254 : et) << 23)) & 0x7fffu);
+    const float x_cut = m + (__logf(cut_lo) - 0.01f);
+    const float l_cut = x_cut / inv;
+    const float l_top = m / inv;
+    const float l_lo = l_cut - __builtin_fabsf(l_cut) * 1e-5f, l_hi = l_top + __builtin_fabsf(l_top) * 1e-5f;
+    constexpr float kMaxFinite = DT == kDtypeBFloat16 ? 3.3895313892515355e38f : 65504.0f;
+    const float l_lo_c = __builtin_fminf(__builtin_fmaxf(l_lo, -kMaxFinite), kMaxFinite);
+    const float l_hi_c = __builtin_fminf(__builtin_fmaxf(l_hi, -kMaxFinite), kMaxFinite);
+    km.key_cut = pattern_key(value_pattern<DT>(l_lo_c), km.mag_min) - 2;
+    const int key_top = pattern_key(value_pattern<DT>(l_hi_c), km.mag_min) + 2;
+    if (km.key_cut < 0) km.key_cut = 0;
+    km.n_bins = key_top - km.key_cut + 1;
+    if (km.n_bins < 1 || km.n_bins > 2 * p.phist_words) km.n_bins = 0;
+  }
+  if (kPatterns && blockIdx.x == 0 && tid == 0) {
+    p.row_state[row].key_cut = km.key_cut;
+    p.row_state[row].n_bins = km.n_bins;
+    p.row_state[row].mag_min = km.mag_min;
+  }
 
   // ---- the slots, no barriers.  Two buffers take turns, so that the entries of the slot after this
   //      one are on their way while this one is worked on (a copy from one buffer to the other
@@ -485,7 +570,7 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
         e[k] = expf_core(d, tab);
       }
     }
-    split_fold_slot<TOPP>(p, row, s, e, sh.cls[s], cut_lo, V, region, sh);
+    split_fold_slot<TOPP, DT>(p, row, s, e, in, sh.cls[s], cut_lo, V, region, sh, km, ph);
   };
   float l2[8];
   while (s_mine < s_end) {
@@ -499,9 +584,13 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
   }
   if (TOPP) {
     __syncthreads();
-    if (tid == 0) p.list_count[static_cast<int64_t>(row) * kMaxRowWorkgroups + blockIdx.x] = sh.list_count;
-    uint32_t* hist_out = p.hist + (static_cast<int64_t>(row) * p.row_wgs + blockIdx.x) * kHistBuckets;
+    if (tid == 0) p.list_count[static_cast<int64_t>(lrow) * kMaxRowWorkgroups + blockIdx.x] = sh.list_count;
+    uint32_t* hist_out = p.hist + (static_cast<int64_t>(lrow) * p.row_wgs + blockIdx.x) * kHistBuckets;
     for (int b = tid; b < kHistBuckets; b += kBlock) hist_out[b] = sh.hist[b];
+    if (kPatterns && km.n_bins > 0) {
+      uint32_t* ph_out = p.phist + (static_cast<int64_t>(lrow) * p.row_wgs + blockIdx.x) * p.phist_words;
+      for (int b = tid; b < (km.n_bins + 1) / 2; b += kBlock) ph_out[b] = ph[b];
+    }
   }
   if (p.timers && blockIdx.x == 0 && tid == 0) {
     uint64_t* t = p.timers + static_cast<int64_t>(gridDim.y) * 8 + static_cast<int64_t>(blockIdx.y) * 4;
@@ -746,6 +835,517 @@ __device__ __forceinline__ HistPlan split_plan(const uint32_t* hist, float a_tot
   return *plan_out;
 }
 
+// ---- top-p draw of 16-bit rows by runs of equal probability ----------------------------------------
+// A row of 16-bit logits has at most 65536 distinct probabilities, and the reference's sorted
+// candidate array (sampler.cpp:145-148) is the row's bit patterns in falling order, each repeated
+// as often as it occurs (among equal probabilities the tie rule orders by token index).  Its two
+// CDF walks (sampler.cpp:150-170) therefore add runs of equal values, and c sequential additions
+// of the same p have a closed form inside one binade of the running sum.  Pass 2 counted the
+// entries per pattern; here the runs are walked with the scheme of the softmax sum: approximate
+// cumulative masses place every group of 64 patterns inside a binade, each group is folded once
+// under that binade's ulp, one wave composes the groups from the exact running sum and works out
+// the few groups in which the sum changes binade, meets a half-ulp tie or crosses the threshold.
+// No sort, no gather; the token is the k-th occurrence, in index order, of the probability the
+// walk stops at.
+
+// c copies of p are added to s one after the other (s = s + p in fp32); the walk stops behind the
+// first copy that takes s above T.  Returns that copy's number (1-based), or 0 when all c copies
+// were added without exceeding T.  One lane.
+__device__ __forceinline__ uint32_t run_walk(float& s, float p, uint32_t c, float T) {
+  uint32_t left = c, done = 0u;
+  while (left > 0u) {
+    const SumState ss = sum_state(s);
+    const float scale = ss.kb >= 64 && ss.kb <= 250 ? __uint_as_float(static_cast<uint32_t>(277 - ss.kb) << 23) : 0.0f;
+    const float t = p * scale;
+    if (scale == 0.0f || !(t < 16777216.0f)) {  // out of the shortcut's range: one native add
+      s = s + p;
+      --left;
+      ++done;
+      if (s > T) return done;
+      continue;
+    }
+    const float r = __builtin_rintf(t);
+    uint32_t n = static_cast<uint32_t>(r);
+    uint32_t S = ss.S;
+    if (__builtin_fabsf(t - r) == 0.5f) {
+      // a half-ulp tie: the first add goes natively and leaves an even integer; from an even integer
+      // every further copy adds floor(t), or one more if that is odd
+      s = s + p;
+      --left;
+      ++done;
+      if (s > T) return done;
+      const SumState s2 = sum_state(s);
+      if (s2.kb != ss.kb) continue;
+      const uint32_t n0 = static_cast<uint32_t>(__builtin_floorf(t));
+      n = n0 + (n0 & 1u);
+      S = s2.S;
+    }
+    if (n == 0u) return 0u;  // absorbed: no copy changes the sum
+    // s' > T  <=>  S' >= floor(T / ulp) + 1; the sum must also stay below 2^24 ulps
+    const float tt = T * scale;
+    uint32_t limit = 1u << 24;
+    if (tt < 16777216.0f) {
+      const uint32_t Tn = tt >= 0.0f ? static_cast<uint32_t>(__builtin_floorf(tt)) + 1u : 0u;
+      limit = Tn < limit ? Tn : limit;
+    }
+    if (S >= limit) {  // (cannot happen: the walk would have stopped) one native add
+      s = s + p;
+      --left;
+      ++done;
+      if (s > T) return done;
+      continue;
+    }
+    const uint32_t stay = (limit - S - 1u) / n;  // copies after which the integer is still below `limit`
+    if (stay >= left) {
+      s = sum_value(S + left * n, ss.kb);
+      return 0u;
+    }
+    s = sum_value(S + stay * n, ss.kb);
+    left -= stay;
+    done += stay;
+    s = s + p;  // the copy that reaches the limit, natively
+    --left;
+    ++done;
+    if (s > T) return done;
+  }
+  return 0u;
+}
+
+struct RunSlotRec {
+  uint32_t meta;  // kind << 8 | kb
+  uint32_t inc_a, inc_b;
+  uint32_t pad;
+};
+
+// Probability and count of the bin at sorted position q (bins in falling key order).
+template <int DT>
+struct RunBins {
+  const uint32_t* cnt;  // LDS: two 16-bit counters per word
+  int key_cut, n_bins, mag_min;
+  float inv, m, cutoff;
+  RowDivisor div;
+  const uint64_t* tab;
+  __device__ __forceinline__ void at(int q, float& prob, uint32_t& count) const {
+    prob = 0.0f;
+    count = 0u;
+    if (q < n_bins) {
+      const int bin = n_bins - 1 - q;
+      const float l = pattern_value<DT>(key_pattern(key_cut + bin, mag_min));
+      const float e = expf_core(__builtin_fmaxf(l * inv - m, -104.0f), tab);
+      prob = div_row(e, div);
+      const uint32_t c = (cnt[bin >> 1] >> ((bin & 1) << 4)) & 0xffffu;
+      count = (prob >= cutoff) ? c : 0u;  // sampler.cpp:137-143
+    }
+  }
+};
+
+// One wave works the 64 bins of group t out exactly from running sum s; `before` is the number of
+// candidates in front of the group.  Returns the sorted position (0-based) behind which s first
+// exceeds T, or -1 (then s is the sum behind the group).
+template <int DT>
+__device__ __forceinline__ int resolve_run_group(float& s, int t, uint32_t before, float T, const RunBins<DT>& bins) {
+  const int lane = threadIdx.x & 63;
+  float prob;
+  uint32_t count;
+  bins.at(64 * t + lane, prob, count);
+  const uint32_t cnt_incl = wave_scan_inclusive_u32(count);
+  int cur = 0;
+  while (cur < 64) {
+    s = uniform_f32(s);
+    const SumState ss = sum_state(s);
+    const bool shortcut = ss.kb >= 64 && ss.kb <= 250;
+    const float scale = shortcut ? __uint_as_float(static_cast<uint32_t>(277 - ss.kb) << 23) : 0.0f;
+    const float tq = prob * scale;
+    const float rq = __builtin_rintf(tq);
+    const bool live = lane >= cur && count != 0u;
+    // a lane is an event when its adds depend on their order or cannot be counted in ulps
+    const bool odd_one = live && (!shortcut || !(tq < 16777216.0f) || __builtin_fabsf(tq - rq) == 0.5f);
+    const float incf = live && !odd_one ? __builtin_fminf(rq * static_cast<float>(count), 33554432.0f) : 0.0f;
+    const uint32_t incl = wave_scan_inclusive_u32(static_cast<uint32_t>(incf));
+    uint32_t limit = 1u << 24;
+    const float tt = T * scale;
+    if (shortcut && tt < 16777216.0f) {
+      const uint32_t Tn = tt >= 0.0f ? static_cast<uint32_t>(__builtin_floorf(tt)) + 1u : 0u;
+      limit = Tn < limit ? Tn : limit;
+    }
+    const uint32_t room = limit > ss.S ? limit - ss.S : 0u;
+    const uint64_t events = __ballot(odd_one || (live && incl >= room));
+    const int j = events ? __ffsll(static_cast<long long>(events)) - 1 : 64;
+    uint32_t S_j = ss.S;
+    if (j > 0) S_j += readlane_u32(incl, j > 63 ? 63 : j - 1);  // lanes below cur hold 0
+    if (j == 64) {
+      s = sum_value(S_j, ss.kb);
+      return -1;
+    }
+    float sj = 0.0f;
+    uint32_t hit = 0u;
+    if (lane == j) {
+      sj = sum_value(S_j, ss.kb);
+      hit = run_walk(sj, prob, count, T);
+    }
+    s = readlane_f32(sj, j);
+    hit = readlane_u32(hit, j);
+    if (hit != 0u) {
+      const uint32_t in_front = readlane_u32(cnt_incl - count, j);
+      return static_cast<int>(before + in_front + hit - 1u);
+    }
+    cur = j + 1;
+  }
+  return -1;
+}
+
+struct RunWalk {
+  int position;  // sorted position behind which the sum first exceeded the threshold, or -1
+  float sum;     // the sum there (or behind the last group walked)
+};
+
+// Needs p.row.lds_keys * 8 bytes of LDS at `lds` (the key buffer); every lane of the workgroup
+// calls it.  Returns false when the runs cannot be used (no pattern histogram, a counter that
+// overflowed, probabilities that do not fall along the patterns): the caller sorts instead.
+// What draw_topp_runs() needs of the launch and the row, by value (a reference to the kernel's
+// argument block would move that block to private memory for the whole kernel).
+struct RunArgs {
+  const uint32_t* phist;  // this row's first region
+  int32_t phist_words, row_wgs, lds_keys, ns;
+  int32_t key_cut, n_bins, mag_min;
+  uint32_t expected;      // candidates pass 2 listed: what the counters must add up to
+  float m;
+};
+
+template <int DT>
+__device__ __noinline__ bool draw_topp_runs(RunArgs a, const char* logits, int V, float inv, float S, float cutoff, float topp,
+                                            float coin, uint64_t* lds, RowDebug& dbg, int32_t& token, BlockScratch& sm) {
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int n_bins = a.n_bins;
+  if (n_bins <= 0) return false;
+  const int n_groups = (n_bins + 63) / 64;
+  const int words = (n_bins + 1) / 2;
+  // ---- LDS: counters | group records | exact sums at group boundaries | candidates in front of
+  //      each group | approximate masses in front of each group
+  uint32_t* cnt = reinterpret_cast<uint32_t*>(lds);
+  RunSlotRec* recs = reinterpret_cast<RunSlotRec*>(cnt + (words + 3) / 4 * 4);
+  float* sbound = reinterpret_cast<float*>(recs + n_groups);
+  uint32_t* cbound = reinterpret_cast<uint32_t*>(sbound + n_groups + 1);
+  float* mbound = reinterpret_cast<float*>(cbound + n_groups + 1);
+  if (reinterpret_cast<char*>(mbound + n_groups + 1) > reinterpret_cast<char*>(lds) + static_cast<size_t>(a.lds_keys) * 8)
+    return false;
+  // ---- the workgroups' counters, added up (16-bit halves add without carries unless one overflows,
+  //      which the totals give away)
+  {
+    const uint32_t* in = a.phist;
+    uint32_t sum16 = 0u;
+    for (int w = tid; w < words; w += kBlock) {
+      uint32_t lo = 0u, hi = 0u;
+      for (int g = 0; g < a.row_wgs; g += 4) {
+        uint32_t v[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) v[k] = in[static_cast<int64_t>(g + k < a.row_wgs ? g + k : g) * a.phist_words + w];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          if (g + k < a.row_wgs) {
+            lo += v[k] & 0xffffu;
+            hi += v[k] >> 16;
+          }
+        }
+      }
+      const bool fits = lo <= 0xffffu && hi <= 0xffffu;
+      cnt[w] = fits ? (lo | (hi << 16)) : 0u;
+      sum16 += fits ? lo + hi : 0x40000000u;  // (spoils the total)
+    }
+    sum16 = wave_sum_u32(sum16);
+    if (lane == 0) sm.red_u[wave] = sum16;
+    __syncthreads();
+    uint32_t total = 0u;
+    for (int w = 0; w < kWaves; ++w) total += sm.red_u[w];
+    __syncthreads();
+    if (total != a.expected) return false;
+  }
+  const RunBins<DT> bins = {cnt, a.key_cut, n_bins, a.mag_min, inv, a.m, cutoff, row_divisor(S), sm.exp2tab};
+  // ---- pass A: per group the candidates and their approximate mass; probabilities must not rise
+  //      along the sorted positions
+  bool rising = false;
+  for (int t = wave; t < n_groups; t += kWaves) {
+    float prob;
+    uint32_t count;
+    bins.at(64 * t + lane, prob, count);
+    float next_prob = 0.0f;  // of the position behind this lane's
+    uint32_t next_count;
+    if (lane == 63) bins.at(64 * t + 64, next_prob, next_count);
+    const float from_right = __shfl_down(prob, 1);
+    if (lane != 63) next_prob = from_right;
+    if (64 * t + lane + 1 < n_bins && next_prob > prob) rising = true;
+    const float mass = wave_sum_f32(static_cast<float>(count) * prob);
+    const uint32_t c = wave_sum_u32(count);
+    if (lane == 0) {
+      mbound[t + 1] = mass;
+      cbound[t + 1] = c;
+    }
+  }
+  {
+    const uint64_t any = __ballot(rising);
+    if (lane == 0) sm.red_u[wave] = any ? 1u : 0u;
+  }
+  __syncthreads();
+  uint32_t bad = 0u;
+  for (int w = 0; w < kWaves; ++w) bad |= sm.red_u[w];
+  // prefix sums over the groups (at most kBlock of them)
+  {
+    const float mine = tid < n_groups ? mbound[tid + 1] : 0.0f;
+    const uint32_t mine_c = tid < n_groups ? cbound[tid + 1] : 0u;
+    const float incl = wave_scan_inclusive_f32(mine, lane);
+    const uint32_t incl_c = wave_scan_inclusive_u32(mine_c);
+    __syncthreads();
+    if (lane == 63) {
+      sm.red_f[wave] = incl;
+      sm.red_u[wave] = incl_c;
+    }
+    __syncthreads();
+    float before = 0.0f;
+    uint32_t before_c = 0u;
+    for (int w = 0; w < wave; ++w) {
+      before += sm.red_f[w];
+      before_c += sm.red_u[w];
+    }
+    if (tid < n_groups) {
+      mbound[tid + 1] = before + incl;
+      cbound[tid + 1] = before_c + incl_c;
+    }
+    if (tid == 0) {
+      mbound[0] = 0.0f;
+      cbound[0] = 0u;
+    }
+    __syncthreads();
+  }
+  if (bad != 0u || n_groups > kBlock) return false;
+  const uint32_t n0 = cbound[n_groups];
+  dbg.n_candidates = static_cast<int>(n0);
+  if (n0 == 0u) {
+    token = -1;  // the reference reads probindex[-1] here
+    return true;
+  }
+  // ---- pass B: fold every group once, under the ulp(s) of the binade(s) the cumulative sum can be
+  //      in while it passes the group.  A group that may hold the place where the sum exceeds topp,
+  //      that spans more than two binades or in which an entry ties is left to the ordered walk.
+  for (int t = wave; t < n_groups; t += kWaves) {
+    const uint32_t c_in = cbound[t], c_out = cbound[t + 1];
+    RunSlotRec rec = {kSlotZero << 8, 0u, 0u, 0u};
+    if (c_out != c_in) {
+      const float eps_in = static_cast<float>(c_in) * (1.02f / 16777216.0f) + 3e-5f;
+      const float eps_out = static_cast<float>(c_out) * (1.02f / 16777216.0f) + 3e-5f;
+      const float lo = mbound[t] * (1.0f - eps_in), hi = mbound[t + 1] * (1.0f + eps_out);
+      const uint32_t kb_lo = __float_as_uint(lo > 0.0f ? lo : 0.0f) >> 23, kb_hi = __float_as_uint(hi) >> 23;
+      const bool near_topp = !(hi < topp * 0.9999f);  // (the walk ends there: nothing behind it is needed)
+      rec.meta = (kSlotSerial << 8) | (kb_lo & 255u);
+      if (!near_topp && lo > 0.0f && kb_lo >= 70u && kb_hi <= 250u && kb_hi <= kb_lo + 1u) {
+        float prob;
+        uint32_t count;
+        bins.at(64 * t + lane, prob, count);
+        const float scale_a = __uint_as_float((277u - kb_lo) << 23), scale_b = __uint_as_float((276u - kb_lo) << 23);
+        const float ta = prob * scale_a, tb = prob * scale_b;
+        const float ra = __builtin_rintf(ta), rb = __builtin_rintf(tb);
+        const bool tie = count != 0u && (__builtin_fabsf(ta - ra) == 0.5f || (kb_hi != kb_lo && __builtin_fabsf(tb - rb) == 0.5f));
+        const float fc = static_cast<float>(count);
+        const uint32_t ia = static_cast<uint32_t>(__builtin_fminf(ra * fc, 33554432.0f));
+        const uint32_t ib = static_cast<uint32_t>(__builtin_fminf(rb * fc, 33554432.0f));
+        const uint32_t inc_a = wave_sum_u32(ia), inc_b = wave_sum_u32(ib);
+        if (__ballot(tie) == 0ull) {
+          rec.meta = ((kb_hi == kb_lo ? kSlotStable : kSlotDual) << 8) | kb_lo;
+          rec.inc_a = inc_a < kSat ? inc_a : kSat;
+          rec.inc_b = inc_b < kSat ? inc_b : kSat;
+        }
+      }
+    }
+    if (lane == 0) recs[t] = rec;
+  }
+  __syncthreads();
+  // ---- walk 1 (sampler.cpp:150-158): the groups in order until the sum exceeds topp.  One wave.
+  if (wave == 0) {
+    float s = 0.0f;
+    int found = -1;
+    int last_group = n_groups - 1;
+    if (lane == 0) sbound[0] = 0.0f;
+    for (int base = 0; base < n_groups && found < 0; base += 64) {
+      RunSlotRec r = {kSlotZero << 8, 0u, 0u, 0u};
+      if (base + lane < n_groups) r = recs[base + lane];
+      const uint32_t kind = (r.meta >> 8) & 7u, kb = r.meta & 255u;
+      int cur = 0;
+      int K_scan = -1;
+      uint32_t incl = 0u;
+      uint64_t plain_mask = 0ull;
+      while (cur < 64 && found < 0) {
+        s = uniform_f32(s);
+        const SumState ss = sum_state(s);
+        const uint32_t K = static_cast<uint32_t>(ss.kb);
+        if (ss.kb != K_scan) {
+          const bool plain = kind == kSlotZero || (kind == kSlotStable && kb == K) || (kind == kSlotDual && (kb == K || kb + 1u == K));
+          const uint32_t inc = kind == kSlotZero ? 0u : ((kind == kSlotDual && kb != K) ? r.inc_b : r.inc_a);
+          incl = wave_scan_inclusive_u32(plain ? inc : 0u);
+          plain_mask = __ballot(plain);
+          K_scan = ss.kb;
+        }
+        const uint64_t not_plain = ~plain_mask & (~0ull << cur);
+        const int jn = not_plain ? __ffsll(static_cast<long long>(not_plain)) - 1 : 64;
+        const uint32_t before = cur > 0 ? readlane_u32(incl, cur - 1) : 0u;
+        const uint32_t S_upto = ss.S + (incl - before);
+        // the sum must stay inside the binade and must not exceed topp inside a folded group
+        uint32_t limit = 1u << 24;
+        if (ss.kb >= 64 && ss.kb <= 250) {
+          const float tt = topp * __uint_as_float(static_cast<uint32_t>(277 - ss.kb) << 23);
+          if (tt < 16777216.0f) {
+            const uint32_t Tn = static_cast<uint32_t>(__builtin_floorf(tt)) + 1u;
+            limit = Tn < limit ? Tn : limit;
+          }
+        }
+        const uint64_t over = __ballot(lane >= cur && lane < jn && S_upto >= limit);
+        const int jo = over ? __ffsll(static_cast<long long>(over)) - 1 : 64;
+        const int j = jn < jo ? jn : jo;
+        if (lane >= cur && lane < j && base + lane < n_groups) sbound[base + lane + 1] = sum_value(S_upto, ss.kb);
+        if (j > cur) s = sum_value(readlane_u32(S_upto, j - 1), ss.kb);
+        if (j == 64) break;
+        const int t = base + j;
+        if (t >= n_groups) break;
+        found = resolve_run_group<DT>(s, t, cbound[t], topp, bins);
+        if (lane == 0) sbound[t + 1] = s;
+        if (found >= 0) last_group = t;
+        cur = j + 1;
+      }
+    }
+    if (lane == 0) {
+      sm.bc_sum = s;
+      sm.bc_found = found;
+      sm.flag = last_group;
+    }
+  }
+  __syncthreads();
+  const float mass = sm.bc_sum;
+  const int last_idx = sm.bc_found >= 0 ? sm.bc_found : static_cast<int>(n0) - 1;
+  const int last_group = sm.flag;
+  const float r = coin * mass;  // sampler.cpp:162
+  __syncthreads();
+  // ---- walk 2 (sampler.cpp:163-168): the same partial sums against r; the group in which they
+  //      first exceed it is worked out once more
+  if (wave == 0) {
+    int t2 = -1;
+    for (int base = 0; base <= last_group && t2 < 0; base += 64) {
+      const int t = base + lane;
+      const uint64_t ballot = __ballot(t <= last_group && sbound[t + 1] > r);
+      if (ballot) t2 = base + __ffsll(static_cast<long long>(ballot)) - 1;
+    }
+    int pos = last_idx;
+    if (t2 >= 0) {
+      float s2 = sbound[t2];
+      const int hit = resolve_run_group<DT>(s2, t2, cbound[t2], r, bins);
+      if (hit >= 0 && hit < last_idx) pos = hit;
+    }
+    if (lane == 0) sm.bc_found = pos;
+  }
+  __syncthreads();
+  const int pos = sm.bc_found;
+  __syncthreads();
+  dbg.last_idx = last_idx;
+  dbg.cumulative = mass;
+  dbg.r = r;
+  dbg.position = pos;
+  // ---- the token: the bins that share the probability at `pos`, and the occurrence wanted of them
+  //      in index order
+  if (wave == 0) {
+    int t = 0;
+    for (int base = 0; base < n_groups; base += 64) {
+      const int g = base + lane;
+      const uint64_t ballot = __ballot(g < n_groups && cbound[g + 1] > static_cast<uint32_t>(pos));
+      if (ballot) {
+        t = base + __ffsll(static_cast<long long>(ballot)) - 1;
+        break;
+      }
+    }
+    float prob;
+    uint32_t count;
+    bins.at(64 * t + lane, prob, count);
+    const uint32_t incl = wave_scan_inclusive_u32(count);
+    const uint64_t holds = __ballot(cbound[t] + incl > static_cast<uint32_t>(pos));
+    const int jl = __ffsll(static_cast<long long>(holds)) - 1;  // not empty: the group's total exceeds pos
+    const float p_star = readlane_f32(prob, jl);
+    // equal probabilities lie next to each other: look 64 positions to either side
+    const int q_star = 64 * t + jl;
+    float p_up, p_down;
+    uint32_t c_up, c_down;
+    bins.at(q_star - 64 + lane >= 0 ? q_star - 64 + lane : n_bins, p_up, c_up);  // positions q_star-64 .. q_star-1
+    bins.at(q_star + 1 + lane, p_down, c_down);                                   // positions q_star+1 .. q_star+64
+    const uint64_t same_up = __ballot(c_up != 0u && p_up == p_star);
+    const uint64_t same_down = __ballot(c_down != 0u && p_down == p_star);
+    const uint32_t group_up = wave_sum_u32((c_up != 0u && p_up == p_star) ? c_up : 0u);
+    // sorted position of the first entry with this probability, and the key range that holds them
+    const uint32_t first_pos = cbound[t] + readlane_u32(incl - count, jl) - group_up;
+    const int q_lo = same_up ? q_star - 64 + (__ffsll(static_cast<long long>(same_up)) - 1) : q_star;
+    const int q_hi = same_down ? q_star + 1 + (63 - __clzll(static_cast<long long>(same_down))) : q_star;
+    if (lane == 0) {
+      // (an equal probability at the window's edge could go on beyond it: then sort instead)
+      sm.flag = ((same_up & 1ull) && q_star - 64 > 0) || (same_down >> 63) ? -1 : static_cast<int>(static_cast<uint32_t>(pos) - first_pos);
+      sm.first_flag[0] = a.key_cut + (n_bins - 1 - q_hi);  // smallest key of the range
+      sm.first_flag[1] = a.key_cut + (n_bins - 1 - q_lo);  // largest
+    }
+  }
+  __syncthreads();
+  const int want = sm.flag;
+  const int key_lo = sm.first_flag[0], key_hi = sm.first_flag[1];
+  __syncthreads();
+  if (want < 0) return false;
+  // occurrences per slot of the row, in index order
+  const int ns = a.ns;
+  uint32_t* occ = reinterpret_cast<uint32_t*>(lds);  // (the counters are dead) ns + 1 words
+  const float kInf = __uint_as_float(0x7f800000u);
+  auto matches = [&](int s_, int lane_) -> uint32_t {
+    float l[8];
+    load_slot_lane<DT>(logits, s_, lane_, V, -kInf, l);
+    uint32_t mask = 0u;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const int key = pattern_key(value_pattern<DT>(l[k]), a.mag_min);
+      mask |= (key >= key_lo && key <= key_hi && s_ * kSlot + lane_ * 8 + k < V) ? (1u << k) : 0u;
+    }
+    return mask;
+  };
+  for (int s_ = wave; s_ < ns; s_ += kWaves) {
+    const uint32_t c = wave_sum_u32(static_cast<uint32_t>(__popc(matches(s_, lane))));
+    if (lane == 0) occ[s_] = c;
+  }
+  __syncthreads();
+  if (wave == 0) {
+    uint32_t seen = 0u;
+    int32_t tok = -1;
+    for (int base = 0; base < ns && tok < 0; base += 64) {
+      const uint32_t c = base + lane < ns ? occ[base + lane] : 0u;
+      const uint32_t incl = wave_scan_inclusive_u32(c);
+      const uint64_t ballot = __ballot(seen + incl > static_cast<uint32_t>(want));
+      if (ballot) {
+        const int js = __ffsll(static_cast<long long>(ballot)) - 1;
+        const uint32_t before = seen + readlane_u32(incl - c, js);
+        const int s_ = base + js;
+        const uint32_t mask = matches(s_, lane);
+        const uint32_t mine = static_cast<uint32_t>(__popc(mask));
+        const uint32_t lincl = wave_scan_inclusive_u32(mine);
+        const uint64_t b2 = __ballot(before + lincl > static_cast<uint32_t>(want));
+        const int jl = __ffsll(static_cast<long long>(b2)) - 1;
+        uint32_t skip = static_cast<uint32_t>(want) - (before + readlane_u32(lincl - mine, jl));
+        uint32_t mk = readlane_u32(mask, jl);
+        while (skip > 0u) {
+          mk &= mk - 1u;
+          --skip;
+        }
+        tok = s_ * kSlot + jl * 8 + (__ffs(static_cast<int>(mk)) - 1);
+      }
+      seen += readlane_u32(incl, 63);
+    }
+    if (lane == 0) sm.bc_found = tok;
+  }
+  __syncthreads();
+  token = sm.bc_found;
+  __syncthreads();
+  return token >= 0;
+}
+
 // grid = rows; dynamic LDS: the key buffer of the draw (p.row.lds_keys keys), which holds the
 // slot records and the prepared slots while the sum is composed.
 template <int DT>
@@ -753,6 +1353,7 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
   extern __shared__ __align__(16) uint64_t lds_keys[];
   __shared__ BlockScratch sm;
   __shared__ FinishShared fs;
+  const int lrow = blockIdx.x;  // row of this launch: indexes the buffers whose layout depends on the launch
   const int row = p.row.row_map ? p.row.row_map[blockIdx.x] : blockIdx.x;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -778,7 +1379,7 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
   if (!row_nan) {
     // ---- how many candidates the workgroups of pass 2 listed; their histograms, added up
     if (tid < 64) {
-      const uint32_t c = tid < p.row_wgs ? p.list_count[static_cast<int64_t>(row) * kMaxRowWorkgroups + tid] : 0u;
+      const uint32_t c = tid < p.row_wgs ? p.list_count[static_cast<int64_t>(lrow) * kMaxRowWorkgroups + tid] : 0u;
       const uint32_t incl = wave_scan_inclusive_u32(c);
       fs.count[tid] = c;
       fs.offset[tid + 1] = incl;
@@ -792,7 +1393,7 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
     }
     {
       // (four workgroups' counts are requested at a time: a loop of one load each would wait for each)
-      const uint32_t* hist_in = p.hist + static_cast<int64_t>(row) * p.row_wgs * kHistBuckets;
+      const uint32_t* hist_in = p.hist + static_cast<int64_t>(lrow) * p.row_wgs * kHistBuckets;
       uint32_t c[kHistBuckets / kBlock];
 #pragma unroll
       for (int q = 0; q < kHistBuckets / kBlock; ++q) c[q] = 0u;
@@ -841,7 +1442,7 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
       // ---- the other waves, meanwhile: one pass over the listed candidates picks out those of the
       //      largest buckets and those that may or may not reach the cutoff
       for (int g = 0; g < p.row_wgs; ++g) {
-        const uint64_t* src = p.list + (static_cast<int64_t>(row) * p.row_wgs + g) * p.list_region;
+        const uint64_t* src = p.list + (static_cast<int64_t>(lrow) * p.row_wgs + g) * p.list_region;
         const int c = static_cast<int>(fs.count[g]);
         for (int j = (wave - 1) * 64 + lane; j < c; j += (kWaves - 1) * 64) {
           const uint64_t ent = src[j];
@@ -941,10 +1542,19 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
         path = 1;
       }
     }
+    if constexpr (DT == kDtypeBFloat16 || DT == kDtypeHalf) {
+      // ---- a longer nucleus of a 16-bit row: runs of equal probabilities
+      if (!done && rs.n_bins > 0 && (!lists_ok || n_listed > 4096)) {
+        const RunArgs ra = {p.phist + static_cast<int64_t>(lrow) * p.row_wgs * p.phist_words, p.phist_words, p.row_wgs,
+                            p.row.lds_keys, ns, rs.key_cut, rs.n_bins, rs.mag_min, static_cast<uint32_t>(n_listed), m};
+        done = draw_topp_runs<DT>(ra, logits, V, inv, S, cutoff, topp, coin, lds_keys, dbg, token, sm);
+        path = 4;
+      }
+    }
     if (!done && lists_ok && n_listed <= p.row.lds_keys - kBlock) {
       // ---- a longer nucleus: the whole list goes to LDS, selection by probability, sort, walks
       for (int g = wave; g < p.row_wgs; g += kWaves) {
-        const uint64_t* src = p.list + (static_cast<int64_t>(row) * p.row_wgs + g) * p.list_region;
+        const uint64_t* src = p.list + (static_cast<int64_t>(lrow) * p.row_wgs + g) * p.list_region;
         uint64_t* dst = lds_keys + kBlock + fs.offset[g];
         const int c = static_cast<int>(fs.count[g]);
         for (int j = lane; j < c; j += 64) dst[j] = src[j];
