@@ -29,7 +29,18 @@ struct ErrorSink {
 
 }  // namespace
 
+// Device memory a call works in beyond its inputs and outputs, when it is not the handle's own:
+// the entry point that allocates nothing lays it out inside the library's static array.
+struct WorkBuffers {
+  ets::SplitParams split = {};
+  uint64_t* scratch = nullptr;  // [rows, scratch_stride] keys of the general draw
+  int64_t scratch_stride = 0;
+  uint64_t* partials = nullptr;  // [rows, kMaxSplits] arg-max partial results
+  int max_row_wgs = 0;           // workgroups of pass 2 per row, at most
+};
+
 struct ets_sampler {
+  const WorkBuffers* wb = nullptr;  // set for the duration of a call that brings its own buffers
   int32_t vocab = 0;
   float inv_temperature = 0.0f;
   float topp = 0.9f;
@@ -169,16 +180,17 @@ ets_status launch_argmax(ets_sampler* s, const void* d_logits, int32_t batch, in
   const int splits = row_splits(s->vocab, batch);
   const size_t esz = ets::ElemSize<DT>::value;
   const bool aligned = (reinterpret_cast<uintptr_t>(d_logits) % 16 == 0) && ((static_cast<size_t>(stride) * esz) % 16 == 0);
+  uint64_t* partials = s->wb ? s->wb->partials : s->d_partials;
   const dim3 grid(splits, batch);
   if (aligned) {
     hipLaunchKernelGGL((ets::argmax_partial_kernel<DT, true>), grid, dim3(ets::kArgmaxBlock), 0, stream, d_logits, stride,
-                       s->vocab, s->d_partials, d_row_map);
+                       s->vocab, partials, d_row_map);
   } else {
     hipLaunchKernelGGL((ets::argmax_partial_kernel<DT, false>), grid, dim3(ets::kArgmaxBlock), 0, stream, d_logits, stride,
-                       s->vocab, s->d_partials, d_row_map);
+                       s->vocab, partials, d_row_map);
   }
   ETS_HIP(s, hipGetLastError());
-  hipLaunchKernelGGL((ets::argmax_finish_kernel<DT>), dim3(batch), dim3(64), 0, stream, d_logits, stride, s->d_partials,
+  hipLaunchKernelGGL((ets::argmax_finish_kernel<DT>), dim3(batch), dim3(64), 0, stream, d_logits, stride, partials,
                      splits, d_tokens, d_row_map);
   ETS_HIP(s, hipGetLastError());
   return ETS_OK;
@@ -239,7 +251,7 @@ float inverse_temperature_ctor(float temperature) {
 }
 
 ets_status ensure_scratch(ets_sampler* s) {
-  if (s->d_scratch) return ETS_OK;
+  if (s->d_scratch || s->wb) return ETS_OK;
   const size_t bytes = static_cast<size_t>(s->max_batch) * static_cast<size_t>(s->scratch_stride) * sizeof(uint64_t);
   ETS_HIP(s, hipMalloc(reinterpret_cast<void**>(&s->d_scratch), bytes));
   return ETS_OK;
@@ -277,6 +289,7 @@ int pass2_workgroups(const ets_sampler* s, int32_t rows, int32_t ns) {
   const int by_len = (ns + 15) / 16;
   if (g > by_len) g = by_len;
   if (g > ets::kMaxRowWorkgroups) g = ets::kMaxRowWorkgroups;
+  if (s->wb && g > s->wb->max_row_wgs) g = s->wb->max_row_wgs;
   return g < 1 ? 1 : g;
 }
 
@@ -356,14 +369,17 @@ bool use_split(const ets_sampler* s, const void* d_logits, int64_t stride, int32
 
 template <int DT>
 ets_status launch_split(ets_sampler* s, const ets::RowParams& p, int32_t rows, hipStream_t stream) {
-  ets_status st = ensure_split(s);
-  if (st != ETS_OK) return st;
+  ets_status st = ETS_OK;
   constexpr bool k16 = DT == ets::kDtypeBFloat16 || DT == ets::kDtypeHalf;
-  if (k16) {
-    st = ensure_phist(s);
+  if (!s->wb) {
+    st = ensure_split(s);
     if (st != ETS_OK) return st;
+    if (k16) {
+      st = ensure_phist(s);
+      if (st != ETS_OK) return st;
+    }
   }
-  ets::SplitParams sp = s->split;
+  ets::SplitParams sp = s->wb ? s->wb->split : s->split;
   sp.row = p;
   sp.phist_words = DT == ets::kDtypeBFloat16 ? kPhistWordsBFloat16 : (DT == ets::kDtypeHalf ? kPhistWordsHalf : 0);
   sp.row_wgs = pass2_workgroups(s, rows, sp.ns);
@@ -428,12 +444,72 @@ ets_status sample_device(ets_sampler* s, const void* d_logits, int32_t dtype, in
   p.tokens = d_tokens;
   p.probs = d_probs;
   p.debug = reinterpret_cast<ets::RowDebug*>(d_debug);
-  p.scratch = s->d_scratch;
-  p.scratch_stride = s->scratch_stride;
+  p.scratch = s->wb ? s->wb->scratch : s->d_scratch;
+  p.scratch_stride = s->wb ? s->wb->scratch_stride : s->scratch_stride;
   p.lds_keys = s->lds_keys;
   p.row_map = nullptr;
   p.row_cfg = nullptr;
   return rows_device(s, p, dtype, batch, stream, draw_mode(s->vocab, s->topp, s->topk));
+}
+
+// ---- the entry point that allocates nothing ------------------------------------------------------
+// Its work buffers live in this array: one copy per GPU the library runs on, held until the
+// process ends.  Host code never uses the array's name as an address: the device address is looked
+// up once per device (at the first handle created there) and kept.
+constexpr size_t kStaticScratchBytes = size_t{32} << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+std::mutex g_static_mutex;
+void* g_static_ptr[kMaxDevices] = {};
+
+// With the handle's device current.
+ets_status static_scratch_address(ets_sampler* s, int device, void** out) {
+  if (device < 0 || device >= kMaxDevices) return fail(s, ETS_NOT_SUPPORTED, "device index beyond the static scratch table");
+  std::lock_guard<std::mutex> lock(g_static_mutex);
+  if (!g_static_ptr[device]) {
+    void* ptr = nullptr;
+    hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return hip_fail(s, e, "hipGetSymbolAddress(scratch)");
+    g_static_ptr[device] = ptr;
+  }
+  *out = g_static_ptr[device];
+  return ETS_OK;
+}
+
+// Lays the work buffers of a call of `rows` rows out from `base`; returns the bytes needed.
+size_t layout_static(const ets_sampler* s, int32_t dtype, int32_t rows, char* base, WorkBuffers* wb) {
+  ets::SplitParams& sp = wb->split;
+  sp = ets::SplitParams{};
+  sp.ns = (s->vocab + ets::kSlot - 1) / ets::kSlot;
+  sp.ns_stride = static_cast<int32_t>(round_up(static_cast<size_t>(sp.ns), 4));
+  sp.prep_cap = ets::kPrepCap;
+  wb->max_row_wgs = 4;
+  int g = ((s->num_cus > 0 ? s->num_cus : 256) + rows - 1) / rows;
+  const int by_len = (sp.ns + 15) / 16;
+  g = g > by_len ? by_len : g;
+  g = g > wb->max_row_wgs ? wb->max_row_wgs : (g < 1 ? 1 : g);
+  const size_t r = static_cast<size_t>(rows);
+  const size_t phist_words = dtype == ETS_DTYPE_HALF ? kPhistWordsHalf : (dtype == ETS_DTYPE_BFLOAT16 ? kPhistWordsBFloat16 : 0);
+  size_t at = 0;
+  auto take = [&](size_t bytes) {
+    const size_t here = at;
+    at = round_up(at + bytes, 256);
+    return base + here;
+  };
+  sp.slot_max = reinterpret_cast<float*>(take(r * sp.ns_stride * sizeof(float)));
+  sp.slot_sum = reinterpret_cast<float*>(take(r * sp.ns_stride * sizeof(float)));
+  sp.slot_rec = reinterpret_cast<ets::SlotRec*>(take(r * sp.ns_stride * sizeof(ets::SlotRec)));
+  sp.prep = reinterpret_cast<ets::PrepSlot*>(take(r * sp.prep_cap * sizeof(ets::PrepSlot)));
+  sp.row_state = reinterpret_cast<ets::RowState*>(take(r * sizeof(ets::RowState)));
+  sp.list_count = reinterpret_cast<uint32_t*>(take(r * ets::kMaxRowWorkgroups * sizeof(uint32_t)));
+  sp.hist = reinterpret_cast<uint32_t*>(take(r * g * ets::kHistBuckets * sizeof(uint32_t)));
+  sp.phist = reinterpret_cast<uint32_t*>(take(r * g * phist_words * sizeof(uint32_t)));
+  sp.list = reinterpret_cast<uint64_t*>(take(r * g * list_region(sp.ns, g) * sizeof(uint64_t)));
+  sp.timers = nullptr;
+  wb->scratch_stride = s->scratch_stride;
+  wb->scratch = reinterpret_cast<uint64_t*>(take(r * static_cast<size_t>(s->scratch_stride) * sizeof(uint64_t)));
+  wb->partials = reinterpret_cast<uint64_t*>(take(r * kMaxSplits * sizeof(uint64_t)));
+  return at;
 }
 
 // ---- per-row parameters ------------------------------------------------------------------------
@@ -570,6 +646,14 @@ ets_status ets_sampler_create(int32_t vocab_size, float temperature, float topp,
   int lds_limit = 0;
   e = hipDeviceGetAttribute(&lds_limit, hipDeviceAttributeMaxSharedMemoryPerBlock, s->device);
   if (e != hipSuccess) return bail(e, "hipDeviceGetAttribute(MaxSharedMemoryPerBlock)");
+  {
+    void* unused = nullptr;  // (kept per device; the entry point that allocates nothing reads it)
+    ets_status sst = static_scratch_address(nullptr, s->device, &unused);
+    if (sst != ETS_OK) {
+      ets_sampler_destroy(s);
+      return sst;
+    }
+  }
   e = hipDeviceGetAttribute(&s->num_cus, hipDeviceAttributeMultiprocessorCount, s->device);
   if (e != hipSuccess) return bail(e, "hipDeviceGetAttribute(MultiprocessorCount)");
   // the row kernel's static LDS (reduction scratch, selection buffer, histogram) stays under 16 KiB
@@ -687,6 +771,35 @@ ets_status ets_sampler_sample_batch(ets_sampler* s, const void* d_logits, int32_
                                     int64_t row_stride_elems, int32_t* d_tokens, void* hip_stream) {
   return ets_sampler_sample_batch_debug(s, d_logits, dtype, batch, row_stride_elems, d_tokens, nullptr, nullptr,
                                         hip_stream);
+}
+
+ets_status ets_sampler_sample_batch_static(ets_sampler* s, const void* d_logits, int32_t dtype, int32_t batch,
+                                           int64_t row_stride_elems, int32_t* d_tokens, void* hip_stream) {
+  if (!s) return fail(nullptr, ETS_INVALID_ARGUMENT, "ets_sampler_sample_batch_static: null handle");
+  s->last_error.clear();
+  if (!d_logits || !d_tokens) return fail(s, ETS_INVALID_ARGUMENT, "ets_sampler_sample_batch_static: null pointer");
+  if (!dtype_ok(dtype)) return fail(s, ETS_INVALID_ARGUMENT, "ets_sampler_sample_batch_static: unsupported dtype");
+  if (batch < 0 || batch > s->max_batch)
+    return fail(s, ETS_INVALID_ARGUMENT, "ets_sampler_sample_batch_static: batch exceeds the handle's max_batch");
+  if (row_stride_elems < s->vocab)
+    return fail(s, ETS_INVALID_ARGUMENT, "ets_sampler_sample_batch_static: row stride smaller than vocab_size");
+  if (batch == 0) return ETS_OK;
+  DeviceGuard g(s->device);
+  void* base = nullptr;
+  ets_status st = static_scratch_address(s, s->device, &base);
+  if (st != ETS_OK) return st;
+  WorkBuffers wb;
+  const size_t need = layout_static(s, dtype, batch, static_cast<char*>(base), &wb);
+  if (need > kStaticScratchBytes) {
+    return fail(s, ETS_INVALID_ARGUMENT,
+                "ets_sampler_sample_batch_static: batch x vocab_size needs " + std::to_string(need) +
+                    " bytes of work buffers, the static scratch holds " + std::to_string(kStaticScratchBytes) +
+                    "; use ets_sampler_sample_batch");
+  }
+  s->wb = &wb;
+  st = sample_device(s, d_logits, dtype, batch, row_stride_elems, d_tokens, nullptr, nullptr, static_cast<hipStream_t>(hip_stream));
+  s->wb = nullptr;
+  return st;
 }
 
 ets_status ets_sampler_sample_batch_configs(ets_sampler* s, const void* d_logits, int32_t dtype, int32_t batch,

@@ -147,6 +147,23 @@ class Sampler:
         self._check(st)
         return out
 
+    def sample_batch_static(self, logits: torch.Tensor, out: torch.Tensor | None = None, dtype: int | None = None) -> torch.Tensor:
+        """``sample_batch`` through the entry point that allocates nothing: the kernels' work buffers
+        come from a fixed array inside the library (so the problem size is limited); ``out`` should
+        be passed by callers that must not allocate either."""
+        if not logits.is_cuda or logits.dim() != 2 or logits.stride(1) != 1:
+            raise SamplerError(_capi.INVALID_ARGUMENT, "sample_batch_static wants a device tensor [B, vocab] with unit inner stride")
+        B, V = logits.shape
+        if V != self.vocab_size:
+            raise SamplerError(_capi.INVALID_ARGUMENT, "last dimension differs from vocab_size")
+        code = dtype_code(logits) if dtype is None else dtype
+        if out is None:
+            out = torch.empty(B, dtype=torch.int32, device=logits.device)
+        stream = torch.cuda.current_stream(logits.device).cuda_stream
+        self._check(_capi.lib().ets_sampler_sample_batch_static(self._h, logits.data_ptr(), code, B, logits.stride(0),
+                                                                out.data_ptr(), stream))
+        return out
+
     def sample_batch_configs(self, logits: torch.Tensor, configs, out: torch.Tensor | None = None,
                              dtype: int | None = None, debug_out: torch.Tensor | None = None) -> torch.Tensor:
         """``sample_batch`` with one ``SamplingConfig`` per row (llm_session.h:29-34): ``configs`` is a

@@ -125,6 +125,20 @@ ETS_API ets_status ets_sampler_sample(ets_sampler* s, const void* logits, int32_
 ETS_API ets_status ets_sampler_sample_batch(ets_sampler* s, const void* d_logits, int32_t dtype, int32_t batch,
                                            int64_t row_stride_elems, int32_t* d_tokens, void* hip_stream);
 
+/* No counterpart in the reference.  ets_sampler_sample_batch() for callers that cannot allocate
+ * device memory at the time of the call -- code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc: same arguments, same tokens and coin states, but every work
+ * buffer of the kernels (partial results, slot records, candidate lists and histograms, sort
+ * keys) lies in a 32 MiB array that is part of the library's device image (one copy per GPU, held
+ * until the process ends), and the call allocates and frees nothing.  The price is a limit: the
+ * buffers of `batch` rows of vocab_size entries must fit (about 17 * batch * vocab_size bytes plus
+ * 0.6 MiB per row; batch 8 at vocab 128256 does), else ETS_INVALID_ARGUMENT with the sizes in
+ * ets_sampler_last_error().  Every call on a GPU, from any handle, uses that GPU's one array:
+ * calls that overlap in time on one GPU race; serialize them (one stream, or events). */
+ETS_API ets_status ets_sampler_sample_batch_static(ets_sampler* s, const void* d_logits, int32_t dtype,
+                                                  int32_t batch, int64_t row_stride_elems, int32_t* d_tokens,
+                                                  void* hip_stream);
+
 /* As above, plus per-row intermediates for the parity tests: `d_probs` (nullable) receives the
  * fp32 softmax probabilities [batch, vocab_size] that the reference would leave in its buffer,
  * `d_debug` (nullable) one ets_row_debug per row.  Both are DEVICE pointers. */
