@@ -57,6 +57,7 @@ SIGNATURES = {
     "ets_sampler_set_rng_states": (C.c_int32, [C.c_void_p, C.c_int32, C.c_int32, C.c_void_p]),
     "ets_sampler_get_rng_states": (C.c_int32, [C.c_void_p, C.c_int32, C.c_int32, C.c_void_p]),
     "ets_sample_from_logits": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.POINTER(C.c_int64), C.POINTER(C.c_int32)]),
+    "ets_sample_from_logits_batch": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.POINTER(C.c_int64), C.c_void_p, C.c_void_p]),
     "ets_logits_to_token": (C.c_int32, [C.c_void_p, C.c_int32, C.c_int32, C.POINTER(C.c_int64), C.c_float, C.POINTER(C.c_int32)]),
     "ets_random_u32": (C.c_uint32, [C.POINTER(C.c_uint64)]),
     "ets_random_f32": (C.c_float, [C.POINTER(C.c_uint64)]),

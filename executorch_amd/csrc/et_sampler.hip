@@ -977,6 +977,31 @@ ets_status ets_sample_from_logits(ets_sampler* s, const void* data, int32_t dtyp
   return ets_sampler_sample(s, p, dtype, token_out);
 }
 
+ets_status ets_sample_from_logits_batch(ets_sampler* s, const void* d_data, int32_t dtype, int32_t rank,
+                                        const int64_t* sizes, int32_t* d_tokens, void* hip_stream) {
+  if (!s) return fail(nullptr, ETS_INVALID_ARGUMENT, "ets_sample_from_logits_batch: null handle");
+  s->last_error.clear();
+  if (!d_data || !sizes || !d_tokens) return fail(s, ETS_INVALID_ARGUMENT, "ets_sample_from_logits_batch: null pointer");
+  if (rank != 2 && rank != 3)
+    return fail(s, ETS_INVALID_ARGUMENT, "ets_sample_from_logits_batch: the tensor must be [batch, vocab] or [batch, seq, vocab]");
+  if (!dtype_ok(dtype)) return fail(s, ETS_INVALID_ARGUMENT, "Unsupported dtype in sample_from_logits");
+  const int64_t vocab = sizes[rank - 1];
+  if (vocab != s->vocab)
+    return fail(s, ETS_INVALID_ARGUMENT, "ets_sample_from_logits_batch: last dimension differs from the sampler's vocab_size");
+  const int64_t batch = sizes[0];
+  if (batch < 0 || batch > s->max_batch)
+    return fail(s, ETS_INVALID_ARGUMENT, "ets_sample_from_logits_batch: batch exceeds the handle's max_batch");
+  const char* first = static_cast<const char*>(d_data);
+  int64_t stride = vocab;
+  if (rank == 3) {
+    if (sizes[1] < 1) return fail(s, ETS_INVALID_ARGUMENT, "ets_sample_from_logits_batch: empty sequence dimension");
+    // the last position of every batch entry (util.h:48-51 takes batch 0's)
+    first += static_cast<size_t>((sizes[1] - 1) * vocab) * dtype_size(dtype);
+    stride = sizes[1] * vocab;
+  }
+  return ets_sampler_sample_batch(s, first, dtype, static_cast<int32_t>(batch), stride, d_tokens, hip_stream);
+}
+
 ets_status ets_logits_to_token(const void* data, int32_t dtype, int32_t rank, const int64_t* sizes, float temperature,
                                int32_t* token_out) {
   if (!data || !sizes || !token_out || rank < 1)

@@ -263,6 +263,23 @@ def sample_from_logits(logits, sampler: Sampler, dtype: int | None = None) -> in
     return tok.value
 
 
+def sample_from_logits_batch(logits: torch.Tensor, sampler: Sampler, out: torch.Tensor | None = None,
+                             dtype: int | None = None) -> torch.Tensor:
+    """The batched adapter over a DEVICE tensor ``[B, V]`` or ``[B, S, V]`` (last position of every
+    batch entry); returns int32 ``[B]`` on the device.  The reference's adapter (util.h:25-55) reads
+    a host tensor and batch 0 only."""
+    if not logits.is_cuda or not logits.is_contiguous() or logits.dim() not in (2, 3):
+        raise SamplerError(_capi.INVALID_ARGUMENT, "sample_from_logits_batch wants a contiguous device tensor of rank 2 or 3")
+    code = dtype_code(logits) if dtype is None else dtype
+    if out is None:
+        out = torch.empty(logits.shape[0], dtype=torch.int32, device=logits.device)
+    sizes = (C.c_int64 * logits.dim())(*logits.shape)
+    stream = torch.cuda.current_stream(logits.device).cuda_stream
+    sampler._check(_capi.lib().ets_sample_from_logits_batch(sampler._h, logits.data_ptr(), code, logits.dim(), sizes,
+                                                            out.data_ptr(), stream))
+    return out
+
+
 def logits_to_token(logits, temperature: float = 0.0, dtype: int | None = None) -> int:
     """util.h:64-71: a temporary 2-argument Sampler over the tensor's last dimension."""
     keep, ptr, code, shape = _host_tensor_args(logits, dtype)

@@ -221,6 +221,17 @@ ETS_API ets_status ets_sampler_get_rng_states(ets_sampler* s, int32_t first_row,
 ETS_API ets_status ets_sample_from_logits(ets_sampler* s, const void* data, int32_t dtype, int32_t rank,
                                           const int64_t* sizes, int32_t* token_out);
 
+/* The batched adapter: sample_from_logits() for a tensor that lives in DEVICE memory and for
+ * every batch entry (the reference's adapter reads a host tensor and batch 0 only, util.h:25-55,
+ * :48-51).  `d_data` is a DEVICE pointer to a contiguous [batch, vocab] (rank 2) or
+ * [batch, seq, vocab] (rank 3: the last position of every batch entry) tensor, `sizes` a HOST
+ * array of `rank` extents, `d_tokens` a DEVICE pointer to `batch` int32.  This is the call a
+ * runner makes when its delegate leaves the logits on the GPU
+ * (backends/cuda/runtime/cuda_backend.cpp:80-81): only the tokens cross to the host.  Row b uses
+ * its own coin stream, as in ets_sampler_sample_batch(); asynchronous on `hip_stream`. */
+ETS_API ets_status ets_sample_from_logits_batch(ets_sampler* s, const void* d_data, int32_t dtype, int32_t rank,
+                                                const int64_t* sizes, int32_t* d_tokens, void* hip_stream);
+
 /* logits_to_token(const Tensor&, float temperature = 0)  -- util.h:64-71: a temporary
  * 2-argument Sampler over the tensor's last dimension. */
 ETS_API ets_status ets_logits_to_token(const void* data, int32_t dtype, int32_t rank, const int64_t* sizes,

@@ -156,6 +156,21 @@ inline int32_t sample_from_logits(const Tensor& logits_tensor, Sampler& sampler)
   return st == ETS_OK ? token : -1;
 }
 
+/// The batched adapter (no counterpart: util.h:48-51 reads batch 0 of a host tensor): `logits_tensor`
+/// describes a DEVICE-resident [batch, vocab] or [batch, seq, vocab] tensor (its const_data_ptr() is
+/// a device pointer, as a delegate that skips the copy to the host leaves it); one token per batch
+/// entry is written to the device array `d_tokens`, asynchronously on `hip_stream`.
+template <typename Tensor>
+inline ets_status sample_from_logits_batch(const Tensor& logits_tensor, Sampler& sampler, int32_t* d_tokens,
+                                           void* hip_stream = nullptr) {
+  const int32_t rank = static_cast<int32_t>(logits_tensor.dim());
+  int64_t sizes[3] = {0, 0, 0};
+  if (rank != 2 && rank != 3) return ETS_INVALID_ARGUMENT;
+  for (int32_t d = 0; d < rank; ++d) sizes[d] = static_cast<int64_t>(logits_tensor.size(d));
+  return ets_sample_from_logits_batch(sampler.handle(), logits_tensor.const_data_ptr(),
+                                      static_cast<int32_t>(logits_tensor.scalar_type()), rank, sizes, d_tokens, hip_stream);
+}
+
 /// util.h:64-71
 template <typename Tensor>
 inline int32_t logits_to_token(const Tensor& logits_tensor, const float temperature = 0.0f) {
