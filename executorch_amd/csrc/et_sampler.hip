@@ -69,6 +69,11 @@ struct ets_sampler {
   void* d_stage = nullptr;
   hipEvent_t stage_event = nullptr;
   bool stage_pending = false;
+  // the last stream a call that uses the staging copy ran on, and the event behind its launches: a
+  // call on another stream waits for it before it overwrites the device copy
+  hipEvent_t stage_done = nullptr;
+  hipStream_t stage_stream = nullptr;
+  bool stage_used = false;
   // opt-in device timing (ets_sampler_set_timing): a ring of event pairs around the launches of a
   // call, harvested when a slot is reused or the totals are read
   bool timing = false;
@@ -537,6 +542,21 @@ ets_status ensure_stage(ets_sampler* s) {
   ETS_HIP(s, hipHostMalloc(&s->h_stage, full.bytes, hipHostMallocDefault));
   ETS_HIP(s, hipMalloc(&s->d_stage, full.bytes));
   ETS_HIP(s, hipEventCreateWithFlags(&s->stage_event, hipEventDisableTiming));
+  ETS_HIP(s, hipEventCreateWithFlags(&s->stage_done, hipEventDisableTiming));
+  return ETS_OK;
+}
+
+// The device copy of the staging data is read by the launches of the call that uploaded it.  A
+// later call on the same stream is ordered behind them; one on another stream waits for the event
+// recorded behind the earlier call's last launch.
+ets_status stage_acquire(ets_sampler* s, hipStream_t stream) {
+  if (s->stage_used && s->stage_stream != stream) ETS_HIP(s, hipStreamWaitEvent(stream, s->stage_done, 0));
+  return ETS_OK;
+}
+ets_status stage_release(ets_sampler* s, hipStream_t stream) {
+  ETS_HIP(s, hipEventRecord(s->stage_done, stream));
+  s->stage_stream = stream;
+  s->stage_used = true;
   return ETS_OK;
 }
 
@@ -574,6 +594,8 @@ ets_status sample_device_configs(ets_sampler* s, const void* d_logits, int32_t d
     st = ensure_scratch(s);
     if (st != ETS_OK) return st;
   }
+  st = stage_acquire(s, stream);
+  if (st != ETS_OK) return st;
   ETS_HIP(s, hipMemcpyAsync(d, h, lay.bytes, hipMemcpyHostToDevice, stream));
   ETS_HIP(s, hipEventRecord(s->stage_event, stream));
   s->stage_pending = true;
@@ -608,7 +630,7 @@ ets_status sample_device_configs(ets_sampler* s, const void* d_logits, int32_t d
     st = rows_device(s, p, dtype, count[1 + draw], stream, draw);
     if (st != ETS_OK) return st;
   }
-  return ETS_OK;
+  return stage_release(s, stream);
 }
 
 }  // namespace
@@ -625,6 +647,8 @@ ets_status ets_sampler_create(int32_t vocab_size, float temperature, float topp,
   // counts of a row's entries are carried in floats in places (exact below 2^24)
   if (vocab_size >= (1 << 24)) return fail(nullptr, ETS_NOT_SUPPORTED, "ets_sampler_create: vocab_size must be below 16777216");
   if (max_batch < 1) return fail(nullptr, ETS_INVALID_ARGUMENT, "ets_sampler_create: max_batch must be >= 1");
+  // rows are the second dimension of several launch grids
+  if (max_batch > 65535) return fail(nullptr, ETS_NOT_SUPPORTED, "ets_sampler_create: max_batch must be at most 65535");
   ets_sampler* s = new (std::nothrow) ets_sampler();
   if (!s) return fail(nullptr, ETS_MEMORY_ALLOCATION_FAILED, "ets_sampler_create: out of host memory");
   s->vocab = vocab_size;
@@ -709,6 +733,7 @@ ets_status ets_sampler_destroy(ets_sampler* s) {
     (void)hipFree(s->d_stage);
     if (s->h_stage) (void)hipHostFree(s->h_stage);
     if (s->stage_event) (void)hipEventDestroy(s->stage_event);
+    if (s->stage_done) (void)hipEventDestroy(s->stage_done);
     for (int i = 0; i < ets_sampler::kTimingSlots; ++i) {
       if (s->t_begin[i]) (void)hipEventDestroy(s->t_begin[i]);
       if (s->t_end[i]) (void)hipEventDestroy(s->t_end[i]);
@@ -855,6 +880,8 @@ ets_status ets_sampler_gumbel_max_batch(ets_sampler* s, const void* d_logits, in
       s->stage_pending = false;
     }
     std::memcpy(s->h_stage, temperatures, sizeof(float) * n_temperatures);
+    st = stage_acquire(s, stream);
+    if (st != ETS_OK) return st;
     ETS_HIP(s, hipMemcpyAsync(s->d_stage, s->h_stage, sizeof(float) * n_temperatures, hipMemcpyHostToDevice, stream));
     ETS_HIP(s, hipEventRecord(s->stage_event, stream));
     s->stage_pending = true;
@@ -890,6 +917,10 @@ ets_status ets_sampler_gumbel_max_batch(ets_sampler* s, const void* d_logits, in
   hipLaunchKernelGGL(ets::gumbel_finish_kernel, dim3(batch), dim3(64), 0, stream, s->d_partials, splits,
                      d_noise ? 0 : 1, s->d_rng, d_tokens);
   ETS_HIP(s, hipGetLastError());
+  if (n_temperatures > 1) {
+    st = stage_release(s, stream);
+    if (st != ETS_OK) return st;
+  }
   return timing_end(s, stream, slot);
 }
 
@@ -1008,12 +1039,36 @@ ets_status ets_logits_to_token(const void* data, int32_t dtype, int32_t rank, co
     return fail(nullptr, ETS_INVALID_ARGUMENT, "ets_logits_to_token: null pointer or rank < 1");
   const int64_t vocab = sizes[rank - 1];
   if (vocab < 1 || vocab > INT32_MAX) return fail(nullptr, ETS_INVALID_ARGUMENT, "ets_logits_to_token: bad vocab size");
-  ets_sampler* s = nullptr;
-  ets_status st = ets_sampler_create_default(static_cast<int32_t>(vocab), temperature, 1, &s);
-  if (st != ETS_OK) return st;
-  st = ets_sample_from_logits(s, data, dtype, rank, sizes, token_out);
+  // The reference builds a temporary Sampler per call (util.h:67-69), which costs it nothing; here
+  // a handle owns device buffers, so each thread keeps the one it built last and reuses it while
+  // the device and the vocabulary stay the same.  What the temporary object would have had -- the
+  // 2-argument constructor's parameters and a clock seed -- is set again on every call.
+  struct Cached {
+    ets_sampler* handle = nullptr;
+    ~Cached() { ets_sampler_destroy(handle); }
+  };
+  thread_local Cached cache;
+  int device = -1;
+  if (hipGetDevice(&device) != hipSuccess) device = -1;
+  ets_sampler* s = cache.handle;
+  if (!s || s->vocab != vocab || s->device != device) {
+    ets_sampler_destroy(cache.handle);
+    cache.handle = nullptr;
+    ets_status st = ets_sampler_create_default(static_cast<int32_t>(vocab), temperature, 1, &cache.handle);
+    if (st != ETS_OK) return st;
+    s = cache.handle;
+  } else {
+    s->inv_temperature = inverse_temperature_ctor(temperature);  // sampler.cpp:183-187
+    s->topp = 0.9f;
+    s->topk = 0;
+    const uint64_t seed = static_cast<uint64_t>(std::time(nullptr));
+    if (s->inv_temperature != 0.0f) {  // (the arg-max draws no coin)
+      ets_status st = ets_sampler_set_rng_states(s, 0, 1, &seed);
+      if (st != ETS_OK) return st;
+    }
+  }
+  ets_status st = ets_sample_from_logits(s, data, dtype, rank, sizes, token_out);
   if (st != ETS_OK) g_thread_error = s->last_error;
-  ets_sampler_destroy(s);
   return st;
 }
 

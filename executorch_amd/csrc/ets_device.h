@@ -427,11 +427,13 @@ __device__ __forceinline__ void wave_resolve(float& s, int& found, const uint32_
       ballot = __ballot(special);
       S_end = __shfl(S_incl, 63);
     }
-    if (!ballot) {
+    // (lanes already consumed hold no increment, but a running sum that is above the threshold
+    // before anything is added flags them too: the walk only ever looks ahead)
+    const int j = next_event(ballot, consumed, 64);
+    if (j == 64) {
       s = sum_value(S_end, ss.kb);
       return;
     }
-    const int j = __ffsll(static_cast<long long>(ballot)) - 1;
     float sj = 0.0f;
     int fj = -1;
     if (lane == j) {
@@ -737,7 +739,7 @@ __device__ __forceinline__ bool seq_sum_rounds(SeqSum& st, const uint32_t (&bits
       bool event = S_upto >= (1u << 24);
       if (!event) event = sum_value(S_upto, ss.kb) > threshold;
       const uint64_t ballot = __ballot(event && lane < kSlots);
-      star = ballot ? __ffsll(static_cast<long long>(ballot)) - 1 : kSlots;
+      star = next_event(ballot, resume, kSlots);  // never a slot that has been consumed: the rounds end
       S_front = star > 0 && star < kSlots ? readlane_u32(S_upto, star - 1) : ss.S;
       S_all = readlane_u32(S_upto, kSlots - 1);
     }

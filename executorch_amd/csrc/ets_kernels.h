@@ -231,8 +231,8 @@ typedef __attribute__((address_space(3))) uint64_t* LdsKeys;
 // ---- sorting candidate keys -----------------------------------------------------------------
 // Ascending sort of N keys (a power of two) that already sit in LDS (and are visible to the
 // workgroup).  Bitonic network; every wave owns a contiguous run of W keys, and the sub-stages
-// whose partners lie inside one run (distance < W) are done by that wave alone, back to back
-// without workgroup barriers -- LDS serves one wave's accesses in order -- so only the
+// whose partners lie inside one run (distance < W) are done by that wave alone, without workgroup
+// barriers (a fence that waits for the wave's own accesses separates them), so only the
 // log2(N / W) long-distance sub-stages of each merge pay a barrier.  Ends with a barrier.
 __device__ void sort_keys_lds(LdsKeys lds, int N) {
   const int lane = threadIdx.x & 63;
@@ -268,9 +268,12 @@ __device__ void sort_keys_lds(LdsKeys lds, int N) {
             mine[l] = a;
           }
         }
-        // other lanes of this wave read these keys next: keep the compiler from carrying values
-        // across sub-stages in registers
-        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        // other lanes of this wave read these keys next.  The stores must have been performed, not
+        // merely issued: a workgroup-scope fence makes the wave wait for its outstanding LDS (and
+        // flat) accesses, whichever instructions the compiler chose for the pointer, and the wave
+        // barrier keeps the sub-stages apart in the instruction stream.
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");
+        __builtin_amdgcn_wave_barrier();
       }
     }
     if (k >= W) __syncthreads();  // the next merge starts with a long-distance sub-stage, or this was the last
@@ -574,7 +577,7 @@ __device__ __forceinline__ bool scan_row(const ScanArgs& a, SeqSum& st, BlockScr
       a.list[slot] = ent;
     }
   };
-  if (ALIGNED) {
+  if (ALIGNED && V >= VE) {  // (a row shorter than one vector has no vector to prefetch)
     const int nvec = V / VE;
     const uint4* vec = reinterpret_cast<const uint4*>(a.logits);
     constexpr int per_iter = kBlock * kGroup;
@@ -699,7 +702,7 @@ __device__ uint64_t* radix_sort_block(uint64_t* a, uint64_t* b, int n, LdsU32 ta
   for (int shift = 32; shift < 64; shift += 8) {
     // ---- count
     for (int d = lane; d < 256; d += 64) mine[d] = 0u;
-    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");
     for (int base = c0; base < c1; base += 64 * 8) {  // eight loads in flight
       uint64_t entry[8];
 #pragma unroll
@@ -767,7 +770,7 @@ __device__ uint64_t* radix_sort_block(uint64_t* a, uint64_t* b, int n, LdsU32 ta
       const uint32_t digit = static_cast<uint32_t>(entry >> shift) & 255u;
       // the lanes with this digit: every lane sets its bit in the digit's word, then reads the word
       if (valid) __hip_atomic_fetch_or(&board[digit], 1ull << lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
-      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");  // (waits for the wave's own LDS accesses)
       const uint64_t peers = valid ? board[digit] : 0ull;
       const uint32_t rank = static_cast<uint32_t>(__popcll(peers & ((1ull << lane) - 1ull)));
       uint32_t position = 0u;
@@ -775,12 +778,12 @@ __device__ uint64_t* radix_sort_block(uint64_t* a, uint64_t* b, int n, LdsU32 ta
         position = mine[digit];
         b[position + rank] = entry;
       }
-      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");  // every peer has read the position
+      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");  // every peer has read the position
       if (valid && rank == 0u) {
         mine[digit] = position + static_cast<uint32_t>(__popcll(peers));
         board[digit] = 0ull;
       }
-      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");
       }
     }
     __syncthreads();
@@ -826,7 +829,6 @@ __device__ int32_t draw_general(const char* logits, int V, float inv, float m, f
   dbg.n_candidates = n0;
   if (n0 == 0) return -1;  // the reference reads probindex[-1] here
   const int N = pow2_ceil(n0);
-  const uint64_t* keys;
   if (N <= cap) {
     __syncthreads();
     if (tid == 0) sm.counter = 0u;
@@ -841,11 +843,13 @@ __device__ int32_t draw_general(const char* logits, int V, float inv, float m, f
     for (int i = n0 + tid; i < N; i += kBlock) lds_keys[i] = ~0ull;
     __syncthreads();
     sort_keys_lds((LdsKeys)lds_keys, N);
-    keys = lds_keys;
-  } else {
-    // the host sizes the scratch for two buffers of V entries and the key buffer for the sort's table
-    keys = radix_sort_block(scratch, scratch + scratch_cap / 2, V, (LdsU32)lds_keys, sm);
+    // (keys in LDS are walked through an LDS-typed pointer, keys in global memory through a global
+    // one: no generic pointer that could stand for either)
+    const int pos = draw_from_sorted((LdsKeys)lds_keys, n0, n0, use_topk, topk, topp, coin, dbg, sm);
+    return static_cast<int32_t>(static_cast<uint32_t>(lds_keys[pos]));
   }
+  // the host sizes the scratch for two buffers of V entries and the key buffer for the sort's table
+  const uint64_t* keys = radix_sort_block(scratch, scratch + scratch_cap / 2, V, (LdsU32)lds_keys, sm);
   const int pos = draw_from_sorted(keys, n0, n0, use_topk, topk, topp, coin, dbg, sm);
   return static_cast<int32_t>(static_cast<uint32_t>(keys[pos]));
 }

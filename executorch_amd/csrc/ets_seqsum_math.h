@@ -79,6 +79,20 @@ ETS_HD ParityInc compose(ParityInc a, ParityInc b) {
   return c;
 }
 
+// Which lane (or slot) an ordered walk works on next: the first one flagged in `events` at or
+// after `from`, or `count` when there is none.  Every ordered walk of the sampler advances with
+//   j = next_event(events, from, 64); ...; from = j + 1;
+// so it takes at most `count` steps whatever the flags say -- also on data that is not what the
+// walk was written for (probabilities that are not sorted, a threshold below the starting sum,
+// NaN), where flags of lanes already consumed could otherwise call the walk back for good.
+ETS_HD int next_event(uint64_t events, int from, int count) {
+  if (from >= 64) return count;
+  const uint64_t ahead = events & (~0ull << from);
+  if (!ahead) return count;
+  const int j = __builtin_ctzll(ahead);
+  return j < count ? j : count;
+}
+
 // Integer view of the running sum: s = S * 2^(kb - 150) with kb the biased exponent (>= 1).
 struct SumState {
   uint32_t S;
@@ -156,6 +170,70 @@ ETS_HD uint32_t fast_inc(uint32_t abits, int kb, bool& tie) {
   const float r = __builtin_rintf(t);
   tie = tie || (__builtin_fabsf(t - r) == 0.5f);
   return static_cast<uint32_t>(r);
+}
+
+// ---- runs of equal addends ----------------------------------------------------------------------
+// c copies of p are added to s one after the other (s = s + p in fp32); the walk stops behind the
+// first copy that takes s above T.  Returns that copy's number (1-based), or 0 when all c copies
+// were added without exceeding T.  One lane.
+ETS_HD uint32_t run_walk(float& s, float p, uint32_t c, float T) {
+  uint32_t left = c, done = 0u;
+  while (left > 0u) {
+    const SumState ss = sum_state(s);
+    const float scale = ss.kb >= 64 && ss.kb <= 250 ? __builtin_bit_cast(float, static_cast<uint32_t>(277 - ss.kb) << 23) : 0.0f;
+    const float t = p * scale;
+    if (scale == 0.0f || !(t < 16777216.0f)) {  // out of the shortcut's range: one native add
+      s = s + p;
+      --left;
+      ++done;
+      if (s > T) return done;
+      continue;
+    }
+    const float r = __builtin_rintf(t);
+    uint32_t n = static_cast<uint32_t>(r);
+    uint32_t S = ss.S;
+    if (__builtin_fabsf(t - r) == 0.5f) {
+      // a half-ulp tie: the first add goes natively and leaves an even integer; from an even integer
+      // every further copy adds floor(t), or one more if that is odd
+      s = s + p;
+      --left;
+      ++done;
+      if (s > T) return done;
+      const SumState s2 = sum_state(s);
+      if (s2.kb != ss.kb) continue;
+      const uint32_t n0 = static_cast<uint32_t>(__builtin_floorf(t));
+      n = n0 + (n0 & 1u);
+      S = s2.S;
+    }
+    if (n == 0u) return 0u;  // absorbed: no copy changes the sum
+    // s' > T  <=>  S' >= floor(T / ulp) + 1; the sum must also stay below 2^24 ulps
+    const float tt = T * scale;
+    uint32_t limit = 1u << 24;
+    if (tt < 16777216.0f) {
+      const uint32_t Tn = tt >= 0.0f ? static_cast<uint32_t>(__builtin_floorf(tt)) + 1u : 0u;
+      limit = Tn < limit ? Tn : limit;
+    }
+    if (S >= limit) {  // (cannot happen: the walk would have stopped) one native add
+      s = s + p;
+      --left;
+      ++done;
+      if (s > T) return done;
+      continue;
+    }
+    const uint32_t stay = (limit - S - 1u) / n;  // copies after which the integer is still below `limit`
+    if (stay >= left) {
+      s = sum_value(S + left * n, ss.kb);
+      return 0u;
+    }
+    s = sum_value(S + stay * n, ss.kb);
+    left -= stay;
+    done += stay;
+    s = s + p;  // the copy that reaches the limit, natively
+    --left;
+    ++done;
+    if (s > T) return done;
+  }
+  return 0u;
 }
 
 }  // namespace ets

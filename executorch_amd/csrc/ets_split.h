@@ -630,8 +630,7 @@ __device__ __forceinline__ void resolve_lanes(float& s, const uint32_t (&bits)[8
     const uint32_t done_before = cur > 0 ? readlane_u32(pre, cur - 1) : 0u;
     const uint32_t room = (1u << 24) - ss.S;
     const uint64_t over = __ballot(lane >= cur && pre - done_before >= room);
-    const uint64_t events = (tie & (~0ull << cur)) | over;
-    const int j = events ? __ffsll(static_cast<long long>(events)) - 1 : 64;
+    const int j = next_event(tie | over, cur, 64);
     uint32_t S_j = ss.S;
     if (j > cur) S_j += readlane_u32(pre, j - 1) - done_before;
     if (j == 64) {
@@ -848,69 +847,6 @@ __device__ __forceinline__ HistPlan split_plan(const uint32_t* hist, float a_tot
 // No sort, no gather; the token is the k-th occurrence, in index order, of the probability the
 // walk stops at.
 
-// c copies of p are added to s one after the other (s = s + p in fp32); the walk stops behind the
-// first copy that takes s above T.  Returns that copy's number (1-based), or 0 when all c copies
-// were added without exceeding T.  One lane.
-__device__ __forceinline__ uint32_t run_walk(float& s, float p, uint32_t c, float T) {
-  uint32_t left = c, done = 0u;
-  while (left > 0u) {
-    const SumState ss = sum_state(s);
-    const float scale = ss.kb >= 64 && ss.kb <= 250 ? __uint_as_float(static_cast<uint32_t>(277 - ss.kb) << 23) : 0.0f;
-    const float t = p * scale;
-    if (scale == 0.0f || !(t < 16777216.0f)) {  // out of the shortcut's range: one native add
-      s = s + p;
-      --left;
-      ++done;
-      if (s > T) return done;
-      continue;
-    }
-    const float r = __builtin_rintf(t);
-    uint32_t n = static_cast<uint32_t>(r);
-    uint32_t S = ss.S;
-    if (__builtin_fabsf(t - r) == 0.5f) {
-      // a half-ulp tie: the first add goes natively and leaves an even integer; from an even integer
-      // every further copy adds floor(t), or one more if that is odd
-      s = s + p;
-      --left;
-      ++done;
-      if (s > T) return done;
-      const SumState s2 = sum_state(s);
-      if (s2.kb != ss.kb) continue;
-      const uint32_t n0 = static_cast<uint32_t>(__builtin_floorf(t));
-      n = n0 + (n0 & 1u);
-      S = s2.S;
-    }
-    if (n == 0u) return 0u;  // absorbed: no copy changes the sum
-    // s' > T  <=>  S' >= floor(T / ulp) + 1; the sum must also stay below 2^24 ulps
-    const float tt = T * scale;
-    uint32_t limit = 1u << 24;
-    if (tt < 16777216.0f) {
-      const uint32_t Tn = tt >= 0.0f ? static_cast<uint32_t>(__builtin_floorf(tt)) + 1u : 0u;
-      limit = Tn < limit ? Tn : limit;
-    }
-    if (S >= limit) {  // (cannot happen: the walk would have stopped) one native add
-      s = s + p;
-      --left;
-      ++done;
-      if (s > T) return done;
-      continue;
-    }
-    const uint32_t stay = (limit - S - 1u) / n;  // copies after which the integer is still below `limit`
-    if (stay >= left) {
-      s = sum_value(S + left * n, ss.kb);
-      return 0u;
-    }
-    s = sum_value(S + stay * n, ss.kb);
-    left -= stay;
-    done += stay;
-    s = s + p;  // the copy that reaches the limit, natively
-    --left;
-    ++done;
-    if (s > T) return done;
-  }
-  return 0u;
-}
-
 struct RunSlotRec {
   uint32_t meta;  // kind << 8 | kb
   uint32_t inc_a, inc_b;
@@ -969,8 +905,7 @@ __device__ __forceinline__ int resolve_run_group(float& s, int t, uint32_t befor
       limit = Tn < limit ? Tn : limit;
     }
     const uint32_t room = limit > ss.S ? limit - ss.S : 0u;
-    const uint64_t events = __ballot(odd_one || (live && incl >= room));
-    const int j = events ? __ffsll(static_cast<long long>(events)) - 1 : 64;
+    const int j = next_event(__ballot(odd_one || (live && incl >= room)), cur, 64);
     uint32_t S_j = ss.S;
     if (j > 0) S_j += readlane_u32(incl, j > 63 ? 63 : j - 1);  // lanes below cur hold 0
     if (j == 64) {

@@ -24,7 +24,9 @@
  *
  * Every function returns an ets_status; none aborts.  Calls on one handle must be serialized
  * by the caller (as for the reference, text_decoder_runner.h:81-82); distinct handles are
- * independent.
+ * independent.  A handle's work buffers are reused from call to call: issue its calls on ONE
+ * stream, or order a call on another stream behind the previous one yourself (the per-row
+ * parameter and temperature tables are the exception: the library orders their reuse).
  */
 #ifndef ET_SAMPLER_H_
 #define ET_SAMPLER_H_
@@ -77,7 +79,7 @@ typedef struct {
  * negative inverse, as there).  `max_batch` (>= 1) is the largest batch later passed to
  * ets_sampler_sample_batch(); row b starts with xorshift64* state rng_seed + b, so row 0 is
  * the reference object's own stream.  The handle lives on the current HIP device.
- * vocab_size must be below 2^24 (ETS_NOT_SUPPORTED otherwise). */
+ * vocab_size must be below 2^24 and max_batch at most 65535 (ETS_NOT_SUPPORTED otherwise). */
 ETS_API ets_status ets_sampler_create(int32_t vocab_size, float temperature, float topp, uint64_t rng_seed,
                                       int32_t max_batch, ets_sampler** out);
 
