@@ -4,14 +4,25 @@
 
 A step is one batched sampling call over one [B, vocab] matrix of synthetic logits already
 resident in HBM.  Steps walk a ring of distinct matrices larger than the 256 MB Infinity Cache so
-that every step reads its logits from HBM.  Prints one JSON line (rows/s, roofline of the
-dominant kernel, the CPU baseline timed on this box's host cores).
+that every step reads its logits from HBM.  Prints one JSON line: rows/s over exactly K steps, the
+roofline of the step's launches (median of five repeats, HIP events on the launch stream), every
+workload of the benchmark contract at its own shape, launch and read floors, and the reference's
+CPU sampler timed on this box's host cores.
+
+    python bench.py --parse-pmc FETCH_DIR WRITE_DIR --out profiles/NAME.json
+
+turns two rocprofv3 --pmc runs of this script (FETCH_SIZE, then WRITE_SIZE, each with --copy-probe)
+into the small JSON file the `roofline.traffic` figure is read from.
 """
 from __future__ import annotations
 
 import argparse
+import csv
+import glob
 import json
 import os
+import platform
+import statistics
 import sys
 import time
 from concurrent.futures import ThreadPoolExecutor
@@ -21,11 +32,8 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
-
-# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by
-# the factors a 256 MiB device copy gives in the same runs (profiles/sample_rows_kernel_cfg2.md has
-# the commands and the raw counters): 9221 KiB * 2.00 fetched + 3780 KiB * 1.00 written.
-MEASURED_TRAFFIC_BYTES = {"cfg2": (8940 * 2.00 + 3817 * 1.00) * 1024}
+COPY_PROBE_BYTES = 256 << 20
+STEP_KERNELS = ("split_pass1_kernel", "split_pass2_kernel", "split_finish_kernel", "sample_rows_kernel")
 
 
 def synth_logits_device(w, count, torch, dev):
@@ -54,10 +62,43 @@ def synth_logits_device(w, count, torch, dev):
             hot = torch.randint(0, w.vocab, (w.batch // 2, 1), generator=g, device=dev)
             gum.scatter_add_(1, hot, torch.full_like(hot, 12.0, dtype=torch.float32))
             x[1::2] = gum
+            del u, gum
         else:
             raise ValueError(w.kind)
         ring.append(x.to(tdt))
+        del x
     return ring
+
+
+def cpu_model() -> str:
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return platform.processor() or "unknown"
+
+
+def physical_cores() -> int:
+    try:
+        seen = set()
+        phys = core = None
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("physical id"):
+                    phys = line.split(":")[1].strip()
+                elif line.startswith("core id"):
+                    core = line.split(":")[1].strip()
+                elif not line.strip() and phys is not None and core is not None:
+                    seen.add((phys, core))
+                    phys = core = None
+        if seen:
+            return len(seen)
+    except OSError:
+        pass
+    return os.cpu_count() or 1
 
 
 def cpu_baseline(w, gpu_tokens, seconds_budget=12.0):
@@ -75,6 +116,8 @@ def cpu_baseline(w, gpu_tokens, seconds_budget=12.0):
     want, _ = O.sample_rows(x, w.dtype, O.inv_temperature(w.temperature), w.topp, 0, W.coin_seeds(w, rows).copy(),
                             mode=O.MODE_UPCAST, tie=O.TIE_STABLE, threads=8)
     mismatches = int((np.asarray(gpu_tokens)[:rows] != want).sum())
+    # worker threads: this job's share of the host (16 threads per GPU on the benchmark boxes), not
+    # every core the machine reports
     cores = max(1, min(16, os.cpu_count() or 1))
     use_ref = O.have_ref()
 
@@ -106,22 +149,30 @@ def cpu_baseline(w, gpu_tokens, seconds_budget=12.0):
         "sample": f"{rows} rows of {w.name} step 0, each sampled {reps} times by its own Sampler, native "
                   f"{W.DTYPE_NAMES[w.dtype]} sample<T>, {cores} threads ({dt:.1f} s)",
         "rows_per_s_one_core": one_core,
+        "cpu_model": cpu_model(),
+        "physical_cores": physical_cores(),
+        "logical_cpus": os.cpu_count(),
+        "compiler": "g++ -std=c++17 -O2 (sampler.cpp as the reference builds it)" if use_ref else "g++ -std=c++17 -O2 (restatement)",
         "parity": {"rows_checked": rows, "token_mismatches_vs_oracle": mismatches},
     }
 
 
-def timed_us(fn, reps, torch):
-    """Mean duration of fn() in microseconds, from events on the current stream."""
+def timed_us(fn, reps, torch, repeats=1):
+    """Duration of fn() in microseconds from events on the current stream: the mean over `reps`
+    calls, or with repeats > 1 the median of that many such means."""
     for _ in range(3):
         fn()
     torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(reps):
-        fn()
-    e1.record()
-    torch.cuda.synchronize()
-    return e0.elapsed_time(e1) * 1e3 / reps
+    means = []
+    for _ in range(repeats):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        means.append(e0.elapsed_time(e1) * 1e3 / reps)
+    return statistics.median(means)
 
 
 def bench_logit_chain(w, logits, torch, dev):
@@ -147,8 +198,11 @@ def bench_logit_chain(w, logits, torch, dev):
 
 def bench_host_buffers(w, s, logits, out, torch):
     """What the same step costs when the boundary is handed HOST memory: one batch copied from
-    pinned host memory to the device and sampled (the PCIe-inclusive rate; never `value`), and the
-    reference-shaped single-row entry ets_sampler_sample() on a pageable host row."""
+    pinned host memory to the device and sampled (the PCIe-inclusive rate; never `value`), the
+    reference-shaped single-row entry ets_sampler_sample() on a pageable host row, and
+    logits_to_token() (util.h:64-71), which the reference calls once per decoded token."""
+    import executorch_amd as ea
+
     host = torch.empty(logits.shape, dtype=logits.dtype, pin_memory=True)
     host.copy_(logits)
     staged = torch.empty_like(logits)
@@ -166,8 +220,14 @@ def bench_host_buffers(w, s, logits, out, torch):
     for _ in range(50):
         one.sample(row)
     row_us = (time.perf_counter() - t0) * 1e6 / 50
+    for _ in range(3):
+        ea.logits_to_token(row, w.temperature)
+    t0 = time.perf_counter()
+    for _ in range(50):
+        ea.logits_to_token(row, w.temperature)
+    l2t_us = (time.perf_counter() - t0) * 1e6 / 50
     return {"batch_from_pinned_host_us": batch_us, "rows_per_s_pcie_inclusive": w.batch / (batch_us * 1e-6),
-            "single_row_host_entry_us": row_us}
+            "single_row_host_entry_us": row_us, "logits_to_token_us": l2t_us}
 
 
 def bench_gumbel(w, s, ring, out, torch):
@@ -204,8 +264,7 @@ def bench_greedy(w, ring, out, torch):
 
 def bench_configs(w, s, ring, out, steps, torch):
     """ets_sampler_sample_batch_configs on the same ring: every row with the workload's own
-    parameters (one launch, plus the upload of the per-row table), and a mix of four kinds of rows
-    (one launch per kind)."""
+    parameters, and a mix of four kinds of rows (one group of launches per kind)."""
     uniform = [(w.temperature, w.topp, 0, 0)] * w.batch
     kinds = [(w.temperature, w.topp, 0, 0), (0.0, w.topp, 0, 0), (1.0, 1.0, 0, 0), (0.8, w.topp, 40, 0)]
     mixed = [kinds[b % 4] for b in range(w.batch)]
@@ -225,7 +284,7 @@ def bench_configs(w, s, ring, out, steps, torch):
 def bench_draw_modes(w, logits, out, torch):
     """The other element types and draws on the headline's shape and rows: the same matrix as
     fp16 / fp32, each with the workload's top-p, the multinomial draw (top-p 1) and top-k 40
-    (microseconds per batch, one launch each)."""
+    (microseconds per batch)."""
     import executorch_amd as ea
 
     res = {}
@@ -239,8 +298,7 @@ def bench_draw_modes(w, logits, out, torch):
 
 
 def bench_batch_sweep(w, torch, dev):
-    """The headline's rows at other batch sizes: one workgroup per row, so a batch of 64 occupies a
-    quarter of the 256 CUs and larger batches run several rows per CU one after another."""
+    """The headline's rows at other batch sizes."""
     import executorch_amd as ea
 
     res = {}
@@ -254,25 +312,149 @@ def bench_batch_sweep(w, torch, dev):
         s = ea.Sampler(w.vocab, w.temperature, w.topp, w.coin_seed, max_batch=rows)
         out = torch.empty(rows, dtype=torch.int32, device=dev)
         us = timed_us(lambda: s.sample_batch(x, out=out), 30, torch)
-        res[f"B{rows}"] = {"us_per_batch": us, "rows_per_s": rows / (us * 1e-6)}
+        gbs = rows * w.vocab * 2 / (us * 1e-6) / 1e9
+        res[f"B{rows}"] = {"us_per_batch": us, "rows_per_s": rows / (us * 1e-6), "frac_of_hbm_peak": gbs / HBM_PEAK_GBS}
     return res
 
 
-def bench_flat_rows(torch, dev):
-    """Near-flat rows, where every entry is a top-p candidate and the draw sorts the whole row
-    (cfg3's rows: vocab 151936, fp16, N(0, 0.5), T=1, top-p 0.95), 64 rows per batch."""
+def bench_all_configs(torch, dev):
+    """Every workload of the benchmark contract at its own batch, element type and parameters:
+    microseconds per step (median of five repeats, device time), rows/s, and the step's algorithmic
+    bytes (B x V x element size, read once) against the HBM peak.  Small rings (at least two
+    matrices, more where they are cheap) keep this bounded; cfg1 also runs at temperature 0."""
+    import dataclasses
+
     import executorch_amd as ea
     from executorch_amd import workloads as W
 
-    w = W.WORKLOADS["cfg3"]
-    rows = 64
-    g = torch.Generator(device=dev)
-    g.manual_seed(7)
-    x = (torch.randn((rows, w.vocab), generator=g, device=dev, dtype=torch.float32) * 0.5).to(torch.float16)
-    s = ea.Sampler(w.vocab, w.temperature, w.topp, w.coin_seed, max_batch=rows)
-    out = torch.empty(rows, dtype=torch.int32, device=dev)
-    us = timed_us(lambda: s.sample_batch(x, out=out), 5, torch)
-    return {"us_per_batch": us, "rows": rows, "rows_per_s": rows / (us * 1e-6)}
+    res = {}
+    for name in ("cfg1_greedy", "cfg1", "cfg2", "cfg3", "cfg4", "cfg5"):
+        w = W.WORKLOADS[name]
+        n_ring = max(2, min(40, (320 << 20) // w.bytes_per_step))
+        ring = synth_logits_device(dataclasses.replace(w, data_seed=w.data_seed + 100), n_ring, torch, dev)
+        s = ea.Sampler(w.vocab, w.temperature, w.topp, w.coin_seed, max_batch=w.batch)
+        out = torch.empty(w.batch, dtype=torch.int32, device=dev)
+        state = {"i": 0}
+
+        def step():
+            s.sample_batch(ring[state["i"] % n_ring], out=out)
+            state["i"] += 1
+
+        reps = 4 if name in ("cfg3", "cfg5") else 20
+        us = timed_us(step, reps, torch, repeats=5)
+        gbs = w.bytes_per_step / (us * 1e-6) / 1e9
+        res[name] = {"vocab": w.vocab, "batch": w.batch, "dtype": W.DTYPE_NAMES[w.dtype], "temperature": w.temperature,
+                     "top_p": w.topp, "us_per_step": us, "rows_per_s": w.batch / (us * 1e-6),
+                     "algorithmic_bytes": w.bytes_per_step, "gbs": gbs, "frac_of_hbm_peak": gbs / HBM_PEAK_GBS,
+                     "ring_matrices": n_ring, "steps_per_repeat": reps, "repeats": 5}
+        del ring, s
+        torch.cuda.empty_cache()
+    return res
+
+
+def bench_floors(w, ring, torch, dev):
+    """What no kernel of this shape can beat on this box: an empty launch, and a kernel that only
+    reads one step's logits (the ring keeps the reads in HBM), with as many workgroups as the step
+    has rows and with enough to fill the chip."""
+    import ctypes as C
+
+    from executorch_amd import _capi
+
+    L = _capi.lib()
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    sink = torch.zeros(4, dtype=torch.int32, device=dev)
+    empty_us = timed_us(lambda: L.ets_test_empty_launch(stream), 200, torch, repeats=5)
+    res = {"empty_launch_us": empty_us}
+    state = {"i": 0}
+    for wgs in (w.batch, 256, 1024, 4096):
+        def step():
+            x = ring[state["i"] % len(ring)]
+            L.ets_test_read_floor(x.data_ptr(), C.c_int64(w.bytes_per_step), wgs, sink.data_ptr(), stream)
+            state["i"] += 1
+        us = timed_us(step, 100, torch, repeats=5)
+        res[f"read_{wgs}_workgroups_us"] = us
+        res[f"read_{wgs}_workgroups_gbs"] = w.bytes_per_step / (us * 1e-6) / 1e9
+    return res
+
+
+def bench_graph(w, s, ring, out, torch, dev):
+    """The same step captured into a HIP graph and replayed (the launches of one call as one graph
+    launch), for the launch-bound batch of the headline.  One graph per ring matrix."""
+    try:
+        side = torch.cuda.Stream(device=dev)
+        graphs = []
+        n = min(len(ring), 8)
+        with torch.cuda.stream(side):
+            for i in range(n):
+                s.sample_batch(ring[i], out=out)  # warm: buffers allocated, attributes set
+            torch.cuda.synchronize()
+            for i in range(n):
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g, stream=side):
+                    s.sample_batch(ring[i], out=out)
+                graphs.append(g)
+        state = {"i": 0}
+
+        def step():
+            graphs[state["i"] % n].replay()
+            state["i"] += 1
+
+        us = timed_us(step, 50, torch, repeats=5)
+        return {"us_per_step": us, "rows_per_s": w.batch / (us * 1e-6), "graphs": n}
+    except Exception as e:  # capture is not supported by every runtime build
+        return {"us_per_step": None, "error": str(e)[:200]}
+
+
+def parse_pmc(fetch_dir, write_dir, out_path):
+    """FETCH_SIZE / WRITE_SIZE (KiB per dispatch) of the step's kernels and of the 256 MiB copy probe
+    from two rocprofv3 counter-collection runs -> HBM bytes per step."""
+    def collect(path, counter):
+        per = {}
+        for f in glob.glob(os.path.join(path, "**", "*counter_collection.csv"), recursive=True):
+            for r in csv.DictReader(open(f)):
+                if r["Counter_Name"] != counter:
+                    continue
+                per.setdefault(r["Kernel_Name"], []).append(float(r["Counter_Value"]))
+        return per
+
+    fetch, write = collect(fetch_dir, "FETCH_SIZE"), collect(write_dir, "WRITE_SIZE")
+
+    def mean_of(per, key):
+        vals = [v for k, vs in per.items() if key in k for v in vs]
+        return (sum(vals) / len(vals), len(vals)) if vals else (None, 0)
+
+    copy_f, _ = mean_of(fetch, "copyBuffer")
+    copy_w, _ = mean_of(write, "copyBuffer")
+    probe_kib = COPY_PROBE_BYTES / 1024
+    res = {"copy_probe_bytes": COPY_PROBE_BYTES, "copy_fetch_kib": copy_f, "copy_write_kib": copy_w,
+           "fetch_factor": probe_kib / copy_f if copy_f else None, "write_factor": probe_kib / copy_w if copy_w else None,
+           "kernels": {}}
+    total = 0.0
+    for k in STEP_KERNELS:
+        f, nf = mean_of(fetch, k)
+        wv, nw = mean_of(write, k)
+        if f is None and wv is None:
+            continue
+        res["kernels"][k] = {"fetch_kib": f, "write_kib": wv, "dispatches": [nf, nw]}
+        if f is not None and res["fetch_factor"]:
+            total += f * res["fetch_factor"] * 1024
+        if wv is not None and res["write_factor"]:
+            total += wv * res["write_factor"] * 1024
+    res["traffic_bytes_per_step"] = total
+    with open(out_path, "w") as fo:
+        json.dump(res, fo, indent=1)
+        fo.write("\n")
+    print(json.dumps(res))
+
+
+def measured_traffic(name):
+    """HBM bytes per step from the committed counter summary of this workload, or None."""
+    path = os.path.join(ROOT, "profiles", f"traffic_{name}.json")
+    try:
+        with open(path) as f:
+            return json.load(f).get("traffic_bytes_per_step"), os.path.relpath(path, ROOT)
+    except (OSError, ValueError):
+        return None, None
 
 
 def main():
@@ -283,12 +465,16 @@ def main():
     ap.add_argument("--workload", default="cfg2")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true",
-                    help="skip the logit-chain, per-row-config and host-buffer figures (a profile of this "
-                         "command then holds the headline kernel only)")
+                    help="only the headline loop (a profile of this command then holds its kernels only)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run five 256 MiB device copies: a kernel of known traffic that calibrates "
                          "FETCH_SIZE / WRITE_SIZE when this command runs under rocprofv3 --pmc")
+    ap.add_argument("--parse-pmc", nargs=2, metavar=("FETCH_DIR", "WRITE_DIR"))
+    ap.add_argument("--out", default=None)
     args = ap.parse_args()
+    if args.parse_pmc:
+        parse_pmc(args.parse_pmc[0], args.parse_pmc[1], args.out or os.path.join(ROOT, "profiles", f"traffic_{args.workload}.json"))
+        return
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; rows are independent, so more GPUs would each take "
               "a slice of the batch with no communication.  Run with --gpus 1.", file=sys.stderr)
@@ -319,7 +505,7 @@ def main():
     got = chk.sample_batch(dx).cpu().numpy()
 
     if args.copy_probe:
-        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_()
+        src = torch.empty(COPY_PROBE_BYTES, dtype=torch.uint8, device=dev).random_()
         dst = torch.empty_like(src)
         for _ in range(5):
             dst.copy_(src)
@@ -329,17 +515,25 @@ def main():
     for i in range(args.warmup):
         s.sample_batch(ring[i % ring_len], out=out)
     torch.cuda.synchronize()
-    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
-    ev0.record()
     for i in range(args.steps):
         s.sample_batch(ring[i % ring_len], out=out)
-    ev1.record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    kernel_ms = ev0.elapsed_time(ev1) / args.steps  # events on the launch stream; one kernel per step
     ms_per_step = wall * 1e3 / args.steps
+    # device time of a step's launches: events on the launch stream, median of five repeats of K steps
+    repeats_ms = []
+    for _ in range(5):
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        ev0.record()
+        for i in range(args.steps):
+            s.sample_batch(ring[i % ring_len], out=out)
+        ev1.record()
+        torch.cuda.synchronize()
+        repeats_ms.append(ev0.elapsed_time(ev1) / args.steps)
+    kernel_ms = statistics.median(repeats_ms)
     achieved = step_bytes / (kernel_ms * 1e-3) / 1e9
+    traffic, traffic_source = measured_traffic(w.name)
 
     line = {
         "metric": f"sampled rows/sec at vocab {w.vocab}, B={w.batch}, {W.DTYPE_NAMES[w.dtype]}, "
@@ -359,21 +553,25 @@ def main():
                                f"temperature {w.temperature}, top-p {w.topp}, per-row xorshift64* coins; "
                                f"ring of {ring_len} distinct matrices ({ring_len * step_bytes >> 20} MiB)"},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES.get(w.name),
-                     "traffic_source": "profiles/sample_rows_kernel_cfg2.md" if w.name in MEASURED_TRAFFIC_BYTES else None,
-                     "kernel": "sample_rows_kernel",
-                     "kernel_ms": kernel_ms, "algorithmic_bytes_per_launch": step_bytes},
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": traffic, "traffic_source": traffic_source,
+                     "kernel": "one step = split_pass1_kernel + split_pass2_kernel + split_finish_kernel (three launches; "
+                               "their summed duration is what the events bracket)",
+                     "kernel_ms": kernel_ms, "kernel_ms_repeats": repeats_ms, "algorithmic_bytes_per_launch": step_bytes},
     }
     if not args.no_extras:
+        line["graph"] = bench_graph(w, s, ring, out, torch, dev)
+        line["floors"] = bench_floors(w, ring, torch, dev)
         line["logit_chain"] = bench_logit_chain(w, ring[0], torch, dev)
         line["host_buffers"] = bench_host_buffers(w, s, ring[0], out, torch)
         line["gumbel_max"] = bench_gumbel(w, s, ring, out, torch)
         line["greedy"] = bench_greedy(w, ring, out, torch)
         line["per_row_configs"] = bench_configs(w, s, ring, out, args.steps, torch)
         line["draw_modes"] = bench_draw_modes(w, ring[0], out, torch)
-        line["flat_rows"] = bench_flat_rows(torch, dev)
         if w.dtype == W.DTYPE_BFLOAT16 and w.kind == "peaked":
             line["batch_sweep"] = bench_batch_sweep(w, torch, dev)
+        del ring
+        torch.cuda.empty_cache()
+        line["configs"] = bench_all_configs(torch, dev)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(w, got)
     print(json.dumps(line))

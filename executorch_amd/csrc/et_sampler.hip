@@ -1108,6 +1108,21 @@ ets_status ets_test_seq_sum(const float* d_a, int32_t n, float s0, float thresho
   return ETS_OK;
 }
 
+ets_status ets_test_empty_launch(void* hip_stream) {
+  hipLaunchKernelGGL(ets::empty_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(hip_stream));
+  ETS_HIP(nullptr, hipGetLastError());
+  return ETS_OK;
+}
+
+ets_status ets_test_read_floor(const void* d_data, int64_t bytes, int32_t workgroups, uint32_t* d_out, void* hip_stream) {
+  if (!d_data || !d_out || bytes < 16 || workgroups < 1 || reinterpret_cast<uintptr_t>(d_data) % 16 != 0)
+    return fail(nullptr, ETS_INVALID_ARGUMENT, "ets_test_read_floor: bad arguments");
+  hipLaunchKernelGGL(ets::read_floor_kernel, dim3(workgroups), dim3(256), 0, static_cast<hipStream_t>(hip_stream),
+                     static_cast<const uint4*>(d_data), bytes / 16, d_out);
+  ETS_HIP(nullptr, hipGetLastError());
+  return ETS_OK;
+}
+
 ets_status ets_test_split_timers(ets_sampler* s, uint64_t* out, int32_t rows) {
   if (!s || !out || rows < 0 || rows > s->max_batch) return fail(s, ETS_INVALID_ARGUMENT, "ets_test_split_timers: bad arguments");
   if (!s->d_split || !s->split.timers)

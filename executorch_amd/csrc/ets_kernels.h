@@ -1776,6 +1776,28 @@ __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
   }
 }
 
+// ---- measurement floors (hooks for the benchmark: what a launch and a plain read cost here) ------
+__global__ void empty_kernel() {}
+
+// Every workgroup reads its share of `n_vec` 16-byte vectors (eight loads in flight per lane) and
+// keeps an XOR of them: nothing but the read.
+__global__ void __launch_bounds__(256) read_floor_kernel(const uint4* data, int64_t n_vec, uint32_t* out) {
+  const int64_t per = (n_vec + gridDim.x - 1) / gridDim.x;
+  const int64_t lo = per * blockIdx.x, hi = lo + per < n_vec ? lo + per : n_vec;
+  uint32_t acc = 0u;
+  for (int64_t j = lo + threadIdx.x; j < hi; j += 8 * 256) {
+    uint4 r[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const int64_t jk = j + k * 256;
+      r[k] = data[jk < hi ? jk : j];
+    }
+#pragma unroll
+    for (int k = 0; k < 8; ++k) acc ^= r[k].x ^ r[k].y ^ r[k].z ^ r[k].w;
+  }
+  if (acc == 0x9e3779b9u) out[0] = acc;  // (keeps the loads alive; practically never taken)
+}
+
 // Evaluates expf_exact over an array (test hook for the exhaustive comparison with libm).
 __global__ void __launch_bounds__(256) expf_exact_kernel(const float* x, float* y, int64_t n) {
   __shared__ uint64_t tab[32];

@@ -1,6 +1,7 @@
-/* Entry points that exist only so that tests can exercise two device building blocks in
- * isolation (the bit-faithful expf and the sequential-sum emulation).  Not part of the
- * drop-in surface; no reference counterpart. */
+/* TEST AND MEASUREMENT HOOKS, not part of the drop-in surface (no reference counterpart): they exist
+ * so that tests can exercise two device building blocks in isolation (the bit-faithful expf and the
+ * sequential-sum emulation) and so that the benchmark can time what a launch and a plain read cost.
+ * A product build may leave them out: nothing in include/ declares them. */
 #ifndef ETS_TEST_HOOKS_H_
 #define ETS_TEST_HOOKS_H_
 
@@ -17,6 +18,12 @@ ETS_API ets_status ets_test_expf(const float* d_x, float* d_y, int64_t n, void* 
  * DEVICE pointers; *d_stop = -1 when the threshold is never exceeded. */
 ETS_API ets_status ets_test_seq_sum(const float* d_a, int32_t n, float s0, float threshold, float* d_sum,
                                     int32_t* d_stop, void* hip_stream);
+
+/* Measurement floors for the benchmark: an empty launch, and a kernel of `workgroups` workgroups
+ * of 256 lanes that does nothing but read `bytes` bytes (16-byte aligned DEVICE pointer). */
+ETS_API ets_status ets_test_empty_launch(void* hip_stream);
+ETS_API ets_status ets_test_read_floor(const void* d_data, int64_t bytes, int32_t workgroups, uint32_t* d_out,
+                                       void* hip_stream);
 
 /* Phase clocks of the finish kernel of the several-workgroups-per-row path, four 64-bit words per
  * row (staging, ordered sum, draw, in ticks of the 100 MHz wall clock; then the candidate and
