@@ -423,8 +423,8 @@ def parse_pmc(fetch_dir, write_dir, out_path):
         vals = [v for k, vs in per.items() if key in k for v in vs]
         return (sum(vals) / len(vals), len(vals)) if vals else (None, 0)
 
-    copy_f, _ = mean_of(fetch, "copyBuffer")
-    copy_w, _ = mean_of(write, "copyBuffer")
+    copy_f, _ = mean_of(fetch, "copy_probe_kernel")
+    copy_w, _ = mean_of(write, "copy_probe_kernel")
     probe_kib = COPY_PROBE_BYTES / 1024
     res = {"copy_probe_bytes": COPY_PROBE_BYTES, "copy_fetch_kib": copy_f, "copy_write_kib": copy_w,
            "fetch_factor": probe_kib / copy_f if copy_f else None, "write_factor": probe_kib / copy_w if copy_w else None,
@@ -508,7 +508,9 @@ def main():
         src = torch.empty(COPY_PROBE_BYTES, dtype=torch.uint8, device=dev).random_()
         dst = torch.empty_like(src)
         for _ in range(5):
-            dst.copy_(src)
+            from executorch_amd import _capi
+            st = _capi.lib().ets_test_copy_probe(src.data_ptr(), dst.data_ptr(), COPY_PROBE_BYTES, torch.cuda.current_stream().cuda_stream)
+            assert st == 0
         torch.cuda.synchronize()
         del src, dst
 

@@ -85,6 +85,7 @@ TEST_HOOKS = {
     "ets_test_seq_sum": (C.c_int32, [C.c_void_p, C.c_int32, C.c_float, C.c_float, C.c_void_p, C.c_void_p, C.c_void_p]),
     "ets_test_split_timers": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int32]),
     "ets_test_empty_launch": (C.c_int32, [C.c_void_p]),
+    "ets_test_copy_probe": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p]),
     "ets_test_read_floor": (C.c_int32, [C.c_void_p, C.c_int64, C.c_int32, C.c_void_p, C.c_void_p]),
 }
 

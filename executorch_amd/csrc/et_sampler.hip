@@ -389,9 +389,8 @@ ets_status launch_split(ets_sampler* s, const ets::RowParams& p, int32_t rows, h
   sp.phist_words = DT == ets::kDtypeBFloat16 ? kPhistWordsBFloat16 : (DT == ets::kDtypeHalf ? kPhistWordsHalf : 0);
   sp.row_wgs = pass2_workgroups(s, rows, sp.ns);
   sp.list_region = list_region(sp.ns, sp.row_wgs);
-  const int per_block = (ets::kPass1Block / 64) * ets::kPass1SlotsPerWave;
-  hipLaunchKernelGGL((ets::split_pass1_kernel<DT>), dim3((sp.ns + per_block - 1) / per_block, rows), dim3(ets::kPass1Block), 0,
-                     stream, sp);
+  // passes 1 and 2 share their grid: a workgroup of pass 2 finds its entries in the L2 of its die
+  hipLaunchKernelGGL((ets::split_pass1_kernel<DT>), dim3(sp.row_wgs, rows), dim3(ets::kBlock), 0, stream, sp);
   ETS_HIP(s, hipGetLastError());
   const size_t lut_bytes = (DT == ets::kDtypeBFloat16 ? sizeof(float) * ets::kLutCountWords : 0) + sizeof(uint32_t) * sp.phist_words;
   static std::atomic<size_t> set_bytes2[kMaxDevices];
@@ -1119,6 +1118,15 @@ ets_status ets_test_read_floor(const void* d_data, int64_t bytes, int32_t workgr
     return fail(nullptr, ETS_INVALID_ARGUMENT, "ets_test_read_floor: bad arguments");
   hipLaunchKernelGGL(ets::read_floor_kernel, dim3(workgroups), dim3(256), 0, static_cast<hipStream_t>(hip_stream),
                      static_cast<const uint4*>(d_data), bytes / 16, d_out);
+  ETS_HIP(nullptr, hipGetLastError());
+  return ETS_OK;
+}
+
+ets_status ets_test_copy_probe(const void* d_src, void* d_dst, int64_t bytes, void* hip_stream) {
+  if (!d_src || !d_dst || bytes < 16 || reinterpret_cast<uintptr_t>(d_src) % 16 != 0 || reinterpret_cast<uintptr_t>(d_dst) % 16 != 0)
+    return fail(nullptr, ETS_INVALID_ARGUMENT, "ets_test_copy_probe: bad arguments");
+  hipLaunchKernelGGL(ets::copy_probe_kernel, dim3(4096), dim3(256), 0, static_cast<hipStream_t>(hip_stream),
+                     static_cast<const uint4*>(d_src), static_cast<uint4*>(d_dst), bytes / 16);
   ETS_HIP(nullptr, hipGetLastError());
   return ETS_OK;
 }

@@ -1713,8 +1713,16 @@ __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
     }
   }
 
-  RowDebug dbg = {m, S, coin, 0.0f, 0.0f, 0, 0, 0};
-  int32_t token = -1;
+  // The draw's results live in LDS: the draw functions are calls, and a result in a lane's own
+  // variable would be passed by address, which puts it (and every lane's copy) in private memory.
+  // Every lane stores the same values.
+  __shared__ RowDebug dbg;
+  __shared__ int32_t token;
+  if (tid == 0) {
+    dbg = RowDebug{m, S, coin, 0.0f, 0.0f, 0, 0, 0};
+    token = -1;
+  }
+  __syncthreads();
   if (row_nan) {
     // Every probability is NaN.  The multinomial walk never fires and returns the last index
     // (sampler.cpp:58-70); top-p keeps no candidate, where the reference reads probindex[-1]:
@@ -1778,6 +1786,13 @@ __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
 
 // ---- measurement floors (hooks for the benchmark: what a launch and a plain read cost here) ------
 __global__ void empty_kernel() {}
+
+// dst = src, 16 bytes per lane and access as in the row kernels: the transfer of known size that the
+// hardware's fetch and write counters are scaled by.
+__global__ void __launch_bounds__(256) copy_probe_kernel(const uint4* src, uint4* dst, int64_t n_vec) {
+  for (int64_t j = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; j < n_vec; j += static_cast<int64_t>(gridDim.x) * 256)
+    dst[j] = src[j];
+}
 
 // Every workgroup reads its share of `n_vec` 16-byte vectors (eight loads in flight per lane) and
 // keeps an XOR of them: nothing but the read.

@@ -24,7 +24,6 @@ namespace ets {
 
 constexpr int kSlot = 512;        // entries per slot: 64 lanes x 8 consecutive entries
 constexpr int kMaxSlots = 2048;   // rows of up to 1048576 entries take this path
-constexpr int kPass1Block = 256;  // lanes per workgroup of pass 1
 constexpr int kPass1SlotsPerWave = 4;
 constexpr int kPrepCap = 40;      // prepared slots per row (a row of the usual kind needs 10 to 20)
 
@@ -165,8 +164,18 @@ __device__ __forceinline__ void load_slot_lane(const char* logits, int s, int la
 }
 
 // ---- pass 1 ---------------------------------------------------------------------------------------
+// Slots of a row that workgroup x of `wgs` takes, in passes 1 and 2 alike: the two launches have
+// the same grid, so a workgroup of pass 2 runs on the die (XCD) whose L2 already holds the entries
+// its namesake of pass 1 read from HBM (workgroups go to the dies in turn, by their linear id).
+__device__ __forceinline__ void split_range(int ns, int wgs, int x, int& s_begin, int& s_end) {
+  const int per_wg = ((ns + wgs - 1) / wgs + kWaves - 1) / kWaves * kWaves;
+  s_begin = x * per_wg;
+  s_end = min(ns, s_begin + per_wg);
+}
+
+// grid = (workgroups per row, rows), kBlock lanes: every wave takes whole slots, four at a time.
 template <int DT>
-__global__ void __launch_bounds__(kPass1Block) split_pass1_kernel(SplitParams p) {
+__global__ void __launch_bounds__(kBlock) split_pass1_kernel(SplitParams p) {
   const int row = p.row.row_map ? p.row.row_map[blockIdx.y] : blockIdx.y;
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -175,39 +184,42 @@ __global__ void __launch_bounds__(kPass1Block) split_pass1_kernel(SplitParams p)
   const char* logits = static_cast<const char*>(p.row.logits) + static_cast<int64_t>(row) * p.row.row_stride * ElemSize<DT>::value;
   const float kInf = __uint_as_float(0x7f800000u);
   const float fill = inv < 0.0f ? kInf : -kInf;  // x = -inf: adds nothing
-  const int slot0 = (blockIdx.x * (kPass1Block / 64) + wave) * kPass1SlotsPerWave;
-  float v[kPass1SlotsPerWave][8];
+  int s_begin, s_end;
+  split_range(p.ns, gridDim.x, blockIdx.x, s_begin, s_end);
+  for (int slot0 = s_begin + wave * kPass1SlotsPerWave; slot0 < s_end; slot0 += kWaves * kPass1SlotsPerWave) {
+    float v[kPass1SlotsPerWave][8];
 #pragma unroll
-  for (int k = 0; k < kPass1SlotsPerWave; ++k) {
-    if (slot0 + k < p.ns) load_slot_lane<DT>(logits, slot0 + k, lane, V, fill, v[k]);
-  }
-#pragma unroll
-  for (int k = 0; k < kPass1SlotsPerWave; ++k) {
-    const int s = slot0 + k;
-    if (s >= p.ns) break;
-    float lmax = -kInf;
-    bool nan = false;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      v[k][e] = v[k][e] * inv;
-      lmax = __builtin_fmaxf(lmax, v[k][e]);  // ignores NaN
-      nan = nan || (v[k][e] != v[k][e]);
+    for (int k = 0; k < kPass1SlotsPerWave; ++k) {
+      if (slot0 + k < s_end) load_slot_lane<DT>(logits, slot0 + k, lane, V, fill, v[k]);
     }
-    const float M = wave_max_ignoring_nan(lmax);
-    const bool any_nan = __ballot(nan) != 0ull;
-    float sum = 0.0f;
-    if (M > -kInf) {
+#pragma unroll
+    for (int k = 0; k < kPass1SlotsPerWave; ++k) {
+      const int s = slot0 + k;
+      if (s >= s_end) break;
+      float lmax = -kInf;
+      bool nan = false;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        const float t = fast_exp2((v[k][e] - M) * kLog2e);
-        sum += (v[k][e] == v[k][e]) ? t : 0.0f;
+        v[k][e] = v[k][e] * inv;
+        lmax = __builtin_fmaxf(lmax, v[k][e]);  // ignores NaN
+        nan = nan || (v[k][e] != v[k][e]);
       }
-    }
-    sum = wave_sum_f32(sum);
-    if (lane == 0) {
-      const int64_t at = static_cast<int64_t>(row) * p.ns_stride + s;
-      p.slot_max[at] = any_nan ? __uint_as_float(0x7fc00000u) : M;
-      p.slot_sum[at] = sum;
+      const float M = wave_max_ignoring_nan(lmax);
+      const bool any_nan = __ballot(nan) != 0ull;
+      float sum = 0.0f;
+      if (M > -kInf) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float t = fast_exp2((v[k][e] - M) * kLog2e);
+          sum += (v[k][e] == v[k][e]) ? t : 0.0f;
+        }
+      }
+      sum = wave_sum_f32(sum);
+      if (lane == 0) {
+        const int64_t at = static_cast<int64_t>(row) * p.ns_stride + s;
+        p.slot_max[at] = any_nan ? __uint_as_float(0x7fc00000u) : M;
+        p.slot_sum[at] = sum;
+      }
     }
   }
 }
@@ -401,9 +413,8 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
 
   // ---- this workgroup's slots: wave w takes s_begin + w, s_begin + w + 16, ...; the first one's
   //      entries are requested before anything else
-  const int per_wg = (((ns + static_cast<int>(gridDim.x) - 1) / static_cast<int>(gridDim.x)) + kWaves - 1) / kWaves * kWaves;
-  const int s_begin = blockIdx.x * per_wg;
-  const int s_end = min(ns, s_begin + per_wg);
+  int s_begin, s_end;
+  split_range(ns, gridDim.x, blockIdx.x, s_begin, s_end);
   float l[8];
   int s_mine = s_begin + wave;
   if (s_mine < s_end) load_slot_lane<DT>(logits, s_mine, lane, V, fill, l);
@@ -1428,8 +1439,16 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
     }
   }
 
-  RowDebug dbg = {m, S, coin, 0.0f, 0.0f, 0, 0, 0};
-  int32_t token = -1;  // a NaN row keeps no candidate, where the reference reads probindex[-1]
+  // The draw's results live in LDS: the draw functions are calls, and a result in a lane's own
+  // variable would be passed by address, which puts it (and every lane's copy) in private memory.
+  // Every lane stores the same values.
+  __shared__ RowDebug dbg;
+  __shared__ int32_t token;
+  if (tid == 0) {
+    dbg = RowDebug{m, S, coin, 0.0f, 0.0f, 0, 0, 0};
+    token = -1;  // a NaN row keeps no candidate, where the reference reads probindex[-1]
+  }
+  __syncthreads();
   int path = 0;
   if (!row_nan) {
     bool done = false;

@@ -25,6 +25,10 @@ ETS_API ets_status ets_test_empty_launch(void* hip_stream);
 ETS_API ets_status ets_test_read_floor(const void* d_data, int64_t bytes, int32_t workgroups, uint32_t* d_out,
                                        void* hip_stream);
 
+/* dst = src with 16-byte accesses (16-byte aligned DEVICE pointers, bytes a multiple of 16): the
+ * transfer of known size that fetch and write counters of a profiler run are scaled by. */
+ETS_API ets_status ets_test_copy_probe(const void* d_src, void* d_dst, int64_t bytes, void* hip_stream);
+
 /* Phase clocks of the finish kernel of the several-workgroups-per-row path, four 64-bit words per
  * row (staging, ordered sum, draw, in ticks of the 100 MHz wall clock; then the candidate and
  * prepared-slot counts), filled when ETS_SPLIT_TIMERS was set before the handle's first stochastic
