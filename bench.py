@@ -175,7 +175,7 @@ def timed_us(fn, reps, torch, repeats=1):
     return statistics.median(means)
 
 
-def bench_logit_chain(w, logits, torch, dev):
+def bench_logit_chain(w, logits, torch, dev, s=None, out=None):
     """The device-side logit processors on a private copy of one batch of the workload: a chain of
     lists (repetition penalty over a 512-token history per row, then a 16-token mask), which touches
     a few hundred entries per row, and a chain of two whole-row processors, which has to read and
@@ -191,7 +191,15 @@ def bench_logit_chain(w, logits, torch, dev):
     lists_us = timed_us(lambda: lists.process(work), 50, torch)
     rows_us = timed_us(lambda: rows.process(work), 50, torch)
     moved = 2 * w.bytes_per_step  # the batch is read once and written once
-    return {"lists_us": lists_us, "lists": "repetition penalty, 512-token history per row + mask of 16 ids",
+    fused = {}
+    if s is not None:
+        # the same two whole-row processors applied while the sampler reads the rows, against the
+        # sampler alone and against the two calls (all three on the same matrix)
+        fused = {"sample_alone_us": timed_us(lambda: s.sample_batch(work, out=out), 100, torch, repeats=5),
+                 "chain_then_sample_us": timed_us(lambda: (rows.process(work), s.sample_batch(work, out=out)), 100, torch, repeats=5),
+                 "chain_fused_into_sample_us": timed_us(lambda: s.sample_batch_chain(work, rows, out=out), 100, torch, repeats=5)}
+        fused["fused_over_alone"] = fused["chain_fused_into_sample_us"] / fused["sample_alone_us"]
+    return {**fused, "lists_us": lists_us, "lists": "repetition penalty, 512-token history per row + mask of 16 ids",
             "whole_rows_us": rows_us, "whole_rows": "scale + bias", "whole_rows_algorithmic_bytes": moved,
             "whole_rows_gbs": moved / (rows_us * 1e-6) / 1e9, "whole_rows_frac_of_hbm_peak": moved / (rows_us * 1e-6) / 1e9 / HBM_PEAK_GBS}
 
@@ -265,9 +273,12 @@ def bench_greedy(w, ring, out, torch):
 def bench_configs(w, s, ring, out, steps, torch):
     """ets_sampler_sample_batch_configs on the same ring: every row with the workload's own
     parameters, and a mix of four kinds of rows (one group of launches per kind)."""
-    uniform = [(w.temperature, w.topp, 0, 0)] * w.batch
+    import numpy as np
+    from executorch_amd.sampler import SAMPLING_CONFIG_DTYPE
     kinds = [(w.temperature, w.topp, 0, 0), (0.0, w.topp, 0, 0), (1.0, 1.0, 0, 0), (0.8, w.topp, 40, 0)]
-    mixed = [kinds[b % 4] for b in range(w.batch)]
+    # (structured arrays, built once: a serving loop keeps its requests' parameters in this form)
+    uniform = np.asarray([kinds[0]] * w.batch, dtype=SAMPLING_CONFIG_DTYPE)
+    mixed = np.asarray([kinds[b % 4] for b in range(w.batch)], dtype=SAMPLING_CONFIG_DTYPE)
     state = {"i": 0}
 
     def run(cfg):
@@ -563,7 +574,7 @@ def main():
     if not args.no_extras:
         line["graph"] = bench_graph(w, s, ring, out, torch, dev)
         line["floors"] = bench_floors(w, ring, torch, dev)
-        line["logit_chain"] = bench_logit_chain(w, ring[0], torch, dev)
+        line["logit_chain"] = bench_logit_chain(w, ring[0], torch, dev, s, out)
         line["host_buffers"] = bench_host_buffers(w, s, ring[0], out, torch)
         line["gumbel_max"] = bench_gumbel(w, s, ring, out, torch)
         line["greedy"] = bench_greedy(w, ring, out, torch)

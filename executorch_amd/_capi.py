@@ -76,6 +76,8 @@ CHAIN_SIGNATURES = {
     "ets_logit_chain_add_token_bias": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32]),
     "ets_logit_chain_add_repetition_penalty": (C.c_int32, [C.c_void_p, C.c_float, C.c_void_p, C.c_int64, C.c_void_p]),
     "ets_logit_chain_process": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.POINTER(C.c_int64), C.c_void_p]),
+    "ets_sampler_sample_batch_chain": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int64, C.c_void_p,
+                                       C.c_void_p]),
     "ets_logit_chain_last_error": (C.c_char_p, [C.c_void_p]),
 }
 

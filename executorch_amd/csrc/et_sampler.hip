@@ -74,6 +74,12 @@ struct ets_sampler {
   hipEvent_t stage_done = nullptr;
   hipStream_t stage_stream = nullptr;
   bool stage_used = false;
+  // ets_sampler_sample_batch_configs(): the groups of rows that draw in different ways run side by
+  // side, each behind the call's stream on a stream of its own (default priority), joined again
+  // before the call returns to the caller's stream
+  hipStream_t aux_stream[3] = {};
+  hipEvent_t fork_event = nullptr;
+  hipEvent_t join_event[3] = {};
   // opt-in device timing (ets_sampler_set_timing): a ring of event pairs around the launches of a
   // call, harvested when a slot is reused or the totals are read
   bool timing = false;
@@ -429,7 +435,8 @@ ets_status rows_device(ets_sampler* s, const ets::RowParams& p, int32_t dtype, i
 }
 
 ets_status sample_device(ets_sampler* s, const void* d_logits, int32_t dtype, int32_t batch, int64_t stride,
-                         int32_t* d_tokens, float* d_probs, ets_row_debug* d_debug, hipStream_t stream) {
+                         int32_t* d_tokens, float* d_probs, ets_row_debug* d_debug, hipStream_t stream,
+                         const ets::FusedOps* fused = nullptr) {
   if (s->inv_temperature == 0.0f) {
     // greedy: no coin is consumed (sampler.cpp:226-228)
     return argmax_device(s, d_logits, dtype, batch, stride, d_tokens, stream, nullptr);
@@ -437,7 +444,8 @@ ets_status sample_device(ets_sampler* s, const void* d_logits, int32_t dtype, in
   if (dtype == ETS_DTYPE_UINT16) return fail(s, ETS_NOT_SUPPORTED, kUint16Message);
   ets_status st = ensure_scratch(s);
   if (st != ETS_OK) return st;
-  ets::RowParams p;
+  ets::RowParams p = {};
+  if (fused) p.fused = *fused;  // (the caller has checked that these rows take the path that applies them)
   p.logits = d_logits;
   p.row_stride = stride;
   p.vocab = s->vocab;
@@ -559,6 +567,16 @@ ets_status stage_release(ets_sampler* s, hipStream_t stream) {
   return ETS_OK;
 }
 
+ets_status ensure_aux_streams(ets_sampler* s) {
+  if (s->fork_event) return ETS_OK;
+  for (int i = 0; i < 3; ++i) {
+    ETS_HIP(s, hipStreamCreateWithFlags(&s->aux_stream[i], hipStreamNonBlocking));
+    ETS_HIP(s, hipEventCreateWithFlags(&s->join_event[i], hipEventDisableTiming));
+  }
+  ETS_HIP(s, hipEventCreateWithFlags(&s->fork_event, hipEventDisableTiming));
+  return ETS_OK;
+}
+
 ets_status sample_device_configs(ets_sampler* s, const void* d_logits, int32_t dtype, int32_t batch, int64_t stride,
                                  const ets_sampling_config* configs, int32_t* d_tokens, ets_row_debug* d_debug,
                                  hipStream_t stream) {
@@ -604,11 +622,30 @@ ets_status sample_device_configs(ets_sampler* s, const void* d_logits, int32_t d
     ETS_HIP(s, hipGetLastError());
   }
   const int32_t* d_maps = reinterpret_cast<const int32_t*>(d + lay.maps);
-  if (count[0] > 0) {
-    st = argmax_device(s, d_logits, dtype, count[0], stride, d_tokens, stream, d_maps);
+  // The groups touch different rows and different work buffers: the first one that has rows runs
+  // on the caller's stream, every further one on a stream of its own between a fork and a join.
+  const int groups = (count[0] > 0) + (count[1] > 0) + (count[2] > 0) + (count[3] > 0);
+  if (groups > 1) {
+    st = ensure_aux_streams(s);
     if (st != ETS_OK) return st;
+    ETS_HIP(s, hipEventRecord(s->fork_event, stream));
   }
-  ets::RowParams p;
+  int forked = 0;
+  bool main_taken = false;
+  hipStream_t side[3] = {};
+  auto group_stream = [&](hipStream_t* out) -> ets_status {
+    if (!main_taken) {
+      main_taken = true;
+      *out = stream;
+      return ETS_OK;
+    }
+    hipStream_t a = s->aux_stream[forked];
+    ETS_HIP(s, hipStreamWaitEvent(a, s->fork_event, 0));
+    side[forked++] = a;
+    *out = a;
+    return ETS_OK;
+  };
+  ets::RowParams p = {};
   p.logits = d_logits;
   p.row_stride = stride;
   p.vocab = s->vocab;
@@ -623,11 +660,28 @@ ets_status sample_device_configs(ets_sampler* s, const void* d_logits, int32_t d
   p.scratch_stride = s->scratch_stride;
   p.lds_keys = s->lds_keys;
   p.row_cfg = reinterpret_cast<const ets::RowConfig*>(d + lay.cfg);
-  for (int draw = 0; draw < 3; ++draw) {
+  // the longest-running groups first (multinomial, top-k, top-p), the arg-max last
+  const int order[3] = {ets::kDrawMultinomial, ets::kDrawTopK, ets::kDrawTopP};
+  for (int k = 0; k < 3; ++k) {
+    const int draw = order[k];
     if (count[1 + draw] == 0) continue;
-    p.row_map = d_maps + (1 + draw) * batch;
-    st = rows_device(s, p, dtype, count[1 + draw], stream, draw);
+    hipStream_t gs = nullptr;
+    st = group_stream(&gs);
     if (st != ETS_OK) return st;
+    p.row_map = d_maps + (1 + draw) * batch;
+    st = rows_device(s, p, dtype, count[1 + draw], gs, draw);
+    if (st != ETS_OK) return st;
+  }
+  if (count[0] > 0) {
+    hipStream_t gs = nullptr;
+    st = group_stream(&gs);
+    if (st != ETS_OK) return st;
+    st = argmax_device(s, d_logits, dtype, count[0], stride, d_tokens, gs, d_maps);
+    if (st != ETS_OK) return st;
+  }
+  for (int i = 0; i < forked; ++i) {
+    ETS_HIP(s, hipEventRecord(s->join_event[i], side[i]));
+    ETS_HIP(s, hipStreamWaitEvent(stream, s->join_event[i], 0));
   }
   return stage_release(s, stream);
 }
@@ -731,6 +785,11 @@ ets_status ets_sampler_destroy(ets_sampler* s) {
     (void)hipFree(s->d_token);
     (void)hipFree(s->d_stage);
     if (s->h_stage) (void)hipHostFree(s->h_stage);
+    for (int i = 0; i < 3; ++i) {
+      if (s->aux_stream[i]) (void)hipStreamDestroy(s->aux_stream[i]);
+      if (s->join_event[i]) (void)hipEventDestroy(s->join_event[i]);
+    }
+    if (s->fork_event) (void)hipEventDestroy(s->fork_event);
     if (s->stage_event) (void)hipEventDestroy(s->stage_event);
     if (s->stage_done) (void)hipEventDestroy(s->stage_done);
     for (int i = 0; i < ets_sampler::kTimingSlots; ++i) {

@@ -28,6 +28,17 @@ struct RowConfig {
   int32_t topk;
 };
 
+// Logit processors that touch every entry of a row the same way (logit_processor.h:19-40: a bias, a
+// factor), applied to each logit as it is read instead of by a pass of their own over the tensor.
+// After each of them the value is rounded to the tensor's element type, as the processor's store
+// into the tensor would.
+constexpr int kMaxFusedOps = 4;
+struct FusedOps {
+  int32_t n;
+  int32_t scale[kMaxFusedOps];  // 1: multiply by value, 0: add value
+  float value[kMaxFusedOps];
+};
+
 struct RowParams {
   const void* logits;
   int64_t row_stride;  // elements between rows
@@ -44,7 +55,66 @@ struct RowParams {
   int32_t lds_keys;   // power of two: keys that fit in the dynamic LDS buffer
   const int32_t* row_map;    // workgroup -> row, or null for the identity
   const RowConfig* row_cfg;  // [batch] per-row parameters (by row), or null for the launch-wide ones
+  FusedOps fused;            // logit processors applied as the logits are read (several-workgroups-per-row path only)
 };
+
+// A float rounded to the row's element type and back (round to nearest even; a NaN stays a NaN).
+template <int DT>
+__device__ __forceinline__ float round_to_elem(float v) {
+  if constexpr (DT == kDtypeBFloat16) {
+    const uint32_t b = __float_as_uint(v);
+    return __uint_as_float((b + 0x7fffu + ((b >> 16) & 1u)) & 0xffff0000u);  // (NaNs made from 16-bit values keep clear low bits)
+  } else if constexpr (DT == kDtypeHalf) {
+    asm volatile("" : "+v"(v));  // round to fp32 first, to half second: no single mixed-precision rounding
+    return static_cast<float>(static_cast<_Float16>(v));
+  } else {
+    return v;
+  }
+}
+
+// Two floats rounded to bf16 and back by the conversion instruction (one for the pair).
+typedef __bf16 ets_bf16x2 __attribute__((ext_vector_type(2)));
+typedef float ets_f32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void round_pair_bf16(float& a, float& b) {
+  const ets_f32x2 v = {a, b};
+  const uint32_t u = __builtin_bit_cast(uint32_t, __builtin_convertvector(v, ets_bf16x2));
+  a = __uint_as_float(u << 16);
+  b = __uint_as_float(u & 0xffff0000u);
+}
+
+// The fused logit processors on R values at once.
+template <int DT, int R>
+__device__ __forceinline__ void apply_fused(float* x, const FusedOps& f) {
+  for (int k = 0; k < f.n; ++k) {
+    const float v = f.value[k];
+    if (f.scale[k]) {
+#pragma unroll
+      for (int e = 0; e < R; ++e) x[e] = x[e] * v;
+    } else {
+#pragma unroll
+      for (int e = 0; e < R; ++e) x[e] = x[e] + v;
+    }
+    if constexpr (DT == kDtypeBFloat16 && R % 2 == 0) {
+#pragma unroll
+      for (int e = 0; e < R; e += 2) round_pair_bf16(x[e], x[e + 1]);
+    } else {
+#pragma unroll
+      for (int e = 0; e < R; ++e) x[e] = round_to_elem<DT>(x[e]);
+    }
+  }
+}
+
+// One logit of the row, processors applied; a NaN comes out as the canonical one a store into the
+// tensor would leave.
+template <int DT>
+__device__ __forceinline__ float load_logit(const char* logits, int64_t i, const FusedOps& f) {
+  float x = load_elem<DT>(logits, i);
+  if (f.n > 0) {
+    apply_fused<DT, 1>(&x, f);
+    if (DT == kDtypeBFloat16 && x != x) x = __uint_as_float(0x7fc00000u);
+  }
+  return x;
+}
 
 // ---- argmax ---------------------------------------------------------------------------------
 // Order-preserving key of a float: larger float <=> larger key; -0 == +0; NaN lowest.
@@ -804,7 +874,7 @@ template <int DT>
 __device__ int32_t draw_general(const char* logits, int V, float inv, float m, float S, bool use_topk,
                                              int topk, float topp, float cutoff, float coin, uint64_t* scratch,
                                              int64_t scratch_cap, uint64_t* lds_keys, int cap, RowDebug& dbg,
-                                             BlockScratch& sm) {
+                                             BlockScratch& sm, const FusedOps* fused = nullptr) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const float cut = use_topk ? 0.0f : cutoff;
@@ -815,7 +885,7 @@ __device__ int32_t draw_general(const char* logits, int V, float inv, float m, f
   for (int base = 0; base < V; base += kBlock) {
     const int i = base + tid;
     if (i < V) {
-      const float x = load_elem<DT>(logits, i) * inv;
+      const float x = (fused ? load_logit<DT>(logits, i, *fused) : load_elem<DT>(logits, i)) * inv;
       const float pi = div_row(expf_nonpositive(x - m, sm.exp2tab), div);
       const bool keep = pi >= cut;
       scratch[i] = keep ? cand_key(pi, i) : ~0ull;

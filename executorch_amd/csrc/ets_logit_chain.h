@@ -196,9 +196,13 @@ ets_status chain_upload(ets_logit_chain* c, const T* host, int32_t count, const 
 
 template <int DT>
 ets_status chain_launch(ets_logit_chain* c, void* d_logits, int64_t row_pitch, int64_t row_offset, int32_t vocab,
-                        int32_t rows, hipStream_t stream) {
+                        int32_t rows, hipStream_t stream, int32_t n_ops = -1) {
+  // (n_ops: only the chain's first processors; the rest is left to the caller)
+  if (n_ops < 0) n_ops = static_cast<int32_t>(c->ops.size());
+  bool whole_rows = false;
+  for (int32_t k = 0; k < n_ops; ++k) whole_rows = whole_rows || c->ops[k].kind == ets::kOpBias || c->ops[k].kind == ets::kOpScale;
   // whole-row processors want many workgroups per row; lists alone are cheapest with one
-  const int32_t tile = c->whole_rows ? ets::kChainTile : vocab;
+  const int32_t tile = whole_rows ? ets::kChainTile : vocab;
   const int32_t tiles = (vocab + tile - 1) / tile;
   const size_t lds = c->repetition ? static_cast<size_t>((tile + 31) / 32) * sizeof(uint32_t) : 0;
   if (lds > 64 * 1024) {
@@ -213,7 +217,7 @@ ets_status chain_launch(ets_logit_chain* c, void* d_logits, int64_t row_pitch, i
     }
   }
   hipLaunchKernelGGL((ets::logit_chain_kernel<DT>), dim3(tiles, rows), dim3(ets::kChainBlock), lds, stream, d_logits,
-                     row_pitch, row_offset, vocab, tile, c->d_ops, static_cast<int32_t>(c->ops.size()));
+                     row_pitch, row_offset, vocab, tile, c->d_ops, n_ops);
   ETS_CHAIN_HIP(c, hipGetLastError());
   return ETS_OK;
 }
@@ -350,6 +354,65 @@ ets_status ets_logit_chain_process(ets_logit_chain* c, void* d_logits, int32_t d
       return chain_launch<ets::kDtypeBFloat16>(c, d_logits, row_pitch, row_offset, static_cast<int32_t>(vocab),
                                                static_cast<int32_t>(rows), stream);
   }
+}
+
+ets_status ets_sampler_sample_batch_chain(ets_sampler* s, ets_logit_chain* c, void* d_logits, int32_t dtype, int32_t batch,
+                                          int64_t row_stride_elems, int32_t* d_tokens, void* hip_stream) {
+  if (!s) return fail(nullptr, ETS_INVALID_ARGUMENT, "ets_sampler_sample_batch_chain: null handle");
+  s->last_error.clear();
+  if (!c) return fail(s, ETS_INVALID_ARGUMENT, "ets_sampler_sample_batch_chain: null chain");
+  if (!d_logits || !d_tokens) return fail(s, ETS_INVALID_ARGUMENT, "ets_sampler_sample_batch_chain: null pointer");
+  if (dtype != ETS_DTYPE_FLOAT && dtype != ETS_DTYPE_HALF && dtype != ETS_DTYPE_BFLOAT16)
+    return fail(s, ETS_INVALID_ARGUMENT, "ets_sampler_sample_batch_chain: element type must be Float, Half or BFloat16");
+  if (batch < 0 || batch > s->max_batch)
+    return fail(s, ETS_INVALID_ARGUMENT, "ets_sampler_sample_batch_chain: batch exceeds the handle's max_batch");
+  if (row_stride_elems < s->vocab)
+    return fail(s, ETS_INVALID_ARGUMENT, "ets_sampler_sample_batch_chain: row stride smaller than vocab_size");
+  if (c->device != s->device) return fail(s, ETS_INVALID_ARGUMENT, "ets_sampler_sample_batch_chain: chain and sampler live on different devices");
+  if (c->repetition && s->vocab > 1048576)
+    return fail(s, ETS_INVALID_ARGUMENT, "ets_sampler_sample_batch_chain: the repetition penalty needs vocab <= 1048576");
+  if (batch == 0) return ETS_OK;
+  DeviceGuard g(s->device);
+  hipStream_t stream = static_cast<hipStream_t>(hip_stream);
+  // The chain's last processors, as far as they are biases and factors, are applied while the
+  // sampler reads the logits -- when the rows take the path that can do that (the top-p draw with
+  // several workgroups per row); everything in front of them runs in place first.
+  const int32_t n_ops = static_cast<int32_t>(c->ops.size());
+  ets::FusedOps fused = {};
+  int32_t n_front = n_ops;
+  const bool can_fuse = s->inv_temperature != 0.0f && !s->wb &&
+                        use_split(s, d_logits, row_stride_elems, dtype, draw_mode(s->vocab, s->topp, s->topk));
+  if (can_fuse) {
+    while (n_front > 0 && fused.n < ets::kMaxFusedOps &&
+           (c->ops[n_front - 1].kind == ets::kOpBias || c->ops[n_front - 1].kind == ets::kOpScale))
+      --n_front, ++fused.n;
+    for (int32_t k = 0; k < fused.n; ++k) {
+      fused.scale[k] = c->ops[n_front + k].kind == ets::kOpScale ? 1 : 0;
+      fused.value[k] = c->ops[n_front + k].value;
+    }
+  }
+  if (n_front > 0) {
+    ets_status st = ETS_OK;
+    switch (dtype) {
+      case ETS_DTYPE_FLOAT:
+        st = chain_launch<ets::kDtypeFloat>(c, d_logits, row_stride_elems, 0, s->vocab, batch, stream, n_front);
+        break;
+      case ETS_DTYPE_HALF:
+        st = chain_launch<ets::kDtypeHalf>(c, d_logits, row_stride_elems, 0, s->vocab, batch, stream, n_front);
+        break;
+      default:
+        st = chain_launch<ets::kDtypeBFloat16>(c, d_logits, row_stride_elems, 0, s->vocab, batch, stream, n_front);
+        break;
+    }
+    if (st != ETS_OK) return fail(s, st, std::string("ets_sampler_sample_batch_chain: ") + c->last_error);
+  }
+  int slot = -1;
+  ets_status st = timing_begin(s, stream, batch, &slot);
+  if (st != ETS_OK) return st;
+  st = sample_device(s, d_logits, dtype, batch, row_stride_elems, d_tokens, nullptr, nullptr, stream,
+                     fused.n > 0 ? &fused : nullptr);
+  if (st != ETS_OK) return st;
+  return timing_end(s, stream, slot);
 }
 
 const char* ets_logit_chain_last_error(const ets_logit_chain* c) {

@@ -158,11 +158,19 @@ constexpr float kLog2e = 1.44269504088896340736f;
 
 // The 8 entries of lane `lane` of slot `s` as floats; positions past the row read as `fill`.
 template <int DT>
-__device__ __forceinline__ void load_slot_lane(const char* logits, int s, int lane, int V, float fill, float* out) {
+__device__ __forceinline__ void load_slot_lane(const char* logits, int s, int lane, int V, float fill, float* out,
+                                               const FusedOps& f) {
   constexpr int VE = VecElems<DT>::value;
   const int first = s * kSlot + lane * 8;
 #pragma unroll
   for (int q = 0; q < 8 / VE; ++q) load_run<DT, true>(logits, first + q * VE, V, fill, out + q * VE);
+  if (f.n > 0) {
+    apply_fused<DT, 8>(out, f);
+    if (first + 8 > V) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) out[e] = first + e < V ? out[e] : fill;
+    }
+  }
 }
 
 // ---- pass 1 ---------------------------------------------------------------------------------------
@@ -192,7 +200,7 @@ __global__ void __launch_bounds__(kBlock) split_pass1_kernel(SplitParams p) {
     float v[kPass1SlotsPerWave][8];
 #pragma unroll
     for (int k = 0; k < kPass1SlotsPerWave; ++k) {
-      if (slot0 + k < s_end) load_slot_lane<DT>(logits, slot0 + k, lane, V, fill, v[k]);
+      if (slot0 + k < s_end) load_slot_lane<DT>(logits, slot0 + k, lane, V, fill, v[k], p.row.fused);
     }
 #pragma unroll
     for (int k = 0; k < kPass1SlotsPerWave; ++k) {
@@ -465,7 +473,7 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
   split_range(ns, gridDim.x, blockIdx.x, s_begin, s_end);
   float l[8];
   int s_mine = s_begin + wave;
-  if (s_mine < s_end) load_slot_lane<DT>(logits, s_mine, lane, V, fill, l);
+  if (s_mine < s_end) load_slot_lane<DT>(logits, s_mine, lane, V, fill, l, p.row.fused);
   if (tid == 0) sh.next_slot = s_begin + kWaves;
 
   // ---- row maximum (sampler.cpp:191-197) from the slots' maxima
@@ -494,7 +502,7 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
     m = (sm.red_f[w] > m) ? sm.red_f[w] : m;
     nan_any |= sm.red_u[w];
   }
-  const float x0 = load_elem<DT>(logits, 0) * inv;
+  const float x0 = load_logit<DT>(logits, 0, p.row.fused) * inv;
   if (x0 != x0) m = x0;  // max_val starts at x[0]; nothing compares greater than NaN
   const bool row_nan = nan_any != 0u || !(m > -kInf && m < kInf);
   if (row_nan) {  // one NaN addend poisons the sum: the finish kernel needs nothing else
@@ -643,12 +651,12 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
   float l2[8];
   while (s_mine < s_end) {
     int s_next = grab();
-    if (s_next < s_end) load_slot_lane<DT>(logits, s_next, lane, V, fill, l2);
+    if (s_next < s_end) load_slot_lane<DT>(logits, s_next, lane, V, fill, l2, p.row.fused);
     work(s_mine, l);
     s_mine = s_next;
     if (s_mine >= s_end) break;
     s_next = grab();
-    if (s_next < s_end) load_slot_lane<DT>(logits, s_next, lane, V, fill, l);
+    if (s_next < s_end) load_slot_lane<DT>(logits, s_next, lane, V, fill, l, p.row.fused);
     work(s_mine, l2);
     s_mine = s_next;
   }
@@ -669,7 +677,7 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
       }
       uint32_t pattern16 = 0u;
       if constexpr (DT == kDtypeBFloat16 || DT == kDtypeHalf)
-        pattern16 = reinterpret_cast<const uint16_t*>(logits)[min(static_cast<uint32_t>(ent), static_cast<uint32_t>(V - 1))];
+        pattern16 = value_pattern<DT>(load_logit<DT>(logits, min(static_cast<uint32_t>(ent), static_cast<uint32_t>(V - 1)), p.row.fused));
       split_count_candidate<DT>(static_cast<uint32_t>(ent >> 32), pattern16, sh, km, ph);
     }
     __syncthreads();
@@ -751,7 +759,7 @@ __device__ __forceinline__ void resolve_lanes(float& s, const uint32_t (&bits)[8
 template <int DT>
 __device__ __forceinline__ float split_chain(const SlotRec* recs, int ns, const PrepSlot* prep, uint32_t n_prep,
                                              const char* logits, int V, float inv, float m, const uint64_t* tab,
-                                             uint64_t* stats = nullptr) {
+                                             const FusedOps& fused, uint64_t* stats = nullptr) {
   const int lane = threadIdx.x & 63;
   const float kInf = __uint_as_float(0x7f800000u);
   const float fill = inv < 0.0f ? kInf : -kInf;
@@ -831,7 +839,7 @@ __device__ __forceinline__ float split_chain(const SlotRec* recs, int ns, const 
           }
         } else {
           float l[8];
-          load_slot_lane<DT>(logits, slot, lane, V, fill, l);
+          load_slot_lane<DT>(logits, slot, lane, V, fill, l, fused);
 #pragma unroll
           for (int k = 0; k < 8; ++k) bits[k] = __float_as_uint(expf_core(__builtin_fmaxf(l[k] * inv - m, -104.0f), tab));
           int found = -1;
@@ -874,6 +882,7 @@ struct FinishShared {
   uint32_t sel_count, band_count;
   uint32_t overflow;
   HistPlan plan;
+  FusedOps fused;  // (the draw functions are calls: they read the launch's processors from here)
 };
 
 // By the whole workgroup, two buckets per lane; `plan_out` is LDS.  Ends with a barrier.
@@ -1034,6 +1043,7 @@ struct RunArgs {
   int32_t key_cut, n_bins, mag_min;
   uint32_t expected;      // candidates pass 2 listed: what the counters must add up to
   float m;
+  const FusedOps* fused;  // (LDS)
 };
 
 template <int DT>
@@ -1322,7 +1332,7 @@ __device__ __noinline__ bool draw_topp_runs(RunArgs a, const char* logits, int V
   const float kInf = __uint_as_float(0x7f800000u);
   auto matches = [&](int s_, int lane_) -> uint32_t {
     float l[8];
-    load_slot_lane<DT>(logits, s_, lane_, V, -kInf, l);
+    load_slot_lane<DT>(logits, s_, lane_, V, -kInf, l, *a.fused);
     uint32_t mask = 0u;
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
@@ -1395,6 +1405,7 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
   uint64_t t0 = 0, t1 = 0, t2 = 0;
   if (p.timers) t0 = wall_clock64();
   if (tid < 32) sm.exp2tab[tid] = kExp2Table[tid];
+  if (tid == 0) fs.fused = p.row.fused;  // (barriers follow before any draw function reads it)
 
   float S = kNaN;
   int n_listed = 0;
@@ -1460,7 +1471,7 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
     if (wave == 0) {
       const float sum = split_chain<DT>(reinterpret_cast<const SlotRec*>(lds_keys), ns,
                                         reinterpret_cast<const PrepSlot*>(prep_dst), n_prep, logits, V, inv, m, sm.exp2tab,
-                                        p.timers ? p.timers + static_cast<int64_t>(row) * 8 : nullptr);
+                                        p.row.fused, p.timers ? p.timers + static_cast<int64_t>(row) * 8 : nullptr);
       if (lane == 0) sm.bc_sum = sum;
     } else if (lists_ok && plan.b_sel >= 0 && plan.n_sel <= 64) {
       // ---- the other waves, meanwhile: one pass over the listed candidates picks out those of the
@@ -1505,13 +1516,13 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
     float* probs = p.row.probs + static_cast<int64_t>(row) * V;
     if (row_nan) {
       for (int i = tid; i < V; i += kBlock) {
-        const float x = load_elem<DT>(logits, i) * inv;
+        const float x = load_logit<DT>(logits, i, p.row.fused) * inv;
         probs[i] = expf_nonpositive(x - m, sm.exp2tab) / S;
       }
     } else {
       const RowDivisor div = row_divisor(S);
       for (int i = tid; i < V; i += kBlock) {
-        const float x = load_elem<DT>(logits, i) * inv;
+        const float x = load_logit<DT>(logits, i, p.row.fused) * inv;
         probs[i] = div_row(expf_nonpositive(x - m, sm.exp2tab), div);
       }
     }
@@ -1578,7 +1589,7 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
       // ---- a longer nucleus of a 16-bit row: runs of equal probabilities
       if (!done && rs.n_bins > 0 && (!lists_ok || n_listed > 4096)) {
         const RunArgs ra = {p.phist + static_cast<int64_t>(lrow) * p.row_wgs * p.phist_words, p.phist_words, p.row_wgs,
-                            p.row.lds_keys, ns, rs.key_cut, rs.n_bins, rs.mag_min, static_cast<uint32_t>(n_listed), m};
+                            p.row.lds_keys, ns, rs.key_cut, rs.n_bins, rs.mag_min, static_cast<uint32_t>(n_listed), m, &fs.fused};
         done = draw_topp_runs<DT>(ra, logits, V, inv, S, cutoff, topp, coin, lds_keys, dbg, token, sm);
         path = 4;
       }
@@ -1599,7 +1610,7 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
     if (!done) {
       uint64_t* scratch = p.row.scratch + static_cast<int64_t>(row) * p.row.scratch_stride;
       token = draw_general<DT>(logits, V, inv, m, S, false, 0, topp, cutoff, coin, scratch, p.row.scratch_stride, lds_keys,
-                               p.row.lds_keys, dbg, sm);
+                               p.row.lds_keys, dbg, sm, p.row.fused.n > 0 ? &fs.fused : nullptr);
       path = 3;
     }
   }

@@ -189,6 +189,24 @@ class Sampler:
         self._check(st)
         return out
 
+    def sample_batch_chain(self, logits: torch.Tensor, chain, out: torch.Tensor | None = None,
+                           dtype: int | None = None) -> torch.Tensor:
+        """``chain.process(logits)`` followed by ``sample_batch(logits)`` in one call
+        (text_token_generator.h:141-148).  Same tokens; the chain's trailing biases and factors may
+        be applied while the sampler reads the rows instead of being stored into ``logits``."""
+        if not logits.is_cuda or logits.dim() != 2 or logits.stride(1) != 1:
+            raise SamplerError(_capi.INVALID_ARGUMENT, "sample_batch_chain wants a device tensor [B, vocab] with unit inner stride")
+        B, V = logits.shape
+        if V != self.vocab_size:
+            raise SamplerError(_capi.INVALID_ARGUMENT, "last dimension differs from vocab_size")
+        code = dtype_code(logits) if dtype is None else dtype
+        if out is None:
+            out = torch.empty(B, dtype=torch.int32, device=logits.device)
+        stream = torch.cuda.current_stream(logits.device).cuda_stream
+        self._check(_capi.lib().ets_sampler_sample_batch_chain(
+            self._h, chain._h, logits.data_ptr(), code, B, logits.stride(0), out.data_ptr(), stream))
+        return out
+
     def gumbel_max_batch(self, logits: torch.Tensor, temperature, noise: torch.Tensor | None = None,
                          out: torch.Tensor | None = None, dtype: int | None = None) -> torch.Tensor:
         """The in-graph Gumbel-max sampler (examples/models/qwen3_5_moe/sampler.py:17-60):

@@ -76,6 +76,21 @@ ETS_API ets_status ets_logit_chain_add_repetition_penalty(ets_logit_chain* c, fl
 ETS_API ets_status ets_logit_chain_process(ets_logit_chain* c, void* d_logits, int32_t dtype, int32_t rank,
                                           const int64_t* sizes, void* hip_stream);
 
+/* The two steps of text_token_generator.h:141-148 in one call: the chain over rows
+ * [batch, vocab] (`row_stride_elems` elements apart), then ets_sampler_sample_batch() on them --
+ * the same tokens, coin streams and errors as ets_logit_chain_process() followed by
+ * ets_sampler_sample_batch() on the same stream.  What differs is what is left in the tensor:
+ * when the rows take the sampler's several-workgroups-per-row path (stochastic top-p rows of at
+ * least 8192 entries, 16-byte aligned), the chain's LAST processors, as far as they are biases
+ * and factors (up to four), are not stored into the tensor but applied while the sampler reads
+ * it -- rounded to the element type after each, as the stores would -- which saves a pass over
+ * the tensor that reads and writes every entry.  The processors in front of those still run in
+ * place.  A caller that reads the logits after sampling uses the two calls instead.
+ * `d_logits` and `d_tokens` are DEVICE pointers; asynchronous on `hip_stream`. */
+ETS_API ets_status ets_sampler_sample_batch_chain(ets_sampler* s, ets_logit_chain* c, void* d_logits, int32_t dtype,
+                                                 int32_t batch, int64_t row_stride_elems, int32_t* d_tokens,
+                                                 void* hip_stream);
+
 /* Text of the last error on this chain ("" if none). */
 ETS_API const char* ets_logit_chain_last_error(const ets_logit_chain* c);
 

@@ -153,3 +153,73 @@ def test_chain_then_sampler_on_one_stream(oracle, dev):
                                  states, mode=oracle.MODE_UPCAST, tie=oracle.TIE_STABLE)
     assert np.array_equal(got, want)
     assert not np.isin(got, banned).any()
+
+
+@pytest.mark.parametrize("dtype_name", ["bf16", "fp16", "fp32"])
+@pytest.mark.parametrize("ops", [
+    (("scale", 1.3), ("bias", -0.75)),
+    (("bias", 2.5),),
+    (("mask", None), ("scale", 0.7), ("bias", 0.3), ("scale", 1.1)),
+    (("scale", 1.3), ("mask", None), ("bias", 0.4)),
+    (("scale", -0.5), ("bias", 1.0)),
+    (("bias", 0.1), ("bias", 0.2), ("scale", 2.0), ("scale", 0.5), ("bias", -0.3), ("scale", 1.7)),
+])
+def test_chain_fused_into_the_sampler(dev, dtype_name, ops):
+    """sample_batch_chain against chain.process followed by sample_batch on a second copy: the same
+    tokens and coin states, whatever part of the chain the sampler applies while it reads the rows
+    (trailing biases and factors; a mask or more than four of them run in place first)."""
+    vocab, rows = 40000, 6
+    rng = np.random.default_rng(17)
+    x = (rng.standard_normal((rows, vocab)) * 2.0).astype(np.float32)
+    hot = rng.integers(0, vocab, size=(rows, 12))
+    np.put_along_axis(x, hot, np.take_along_axis(x, hot, 1) + 7.0, 1)
+    x[1, vocab - 3:] = -np.inf   # entries that drop out
+    x[2, 5] = np.inf if ops[0][0] != "scale" or ops[0][1] > 0 else -np.inf  # an infinite maximum: every probability NaN or one hot
+    tdt = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}[dtype_name]
+    if dtype_name == "fp16":
+        x = np.clip(x, -60000.0, 60000.0)
+    base = torch.from_numpy(x).to(dev).to(tdt)
+    banned = np.array([int(hot[0, 0]), 3, vocab - 1], dtype=np.int32)
+
+    def chain():
+        c = LogitChain()
+        for kind, v in ops:
+            if kind == "scale":
+                c.add_scale(v)
+            elif kind == "bias":
+                c.add_bias(v)
+            else:
+                c.add_mask(banned)
+        return c
+
+    for topp in (0.9, 0.5):
+        a, b = base.clone(), base.clone()
+        s1 = ea.Sampler(vocab, 0.8, topp, 1234, max_batch=rows)
+        s2 = ea.Sampler(vocab, 0.8, topp, 1234, max_batch=rows)
+        c1, c2 = chain(), chain()
+        c1.process(a)
+        want = s1.sample_batch(a).cpu().numpy()
+        got = s2.sample_batch_chain(b, c2).cpu().numpy()
+        assert np.array_equal(got, want), (dtype_name, ops, topp, got, want)
+        # a second call continues both coin streams alike
+        a2, b2 = base.clone(), base.clone()
+        c1.process(a2)
+        assert np.array_equal(s2.sample_batch_chain(b2, c2).cpu().numpy(), s1.sample_batch(a2).cpu().numpy())
+
+
+def test_chain_fused_falls_back_in_place(dev):
+    """Rows that do not take the several-workgroups path (here: too short, and temperature 0) get
+    the whole chain in place, then the sampler: the tensor then holds the processed logits."""
+    vocab, rows = 3000, 4
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((rows, vocab)).astype(np.float32)
+    for temperature in (0.7, 0.0):
+        a, b = torch.from_numpy(x).to(dev), torch.from_numpy(x).to(dev)
+        c1, c2 = LogitChain().add_scale(1.5).add_bias(0.25), LogitChain().add_scale(1.5).add_bias(0.25)
+        s1 = ea.Sampler(vocab, temperature, 0.9, 7, max_batch=rows)
+        s2 = ea.Sampler(vocab, temperature, 0.9, 7, max_batch=rows)
+        c1.process(a)
+        want = s1.sample_batch(a).cpu().numpy()
+        got = s2.sample_batch_chain(b, c2).cpu().numpy()
+        assert np.array_equal(got, want)
+        assert torch.equal(a, b)
