@@ -34,6 +34,8 @@ struct ErrorSink {
 struct WorkBuffers {
   ets::SplitParams split = {};
   uint64_t* scratch = nullptr;  // [rows, scratch_stride] keys of the general draw
+  uint32_t* tickets = nullptr;
+  int32_t scratch_rows = 0;
   int64_t scratch_stride = 0;
   uint64_t* partials = nullptr;  // [rows, kMaxSplits] arg-max partial results
   int max_row_wgs = 0;           // workgroups of pass 2 per row, at most
@@ -51,6 +53,8 @@ struct ets_sampler {
   size_t lds_bytes = 0;
   int64_t scratch_stride = 0;  // keys per row of candidate scratch (twice the vocabulary, rounded up)
   uint64_t* d_rng = nullptr;       // [max_batch]
+  uint32_t* d_tickets = nullptr;   // row counters of the row kernels' launches (0 between launches), one per draw
+  int32_t scratch_rows = 0;        // rows of candidate scratch: one per workgroup that can be resident, not one per row
   uint64_t* d_scratch = nullptr;   // [max_batch, scratch_stride], allocated on first stochastic use
   uint64_t* d_partials = nullptr;  // [max_batch, kMaxSplits] argmax partial results
   void* d_row = nullptr;           // staging for one host row (vocab * 4 bytes)
@@ -219,12 +223,16 @@ ets_status allow_dynamic_lds(ets_sampler* s, const void* kernel, size_t bytes, s
 }
 
 template <int DT, bool ALIGNED, int DRAW>
-ets_status launch_rows_impl(ets_sampler* s, const ets::RowParams& p, int32_t batch, hipStream_t stream) {
+ets_status launch_rows_impl(ets_sampler* s, const ets::RowParams& p_in, int32_t batch, hipStream_t stream) {
   static std::atomic<size_t> set_bytes[kMaxDevices];
   const size_t lds = s->lds_bytes;
   ets_status st = allow_dynamic_lds(s, reinterpret_cast<const void*>(&ets::sample_rows_kernel<DT, ALIGNED, DRAW>), lds, set_bytes);
   if (st != ETS_OK) return st;
-  hipLaunchKernelGGL((ets::sample_rows_kernel<DT, ALIGNED, DRAW>), dim3(batch), dim3(ets::kBlock), lds, stream, p);
+  ets::RowParams p = p_in;
+  p.rows = batch;
+  p.ticket = (s->wb ? s->wb->tickets : s->d_tickets) + DRAW;
+  const int grid = batch < p.grid_cap ? batch : p.grid_cap;
+  hipLaunchKernelGGL((ets::sample_rows_kernel<DT, ALIGNED, DRAW>), dim3(grid), dim3(ets::kBlock), lds, stream, p);
   ETS_HIP(s, hipGetLastError());
   return ETS_OK;
 }
@@ -263,7 +271,7 @@ float inverse_temperature_ctor(float temperature) {
 
 ets_status ensure_scratch(ets_sampler* s) {
   if (s->d_scratch || s->wb) return ETS_OK;
-  const size_t bytes = static_cast<size_t>(s->max_batch) * static_cast<size_t>(s->scratch_stride) * sizeof(uint64_t);
+  const size_t bytes = static_cast<size_t>(s->scratch_rows) * static_cast<size_t>(s->scratch_stride) * sizeof(uint64_t);
   ETS_HIP(s, hipMalloc(reinterpret_cast<void**>(&s->d_scratch), bytes));
   return ETS_OK;
 }
@@ -392,6 +400,8 @@ ets_status launch_split(ets_sampler* s, const ets::RowParams& p, int32_t rows, h
   }
   ets::SplitParams sp = s->wb ? s->wb->split : s->split;
   sp.row = p;
+  sp.row.rows = rows;
+  sp.row.ticket = (s->wb ? s->wb->tickets : s->d_tickets) + 3;  // (0 .. 2 are the one-workgroup-per-row kernel's, by draw)
   sp.phist_words = DT == ets::kDtypeBFloat16 ? kPhistWordsBFloat16 : (DT == ets::kDtypeHalf ? kPhistWordsHalf : 0);
   sp.row_wgs = pass2_workgroups(s, rows, sp.ns);
   sp.list_region = list_region(sp.ns, sp.row_wgs);
@@ -404,10 +414,17 @@ ets_status launch_split(ets_sampler* s, const ets::RowParams& p, int32_t rows, h
   if (st != ETS_OK) return st;
   hipLaunchKernelGGL((ets::split_pass2_kernel<DT, true>), dim3(sp.row_wgs, rows), dim3(ets::kBlock), lut_bytes, stream, sp);
   ETS_HIP(s, hipGetLastError());
-  static std::atomic<size_t> set_bytes[kMaxDevices];
-  st = allow_dynamic_lds(s, reinterpret_cast<const void*>(&ets::split_finish_kernel<DT>), s->lds_bytes, set_bytes);
-  if (st != ETS_OK) return st;
-  hipLaunchKernelGGL((ets::split_finish_kernel<DT>), dim3(rows), dim3(ets::kBlock), s->lds_bytes, stream, sp);
+  if (rows > p.grid_cap) {
+    static std::atomic<size_t> set_bytes[kMaxDevices];
+    st = allow_dynamic_lds(s, reinterpret_cast<const void*>(&ets::split_finish_kernel<DT, true>), s->lds_bytes, set_bytes);
+    if (st != ETS_OK) return st;
+    hipLaunchKernelGGL((ets::split_finish_kernel<DT, true>), dim3(p.grid_cap), dim3(ets::kBlock), s->lds_bytes, stream, sp);
+  } else {
+    static std::atomic<size_t> set_bytes[kMaxDevices];
+    st = allow_dynamic_lds(s, reinterpret_cast<const void*>(&ets::split_finish_kernel<DT, false>), s->lds_bytes, set_bytes);
+    if (st != ETS_OK) return st;
+    hipLaunchKernelGGL((ets::split_finish_kernel<DT, false>), dim3(rows), dim3(ets::kBlock), s->lds_bytes, stream, sp);
+  }
   ETS_HIP(s, hipGetLastError());
   return ETS_OK;
 }
@@ -458,6 +475,7 @@ ets_status sample_device(ets_sampler* s, const void* d_logits, int32_t dtype, in
   p.debug = reinterpret_cast<ets::RowDebug*>(d_debug);
   p.scratch = s->wb ? s->wb->scratch : s->d_scratch;
   p.scratch_stride = s->wb ? s->wb->scratch_stride : s->scratch_stride;
+  p.grid_cap = s->wb ? s->wb->scratch_rows : s->scratch_rows;
   p.lds_keys = s->lds_keys;
   p.row_map = nullptr;
   p.row_cfg = nullptr;
@@ -508,6 +526,7 @@ size_t layout_static(const ets_sampler* s, int32_t dtype, int32_t rows, char* ba
     at = round_up(at + bytes, 256);
     return base + here;
   };
+  wb->tickets = reinterpret_cast<uint32_t*>(take(16 * sizeof(uint32_t)));  // always the array's first bytes: 0 between launches
   sp.slot_max = reinterpret_cast<float*>(take(r * sp.ns_stride * sizeof(float)));
   sp.slot_sum = reinterpret_cast<float*>(take(r * sp.ns_stride * sizeof(float)));
   sp.slot_rec = reinterpret_cast<ets::SlotRec*>(take(r * sp.ns_stride * sizeof(ets::SlotRec)));
@@ -519,7 +538,8 @@ size_t layout_static(const ets_sampler* s, int32_t dtype, int32_t rows, char* ba
   sp.list = reinterpret_cast<uint64_t*>(take(r * g * list_region(sp.ns, g) * sizeof(uint64_t)));
   sp.timers = nullptr;
   wb->scratch_stride = s->scratch_stride;
-  wb->scratch = reinterpret_cast<uint64_t*>(take(r * static_cast<size_t>(s->scratch_stride) * sizeof(uint64_t)));
+  wb->scratch_rows = rows < s->scratch_rows ? rows : s->scratch_rows;
+  wb->scratch = reinterpret_cast<uint64_t*>(take(static_cast<size_t>(wb->scratch_rows) * static_cast<size_t>(s->scratch_stride) * sizeof(uint64_t)));
   wb->partials = reinterpret_cast<uint64_t*>(take(r * kMaxSplits * sizeof(uint64_t)));
   return at;
 }
@@ -656,10 +676,15 @@ ets_status sample_device_configs(ets_sampler* s, const void* d_logits, int32_t d
   p.tokens = d_tokens;
   p.probs = nullptr;
   p.debug = reinterpret_cast<ets::RowDebug*>(d_debug);
-  p.scratch = s->d_scratch;
   p.scratch_stride = s->scratch_stride;
   p.lds_keys = s->lds_keys;
   p.row_cfg = reinterpret_cast<const ets::RowConfig*>(d + lay.cfg);
+  // The groups that draw run side by side: each gets its share of the scratch rows (a workgroup
+  // owns the scratch row of its index in its launch).
+  const int drawing = (count[1] > 0) + (count[2] > 0) + (count[3] > 0);
+  const int32_t share = drawing > 0 ? s->scratch_rows / drawing : 0;
+  if (drawing > 0 && share < 1) return fail(s, ETS_INTERNAL, "ets_sampler_sample_batch_configs: no scratch rows");
+  int32_t next_scratch_row = 0;
   // the longest-running groups first (multinomial, top-k, top-p), the arg-max last
   const int order[3] = {ets::kDrawMultinomial, ets::kDrawTopK, ets::kDrawTopP};
   for (int k = 0; k < 3; ++k) {
@@ -668,6 +693,9 @@ ets_status sample_device_configs(ets_sampler* s, const void* d_logits, int32_t d
     hipStream_t gs = nullptr;
     st = group_stream(&gs);
     if (st != ETS_OK) return st;
+    p.scratch = s->d_scratch + static_cast<int64_t>(next_scratch_row) * s->scratch_stride;
+    p.grid_cap = share;
+    next_scratch_row += share;
     p.row_map = d_maps + (1 + draw) * batch;
     st = rows_device(s, p, dtype, count[1 + draw], gs, draw);
     if (st != ETS_OK) return st;
@@ -746,6 +774,12 @@ ets_status ets_sampler_create(int32_t vocab_size, float temperature, float topp,
   // two buffers of a row's sort keys (the radix sort of large candidate sets moves between them)
   s->scratch_stride = 2 * ((static_cast<int64_t>(vocab_size) + 63) / 64 * 64);
 
+  // the row kernels keep one workgroup per CU resident (their LDS): that many rows of scratch
+  s->scratch_rows = max_batch < s->num_cus ? max_batch : (s->num_cus > 0 ? s->num_cus : 1);
+  e = hipMalloc(reinterpret_cast<void**>(&s->d_tickets), sizeof(uint32_t) * 16);
+  if (e != hipSuccess) return bail(e, "hipMalloc(tickets)");
+  e = hipMemset(s->d_tickets, 0, sizeof(uint32_t) * 16);
+  if (e != hipSuccess) return bail(e, "hipMemset(tickets)");
   e = hipMalloc(reinterpret_cast<void**>(&s->d_rng), sizeof(uint64_t) * max_batch);
   if (e != hipSuccess) return bail(e, "hipMalloc(rng states)");
   e = hipMalloc(reinterpret_cast<void**>(&s->d_partials), sizeof(uint64_t) * max_batch * kMaxSplits);
@@ -777,6 +811,7 @@ ets_status ets_sampler_destroy(ets_sampler* s) {
   {
     DeviceGuard g(s->device);
     (void)hipFree(s->d_rng);
+    (void)hipFree(s->d_tickets);
     (void)hipFree(s->d_scratch);
     (void)hipFree(s->d_split);
     (void)hipFree(s->d_phist);

@@ -56,7 +56,34 @@ struct RowParams {
   const int32_t* row_map;    // workgroup -> row, or null for the identity
   const RowConfig* row_cfg;  // [batch] per-row parameters (by row), or null for the launch-wide ones
   FusedOps fused;            // logit processors applied as the logits are read (several-workgroups-per-row path only)
+  // One workgroup per row, but no more workgroups than the launch's grid: a workgroup that is done
+  // with a row takes the next one from `ticket` (0 before and after every launch), and the row's
+  // scratch is the workgroup's, not the row's.
+  int32_t rows;
+  uint32_t* ticket;
+  int32_t grid_cap;  // (host side only: the most workgroups the launch may have, i.e. scratch rows behind `scratch`)
 };
+
+// Rows beyond the launch's workgroups are handed out by `ticket`: a workgroup asks for its next row
+// when it starts on one (the answer has arrived long before the row is done) and picks it up with
+// take_row().  Rows 0 .. gridDim.x - 1 are the workgroups' first ones, asked for by nobody; every
+// row a workgroup works on costs one request, so the launch makes p.rows of them, and whoever makes
+// the last one puts the counter back to 0 for the next launch.  A launch with a workgroup per row
+// touches no counter.
+__device__ __forceinline__ void request_row(const RowParams& p, int* lds_slot) {
+  if (static_cast<int>(gridDim.x) < p.rows && threadIdx.x == 0) {
+    const uint32_t t = atomicAdd(p.ticket, 1u);
+    if (t + 1u == static_cast<uint32_t>(p.rows)) atomicExch(p.ticket, 0u);
+    *lds_slot = static_cast<int>(gridDim.x + t);
+  }
+}
+__device__ __forceinline__ int take_row(const RowParams& p, const int* lds_slot) {
+  if (static_cast<int>(gridDim.x) >= p.rows) return p.rows;
+  __syncthreads();
+  const int next = *lds_slot;
+  __syncthreads();
+  return next;
+}
 
 // A float rounded to the row's element type and back (round to nearest even; a NaN stays a NaN).
 template <int DT>
@@ -1558,19 +1585,22 @@ template <int DT, bool ALIGNED, int DRAW>
 __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
   extern __shared__ __align__(16) uint64_t lds_keys[];
   __shared__ BlockScratch sm;
+  __shared__ int next_lrow;
   constexpr int VE = VecElems<DT>::value;
-  const int row = p.row_map ? p.row_map[blockIdx.x] : blockIdx.x;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int V = p.vocab;
+  uint64_t* scratch = p.scratch + static_cast<int64_t>(blockIdx.x) * p.scratch_stride;
+  const float kInf = __uint_as_float(0x7f800000u);
+  const float kNaN = __uint_as_float(0x7fc00000u);
+  for (int lrow = blockIdx.x; lrow < p.rows; lrow = take_row(p, &next_lrow)) {
+  request_row(p, &next_lrow);
+  const int row = p.row_map ? p.row_map[lrow] : lrow;
   const float inv = p.row_cfg ? p.row_cfg[row].inv_temperature : p.inv_temperature;
   const float topp = p.row_cfg ? p.row_cfg[row].topp : p.topp;
   const int32_t topk = p.row_cfg ? p.row_cfg[row].topk : p.topk;
   const char* logits = static_cast<const char*>(p.logits) + static_cast<int64_t>(row) * p.row_stride * ElemSize<DT>::value;
-  uint64_t* scratch = p.scratch + static_cast<int64_t>(row) * p.scratch_stride;
-  const float kInf = __uint_as_float(0x7f800000u);
-  const float kNaN = __uint_as_float(0x7fc00000u);
 
   if (tid < 32) sm.exp2tab[tid] = kExp2Table[tid];
   if (tid == 0) sm.counter = 0u;
@@ -1852,6 +1882,7 @@ __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
     p.tokens[row] = token;
     if (p.debug) p.debug[row] = dbg;
   }
+  }  // rows of this workgroup
 }
 
 // ---- measurement floors (hooks for the benchmark: what a launch and a plain read cost here) ------

@@ -75,8 +75,6 @@ constexpr int kListRegion = 16384;     // candidates one workgroup of pass 2 can
 // Bucket b holds exp bit patterns in (0x3F800000 - (b + 1) * 2^17, 0x3F800000 - b * 2^17]; the last
 // bucket also takes everything below.
 constexpr int kHistBuckets = 2048;
-constexpr int kLdsList = 2048;  // candidates and slot records a workgroup of pass 2 keeps in LDS during its sweep
-constexpr int kLdsRecs = 512;
 __device__ __forceinline__ uint32_t hist_bucket(uint32_t e_bits) {
   const uint32_t b = (0x3F800000u - e_bits) >> 17;  // (exp <= 1)
   return b < static_cast<uint32_t>(kHistBuckets - 1) ? b : static_cast<uint32_t>(kHistBuckets - 1);
@@ -242,89 +240,43 @@ struct Pass2Shared {
   uint32_t cls[kMaxSlots];    // per slot: kb_lo | kb_hi << 8 | kind << 16 | prepared-slot index << 19
   uint32_t hist[kHistBuckets];
   uint32_t list_count;        // candidates this workgroup has listed
-  int next_slot;              // the next slot no wave has taken yet
-  // What the sweep produces is kept here and stored after it: a wave that stores to global memory
-  // between its loads waits for those stores whenever it waits for the next slot's entries.
-  uint64_t list[kLdsList];    // the first candidates of the workgroup's list
-  SlotRec recs[kLdsRecs];     // the records of the workgroup's first slots
 };
-
-// One candidate into the workgroup's histograms: by the size of exp and, for 16-bit rows, by bit
-// pattern (one outside the range of bins is missed there, which the totals give away).
-template <int DT>
-__device__ __forceinline__ void split_count_candidate(uint32_t e_bits, uint32_t pattern16, Pass2Shared& sh, const KeyMap& km,
-                                                      uint32_t* ph) {
-  atomicAdd(&sh.hist[hist_bucket(e_bits)], 1u);
-  if constexpr (DT == kDtypeBFloat16 || DT == kDtypeHalf) {
-    const int bin = pattern_key(pattern16, km.mag_min) - km.key_cut;
-    if (bin >= 0 && bin < km.n_bins) atomicAdd(&ph[bin >> 1], 1u << ((bin & 1) << 4));
-  }
-}
 
 // One wave, one slot: e[] are the lane's 8 entries; `cls` is the slot's entry of Pass2Shared::cls.
 template <bool TOPP, int DT>
-__device__ __forceinline__ void split_fold_slot(const SplitParams& p, int row, int s, int s_begin, const float (&e)[8],
+__device__ __forceinline__ void split_fold_slot(const SplitParams& p, int row, int s, const float (&e)[8],
                                                 const float (&logit)[8], uint32_t cls, float cut_lo, int V, uint64_t* region,
                                                 Pass2Shared& sh, const KeyMap& km, uint32_t* ph) {
   const int lane = threadIdx.x & 63;
-  auto put_rec = [&](const SlotRec& r) {
-    if (s - s_begin < kLdsRecs) {
-      sh.recs[s - s_begin] = r;
-    } else {
-      p.slot_rec[static_cast<int64_t>(row) * p.ns_stride + s] = r;
-    }
-  };
+  const int64_t rec_at = static_cast<int64_t>(row) * p.ns_stride + s;
   // ---- candidates of the top-p draw (sampler.cpp:137-143), by a cut that is safely below the
   //      reference's once the exact normaliser is known
   if (TOPP) {
     uint32_t cmask = 0u;
 #pragma unroll
-    for (int k = 0; k < 8; ++k) cmask |= e[k] >= cut_lo ? (1u << k) : 0u;
-    if (s == p.ns - 1) {  // entries past the row's end
-      const int left = V - (s * kSlot + lane * 8);
-      cmask &= left >= 8 ? 0xffu : (left > 0 ? (1u << left) - 1u : 0u);
-    }
+    for (int k = 0; k < 8; ++k) cmask |= (e[k] >= cut_lo && s * kSlot + lane * 8 + k < V) ? (1u << k) : 0u;
     if (__ballot(cmask != 0u) != 0ull) {
-      // The list's order does not matter: every lane reserves its own places.  A listed candidate
-      // is counted into the histograms after the sweep, by all lanes side by side
-      // (split_count_listed); one that does not fit the list is counted here.
       const uint32_t mine = static_cast<uint32_t>(__popc(cmask));
-      uint32_t at = 0u;
-      if (mine) at = atomicAdd(&sh.list_count, mine);
+      const uint32_t incl = wave_scan_inclusive_u32(mine);
+      const uint32_t total = readlane_u32(incl, 63);
+      uint32_t base = 0u;
+      if (lane == 0) base = atomicAdd(&sh.list_count, total);
+      base = readlane_u32(base, 0);
+      uint32_t at = base + incl - mine;
       const int first = s * kSlot + lane * 8;
-      auto note = [&](float ek, float lk, int k) {
-        const uint32_t eb = __float_as_uint(ek);
-        const uint64_t ent = (static_cast<uint64_t>(eb) << 32) | static_cast<uint32_t>(first + k);
-        if (at < static_cast<uint32_t>(kLdsList)) {
-          sh.list[at] = ent;
-        } else if (at < static_cast<uint32_t>(p.list_region)) {
-          region[at] = ent;
-        } else {
-          split_count_candidate<DT>(eb, value_pattern<DT>(lk), sh, km, ph);
-        }
-        ++at;
-      };
-      if (__ballot(mine > 2u) != 0ull) {
-        // dense: entry by entry
 #pragma unroll
-        for (int k = 0; k < 8; ++k) {
-          if ((cmask >> k) & 1u) note(e[k], logit[k], k);
-        }
-      } else {
-        // sparse (the usual row: a few candidates in a slot): as many rounds as the busiest lane has candidates
-        for (int round = 0; round < 2; ++round) {
-          if (__ballot(cmask != 0u) == 0ull) break;
-          if (cmask) {
-            const int k = __ffs(static_cast<int>(cmask)) - 1;
-            cmask &= cmask - 1u;
-            float ek = e[0], lk = logit[0];
-#pragma unroll
-            for (int j = 1; j < 8; ++j) {
-              ek = k == j ? e[j] : ek;
-              lk = k == j ? logit[j] : lk;
-            }
-            note(ek, lk, k);
+      for (int k = 0; k < 8; ++k) {
+        if ((cmask >> k) & 1u) {
+          const uint32_t eb = __float_as_uint(e[k]);
+          atomicAdd(&sh.hist[hist_bucket(eb)], 1u);
+          if constexpr (DT == kDtypeBFloat16 || DT == kDtypeHalf) {
+            // 16-bit rows: the same candidates per bit pattern (one outside the range of bins is
+            // missed there, which the totals give away)
+            const int bin = pattern_key(value_pattern<DT>(logit[k]), km.mag_min) - km.key_cut;
+            if (bin >= 0 && bin < km.n_bins) atomicAdd(&ph[bin >> 1], 1u << ((bin & 1) << 4));
           }
+          if (at < static_cast<uint32_t>(p.list_region)) region[at] = (static_cast<uint64_t>(eb) << 32) | static_cast<uint32_t>(first + k);
+          ++at;
         }
       }
     }
@@ -337,7 +289,7 @@ __device__ __forceinline__ void split_fold_slot(const SplitParams& p, int row, i
     float sum = 0.0f;
     int found = -1;
     wave_resolve<8>(sum, found, bits, lane * 8, V, __uint_as_float(0x7f800000u));
-    if (lane == 0) put_rec(SlotRec{kSlotExact << 8, __float_as_uint(sum), 0u, 0xffffffffu});
+    if (lane == 0) p.slot_rec[rec_at] = {kSlotExact << 8, __float_as_uint(sum), 0u, 0xffffffffu};
     return;
   }
   // ---- every entry 0: no effect on any running sum
@@ -345,7 +297,7 @@ __device__ __forceinline__ void split_fold_slot(const SplitParams& p, int row, i
 #pragma unroll
   for (int k = 0; k < 8; ++k) nonzero = nonzero || e[k] != 0.0f;
   if (__ballot(nonzero) == 0ull) {
-    if (lane == 0) put_rec(SlotRec{kSlotZero << 8, 0u, 0u, 0xffffffffu});
+    if (lane == 0) p.slot_rec[rec_at] = {kSlotZero << 8, 0u, 0u, 0xffffffffu};
     return;
   }
   const uint32_t kb_lo = cls & 255u, kb_hi = (cls >> 8) & 255u;
@@ -367,7 +319,7 @@ __device__ __forceinline__ void split_fold_slot(const SplitParams& p, int row, i
       slot.even = readlane_u32(upto.even, 63);
       slot.odd = readlane_u32(upto.odd, 63);
     }
-    if (lane == 0) put_rec(SlotRec{kb_lo | (kSlotStable << 8), slot.even, slot.odd, 0xffffffffu});
+    if (lane == 0) p.slot_rec[rec_at] = {kb_lo | (kSlotStable << 8), slot.even, slot.odd, 0xffffffffu};
     return;
   }
   if (kind == kSlotDual) {
@@ -383,10 +335,10 @@ __device__ __forceinline__ void split_fold_slot(const SplitParams& p, int row, i
     const float inc_a = wave_sum_f32(fa.inc), inc_b = wave_sum_f32(fb.inc);
     if (lane == 0) {
       if (ties) {  // (rare) the finish kernel works the slot out from the logits
-        put_rec(SlotRec{kb_lo | (kSlotSerial << 8), 0u, 0u, 0xffffffffu});
+        p.slot_rec[rec_at] = {kb_lo | (kSlotSerial << 8), 0u, 0u, 0xffffffffu};
       } else {
-        put_rec(SlotRec{kb_lo | (kSlotDual << 8), inc_a < 67108864.0f ? static_cast<uint32_t>(inc_a) : kSat,
-                              inc_b < 67108864.0f ? static_cast<uint32_t>(inc_b) : kSat, 0xffffffffu});
+        p.slot_rec[rec_at] = {kb_lo | (kSlotDual << 8), inc_a < 67108864.0f ? static_cast<uint32_t>(inc_a) : kSat,
+                              inc_b < 67108864.0f ? static_cast<uint32_t>(inc_b) : kSat, 0xffffffffu};
       }
     }
     return;
@@ -425,8 +377,8 @@ __device__ __forceinline__ void split_fold_slot(const SplitParams& p, int row, i
     }
   }
   if (lane == 0) {
-    put_rec(SlotRec{kb_a | (kSlotSerial << 8), 0u, 0u,
-                          idx < static_cast<uint32_t>(p.prep_cap) ? idx : 0xffffffffu});
+    p.slot_rec[rec_at] = {kb_a | (kSlotSerial << 8), 0u, 0u,
+                          idx < static_cast<uint32_t>(p.prep_cap) ? idx : 0xffffffffu};
   }
 }
 
@@ -467,14 +419,13 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
     }
   }
 
-  // ---- this workgroup's slots: wave w starts with slot s_begin + w, whose entries are requested
-  //      before anything else
+  // ---- this workgroup's slots: wave w takes s_begin + w, s_begin + w + 16, ...; the first one's
+  //      entries are requested before anything else
   int s_begin, s_end;
   split_range(ns, gridDim.x, blockIdx.x, s_begin, s_end);
   float l[8];
   int s_mine = s_begin + wave;
   if (s_mine < s_end) load_slot_lane<DT>(logits, s_mine, lane, V, fill, l, p.row.fused);
-  if (tid == 0) sh.next_slot = s_begin + kWaves;
 
   // ---- row maximum (sampler.cpp:191-197) from the slots' maxima
   float m = -kInf;
@@ -638,48 +589,19 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
         e[k] = expf_core(d, tab);
       }
     }
-    split_fold_slot<TOPP, DT>(p, row, s, s_begin, e, in, sh.cls[s], cut_lo, V, region, sh, km, ph);
-  };
-  // A wave's first slot is fixed (s_begin + wave, on its way since the kernel's start); the others
-  // are taken from a counter as the waves get to them, one ahead of the slot being worked on: slots
-  // differ a lot in cost (the row's first one is summed entry by entry, some hold many candidates).
-  auto grab = [&]() {
-    int s = 0;
-    if (lane == 0) s = atomicAdd(&sh.next_slot, 1);
-    return __builtin_amdgcn_readfirstlane(s);
+    split_fold_slot<TOPP, DT>(p, row, s, e, in, sh.cls[s], cut_lo, V, region, sh, km, ph);
   };
   float l2[8];
   while (s_mine < s_end) {
-    int s_next = grab();
-    if (s_next < s_end) load_slot_lane<DT>(logits, s_next, lane, V, fill, l2, p.row.fused);
+    if (s_mine + kWaves < s_end) load_slot_lane<DT>(logits, s_mine + kWaves, lane, V, fill, l2, p.row.fused);
     work(s_mine, l);
-    s_mine = s_next;
+    s_mine += kWaves;
     if (s_mine >= s_end) break;
-    s_next = grab();
-    if (s_next < s_end) load_slot_lane<DT>(logits, s_next, lane, V, fill, l, p.row.fused);
+    if (s_mine + kWaves < s_end) load_slot_lane<DT>(logits, s_mine + kWaves, lane, V, fill, l, p.row.fused);
     work(s_mine, l2);
-    s_mine = s_next;
+    s_mine += kWaves;
   }
-  __syncthreads();
-  for (int i = tid; i < min(s_end - s_begin, kLdsRecs); i += kBlock)
-    p.slot_rec[static_cast<int64_t>(row) * p.ns_stride + s_begin + i] = sh.recs[i];
   if (TOPP) {
-    // (the barrier above also orders the list's stores in front of the loads below: one workgroup, one L1)
-    // ---- the listed candidates into the histograms, one per lane
-    const int n_here = static_cast<int>(min(sh.list_count, static_cast<uint32_t>(p.list_region)));
-    for (int j = tid; j < n_here; j += kBlock) {
-      uint64_t ent;
-      if (j < kLdsList) {
-        ent = sh.list[j];
-        region[j] = ent;
-      } else {
-        ent = region[j];
-      }
-      uint32_t pattern16 = 0u;
-      if constexpr (DT == kDtypeBFloat16 || DT == kDtypeHalf)
-        pattern16 = value_pattern<DT>(load_logit<DT>(logits, min(static_cast<uint32_t>(ent), static_cast<uint32_t>(V - 1)), p.row.fused));
-      split_count_candidate<DT>(static_cast<uint32_t>(ent >> 32), pattern16, sh, km, ph);
-    }
     __syncthreads();
     if (tid == 0) p.list_count[static_cast<int64_t>(lrow) * kMaxRowWorkgroups + blockIdx.x] = sh.list_count;
     uint32_t* hist_out = p.hist + (static_cast<int64_t>(lrow) * p.row_wgs + blockIdx.x) * kHistBuckets;
@@ -1382,18 +1304,23 @@ __device__ __noinline__ bool draw_topp_runs(RunArgs a, const char* logits, int V
 
 // grid = rows; dynamic LDS: the key buffer of the draw (p.row.lds_keys keys), which holds the
 // slot records and the prepared slots while the sum is composed.
-template <int DT>
+// LOOP: fewer workgroups than rows, a workgroup takes one row after the other (the loop costs
+// registers, so a launch with a workgroup per row uses the instantiation without it).
+template <int DT, bool LOOP>
 __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
   extern __shared__ __align__(16) uint64_t lds_keys[];
   __shared__ BlockScratch sm;
   __shared__ FinishShared fs;
-  const int lrow = blockIdx.x;  // row of this launch: indexes the buffers whose layout depends on the launch
-  const int row = p.row.row_map ? p.row.row_map[blockIdx.x] : blockIdx.x;
+  __shared__ int next_lrow;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int V = p.row.vocab;
   const int ns = p.ns;
+  // lrow, the row of this launch, indexes the buffers whose layout depends on the launch
+  for (int lrow = blockIdx.x; lrow < p.row.rows; lrow = LOOP ? take_row(p.row, &next_lrow) : p.row.rows) {
+  if (LOOP) request_row(p.row, &next_lrow);
+  const int row = p.row.row_map ? p.row.row_map[lrow] : lrow;
   const float inv = p.row.row_cfg ? p.row.row_cfg[row].inv_temperature : p.row.inv_temperature;
   const float topp = p.row.row_cfg ? p.row.row_cfg[row].topp : p.row.topp;
   const char* logits = static_cast<const char*>(p.row.logits) + static_cast<int64_t>(row) * p.row.row_stride * ElemSize<DT>::value;
@@ -1608,7 +1535,7 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
       path = 2;
     }
     if (!done) {
-      uint64_t* scratch = p.row.scratch + static_cast<int64_t>(row) * p.row.scratch_stride;
+      uint64_t* scratch = p.row.scratch + static_cast<int64_t>(blockIdx.x) * p.row.scratch_stride;
       token = draw_general<DT>(logits, V, inv, m, S, false, 0, topp, cutoff, coin, scratch, p.row.scratch_stride, lds_keys,
                                p.row.lds_keys, dbg, sm, p.row.fused.n > 0 ? &fs.fused : nullptr);
       path = 3;
@@ -1626,6 +1553,7 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
       t[4] = static_cast<uint64_t>(path) | (static_cast<uint64_t>(plan.n_sel) << 8) | (static_cast<uint64_t>(fs.band_count) << 32);
     }
   }
+  }  // rows of this workgroup
 }
 
 }  // namespace ets

@@ -110,3 +110,29 @@ def test_row_pitch_and_row_map_when_split(oracle, dev):
         o = oracle.Sampler(V, t, p, 400 + b, mode=oracle.MODE_UPCAST, tie=oracle.TIE_STABLE)
         o.set_topk(k)
         assert got2[b] == o.sample(x[b].copy(), W.DTYPE_FLOAT), b
+
+
+@pytest.mark.parametrize("topp,topk", [(0.9, 0), (1.0, 0), (0.9, 30)])
+@pytest.mark.parametrize("mode", [SPLIT_ON, SPLIT_OFF])
+def test_more_rows_than_workgroups(oracle, dev, topp, topk, mode):
+    """The row kernels launch no more workgroups than the GPU keeps resident and hand the other rows
+    out from a counter that is 0 again after every launch: 700 rows, then 300 on the same handle,
+    then 700 again, against the oracle (top-p, multinomial, top-k; both paths)."""
+    V, rows = 9000, 700
+    rng = np.random.default_rng(3)
+    s = ea.Sampler(V, 0.8, topp, 41, max_batch=rows)
+    s.set_row_split(mode)
+    if topk:
+        s.set_topk(topk)
+    states = (np.uint64(41) + np.arange(rows, dtype=np.uint64)).astype(np.uint64)
+    inv = oracle.inv_temperature(0.8)
+    for n in (rows, 300, rows):
+        x = (rng.standard_normal((n, V)) * 1.5).astype(np.float32)
+        hot = rng.integers(0, V, size=(n, 6))
+        np.put_along_axis(x, hot, np.take_along_axis(x, hot, 1) + 6.0, 1)
+        got = s.sample_batch(to_device(x, W.DTYPE_FLOAT, dev)).cpu().numpy()
+        st = states[:n].copy()
+        want, _ = oracle.sample_rows(x, W.DTYPE_FLOAT, inv, topp, topk, st, mode=oracle.MODE_UPCAST, tie=oracle.TIE_STABLE, threads=8)
+        states[:n] = st
+        assert np.array_equal(got, want), (n, np.nonzero(got != want)[0][:8])
+        assert np.array_equal(s.get_rng_states(n), states[:n])
