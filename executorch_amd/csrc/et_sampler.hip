@@ -222,19 +222,25 @@ ets_status allow_dynamic_lds(ets_sampler* s, const void* kernel, size_t bytes, s
   return ETS_OK;
 }
 
-template <int DT, bool ALIGNED, int DRAW>
-ets_status launch_rows_impl(ets_sampler* s, const ets::RowParams& p_in, int32_t batch, hipStream_t stream) {
+template <int DT, bool ALIGNED, int DRAW, bool LOOP>
+ets_status launch_rows_looped(ets_sampler* s, const ets::RowParams& p, int grid, hipStream_t stream) {
   static std::atomic<size_t> set_bytes[kMaxDevices];
   const size_t lds = s->lds_bytes;
-  ets_status st = allow_dynamic_lds(s, reinterpret_cast<const void*>(&ets::sample_rows_kernel<DT, ALIGNED, DRAW>), lds, set_bytes);
+  ets_status st = allow_dynamic_lds(s, reinterpret_cast<const void*>(&ets::sample_rows_kernel<DT, ALIGNED, DRAW, LOOP>), lds, set_bytes);
   if (st != ETS_OK) return st;
+  hipLaunchKernelGGL((ets::sample_rows_kernel<DT, ALIGNED, DRAW, LOOP>), dim3(grid), dim3(ets::kBlock), lds, stream, p);
+  ETS_HIP(s, hipGetLastError());
+  return ETS_OK;
+}
+
+template <int DT, bool ALIGNED, int DRAW>
+ets_status launch_rows_impl(ets_sampler* s, const ets::RowParams& p_in, int32_t batch, hipStream_t stream) {
   ets::RowParams p = p_in;
   p.rows = batch;
   p.ticket = (s->wb ? s->wb->tickets : s->d_tickets) + DRAW;
-  const int grid = batch < p.grid_cap ? batch : p.grid_cap;
-  hipLaunchKernelGGL((ets::sample_rows_kernel<DT, ALIGNED, DRAW>), dim3(grid), dim3(ets::kBlock), lds, stream, p);
-  ETS_HIP(s, hipGetLastError());
-  return ETS_OK;
+  // a workgroup per row while the scratch rows last; beyond that the rows are handed out by ticket
+  return batch > p.grid_cap ? launch_rows_looped<DT, ALIGNED, DRAW, true>(s, p, p.grid_cap, stream)
+                            : launch_rows_looped<DT, ALIGNED, DRAW, false>(s, p, batch, stream);
 }
 
 // Which draw follows the softmax (sampler.cpp:238-249).

@@ -1581,7 +1581,9 @@ __device__ __noinline__ bool draw_topk_listed(uint64_t* lds_keys, int cap, int l
 // the list of possible top-p candidates.  Then the coin and the draw.
 constexpr int kDrawTopP = 0, kDrawMultinomial = 1, kDrawTopK = 2;  // sampler.cpp:238-249, chosen by the host
 
-template <int DT, bool ALIGNED, int DRAW>
+// LOOP: fewer workgroups than rows, a workgroup takes one row after the other (the loop costs
+// registers, so a launch with a workgroup per row uses the instantiation without it).
+template <int DT, bool ALIGNED, int DRAW, bool LOOP>
 __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
   extern __shared__ __align__(16) uint64_t lds_keys[];
   __shared__ BlockScratch sm;
@@ -1594,8 +1596,8 @@ __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
   uint64_t* scratch = p.scratch + static_cast<int64_t>(blockIdx.x) * p.scratch_stride;
   const float kInf = __uint_as_float(0x7f800000u);
   const float kNaN = __uint_as_float(0x7fc00000u);
-  for (int lrow = blockIdx.x; lrow < p.rows; lrow = take_row(p, &next_lrow)) {
-  request_row(p, &next_lrow);
+  for (int lrow = blockIdx.x; lrow < p.rows; lrow = LOOP ? take_row(p, &next_lrow) : p.rows) {
+  if (LOOP) request_row(p, &next_lrow);
   const int row = p.row_map ? p.row_map[lrow] : lrow;
   const float inv = p.row_cfg ? p.row_cfg[row].inv_temperature : p.inv_temperature;
   const float topp = p.row_cfg ? p.row_cfg[row].topp : p.topp;
