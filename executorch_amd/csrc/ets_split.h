@@ -254,29 +254,68 @@ __device__ __forceinline__ void split_fold_slot(const SplitParams& p, int row, i
   if (TOPP) {
     uint32_t cmask = 0u;
 #pragma unroll
-    for (int k = 0; k < 8; ++k) cmask |= (e[k] >= cut_lo && s * kSlot + lane * 8 + k < V) ? (1u << k) : 0u;
-    if (__ballot(cmask != 0u) != 0ull) {
-      const uint32_t mine = static_cast<uint32_t>(__popc(cmask));
-      const uint32_t incl = wave_scan_inclusive_u32(mine);
-      const uint32_t total = readlane_u32(incl, 63);
-      uint32_t base = 0u;
-      if (lane == 0) base = atomicAdd(&sh.list_count, total);
-      base = readlane_u32(base, 0);
-      uint32_t at = base + incl - mine;
+    for (int k = 0; k < 8; ++k) cmask |= e[k] >= cut_lo ? (1u << k) : 0u;
+    if (s == p.ns - 1) {  // entries past the row's end
+      const int left = V - (s * kSlot + lane * 8);
+      cmask &= left >= 8 ? 0xffu : (left > 0 ? (1u << left) - 1u : 0u);
+    }
+    const uint64_t has1 = __ballot(cmask != 0u);
+    if (has1 != 0ull) {
       const int first = s * kSlot + lane * 8;
+      uint32_t at = 0u;
+      auto note = [&](float ek, float lk, int k) {
+        const uint32_t eb = __float_as_uint(ek);
+        atomicAdd(&sh.hist[hist_bucket(eb)], 1u);
+        if constexpr (DT == kDtypeBFloat16 || DT == kDtypeHalf) {
+          // 16-bit rows: the same candidates per bit pattern (one outside the range of bins is
+          // missed there, which the totals give away)
+          const int bin = pattern_key(value_pattern<DT>(lk), km.mag_min) - km.key_cut;
+          if (bin >= 0 && bin < km.n_bins) atomicAdd(&ph[bin >> 1], 1u << ((bin & 1) << 4));
+        }
+        if (at < static_cast<uint32_t>(p.list_region)) region[at] = (static_cast<uint64_t>(eb) << 32) | static_cast<uint32_t>(first + k);
+        ++at;
+      };
+      const uint32_t rest1 = cmask & (cmask - 1u);   // without the lane's first candidate
+      const uint32_t rest2 = rest1 & (rest1 - 1u);   // without its second
+      if (__ballot(rest2 != 0u) != 0ull) {
+        // dense (some lane holds three or more): entry by entry, places from a scan over the lanes
+        const uint32_t mine = static_cast<uint32_t>(__popc(cmask));
+        const uint32_t incl = wave_scan_inclusive_u32(mine);
+        const uint32_t total = readlane_u32(incl, 63);
+        uint32_t base = 0u;
+        if (lane == 0) base = atomicAdd(&sh.list_count, total);
+        base = readlane_u32(base, 0);
+        at = base + incl - mine;
 #pragma unroll
-      for (int k = 0; k < 8; ++k) {
-        if ((cmask >> k) & 1u) {
-          const uint32_t eb = __float_as_uint(e[k]);
-          atomicAdd(&sh.hist[hist_bucket(eb)], 1u);
-          if constexpr (DT == kDtypeBFloat16 || DT == kDtypeHalf) {
-            // 16-bit rows: the same candidates per bit pattern (one outside the range of bins is
-            // missed there, which the totals give away)
-            const int bin = pattern_key(value_pattern<DT>(logit[k]), km.mag_min) - km.key_cut;
-            if (bin >= 0 && bin < km.n_bins) atomicAdd(&ph[bin >> 1], 1u << ((bin & 1) << 4));
+        for (int k = 0; k < 8; ++k) {
+          if ((cmask >> k) & 1u) note(e[k], logit[k], k);
+        }
+      } else {
+        // sparse (the usual row: a few candidates in a slot, at most two in a lane): two rounds,
+        // every lane taking its next candidate; places from the two ballots, no scan
+        const uint64_t has2 = __ballot(rest1 != 0u);
+        const uint32_t n1 = static_cast<uint32_t>(__popcll(has1)), n2 = static_cast<uint32_t>(__popcll(has2));
+        uint32_t base = 0u;
+        if (lane == 0) base = atomicAdd(&sh.list_count, n1 + n2);
+        base = readlane_u32(base, 0);
+        const uint64_t below = (1ull << lane) - 1ull;
+        auto one = [&](uint32_t mask) {
+          const int k = __ffs(static_cast<int>(mask)) - 1;
+          float ek = e[0], lk = logit[0];
+#pragma unroll
+          for (int j = 1; j < 8; ++j) {
+            ek = k == j ? e[j] : ek;
+            lk = k == j ? logit[j] : lk;
           }
-          if (at < static_cast<uint32_t>(p.list_region)) region[at] = (static_cast<uint64_t>(eb) << 32) | static_cast<uint32_t>(first + k);
-          ++at;
+          note(ek, lk, k);
+        };
+        if (cmask) {
+          at = base + static_cast<uint32_t>(__popcll(has1 & below));
+          one(cmask);
+        }
+        if (has2 != 0ull && rest1) {
+          at = base + n1 + static_cast<uint32_t>(__popcll(has2 & below));
+          one(rest1);
         }
       }
     }
