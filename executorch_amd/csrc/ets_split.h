@@ -252,9 +252,11 @@ __device__ __forceinline__ void split_fold_slot(const SplitParams& p, int row, i
   // ---- candidates of the top-p draw (sampler.cpp:137-143), by a cut that is safely below the
   //      reference's once the exact normaliser is known
   if (TOPP) {
+    // bit k: entry k is a candidate (two instructions per entry: compare, shift the outcome in)
     uint32_t cmask = 0u;
 #pragma unroll
-    for (int k = 0; k < 8; ++k) cmask |= e[k] >= cut_lo ? (1u << k) : 0u;
+    for (int k = 7; k >= 0; --k)
+      asm("v_cmp_le_f32 vcc, %2, %1\n\tv_addc_co_u32 %0, vcc, %0, %0, vcc" : "+v"(cmask) : "v"(e[k]), "s"(cut_lo) : "vcc");
     if (s == p.ns - 1) {  // entries past the row's end
       const int left = V - (s * kSlot + lane * 8);
       cmask &= left >= 8 ? 0xffu : (left > 0 ? (1u << left) - 1u : 0u);
@@ -332,10 +334,8 @@ __device__ __forceinline__ void split_fold_slot(const SplitParams& p, int row, i
     return;
   }
   // ---- every entry 0: no effect on any running sum
-  bool nonzero = false;
-#pragma unroll
-  for (int k = 0; k < 8; ++k) nonzero = nonzero || e[k] != 0.0f;
-  if (__ballot(nonzero) == 0ull) {
+  const uint32_t any_bits = bits[0] | bits[1] | bits[2] | bits[3] | bits[4] | bits[5] | bits[6] | bits[7];  // (no -0 among exps)
+  if (__ballot(any_bits != 0u) == 0ull) {
     if (lane == 0) p.slot_rec[rec_at] = {kSlotZero << 8, 0u, 0u, 0xffffffffu};
     return;
   }
