@@ -932,6 +932,25 @@ struct RunBins {
       count = (prob >= cutoff) ? c : 0u;  // sampler.cpp:137-143
     }
   }
+  // The same with the probability from the hardware's exp2 (relative error below 1e-5): enough to
+  // place the cumulative masses; the count is exact (a bin whose probability is within 1e-3 of
+  // the cutoff is evaluated exactly).
+  __device__ __forceinline__ void at_approx(int q, float& prob, uint32_t& count) const {
+    prob = 0.0f;
+    count = 0u;
+    if (q < n_bins) {
+      const int bin = n_bins - 1 - q;
+      const uint32_t c = (cnt[bin >> 1] >> ((bin & 1) << 4)) & 0xffffu;
+      if (c != 0u) {
+        const float l = pattern_value<DT>(key_pattern(key_cut + bin, mag_min));
+        const float x = __builtin_fmaxf(l * inv - m, -104.0f);
+        prob = fast_exp2(x * kLog2e) * static_cast<float>(div.recip);
+        bool in = prob >= cutoff;
+        if (__builtin_fabsf(prob - cutoff) <= cutoff * 1e-3f) in = div_row(expf_core(x, tab), div) >= cutoff;
+        count = in ? c : 0u;
+      }
+    }
+  }
 };
 
 // One wave works the 64 bins of group t out exactly from running sum s; `before` is the number of
@@ -1024,7 +1043,9 @@ __device__ __noinline__ bool draw_topp_runs(RunArgs a, const char* logits, int V
   float* sbound = reinterpret_cast<float*>(recs + n_groups);
   uint32_t* cbound = reinterpret_cast<uint32_t*>(sbound + n_groups + 1);
   float* mbound = reinterpret_cast<float*>(cbound + n_groups + 1);
-  if (reinterpret_cast<char*>(mbound + n_groups + 1) > reinterpret_cast<char*>(lds) + static_cast<size_t>(a.lds_keys) * 8)
+  float* gfirst = mbound + n_groups + 1;  // probability of a group's first and last candidate bin (-1: none)
+  float* glast = gfirst + n_groups;
+  if (reinterpret_cast<char*>(glast + n_groups) > reinterpret_cast<char*>(lds) + static_cast<size_t>(a.lds_keys) * 8)
     return false;
   // ---- the workgroups' counters, added up (16-bit halves add without carries unless one overflows,
   //      which the totals give away)
@@ -1058,19 +1079,11 @@ __device__ __noinline__ bool draw_topp_runs(RunArgs a, const char* logits, int V
     if (total != a.expected) return false;
   }
   const RunBins<DT> bins = {cnt, a.key_cut, n_bins, a.mag_min, inv, a.m, cutoff, row_divisor(S), sm.exp2tab};
-  // ---- pass A: per group the candidates and their approximate mass; probabilities must not rise
-  //      along the sorted positions
-  bool rising = false;
+  // ---- pass A: per group the candidates (exactly) and their approximate mass
   for (int t = wave; t < n_groups; t += kWaves) {
     float prob;
     uint32_t count;
-    bins.at(64 * t + lane, prob, count);
-    float next_prob = 0.0f;  // of the position behind this lane's
-    uint32_t next_count;
-    if (lane == 63) bins.at(64 * t + 64, next_prob, next_count);
-    const float from_right = __shfl_down(prob, 1);
-    if (lane != 63) next_prob = from_right;
-    if (64 * t + lane + 1 < n_bins && next_prob > prob) rising = true;
+    bins.at_approx(64 * t + lane, prob, count);
     const float mass = wave_sum_f32(static_cast<float>(count) * prob);
     const uint32_t c = wave_sum_u32(count);
     if (lane == 0) {
@@ -1078,13 +1091,7 @@ __device__ __noinline__ bool draw_topp_runs(RunArgs a, const char* logits, int V
       cbound[t + 1] = c;
     }
   }
-  {
-    const uint64_t any = __ballot(rising);
-    if (lane == 0) sm.red_u[wave] = any ? 1u : 0u;
-  }
   __syncthreads();
-  uint32_t bad = 0u;
-  for (int w = 0; w < kWaves; ++w) bad |= sm.red_u[w];
   // prefix sums over the groups (at most kBlock of them)
   {
     const float mine = tid < n_groups ? mbound[tid + 1] : 0.0f;
@@ -1113,48 +1120,100 @@ __device__ __noinline__ bool draw_topp_runs(RunArgs a, const char* logits, int V
     }
     __syncthreads();
   }
-  if (bad != 0u || n_groups > kBlock) return false;
+  if (n_groups > kBlock) return false;
   const uint32_t n0 = cbound[n_groups];
   dbg.n_candidates = static_cast<int>(n0);
   if (n0 == 0u) {
     token = -1;  // the reference reads probindex[-1] here
     return true;
   }
-  // ---- pass B: fold every group once, under the ulp(s) of the binade(s) the cumulative sum can be
-  //      in while it passes the group.  A group that may hold the place where the sum exceeds topp,
-  //      that spans more than two binades or in which an entry ties is left to the ordered walk.
+  // ---- pass B: the exact probabilities, group by group, as far as the walk can get (cumulative mass
+  //      up to topp).  They must not rise along the sorted positions (a larger logit with a smaller
+  //      probability would not be where the reference's sort puts it).  Every group is folded once,
+  //      under the ulp(s) of the binade(s) the cumulative sum can be in while it passes the group;
+  //      one that may hold the place where the sum exceeds topp, that spans more than two binades
+  //      or in which an entry ties is left to the ordered walk.
+  bool rising = false;
   for (int t = wave; t < n_groups; t += kWaves) {
     const uint32_t c_in = cbound[t], c_out = cbound[t + 1];
     RunSlotRec rec = {kSlotZero << 8, 0u, 0u, 0u};
+    float first_p = -1.0f, last_p = -1.0f;
     if (c_out != c_in) {
-      const float eps_in = static_cast<float>(c_in) * (1.02f / 16777216.0f) + 3e-5f;
-      const float eps_out = static_cast<float>(c_out) * (1.02f / 16777216.0f) + 3e-5f;
+      const float eps_in = static_cast<float>(c_in) * (1.02f / 16777216.0f) + 6e-5f;
+      const float eps_out = static_cast<float>(c_out) * (1.02f / 16777216.0f) + 6e-5f;
       const float lo = mbound[t] * (1.0f - eps_in), hi = mbound[t + 1] * (1.0f + eps_out);
       const uint32_t kb_lo = __float_as_uint(lo > 0.0f ? lo : 0.0f) >> 23, kb_hi = __float_as_uint(hi) >> 23;
       const bool near_topp = !(hi < topp * 0.9999f);  // (the walk ends there: nothing behind it is needed)
       rec.meta = (kSlotSerial << 8) | (kb_lo & 255u);
-      if (!near_topp && lo > 0.0f && kb_lo >= 70u && kb_hi <= 250u && kb_hi <= kb_lo + 1u) {
+      if (!(lo > topp * 1.001f)) {  // (a group the walk cannot reach stays "serial": worked out exactly if reached after all)
         float prob;
         uint32_t count;
         bins.at(64 * t + lane, prob, count);
-        const float scale_a = __uint_as_float((277u - kb_lo) << 23), scale_b = __uint_as_float((276u - kb_lo) << 23);
-        const float ta = prob * scale_a, tb = prob * scale_b;
-        const float ra = __builtin_rintf(ta), rb = __builtin_rintf(tb);
-        const bool tie = count != 0u && (__builtin_fabsf(ta - ra) == 0.5f || (kb_hi != kb_lo && __builtin_fabsf(tb - rb) == 0.5f));
-        const float fc = static_cast<float>(count);
-        const uint32_t ia = static_cast<uint32_t>(__builtin_fminf(ra * fc, 33554432.0f));
-        const uint32_t ib = static_cast<uint32_t>(__builtin_fminf(rb * fc, 33554432.0f));
-        const uint32_t inc_a = wave_sum_u32(ia), inc_b = wave_sum_u32(ib);
-        if (__ballot(tie) == 0ull) {
-          rec.meta = ((kb_hi == kb_lo ? kSlotStable : kSlotDual) << 8) | kb_lo;
-          rec.inc_a = inc_a < kSat ? inc_a : kSat;
-          rec.inc_b = inc_b < kSat ? inc_b : kSat;
+        // among the group's candidate bins: each against the next one
+        const uint64_t occ = __ballot(count != 0u);
+        const uint64_t above = lane == 63 ? 0ull : occ >> (lane + 1);
+        const int next = above ? lane + __ffsll(static_cast<long long>(above)) : lane;
+        const float next_prob = __shfl(prob, next);
+        if (count != 0u && above != 0ull && next_prob > prob) rising = true;
+        if (occ != 0ull) {
+          first_p = readlane_f32(prob, __ffsll(static_cast<long long>(occ)) - 1);
+          last_p = readlane_f32(prob, 63 - __clzll(static_cast<long long>(occ)));
+        }
+        if (!near_topp && lo > 0.0f && kb_lo >= 70u && kb_hi <= 250u && kb_hi <= kb_lo + 1u) {
+          const float scale_a = __uint_as_float((277u - kb_lo) << 23), scale_b = __uint_as_float((276u - kb_lo) << 23);
+          const float ta = prob * scale_a, tb = prob * scale_b;
+          const float ra = __builtin_rintf(ta), rb = __builtin_rintf(tb);
+          const bool tie = count != 0u && (__builtin_fabsf(ta - ra) == 0.5f || (kb_hi != kb_lo && __builtin_fabsf(tb - rb) == 0.5f));
+          const float fc = static_cast<float>(count);
+          const uint32_t ia = static_cast<uint32_t>(__builtin_fminf(ra * fc, 33554432.0f));
+          const uint32_t ib = static_cast<uint32_t>(__builtin_fminf(rb * fc, 33554432.0f));
+          const uint32_t inc_a = wave_sum_u32(ia), inc_b = wave_sum_u32(ib);
+          if (__ballot(tie) == 0ull) {
+            rec.meta = ((kb_hi == kb_lo ? kSlotStable : kSlotDual) << 8) | kb_lo;
+            rec.inc_a = inc_a < kSat ? inc_a : kSat;
+            rec.inc_b = inc_b < kSat ? inc_b : kSat;
+          }
         }
       }
     }
-    if (lane == 0) recs[t] = rec;
+    if (lane == 0) {
+      recs[t] = rec;
+      gfirst[t] = first_p;
+      glast[t] = last_p;
+    }
+  }
+  {
+    const uint64_t any = __ballot(rising);
+    if (lane == 0) sm.red_u[wave] = any ? 1u : 0u;
   }
   __syncthreads();
+  {
+    uint32_t bad = 0u;
+    for (int w = 0; w < kWaves; ++w) bad |= sm.red_u[w];
+    // ... and from group to group: a group's first candidate against the last one in front of it
+    if (wave == 0) {
+      float prev_last = __uint_as_float(0x7f800000u);
+      bool up = false;
+      for (int base = 0; base < n_groups; base += 64) {
+        const int g = base + lane;
+        const float f = g < n_groups ? gfirst[g] : -1.0f;
+        const float l = g < n_groups ? glast[g] : -1.0f;
+        const uint64_t occ = __ballot(f >= 0.0f);
+        const uint64_t below = occ & ((1ull << lane) - 1ull);
+        const int prev = below ? 63 - __clzll(static_cast<long long>(below)) : lane;
+        float before = __shfl(l, prev);
+        if (!below) before = prev_last;
+        if (f >= 0.0f && f > before) up = true;
+        if (occ) prev_last = readlane_f32(l, 63 - __clzll(static_cast<long long>(occ)));
+      }
+      const uint64_t any = __ballot(up);
+      if (lane == 0) sm.flag = any ? 1 : 0;
+    }
+    __syncthreads();
+    bad |= static_cast<uint32_t>(sm.flag);
+    __syncthreads();
+    if (bad != 0u) return false;
+  }
   // ---- walk 1 (sampler.cpp:150-158): the groups in order until the sum exceeds topp.  One wave.
   if (wave == 0) {
     float s = 0.0f;
