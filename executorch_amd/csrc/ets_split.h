@@ -673,6 +673,45 @@ __device__ __forceinline__ void resolve_lanes(float& s, const uint32_t (&bits)[8
                                               uint32_t* inner = nullptr) {
   const int lane = threadIdx.x & 63;
   int cur = 0;
+  // ---- the usual slot, in one go: the sum enters in binade a, no tie in front of the lane in which
+  //      it leaves a, that lane's native adds land in binade b, nothing ties behind it and the rest
+  //      stays inside b.  Anything else: the general rounds below, from the lane reached.
+  {
+    s = uniform_f32(s);
+    const SumState ss = sum_state(s);
+    if (static_cast<uint32_t>(ss.kb) == kb_a) {
+      const uint32_t room = (1u << 24) - ss.S;
+      const uint64_t over = __ballot(pre_a >= room);  // (prefix sums rise: the lanes from the crossing one on)
+      if (over == 0ull) {
+        if (tie_a == 0ull) {
+          s = sum_value(ss.S + readlane_u32(pre_a, 63), ss.kb);
+          return;
+        }
+      } else {
+        const int j = __ffsll(static_cast<long long>(over)) - 1;
+        if ((tie_a & ((1ull << j) - 1ull)) == 0ull) {
+          const uint32_t S_j = ss.S + (j > 0 ? readlane_u32(pre_a, j - 1) : 0u);
+          float sj = 0.0f;
+          if (lane == j) {
+            sj = sum_value(S_j, ss.kb);
+#pragma unroll
+            for (int k = 0; k < 8; ++k) sj = sj + __uint_as_float(bits[k]);  // (entries past the row hold 0)
+          }
+          s = readlane_f32(sj, j);
+          cur = j + 1;
+          if (cur == 64) return;
+          const SumState s2 = sum_state(s);
+          if (static_cast<uint32_t>(s2.kb) == kb_b && (tie_b >> cur) == 0ull) {
+            const uint32_t rest = readlane_u32(pre_b, 63) - readlane_u32(pre_b, j);
+            if (s2.S + rest < (1u << 24)) {
+              s = sum_value(s2.S + rest, s2.kb);
+              return;
+            }
+          }
+        }
+      }
+    }
+  }
   while (cur < 64) {
     if (inner) ++*inner;
     s = uniform_f32(s);
