@@ -411,8 +411,9 @@ ets_status launch_split(ets_sampler* s, const ets::RowParams& p, int32_t rows, h
   sp.phist_words = DT == ets::kDtypeBFloat16 ? kPhistWordsBFloat16 : (DT == ets::kDtypeHalf ? kPhistWordsHalf : 0);
   sp.row_wgs = pass2_workgroups(s, rows, sp.ns);
   sp.list_region = list_region(sp.ns, sp.row_wgs);
-  // passes 1 and 2 share their grid: a workgroup of pass 2 finds its entries in the L2 of its die
-  hipLaunchKernelGGL((ets::split_pass1_kernel<DT>), dim3(sp.row_wgs, rows), dim3(ets::kBlock), 0, stream, sp);
+  const int per_block = (ets::kPass1Block / 64) * ets::kPass1SlotsPerWave;
+  hipLaunchKernelGGL((ets::split_pass1_kernel<DT>), dim3((sp.ns + per_block - 1) / per_block, rows), dim3(ets::kPass1Block), 0,
+                     stream, sp);
   ETS_HIP(s, hipGetLastError());
   const size_t lut_bytes = (DT == ets::kDtypeBFloat16 ? sizeof(float) * ets::kLutCountWords : 0) + sizeof(uint32_t) * sp.phist_words;
   static std::atomic<size_t> set_bytes2[kMaxDevices];

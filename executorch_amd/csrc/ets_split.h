@@ -181,9 +181,11 @@ __device__ __forceinline__ void split_range(int ns, int wgs, int x, int& s_begin
   s_end = min(ns, s_begin + per_wg);
 }
 
-// grid = (workgroups per row, rows), kBlock lanes: every wave takes whole slots, four at a time.
+// grid = (ceil(ns / 16), rows), 256 lanes: every wave takes four slots, all loads issued first.
+// (Small workgroups: many are resident per CU, which is what a kernel bound by HBM wants.)
+constexpr int kPass1Block = 256;
 template <int DT>
-__global__ void __launch_bounds__(kBlock) split_pass1_kernel(SplitParams p) {
+__global__ void __launch_bounds__(kPass1Block) split_pass1_kernel(SplitParams p) {
   const int row = p.row.row_map ? p.row.row_map[blockIdx.y] : blockIdx.y;
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -192,35 +194,52 @@ __global__ void __launch_bounds__(kBlock) split_pass1_kernel(SplitParams p) {
   const char* logits = static_cast<const char*>(p.row.logits) + static_cast<int64_t>(row) * p.row.row_stride * ElemSize<DT>::value;
   const float kInf = __uint_as_float(0x7f800000u);
   const float fill = inv < 0.0f ? kInf : -kInf;  // x = -inf: adds nothing
-  int s_begin, s_end;
-  split_range(p.ns, gridDim.x, blockIdx.x, s_begin, s_end);
-  for (int slot0 = s_begin + wave * kPass1SlotsPerWave; slot0 < s_end; slot0 += kWaves * kPass1SlotsPerWave) {
+  const int s_end = p.ns;
+  for (int slot0 = (blockIdx.x * (kPass1Block / 64) + wave) * kPass1SlotsPerWave; slot0 < s_end; slot0 = s_end) {
     float v[kPass1SlotsPerWave][8];
 #pragma unroll
     for (int k = 0; k < kPass1SlotsPerWave; ++k) {
       if (slot0 + k < s_end) load_slot_lane<DT>(logits, slot0 + k, lane, V, fill, v[k], p.row.fused);
     }
+    // Few instructions per entry (with a workgroup per row the kernel would otherwise be bound by
+    // them, not by HBM): the maximum is taken over the raw logits -- rounding is monotone, so the
+    // largest product l * inv is the product of the largest (smallest, for a negative inv) logit --
+    // and the exponent comes from one fused multiply-add per entry.
+    // (An infinite inv can turn a finite logit into a NaN product: then the products themselves
+    // are reduced, with a factor of 1.)
+    float inv_u = inv;
+    if (!(__builtin_fabsf(inv) < kInf)) {
+#pragma unroll
+      for (int k = 0; k < kPass1SlotsPerWave; ++k) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[k][e] = v[k][e] * inv;
+      }
+      inv_u = 1.0f;
+    }
+    const float c1 = inv_u * kLog2e;
 #pragma unroll
     for (int k = 0; k < kPass1SlotsPerWave; ++k) {
       const int s = slot0 + k;
       if (s >= s_end) break;
-      float lmax = -kInf;
+      float ext = inv_u < 0.0f ? kInf : -kInf;
       bool nan = false;
+      if (inv_u < 0.0f) {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        v[k][e] = v[k][e] * inv;
-        lmax = __builtin_fmaxf(lmax, v[k][e]);  // ignores NaN
-        nan = nan || (v[k][e] != v[k][e]);
+        for (int e = 0; e < 8; ++e) ext = __builtin_fminf(ext, v[k][e]);  // ignores NaN
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) ext = __builtin_fmaxf(ext, v[k][e]);
       }
-      const float M = wave_max_ignoring_nan(lmax);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) nan = nan || (v[k][e] != v[k][e]);
+      // (a lane whose entries all lie past the row's end holds the fill value, whose product is -inf)
+      const float M = wave_max_ignoring_nan(ext * inv_u);
       const bool any_nan = __ballot(nan) != 0ull;
       float sum = 0.0f;
       if (M > -kInf) {
+        const float c2 = -M * kLog2e;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const float t = fast_exp2((v[k][e] - M) * kLog2e);
-          sum += (v[k][e] == v[k][e]) ? t : 0.0f;
-        }
+        for (int e = 0; e < 8; ++e) sum += fast_exp2(__builtin_fmaf(v[k][e], c1, c2));  // (a NaN here: the row is one)
       }
       sum = wave_sum_f32(sum);
       if (lane == 0) {
