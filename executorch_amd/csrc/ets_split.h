@@ -322,11 +322,18 @@ __device__ __forceinline__ void split_fold_slot(const SplitParams& p, int row, i
         const uint64_t below = (1ull << lane) - 1ull;
         auto one = [&](uint32_t mask) {
           const int k = __ffs(static_cast<int>(mask)) - 1;
-          float ek = e[0], lk = logit[0];
-#pragma unroll
-          for (int j = 1; j < 8; ++j) {
-            ek = k == j ? e[j] : ek;
-            lk = k == j ? logit[j] : lk;
+          // entry k of the lane's eight, by three levels of selects (kept in registers: indexing the
+          // arrays with k would move them to private memory)
+          const bool b0 = (k & 1) != 0, b1 = (k & 2) != 0, b2 = (k & 4) != 0;
+          const float e01 = b0 ? e[1] : e[0], e23 = b0 ? e[3] : e[2], e45 = b0 ? e[5] : e[4], e67 = b0 ? e[7] : e[6];
+          const float e03 = b1 ? e23 : e01, e47 = b1 ? e67 : e45;
+          const float ek = b2 ? e47 : e03;
+          float lk = 0.0f;
+          if constexpr (DT == kDtypeBFloat16 || DT == kDtypeHalf) {
+            const float l01 = b0 ? logit[1] : logit[0], l23 = b0 ? logit[3] : logit[2], l45 = b0 ? logit[5] : logit[4],
+                        l67 = b0 ? logit[7] : logit[6];
+            const float l03 = b1 ? l23 : l01, l47 = b1 ? l67 : l45;
+            lk = b2 ? l47 : l03;
           }
           note(ek, lk, k);
         };
