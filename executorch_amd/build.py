@@ -5,7 +5,9 @@ hipcc cross-compiles, so no GPU is needed to build.
 """
 from __future__ import annotations
 
+import json
 import os
+import re
 import shutil
 import subprocess
 import sys
@@ -36,12 +38,52 @@ def hipcc() -> str:
     return exe
 
 
+RESOURCES = os.path.join(HERE, "kernel_resources.json")
+
+# hipcc's host pass does not know the device feature that the packed-fp32 switch names and says so
+# once per pass; the device pass honours it (tests/test_build_hygiene.py looks for the packed
+# instructions in the library's device code).
+_HOST_PASS_NOISE = "is not a recognized feature for this target"
+
+
 def build_library(verbose: bool = True, extra_flags: list[str] | None = None, out: str = LIB) -> str:
-    cmd = [hipcc(), *HIPCC_FLAGS, *(extra_flags or []), os.path.join(CSRC, "et_sampler.hip"), "-o", out]
+    """One hipcc command.  Also records what every kernel needs (registers, private memory, LDS) in
+    kernel_resources.json next to the library: private memory in a hot kernel is a regression that
+    no test of results would notice."""
+    cmd = [hipcc(), *HIPCC_FLAGS, "-Rpass-analysis=kernel-resource-usage", *(extra_flags or []),
+           os.path.join(CSRC, "et_sampler.hip"), "-o", out]
     if verbose:
         print(" ".join(cmd), flush=True)
-    subprocess.check_call(cmd)
-    return LIB
+    proc = subprocess.run(cmd, stderr=subprocess.PIPE, text=True)
+    kernels: dict[str, dict[str, int]] = {}
+    name = None
+    quoted = 0
+    for line in proc.stderr.splitlines():
+        m = re.search(r"remark: +Function Name: (\S+)", line)
+        if m:
+            name = m.group(1)
+            kernels[name] = {}
+            continue
+        m = re.search(r"remark: +(VGPRs|AGPRs|TotalSGPRs|ScratchSize \[bytes/lane\]|LDS Size \[bytes/block\]|"
+                      r"Occupancy \[waves/SIMD\]|SGPRs Spill|VGPRs Spill): (\d+)", line)
+        if m and name:
+            kernels[name][m.group(1).split(" [")[0]] = int(m.group(2))
+            continue
+        if "-Rpass-analysis" in line or _HOST_PASS_NOISE in line or not line.strip():
+            quoted = 2  # (a remark is followed by the source line it points at and a caret line)
+            continue
+        if quoted > 0 and re.match(r"\s*(\d+\s*)?\|", line):
+            quoted -= 1
+            continue
+        quoted = 0
+        print(line, file=sys.stderr)
+    if proc.returncode != 0:
+        raise subprocess.CalledProcessError(proc.returncode, cmd)
+    if out == LIB:
+        with open(RESOURCES, "w") as f:
+            json.dump(kernels, f, indent=1, sort_keys=True)
+            f.write("\n")
+    return out
 
 
 if __name__ == "__main__":
