@@ -57,26 +57,33 @@ def build_library(verbose: bool = True, extra_flags: list[str] | None = None, ou
     proc = subprocess.run(cmd, stderr=subprocess.PIPE, text=True)
     kernels: dict[str, dict[str, int]] = {}
     name = None
-    quoted = 0
+    keep, pending = True, []
     for line in proc.stderr.splitlines():
         m = re.search(r"remark: +Function Name: (\S+)", line)
         if m:
             name = m.group(1)
             kernels[name] = {}
+            keep, pending = False, []
             continue
         m = re.search(r"remark: +(VGPRs|AGPRs|TotalSGPRs|ScratchSize \[bytes/lane\]|LDS Size \[bytes/block\]|"
                       r"Occupancy \[waves/SIMD\]|SGPRs Spill|VGPRs Spill): (\d+)", line)
         if m and name:
             kernels[name][m.group(1).split(" [")[0]] = int(m.group(2))
+            keep, pending = False, []
             continue
-        if "-Rpass-analysis" in line or _HOST_PASS_NOISE in line or not line.strip():
-            quoted = 2  # (a remark is followed by the source line it points at and a caret line)
+        # the rest goes to stderr diagnostic by diagnostic: a remark's or the host pass's own lines
+        # (header, include chain, quoted source line, caret) are dropped, warnings and errors kept
+        if re.search(r": (remark|warning|error|note|fatal error):", line):
+            keep = not ("remark:" in line or _HOST_PASS_NOISE in line)
+            if keep:
+                for held in pending:
+                    print(held, file=sys.stderr)
+            pending = []
+        elif line.startswith("In file included from") or line.startswith("                 from"):
+            pending.append(line)
             continue
-        if quoted > 0 and re.match(r"\s*(\d+\s*)?\|", line):
-            quoted -= 1
-            continue
-        quoted = 0
-        print(line, file=sys.stderr)
+        if keep:
+            print(line, file=sys.stderr)
     if proc.returncode != 0:
         raise subprocess.CalledProcessError(proc.returncode, cmd)
     if out == LIB:
