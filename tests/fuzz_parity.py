@@ -51,14 +51,9 @@ def make_rows(rng, kind, rows, vocab):
     return np.ascontiguousarray(x)
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--cases", type=int, default=2000)
-    ap.add_argument("--seed", type=int, default=1)
-    ap.add_argument("--max-vocab", type=int, default=300000)
-    ap.add_argument("--configs", action="store_true",
-                    help="give every row its own (temperature, top-p, top-k, seed) through sample_batch_configs")
-    args = ap.parse_args()
+def run(cases=2000, seed=1, max_vocab=300000, configs=False):
+    """The cases; returns {"cases", "failures", "first_failures", "seconds"}."""
+    args = argparse.Namespace(cases=cases, seed=seed, max_vocab=max_vocab, configs=configs)
 
     import torch
 
@@ -156,8 +151,20 @@ def main():
                 break
         if case % 100 == 99:
             print(f"fuzz_parity: {case + 1} cases, {len(failures)} failures, {time.time() - t0:.0f} s", file=sys.stderr, flush=True)
-    print(json.dumps({"cases": case + 1, "failures": len(failures), "first_failures": failures[:3], "seconds": round(time.time() - t0, 1)}))
-    sys.exit(1 if failures else 0)
+    return {"cases": case + 1, "failures": len(failures), "first_failures": failures[:3], "seconds": round(time.time() - t0, 1)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--cases", type=int, default=2000)
+    ap.add_argument("--seed", type=int, default=1)
+    ap.add_argument("--max-vocab", type=int, default=300000)
+    ap.add_argument("--configs", action="store_true",
+                    help="give every row its own (temperature, top-p, top-k, seed) through sample_batch_configs")
+    args = ap.parse_args()
+    res = run(args.cases, args.seed, args.max_vocab, args.configs)
+    print(json.dumps(res))
+    sys.exit(1 if res["failures"] else 0)
 
 
 if __name__ == "__main__":

@@ -54,14 +54,9 @@ def device_rows(w, rows, gen, torch, dev):
     return x.to(tdt).contiguous()
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--workload", default="cfg2")
-    ap.add_argument("--rows", type=int, default=100000)
-    ap.add_argument("--chunk", type=int, default=1024)
-    ap.add_argument("--threads", type=int, default=16)
-    ap.add_argument("--seed", type=int, default=20240607)
-    args = ap.parse_args()
+def run(workload="cfg2", rows=100000, chunk=1024, threads=16, seed=20240607):
+    """The comparison; returns the report as a dict."""
+    args = argparse.Namespace(workload=workload, rows=rows, chunk=chunk, threads=threads, seed=seed)
 
     import torch
 
@@ -112,7 +107,7 @@ def main():
         done += n
         print(f"parity_report: {done} rows, {mismatches} mismatches, {time.time() - t0:.0f} s", file=sys.stderr, flush=True)
 
-    print(json.dumps({
+    return {
         "workload": f"{w.name}: vocab {w.vocab}, {W.DTYPE_NAMES[w.dtype]} ({w.kind}), temperature {w.temperature}, top-p {w.topp}",
         "rows": done,
         "token_mismatches_vs_oracle_fp32_index_ties": mismatches,
@@ -121,8 +116,22 @@ def main():
         "of_which_not_between_equal_probabilities": tie_not_equal,
         "rows_equal_to_native_16bit_reference_arithmetic": native_agree,
         "seconds": round(time.time() - t0, 1),
-    }))
-    sys.exit(0 if mismatches == 0 and sum_mismatches == 0 and tie_not_equal == 0 else 1)
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--workload", default="cfg2")
+    ap.add_argument("--rows", type=int, default=100000)
+    ap.add_argument("--chunk", type=int, default=1024)
+    ap.add_argument("--threads", type=int, default=16)
+    ap.add_argument("--seed", type=int, default=20240607)
+    args = ap.parse_args()
+    res = run(args.workload, args.rows, args.chunk, args.threads, args.seed)
+    print(json.dumps(res))
+    ok = res["token_mismatches_vs_oracle_fp32_index_ties"] == 0 and res["normaliser_bit_mismatches_vs_oracle"] == 0 and \
+        res["of_which_not_between_equal_probabilities"] == 0
+    sys.exit(0 if ok else 1)
 
 
 if __name__ == "__main__":

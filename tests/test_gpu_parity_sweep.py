@@ -1,0 +1,34 @@
+"""Parity at a scale the fixed cases do not reach, as part of the GPU suite: the randomised cases of
+fuzz_parity.py in the three settings of the row split (automatic, forced, off) and with per-row
+parameters, and a few thousand rows of the headline workload's distribution against the oracle
+(tokens, the softmax normaliser bit for bit, the reference's own tie order).  The same code runs
+longer from the command line: `python tests/fuzz_parity.py --cases N`, `python tests/parity_report.py`."""
+import pytest
+
+import fuzz_parity
+import parity_report
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("split,seed", [("0", 101), ("1", 102), ("2", 103)])
+def test_randomised_cases(monkeypatch, split, seed):
+    monkeypatch.setenv("ETS_ROW_SPLIT", split)  # the default of new handles: 0 automatic, 1 on, 2 off
+    res = fuzz_parity.run(cases=500, seed=seed)
+    assert res["failures"] == 0, res["first_failures"]
+    assert res["cases"] == 500
+
+
+def test_randomised_cases_with_per_row_parameters(monkeypatch):
+    monkeypatch.setenv("ETS_ROW_SPLIT", "1")
+    res = fuzz_parity.run(cases=300, seed=104, configs=True)
+    assert res["failures"] == 0, res["first_failures"]
+
+
+@pytest.mark.parametrize("workload,rows", [("cfg2", 4096), ("cfg1", 1024)])
+def test_rows_of_a_workload_at_scale(workload, rows):
+    res = parity_report.run(workload=workload, rows=rows, chunk=1024, threads=8, seed=7)
+    assert res["rows"] == rows
+    assert res["token_mismatches_vs_oracle_fp32_index_ties"] == 0, res
+    assert res["normaliser_bit_mismatches_vs_oracle"] == 0, res
+    assert res["of_which_not_between_equal_probabilities"] == 0, res
