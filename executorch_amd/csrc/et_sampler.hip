@@ -348,6 +348,7 @@ ets_status ensure_split(ets_sampler* s) {
     return here;
   };
   const size_t o_max = take(rows * sp.ns_stride * sizeof(float));
+  const size_t o_max2 = take(rows * sp.ns_stride * sizeof(float));
   const size_t o_sum = take(rows * sp.ns_stride * sizeof(float));
   const size_t o_rec = take(rows * sp.ns_stride * sizeof(ets::SlotRec));
   const size_t o_prep = take(rows * sp.prep_cap * sizeof(ets::PrepSlot));
@@ -359,6 +360,7 @@ ets_status ensure_split(ets_sampler* s) {
   ETS_HIP(s, hipMalloc(&s->d_split, at));
   char* base = static_cast<char*>(s->d_split);
   sp.slot_max = reinterpret_cast<float*>(base + o_max);
+  sp.slot_max2 = reinterpret_cast<float*>(base + o_max2);
   sp.slot_sum = reinterpret_cast<float*>(base + o_sum);
   sp.slot_rec = reinterpret_cast<ets::SlotRec*>(base + o_rec);
   sp.prep = reinterpret_cast<ets::PrepSlot*>(base + o_prep);
@@ -411,6 +413,11 @@ ets_status launch_split(ets_sampler* s, const ets::RowParams& p, int32_t rows, h
   sp.phist_words = DT == ets::kDtypeBFloat16 ? kPhistWordsBFloat16 : (DT == ets::kDtypeHalf ? kPhistWordsHalf : 0);
   sp.row_wgs = pass2_workgroups(s, rows, sp.ns);
   sp.list_region = list_region(sp.ns, sp.row_wgs);
+  static const int short_lists = [] {
+    const char* e = std::getenv("ETS_SHORT_LISTS");  // 0: pass 2 lists every possible candidate, always
+    return e ? std::atoi(e) : 1;
+  }();
+  sp.short_lists = short_lists;
   const int per_block = (ets::kPass1Block / 64) * ets::kPass1SlotsPerWave;
   hipLaunchKernelGGL((ets::split_pass1_kernel<DT>), dim3((sp.ns + per_block - 1) / per_block, rows), dim3(ets::kPass1Block), 0,
                      stream, sp);
@@ -535,6 +542,7 @@ size_t layout_static(const ets_sampler* s, int32_t dtype, int32_t rows, char* ba
   };
   wb->tickets = reinterpret_cast<uint32_t*>(take(16 * sizeof(uint32_t)));  // always the array's first bytes: 0 between launches
   sp.slot_max = reinterpret_cast<float*>(take(r * sp.ns_stride * sizeof(float)));
+  sp.slot_max2 = reinterpret_cast<float*>(take(r * sp.ns_stride * sizeof(float)));
   sp.slot_sum = reinterpret_cast<float*>(take(r * sp.ns_stride * sizeof(float)));
   sp.slot_rec = reinterpret_cast<ets::SlotRec*>(take(r * sp.ns_stride * sizeof(ets::SlotRec)));
   sp.prep = reinterpret_cast<ets::PrepSlot*>(take(r * sp.prep_cap * sizeof(ets::PrepSlot)));

@@ -1052,10 +1052,11 @@ __device__ int draw_small_wave(LdsKeys lds, int n, int n_total, float topp, floa
 //      safely more than topp (any-order float sums with a 0.4 % margin): the nucleus is among them;
 //   C. only those entries are sorted (in LDS) and the reference's two CDF walks run over them.
 // Returns false when the entries to sort do not fit in LDS or, against expectation, do not reach
-// topp (the caller takes the general path).
+// topp (the caller takes the general path).  more_exist: the list is the row's largest entries,
+// not every candidate.
 __device__ bool draw_topp_listed(uint64_t* list, uint64_t* lds_list, int lds_list_cap, int list_base, int n_listed,
                                  float S, float cutoff, float topp, float coin, uint64_t* lds_keys, int cap,
-                                 RowDebug& dbg, int32_t& token, BlockScratch& sm) {
+                                 RowDebug& dbg, int32_t& token, BlockScratch& sm, bool more_exist = false) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   uint32_t buf = 0u;
@@ -1099,9 +1100,13 @@ __device__ bool draw_topp_listed(uint64_t* list, uint64_t* lds_list, int lds_lis
   const int n0 = static_cast<int>(cnt);
   dbg.n_candidates = n0;
   if (n0 == 0) {
+    if (more_exist) return false;
     token = -1;  // the reference reads probindex[-1] here
     return true;
   }
+  // more_exist: the list holds the row's largest entries only (every entry that is not listed is
+  // smaller than every listed one), so the walks below must end inside it
+  const int n_total = more_exist ? 0x7fffffff : n0;
   // ---- B
   const float target = topp * 1.004f + 1e-6f;
   float tau = 0.0f;  // select everything
@@ -1165,9 +1170,9 @@ __device__ bool draw_topp_listed(uint64_t* list, uint64_t* lds_list, int lds_lis
   __syncthreads();
   for (int i = n_sel + tid; i < N; i += kBlock) lds_keys[i] = ~0ull;
   __syncthreads();
-  if (n_sel <= 64) return draw_small_wave((LdsKeys)lds_keys, n_sel, n0, topp, coin, dbg, token, sm) != -2;
+  if (n_sel <= 64) return draw_small_wave((LdsKeys)lds_keys, n_sel, n_total, topp, coin, dbg, token, sm) != -2;
   sort_keys_lds((LdsKeys)lds_keys, N);
-  const int pos = draw_from_sorted((LdsKeys)lds_keys, n_sel, n0, false, 0, topp, coin, dbg, sm);
+  const int pos = draw_from_sorted((LdsKeys)lds_keys, n_sel, n_total, false, 0, topp, coin, dbg, sm);
   if (pos == -2) return false;  // the pre-selection did not reach topp after all
   token = static_cast<int32_t>(static_cast<uint32_t>(lds_keys[pos]));
   return true;

@@ -65,7 +65,8 @@ struct RowState {
   int32_t key_cut;      // 16-bit rows: order key of the first bin of the pattern histogram,
   int32_t n_bins;       //   how many bins it has (0: no pattern histogram)
   int32_t mag_min;      //   and the KeyMap's first magnitude with a key of its own
-  uint32_t pad;
+  uint32_t listed_buckets;  // 0: every possible candidate is listed; else only those of the histogram's
+                            //   first `listed_buckets` buckets (which carry more than topp of the mass)
 };
 
 constexpr int kMaxRowWorkgroups = 64;  // workgroups of pass 2 per row
@@ -122,8 +123,9 @@ __device__ __forceinline__ uint32_t value_pattern(float v) {
 
 struct SplitParams {
   RowParams row;        // what the one-workgroup kernel takes
-  float* slot_max;      // [rows, ns_stride]
-  float* slot_sum;      // [rows, ns_stride]
+  float* slot_max;      // [rows, ns_stride] largest x = logit * inv_temperature of the slot (NaN: the slot holds one)
+  float* slot_max2;     // [rows, ns_stride] largest x among the other 63 lanes' entries
+  float* slot_sum;      // [rows, ns_stride] sum of exp(x - slot_max), approximate
   SlotRec* slot_rec;    // [rows, ns_stride]
   PrepSlot* prep;       // [rows, prep_cap]
   RowState* row_state;  // [rows]
@@ -136,6 +138,7 @@ struct SplitParams {
   int32_t phist_words;  // words per (row, workgroup) region; 0 disables the pattern histogram
   uint64_t* timers;     // phase clocks (profiling), or null
   int32_t list_region;  // entries per region
+  int32_t short_lists;  // 1: pass 2 may list only the largest candidates of a peaked row (see RowState::listed_buckets)
   int32_t row_wgs;      // workgroups of pass 2 per row
   int32_t ns;           // slots per row
   int32_t ns_stride;
@@ -233,8 +236,14 @@ __global__ void __launch_bounds__(kPass1Block) split_pass1_kernel(SplitParams p)
 #pragma unroll
       for (int e = 0; e < 8; ++e) nan = nan || (v[k][e] != v[k][e]);
       // (a lane whose entries all lie past the row's end holds the fill value, whose product is -inf)
-      const float M = wave_max_ignoring_nan(ext * inv_u);
+      const float xm = ext * inv_u;
+      const float M = wave_max_ignoring_nan(xm);
       const bool any_nan = __ballot(nan) != 0ull;
+      // the largest entry of the other lanes (pass 2 bounds the mass of the row's largest entries
+      // from below with the two)
+      const uint64_t holds = __ballot(xm == M);
+      const int holder = holds ? __ffsll(static_cast<long long>(holds)) - 1 : 64;
+      const float M2 = wave_max_ignoring_nan(lane == holder ? -kInf : xm);
       float sum = 0.0f;
       if (M > -kInf) {
         const float c2 = -M * kLog2e;
@@ -245,6 +254,7 @@ __global__ void __launch_bounds__(kPass1Block) split_pass1_kernel(SplitParams p)
       if (lane == 0) {
         const int64_t at = static_cast<int64_t>(row) * p.ns_stride + s;
         p.slot_max[at] = any_nan ? __uint_as_float(0x7fc00000u) : M;
+        p.slot_max2[at] = M2;
         p.slot_sum[at] = sum;
       }
     }
@@ -259,6 +269,7 @@ struct Pass2Shared {
   uint32_t cls[kMaxSlots];    // per slot: kb_lo | kb_hi << 8 | kind << 16 | prepared-slot index << 19
   uint32_t hist[kHistBuckets];
   uint32_t list_count;        // candidates this workgroup has listed
+  uint32_t top_mass[32];      // the slots' two largest exps, added up per binade (bin j: [2^-j, 2^(1-j))), in units of 2^-20
 };
 
 // One wave, one slot: e[] are the lane's 8 entries; `cls` is the slot's entry of Pass2Shared::cls.
@@ -468,12 +479,14 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
   const char* logits = static_cast<const char*>(p.row.logits) + static_cast<int64_t>(row) * p.row.row_stride * ElemSize<DT>::value;
   const float* slot_max = p.slot_max + static_cast<int64_t>(row) * p.ns_stride;
   const float* slot_sum = p.slot_sum + static_cast<int64_t>(row) * p.ns_stride;
+  const float* slot_max2 = p.slot_max2 + static_cast<int64_t>(row) * p.ns_stride;
   const float kInf = __uint_as_float(0x7f800000u);
   const float fill = inv < 0.0f ? kInf : -kInf;
   uint64_t c0 = 0, c1 = 0, c2 = 0, c3 = 0;
   if (p.timers) c0 = wall_clock64();
   if (tid < 32) sm.exp2tab[tid] = kExp2Table[tid];
   if (tid == 0) sh.list_count = 0u;
+  if (TOPP && tid < 32) sh.top_mass[tid] = 0u;
   // 16-bit rows: entries per bit pattern, behind the expf table
   constexpr bool kPatterns = TOPP && (DT == kDtypeBFloat16 || DT == kDtypeHalf);
   uint32_t* ph = reinterpret_cast<uint32_t*>(lut_mem + (DT == kDtypeBFloat16 ? kLutCountWords : 0));
@@ -495,12 +508,13 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
   // ---- row maximum (sampler.cpp:191-197) from the slots' maxima
   float m = -kInf;
   bool any_nan = false;
-  float first_max = 0.0f, first_sum = 0.0f;  // the scan below starts with the same slots
+  float first_max = 0.0f, first_sum = 0.0f, first_max2 = -kInf;  // the scan below starts with the same slots
   for (int s = tid; s < ns; s += kBlock) {
     const float v = slot_max[s];
     if (s == tid) {
       first_max = v;
       first_sum = slot_sum[s];
+      if (TOPP) first_max2 = slot_max2[s];
     }
     any_nan = any_nan || (v != v);
     m = __builtin_fmaxf(m, v);
@@ -540,7 +554,20 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
     if (s < ns) {
       const float sum = base == 0 ? first_sum : slot_sum[s];
       const float smax = base == 0 ? first_max : slot_max[s];
-      a = sum > 0.0f ? sum * fast_exp2((smax - m) * kLog2e) : 0.0f;
+      const float f = sum > 0.0f ? fast_exp2((smax - m) * kLog2e) : 0.0f;  // exp of the slot's largest entry
+      a = sum > 0.0f ? sum * f : 0.0f;
+      if (TOPP && f > 0.0f) {
+        // lower bounds of the exact exps of the slot's two largest entries, into the bins of their
+        // binades (integers: every workgroup of the row arrives at the same totals)
+        const float smax2 = base == 0 ? first_max2 : slot_max2[s];
+        const float f2 = smax2 > -kInf ? fast_exp2((smax2 - m) * kLog2e) : 0.0f;
+        const float below[2] = {f * 0.9999f, f2 * 0.9999f};
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+          const int j = 127 - static_cast<int>(__float_as_uint(below[q]) >> 23);
+          if (below[q] > 0.0f && j >= 0 && j < 32) atomicAdd(&sh.top_mass[j], static_cast<uint32_t>(below[q] * 1048576.0f));
+        }
+      }
     }
     const float incl = wave_scan_inclusive_f32(a, lane);
     if (lane == 63) sm.group_total[0][wave] = incl;
@@ -582,7 +609,6 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
     serial_before += chunk_total;
   }
   const float a_total = carry;
-  if (blockIdx.x == 0 && tid == 0) p.row_state[row] = {serial_before, m, 0u, a_total, 0, 0, 0, 0u};
   if (p.timers) c2 = wall_clock64();
 
   // ---- bf16 rows: expf by bit pattern
@@ -597,6 +623,28 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
 
   const float cutoff = TOPP ? (1.0f - topp) / static_cast<float>(V - 1) : 0.0f;  // sampler.cpp:136
   const float cut_lo = cutoff * a_total * (1.0f - split_eps(V)) * 0.999f;
+  // ---- a peaked row: when the largest entries of the slots alone carry safely more than topp of
+  //      the mass, the nucleus lies among the entries of their binades, and only those are listed
+  //      (whole buckets of the histogram, so that the finish kernel knows what the lists hold).  The
+  //      count of all candidates is lost then, which only the debug record reports: a launch that
+  //      asks for debug records lists everything.
+  float list_cut = cut_lo;
+  uint32_t listed_buckets = 0u;
+  if (TOPP && p.short_lists != 0 && p.row.debug == nullptr) {
+    const uint32_t mine = lane < 32 ? sh.top_mass[lane] : 0u;
+    const uint32_t incl = wave_scan_inclusive_u32(mine);
+    const float need = topp * a_total * 1.04f * 1048576.0f;
+    const uint64_t reach = __ballot(lane < 32 && static_cast<float>(incl) >= need);
+    if (reach != 0ull) {
+      const uint32_t j = static_cast<uint32_t>(__ffsll(static_cast<long long>(reach)) - 1);  // binades 1 .. j are enough
+      // buckets 0 .. 64 j hold every exp from 2^-j up (bucket 64 j starts with 2^-j itself and is listed whole)
+      const float whole = __uint_as_float(0x3F800000u - ((64u * j + 1u) << 17) + 1u);
+      if (whole > cut_lo) {
+        list_cut = whole;
+        listed_buckets = 64u * j + 1u;
+      }
+    }
+  }
   uint64_t* region = p.list + (static_cast<int64_t>(lrow) * p.row_wgs + blockIdx.x) * p.list_region;
   // ---- the pattern histogram's range of order keys: from safely below the smallest logit whose exp
   //      can reach cut_lo up to the row's largest logit (every workgroup of the row arrives at the
@@ -621,11 +669,7 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
     km.n_bins = key_top - km.key_cut + 1;
     if (km.n_bins < 1 || km.n_bins > 2 * p.phist_words) km.n_bins = 0;
   }
-  if (kPatterns && blockIdx.x == 0 && tid == 0) {
-    p.row_state[row].key_cut = km.key_cut;
-    p.row_state[row].n_bins = km.n_bins;
-    p.row_state[row].mag_min = km.mag_min;
-  }
+  if (blockIdx.x == 0 && tid == 0) p.row_state[row] = {serial_before, m, 0u, a_total, km.key_cut, km.n_bins, km.mag_min, listed_buckets};
 
   // ---- the slots, no barriers.  Two buffers take turns, so that the entries of the slot after this
   //      one are on their way while this one is worked on (a copy from one buffer to the other
@@ -654,7 +698,7 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
         e[k] = expf_core(d, tab);
       }
     }
-    split_fold_slot<TOPP, DT>(p, row, s, e, in, sh.cls[s], cut_lo, V, region, sh, km, ph);
+    split_fold_slot<TOPP, DT>(p, row, s, e, in, sh.cls[s], list_cut, V, region, sh, km, ph);
   };
   float l2[8];
   while (s_mine < s_end) {
@@ -1632,14 +1676,21 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
   if (!row_nan) {
     bool done = false;
     const RowDivisor div = row_divisor(S);
-    if (lists_ok && n_listed == 0) {
+    // Short lists (RowState::listed_buckets): the lists hold every entry of the histogram's first
+    // buckets and nothing else, so the number of candidates is unknown ("more exist") and a walk
+    // that does not end inside the listed entries is redone from the row.
+    const bool short_lists = rs.listed_buckets != 0u;
+    const int kMore = 0x7fffffff;
+    if (lists_ok && n_listed == 0 && !short_lists) {
       done = true;  // no candidate (the reference reads probindex[-1] here)
     } else if (lists_ok && plan.b_sel >= 0 && plan.n_sel >= 1 && plan.n_sel <= 64 &&
-               fs.sel_count == static_cast<uint32_t>(plan.n_sel) && fs.band_count <= static_cast<uint32_t>(kBandCap) &&
-               fs.band_count + static_cast<uint32_t>(plan.n_certain) == static_cast<uint32_t>(n_listed)) {
+               fs.sel_count == static_cast<uint32_t>(plan.n_sel) &&
+               (short_lists ? plan.b_sel < static_cast<int>(rs.listed_buckets)
+                            : (fs.band_count <= static_cast<uint32_t>(kBandCap) &&
+                               fs.band_count + static_cast<uint32_t>(plan.n_certain) == static_cast<uint32_t>(n_listed)))) {
       // ---- exact candidate count (sampler.cpp:137-143): the certain ones, plus those of the band
       //      whose probability reaches the cutoff
-      const int n_band = static_cast<int>(fs.band_count);
+      const int n_band = short_lists ? 0 : static_cast<int>(fs.band_count);
       uint32_t cnt = 0u;
       for (int j = tid; j < n_band; j += kBlock) cnt += div_row(__uint_as_float(fs.band[j]), div) >= cutoff ? 1u : 0u;
       cnt = wave_sum_u32(cnt);
@@ -1662,6 +1713,7 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
       __syncthreads();
       uint32_t n0 = static_cast<uint32_t>(plan.n_certain);
       for (int w = 0; w < kWaves; ++w) n0 += sm.red_u[w];
+      if (short_lists) n0 = static_cast<uint32_t>(kMore);
       const bool ok = sm.flag != 0;
       __syncthreads();
       if (n0 == 0u) {
@@ -1677,14 +1729,14 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
     }
     if constexpr (DT == kDtypeBFloat16 || DT == kDtypeHalf) {
       // ---- a longer nucleus of a 16-bit row: runs of equal probabilities
-      if (!done && rs.n_bins > 0 && (!lists_ok || n_listed > 4096)) {
+      if (!done && !short_lists && rs.n_bins > 0 && (!lists_ok || n_listed > 4096)) {
         const RunArgs ra = {p.phist + static_cast<int64_t>(lrow) * p.row_wgs * p.phist_words, p.phist_words, p.row_wgs,
                             p.row.lds_keys, ns, rs.key_cut, rs.n_bins, rs.mag_min, static_cast<uint32_t>(n_listed), m, &fs.fused};
         done = draw_topp_runs<DT>(ra, logits, V, inv, S, cutoff, topp, coin, lds_keys, dbg, token, sm);
         path = 4;
       }
     }
-    if (!done && lists_ok && n_listed <= p.row.lds_keys - kBlock) {
+    if (!done && lists_ok && n_listed > 0 && n_listed <= p.row.lds_keys - kBlock) {
       // ---- a longer nucleus: the whole list goes to LDS, selection by probability, sort, walks
       for (int g = wave; g < p.row_wgs; g += kWaves) {
         const uint64_t* src = p.list + (static_cast<int64_t>(lrow) * p.row_wgs + g) * p.list_region;
@@ -1694,7 +1746,7 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
       }
       __syncthreads();
       done = draw_topp_listed(nullptr, lds_keys + kBlock, p.row.lds_keys - kBlock, kBlock, n_listed, S, cutoff, topp, coin,
-                              lds_keys, p.row.lds_keys, dbg, token, sm);
+                              lds_keys, p.row.lds_keys, dbg, token, sm, short_lists);
       path = 2;
     }
     if (!done) {

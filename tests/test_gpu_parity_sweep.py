@@ -30,5 +30,6 @@ def test_rows_of_a_workload_at_scale(workload, rows):
     res = parity_report.run(workload=workload, rows=rows, chunk=1024, threads=8, seed=7)
     assert res["rows"] == rows
     assert res["token_mismatches_vs_oracle_fp32_index_ties"] == 0, res
+    assert res["token_mismatches_without_debug_records"] == 0, res
     assert res["normaliser_bit_mismatches_vs_oracle"] == 0, res
     assert res["of_which_not_between_equal_probabilities"] == 0, res

@@ -136,3 +136,50 @@ def test_more_rows_than_workgroups(oracle, dev, topp, topk, mode):
         states[:n] = st
         assert np.array_equal(got, want), (n, np.nonzero(got != want)[0][:8])
         assert np.array_equal(s.get_rng_states(n), states[:n])
+
+
+@pytest.mark.parametrize("dtype", [W.DTYPE_BFLOAT16, W.DTYPE_FLOAT, W.DTYPE_HALF])
+def test_short_candidate_lists_do_not_change_tokens(oracle, dev, dtype):
+    """A call without debug records lets pass 2 list only the largest candidates of a row whose
+    largest entries carry the nucleus; a call with them lists every candidate.  Rows on which that
+    matters: few to thousands of raised entries (in distinct slots, sharing slots, sharing a lane's
+    eight entries, equal to each other), raised by little (the shortcut must not apply) or by much
+    (the nucleus is one entry), nuclei of more than 64 entries, a nucleus that ends among equal
+    probabilities.  Tokens and coin states of both calls must be the oracle's."""
+    rng = np.random.default_rng(21)
+    V = 128256 if dtype == W.DTYPE_BFLOAT16 else 70001
+    rows = []
+    for k, boost in ((1, 14.0), (3, 9.0), (20, 8.0), (20, 3.0), (70, 7.0), (300, 7.0), (2500, 6.0), (9000, 5.0)):
+        x = rng.standard_normal(V).astype(np.float32)
+        ids = rng.choice(V, size=k, replace=False)
+        x[ids] += boost
+        rows.append(x)
+    x = rng.standard_normal(V).astype(np.float32)  # raised entries side by side: one slot, some in one lane's eight
+    x[40000:40012] += 9.0
+    rows.append(x)
+    x = rng.standard_normal(V).astype(np.float32)  # equal raised entries: the nucleus ends inside a run of ties
+    x[rng.choice(V, size=40, replace=False)] = 7.5
+    rows.append(x)
+    x = rng.standard_normal(V).astype(np.float32)  # two groups of ties a power of two apart in probability
+    x[rng.choice(V, size=16, replace=False)] = 8.0
+    x[rng.choice(V, size=16, replace=False)] = 8.0 - np.float32(np.log(2.0))
+    rows.append(x)
+    x = np.full(V, -30.0, dtype=np.float32)  # almost everything negligible, 100 entries of falling size
+    x[rng.choice(V, size=100, replace=False)] = np.linspace(0.0, -6.0, 100, dtype=np.float32)
+    rows.append(x)
+    base = W.to_storage(np.stack(rows), dtype)
+    B = base.shape[0]
+    for temperature, topp in ((0.6, 0.9), (1.0, 0.5), (1.0, 0.99), (0.3, 0.9), (2.0, 0.95)):
+        for seed in (5, 6, 7):
+            states = (np.uint64(seed * 1000) + np.arange(B, dtype=np.uint64)).astype(np.uint64)
+            after = states.copy()  # (the oracle advances the states it is given)
+            want, _ = oracle.sample_rows(base, dtype, oracle.inv_temperature(temperature), topp, 0, after,
+                                         mode=oracle.MODE_UPCAST, tie=oracle.TIE_STABLE, threads=8)
+            for with_debug in (False, True):
+                s = ea.Sampler(V, temperature, topp, 1, max_batch=B)
+                s.set_row_split(SPLIT_ON)
+                s.set_rng_states(states)
+                dbg = torch.zeros((B, 8), dtype=torch.int32, device=dev) if with_debug else None
+                got = s.sample_batch(to_device(base, dtype, dev), debug_out=dbg).cpu().numpy()
+                assert np.array_equal(got, want), (temperature, topp, seed, with_debug, np.nonzero(got != want)[0])
+                assert np.array_equal(s.get_rng_states(B), after)
