@@ -202,6 +202,29 @@ __device__ __forceinline__ int wave_max_i32(int v) {
   return static_cast<int>(__builtin_amdgcn_readlane(static_cast<uint32_t>(v), 63));
 }
 
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
+  // (lanes without a source read 0, the identity of the maximum: one instruction per step)
+#define ETS_MAX_STEP(CTRL, MASK)                      \
+  {                                                   \
+    const uint32_t o = dpp_u32_or<CTRL, MASK>(0u, v); \
+    v = o > v ? o : v;                                \
+  }
+  ETS_MAX_STEP(0x111, 0xf) ETS_MAX_STEP(0x112, 0xf) ETS_MAX_STEP(0x114, 0xf) ETS_MAX_STEP(0x118, 0xf)
+  ETS_MAX_STEP(0x142, 0xa) ETS_MAX_STEP(0x143, 0xc)
+#undef ETS_MAX_STEP
+  return __builtin_amdgcn_readlane(v, 63);
+}
+
+// Unsigned key of a float: a larger value has a larger key (-0 below +0; a NaN with the sign bit
+// clear above +inf), and back.
+__device__ __forceinline__ uint32_t float_max_key(float x) {
+  const uint32_t u = __float_as_uint(x);
+  return u ^ (static_cast<uint32_t>(static_cast<int32_t>(u) >> 31) | 0x80000000u);
+}
+__device__ __forceinline__ float float_of_max_key(uint32_t k) {
+  return __uint_as_float((k & 0x80000000u) ? (k ^ 0x80000000u) : ~k);
+}
+
 __device__ __forceinline__ float wave_max_ignoring_nan(float v) {
 #define ETS_MAX_STEP(CTRL, MASK)                                                                      \
   {                                                                                                   \

@@ -163,8 +163,16 @@ __device__ __forceinline__ void load_slot_lane(const char* logits, int s, int la
                                                const FusedOps& f) {
   constexpr int VE = VecElems<DT>::value;
   const int first = s * kSlot + lane * 8;
+  if ((s + 1) * kSlot <= V) {  // (the same for every lane) a slot inside the row: no position is tested
 #pragma unroll
-  for (int q = 0; q < 8 / VE; ++q) load_run<DT, true>(logits, first + q * VE, V, fill, out + q * VE);
+    for (int q = 0; q < 8 / VE; ++q) {
+      const uint4 raw = *reinterpret_cast<const uint4*>(logits + static_cast<int64_t>(first + q * VE) * ElemSize<DT>::value);
+      decode_vec<DT>(raw, out + q * VE);
+    }
+  } else {
+#pragma unroll
+    for (int q = 0; q < 8 / VE; ++q) load_run<DT, true>(logits, first + q * VE, V, fill, out + q * VE);
+  }
   if (f.n > 0) {
     apply_fused<DT, 8>(out, f);
     if (first + 8 > V) {
@@ -225,7 +233,6 @@ __global__ void __launch_bounds__(kPass1Block) split_pass1_kernel(SplitParams p)
       const int s = slot0 + k;
       if (s >= s_end) break;
       float ext = inv_u < 0.0f ? kInf : -kInf;
-      bool nan = false;
       if (inv_u < 0.0f) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) ext = __builtin_fminf(ext, v[k][e]);  // ignores NaN
@@ -233,24 +240,38 @@ __global__ void __launch_bounds__(kPass1Block) split_pass1_kernel(SplitParams p)
 #pragma unroll
         for (int e = 0; e < 8; ++e) ext = __builtin_fmaxf(ext, v[k][e]);
       }
-#pragma unroll
-      for (int e = 0; e < 8; ++e) nan = nan || (v[k][e] != v[k][e]);
       // (a lane whose entries all lie past the row's end holds the fill value, whose product is -inf)
-      const float xm = ext * inv_u;
-      const float M = wave_max_ignoring_nan(xm);
-      const bool any_nan = __ballot(nan) != 0ull;
+      // (reduced as integer keys: one instruction per step.  A NaN product -- the row is one then --
+      // may come out as the maximum: the slot's maximum is stored as NaN in that case anyway.)
+      const uint32_t xk = float_max_key(ext * inv_u);
+      const uint32_t Mk = wave_max_u32(xk);
+      const float M = float_of_max_key(Mk);
       // the largest entry of the other lanes (pass 2 bounds the mass of the row's largest entries
       // from below with the two)
-      const uint64_t holds = __ballot(xm == M);
-      const int holder = holds ? __ffsll(static_cast<long long>(holds)) - 1 : 64;
-      const float M2 = wave_max_ignoring_nan(lane == holder ? -kInf : xm);
+      const uint64_t holds = __ballot(xk == Mk);
+      const int holder = __ffsll(static_cast<long long>(holds)) - 1;  // (some lane holds the maximum)
+      const float M2 = float_of_max_key(wave_max_u32(lane == holder ? float_max_key(-kInf) : xk));
+      // With a finite maximum of ordinary size every entry's exponent below is finite or -inf unless
+      // the entry is NaN, so the sum itself tells whether the slot holds a NaN; otherwise the
+      // entries are tested one by one.
+      const bool ordinary = M > -kInf && __builtin_fabsf(M) < 1e38f;
       float sum = 0.0f;
-      if (M > -kInf) {
+      bool nan = false;
+      if (ordinary) {
         const float c2 = -M * kLog2e;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) sum += fast_exp2(__builtin_fmaf(v[k][e], c1, c2));  // (a NaN here: the row is one)
+        for (int e = 0; e < 8; ++e) sum += fast_exp2(__builtin_fmaf(v[k][e], c1, c2));
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) nan = nan || (v[k][e] != v[k][e]);
+        if (M > -kInf) {
+          const float c2 = -M * kLog2e;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) sum += fast_exp2(__builtin_fmaf(v[k][e], c1, c2));  // (a NaN here: the row is one)
+        }
       }
       sum = wave_sum_f32(sum);
+      const bool any_nan = ordinary ? sum != sum : __ballot(nan) != 0ull;
       if (lane == 0) {
         const int64_t at = static_cast<int64_t>(row) * p.ns_stride + s;
         p.slot_max[at] = any_nan ? __uint_as_float(0x7fc00000u) : M;
@@ -267,6 +288,7 @@ struct Pass2Shared {
   BlockScratch sm;
   float upto[kMaxSlots + 1];  // approximate running sum in front of every slot, in units of exp(-m)
   uint32_t cls[kMaxSlots];    // per slot: kb_lo | kb_hi << 8 | kind << 16 | prepared-slot index << 19
+  float top[kMaxSlots];       // per slot: an upper bound of its largest exp (top-p: a slot below the listing cut is not searched)
   uint32_t hist[kHistBuckets];
   uint32_t list_count;        // candidates this workgroup has listed
   uint32_t top_mass[32];      // the slots' two largest exps, added up per binade (bin j: [2^-j, 2^(1-j))), in units of 2^-20
@@ -275,13 +297,13 @@ struct Pass2Shared {
 // One wave, one slot: e[] are the lane's 8 entries; `cls` is the slot's entry of Pass2Shared::cls.
 template <bool TOPP, int DT>
 __device__ __forceinline__ void split_fold_slot(const SplitParams& p, int row, int s, const float (&e)[8],
-                                                const float (&logit)[8], uint32_t cls, float cut_lo, int V, uint64_t* region,
-                                                Pass2Shared& sh, const KeyMap& km, uint32_t* ph) {
+                                                const float (&logit)[8], uint32_t cls, float cut_lo, bool search, int V,
+                                                uint64_t* region, Pass2Shared& sh, const KeyMap& km, uint32_t* ph) {
   const int lane = threadIdx.x & 63;
   const int64_t rec_at = static_cast<int64_t>(row) * p.ns_stride + s;
   // ---- candidates of the top-p draw (sampler.cpp:137-143), by a cut that is safely below the
   //      reference's once the exact normaliser is known
-  if (TOPP) {
+  if (TOPP && search) {
     // bit k: entry k is a candidate (two instructions per entry: compare, shift the outcome in)
     uint32_t cmask = 0u;
 #pragma unroll
@@ -556,6 +578,7 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
       const float smax = base == 0 ? first_max : slot_max[s];
       const float f = sum > 0.0f ? fast_exp2((smax - m) * kLog2e) : 0.0f;  // exp of the slot's largest entry
       a = sum > 0.0f ? sum * f : 0.0f;
+      if (TOPP) sh.top[s] = f * 1.0001f;  // (the hardware's exp2 is within 1e-5 of the exact exp)
       if (TOPP && f > 0.0f) {
         // lower bounds of the exact exps of the slot's two largest entries, into the bins of their
         // binades (integers: every workgroup of the row arrives at the same totals)
@@ -650,7 +673,9 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
   //      can reach cut_lo up to the row's largest logit (every workgroup of the row arrives at the
   //      same two numbers).  Too many bins for the LDS set aside: no pattern histogram.
   KeyMap km = {0, 0, 0};
-  if (kPatterns && p.phist_words > 0 && inv > 0.0f && inv < kInf && cut_lo > 0.0f && (__float_as_uint(inv) >> 23) != 0u) {
+  // (short lists are drawn from directly: no pattern histogram then)
+  if (kPatterns && listed_buckets == 0u && p.phist_words > 0 && inv > 0.0f && inv < kInf && cut_lo > 0.0f &&
+      (__float_as_uint(inv) >> 23) != 0u) {
     // magnitudes below 2^(em - ei - 27) vanish against m (em, ei: biased exponents of |m| and inv)
     const uint32_t mb = __float_as_uint(__builtin_fabsf(m));
     const int em = (mb >> 23) ? static_cast<int>(mb >> 23) : 1;
@@ -698,7 +723,8 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
         e[k] = expf_core(d, tab);
       }
     }
-    split_fold_slot<TOPP, DT>(p, row, s, e, in, sh.cls[s], list_cut, V, region, sh, km, ph);
+    const bool search = TOPP && __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(sh.top[s]))) >= list_cut;
+    split_fold_slot<TOPP, DT>(p, row, s, e, in, sh.cls[s], list_cut, search, V, region, sh, km, ph);
   };
   float l2[8];
   while (s_mine < s_end) {
@@ -714,7 +740,9 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
     __syncthreads();
     if (tid == 0) p.list_count[static_cast<int64_t>(lrow) * kMaxRowWorkgroups + blockIdx.x] = sh.list_count;
     uint32_t* hist_out = p.hist + (static_cast<int64_t>(lrow) * p.row_wgs + blockIdx.x) * kHistBuckets;
-    for (int b = tid; b < kHistBuckets; b += kBlock) hist_out[b] = sh.hist[b];
+    // (short lists: the buckets behind the listed ones are empty, and the finish kernel does not read them)
+    const int n_hist = listed_buckets != 0u ? static_cast<int>(listed_buckets) : kHistBuckets;
+    for (int b = tid; b < n_hist; b += kBlock) hist_out[b] = sh.hist[b];
     if (kPatterns && km.n_bins > 0) {
       uint32_t* ph_out = p.phist + (static_cast<int64_t>(lrow) * p.row_wgs + blockIdx.x) * p.phist_words;
       for (int b = tid; b < (km.n_bins + 1) / 2; b += kBlock) ph_out[b] = ph[b];
@@ -1563,6 +1591,7 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
     {
       // (four workgroups' counts are requested at a time: a loop of one load each would wait for each)
       const uint32_t* hist_in = p.hist + static_cast<int64_t>(lrow) * p.row_wgs * kHistBuckets;
+      const int n_hist = rs.listed_buckets != 0u ? static_cast<int>(rs.listed_buckets) : kHistBuckets;  // (the rest was not written)
       uint32_t c[kHistBuckets / kBlock];
 #pragma unroll
       for (int q = 0; q < kHistBuckets / kBlock; ++q) c[q] = 0u;
@@ -1572,7 +1601,9 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
         for (int k = 0; k < 4; ++k) {
           const int gk = g + k < p.row_wgs ? g + k : g;
 #pragma unroll
-          for (int q = 0; q < kHistBuckets / kBlock; ++q) v[k][q] = hist_in[gk * kHistBuckets + q * kBlock + tid];
+          for (int q = 0; q < kHistBuckets / kBlock; ++q) {
+            v[k][q] = q * kBlock + tid < n_hist ? hist_in[gk * kHistBuckets + q * kBlock + tid] : 0u;
+          }
         }
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
