@@ -78,12 +78,12 @@ struct ets_sampler {
   hipEvent_t stage_done = nullptr;
   hipStream_t stage_stream = nullptr;
   bool stage_used = false;
-  // ets_sampler_sample_batch_configs(): the groups of rows that draw in different ways run side by
-  // side, each behind the call's stream on a stream of its own (default priority), joined again
-  // before the call returns to the caller's stream
-  hipStream_t aux_stream[3] = {};
+  // ets_sampler_sample_batch_configs(): rows that take different launches run side by side, one
+  // group on the call's stream and the others on a second stream (default priority) that starts
+  // behind the call's stream and is joined again before the call returns
+  hipStream_t aux_stream = nullptr;
   hipEvent_t fork_event = nullptr;
-  hipEvent_t join_event[3] = {};
+  hipEvent_t join_event = nullptr;
   // opt-in device timing (ets_sampler_set_timing): a ring of event pairs around the launches of a
   // call, harvested when a slot is reused or the totals are read
   bool timing = false;
@@ -258,6 +258,15 @@ ets_status launch_rows(ets_sampler* s, const ets::RowParams& p, int32_t batch, h
   // one kernel instantiation per draw
   const bool use_topk = draw == ets::kDrawTopK;
   const bool use_mult = draw == ets::kDrawMultinomial;
+  if (draw == ets::kDrawAny) {
+    // rows of different draws in one launch (the looping instantiation serves every batch size)
+    ets::RowParams q = p;
+    q.rows = batch;
+    q.ticket = (s->wb ? s->wb->tickets : s->d_tickets) + 4;  // (0 .. 2: the launches of one draw, 3: the finish kernel)
+    const int grid = batch < q.grid_cap ? batch : q.grid_cap;
+    return aligned ? launch_rows_looped<DT, true, ets::kDrawAny, true>(s, q, grid, stream)
+                   : launch_rows_looped<DT, false, ets::kDrawAny, true>(s, q, grid, stream);
+  }
   if (use_topk) {
     return aligned ? launch_rows_impl<DT, true, ets::kDrawTopK>(s, p, batch, stream)
                    : launch_rows_impl<DT, false, ets::kDrawTopK>(s, p, batch, stream);
@@ -604,10 +613,8 @@ ets_status stage_release(ets_sampler* s, hipStream_t stream) {
 
 ets_status ensure_aux_streams(ets_sampler* s) {
   if (s->fork_event) return ETS_OK;
-  for (int i = 0; i < 3; ++i) {
-    ETS_HIP(s, hipStreamCreateWithFlags(&s->aux_stream[i], hipStreamNonBlocking));
-    ETS_HIP(s, hipEventCreateWithFlags(&s->join_event[i], hipEventDisableTiming));
-  }
+  ETS_HIP(s, hipStreamCreateWithFlags(&s->aux_stream, hipStreamNonBlocking));
+  ETS_HIP(s, hipEventCreateWithFlags(&s->join_event, hipEventDisableTiming));
   ETS_HIP(s, hipEventCreateWithFlags(&s->fork_event, hipEventDisableTiming));
   return ETS_OK;
 }
@@ -627,7 +634,12 @@ ets_status sample_device_configs(ets_sampler* s, const void* d_logits, int32_t d
   uint64_t* h_reseed = reinterpret_cast<uint64_t*>(h + lay.reseed);
   ets::RowConfig* h_cfg = reinterpret_cast<ets::RowConfig*>(h + lay.cfg);
   int32_t* h_maps = reinterpret_cast<int32_t*>(h + lay.maps);
-  int32_t count[4] = {0, 0, 0, 0};  // greedy, then ets::kDrawTopP / Multinomial / TopK + 1
+  // Three groups of rows: arg-max rows, top-p rows that take the three-launch path, and every other
+  // row that draws (one launch of the one-workgroup-per-row kernel, which picks each row's draw
+  // from its parameters).  maps[g * batch + i]: the i-th row of group g.
+  enum { kGreedy = 0, kSplit = 1, kRows = 2 };
+  int32_t count[3] = {0, 0, 0};
+  const bool split_ok = use_split(s, d_logits, stride, dtype, ets::kDrawTopP);
   bool any_reseed = false;
   for (int32_t b = 0; b < batch; ++b) {
     const ets_sampling_config& c = configs[b];
@@ -638,11 +650,12 @@ ets_status sample_device_configs(ets_sampler* s, const void* d_logits, int32_t d
     h_cfg[b].topk = c.top_k;
     h_reseed[b] = c.seed;
     any_reseed = any_reseed || c.seed != 0;
-    const int group = inv == 0.0f ? 0 : 1 + draw_mode(s->vocab, c.top_p, c.top_k);
-    if (group != 0 && dtype == ETS_DTYPE_UINT16) return fail(s, ETS_NOT_SUPPORTED, kUint16Message);
+    int group = kGreedy;
+    if (inv != 0.0f) group = (split_ok && draw_mode(s->vocab, c.top_p, c.top_k) == ets::kDrawTopP) ? kSplit : kRows;
+    if (group != kGreedy && dtype == ETS_DTYPE_UINT16) return fail(s, ETS_NOT_SUPPORTED, kUint16Message);
     h_maps[group * batch + count[group]++] = b;
   }
-  if (count[1] + count[2] + count[3] > 0) {
+  if (count[kSplit] + count[kRows] > 0) {
     st = ensure_scratch(s);
     if (st != ETS_OK) return st;
   }
@@ -657,29 +670,6 @@ ets_status sample_device_configs(ets_sampler* s, const void* d_logits, int32_t d
     ETS_HIP(s, hipGetLastError());
   }
   const int32_t* d_maps = reinterpret_cast<const int32_t*>(d + lay.maps);
-  // The groups touch different rows and different work buffers: the first one that has rows runs
-  // on the caller's stream, every further one on a stream of its own between a fork and a join.
-  const int groups = (count[0] > 0) + (count[1] > 0) + (count[2] > 0) + (count[3] > 0);
-  if (groups > 1) {
-    st = ensure_aux_streams(s);
-    if (st != ETS_OK) return st;
-    ETS_HIP(s, hipEventRecord(s->fork_event, stream));
-  }
-  int forked = 0;
-  bool main_taken = false;
-  hipStream_t side[3] = {};
-  auto group_stream = [&](hipStream_t* out) -> ets_status {
-    if (!main_taken) {
-      main_taken = true;
-      *out = stream;
-      return ETS_OK;
-    }
-    hipStream_t a = s->aux_stream[forked];
-    ETS_HIP(s, hipStreamWaitEvent(a, s->fork_event, 0));
-    side[forked++] = a;
-    *out = a;
-    return ETS_OK;
-  };
   ets::RowParams p = {};
   p.logits = d_logits;
   p.row_stride = stride;
@@ -694,37 +684,45 @@ ets_status sample_device_configs(ets_sampler* s, const void* d_logits, int32_t d
   p.scratch_stride = s->scratch_stride;
   p.lds_keys = s->lds_keys;
   p.row_cfg = reinterpret_cast<const ets::RowConfig*>(d + lay.cfg);
-  // The groups that draw run side by side: each gets its share of the scratch rows (a workgroup
-  // owns the scratch row of its index in its launch).
-  const int drawing = (count[1] > 0) + (count[2] > 0) + (count[3] > 0);
-  const int32_t share = drawing > 0 ? s->scratch_rows / drawing : 0;
-  if (drawing > 0 && share < 1) return fail(s, ETS_INTERNAL, "ets_sampler_sample_batch_configs: no scratch rows");
-  int32_t next_scratch_row = 0;
-  // the longest-running groups first (multinomial, top-k, top-p), the arg-max last
-  const int order[3] = {ets::kDrawMultinomial, ets::kDrawTopK, ets::kDrawTopP};
-  for (int k = 0; k < 3; ++k) {
-    const int draw = order[k];
-    if (count[1 + draw] == 0) continue;
-    hipStream_t gs = nullptr;
-    st = group_stream(&gs);
+  // The groups touch different rows and different work buffers.  The one-workgroup-per-row launch
+  // is the longest and runs on the caller's stream; when there is one, the other groups run
+  // beside it on a second stream, between a fork and a join (one of each: they cost more on the
+  // host than the kernels they order).  The two launches that draw share the scratch rows (a
+  // workgroup owns the scratch row of its index in its launch).
+  const bool fork = count[kRows] > 0 && count[kSplit] + count[kGreedy] > 0;
+  hipStream_t side = stream;
+  if (fork) {
+    st = ensure_aux_streams(s);
     if (st != ETS_OK) return st;
-    p.scratch = s->d_scratch + static_cast<int64_t>(next_scratch_row) * s->scratch_stride;
+    side = s->aux_stream;
+    ETS_HIP(s, hipEventRecord(s->fork_event, stream));
+    ETS_HIP(s, hipStreamWaitEvent(side, s->fork_event, 0));
+  }
+  const bool both_draw = count[kRows] > 0 && count[kSplit] > 0;
+  const int32_t share = both_draw ? s->scratch_rows / 2 : s->scratch_rows;
+  if (count[kSplit] + count[kRows] > 0 && share < 1)
+    return fail(s, ETS_INTERNAL, "ets_sampler_sample_batch_configs: no scratch rows");
+  if (count[kRows] > 0) {
+    p.scratch = s->d_scratch;
     p.grid_cap = share;
-    next_scratch_row += share;
-    p.row_map = d_maps + (1 + draw) * batch;
-    st = rows_device(s, p, dtype, count[1 + draw], gs, draw);
+    p.row_map = d_maps + kRows * batch;
+    st = rows_device(s, p, dtype, count[kRows], stream, ets::kDrawAny);
     if (st != ETS_OK) return st;
   }
-  if (count[0] > 0) {
-    hipStream_t gs = nullptr;
-    st = group_stream(&gs);
-    if (st != ETS_OK) return st;
-    st = argmax_device(s, d_logits, dtype, count[0], stride, d_tokens, gs, d_maps);
+  if (count[kSplit] > 0) {
+    p.scratch = s->d_scratch + (both_draw ? static_cast<int64_t>(share) * s->scratch_stride : 0);
+    p.grid_cap = share;
+    p.row_map = d_maps + kSplit * batch;
+    st = rows_device(s, p, dtype, count[kSplit], side, ets::kDrawTopP);
     if (st != ETS_OK) return st;
   }
-  for (int i = 0; i < forked; ++i) {
-    ETS_HIP(s, hipEventRecord(s->join_event[i], side[i]));
-    ETS_HIP(s, hipStreamWaitEvent(stream, s->join_event[i], 0));
+  if (count[kGreedy] > 0) {
+    st = argmax_device(s, d_logits, dtype, count[kGreedy], stride, d_tokens, side, d_maps + kGreedy * batch);
+    if (st != ETS_OK) return st;
+  }
+  if (fork) {
+    ETS_HIP(s, hipEventRecord(s->join_event, side));
+    ETS_HIP(s, hipStreamWaitEvent(stream, s->join_event, 0));
   }
   return stage_release(s, stream);
 }
@@ -835,10 +833,8 @@ ets_status ets_sampler_destroy(ets_sampler* s) {
     (void)hipFree(s->d_token);
     (void)hipFree(s->d_stage);
     if (s->h_stage) (void)hipHostFree(s->h_stage);
-    for (int i = 0; i < 3; ++i) {
-      if (s->aux_stream[i]) (void)hipStreamDestroy(s->aux_stream[i]);
-      if (s->join_event[i]) (void)hipEventDestroy(s->join_event[i]);
-    }
+    if (s->aux_stream) (void)hipStreamDestroy(s->aux_stream);
+    if (s->join_event) (void)hipEventDestroy(s->join_event);
     if (s->fork_event) (void)hipEventDestroy(s->fork_event);
     if (s->stage_event) (void)hipEventDestroy(s->stage_event);
     if (s->stage_done) (void)hipEventDestroy(s->stage_done);

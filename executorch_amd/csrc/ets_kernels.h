@@ -1585,6 +1585,7 @@ __device__ __noinline__ bool draw_topk_listed(uint64_t* lds_keys, int cap, int l
 // Pass 2 re-reads it (L2 / Infinity Cache): exact expf, the sequential sum in index order, and
 // the list of possible top-p candidates.  Then the coin and the draw.
 constexpr int kDrawTopP = 0, kDrawMultinomial = 1, kDrawTopK = 2;  // sampler.cpp:238-249, chosen by the host
+constexpr int kDrawAny = 3;  // chosen per row from its top-k and top-p (rows with parameters of their own)
 
 // LOOP: fewer workgroups than rows, a workgroup takes one row after the other (the loop costs
 // registers, so a launch with a workgroup per row uses the instantiation without it).
@@ -1612,9 +1613,12 @@ __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
   if (tid < 32) sm.exp2tab[tid] = kExp2Table[tid];
   if (tid == 0) sm.counter = 0u;
 
-  constexpr bool use_topk = DRAW == kDrawTopK;
-  constexpr bool use_mult = DRAW == kDrawMultinomial;
-  constexpr bool use_topp = DRAW == kDrawTopP;
+  // (compile-time constants but for kDrawAny, where the row's parameters decide: sampler.cpp:238-249)
+  const int draw = DRAW != kDrawAny ? DRAW
+                                    : ((topk > 0 && topk < V) ? kDrawTopK : ((topp <= 0.0f || topp >= 1.0f) ? kDrawMultinomial : kDrawTopP));
+  const bool use_topk = draw == kDrawTopK;
+  const bool use_mult = draw == kDrawMultinomial;
+  const bool use_topp = draw == kDrawTopP;
 
   // ---- pass 1: row maximum (sampler.cpp:231-233, 191-197)
   float m = -kInf;
