@@ -438,10 +438,20 @@ ets_status launch_split(ets_sampler* s, const ets::RowParams& p, int32_t rows, h
   hipLaunchKernelGGL((ets::split_pass2_kernel<DT, true>), dim3(sp.row_wgs, rows), dim3(ets::kBlock), lut_bytes, stream, sp);
   ETS_HIP(s, hipGetLastError());
   if (rows > p.grid_cap) {
+    // more rows than workgroups: a workgroup takes up to kChainRows rows at a time
+    static const int chain_rows_max = [] {
+      const char* e = std::getenv("ETS_CHAIN_ROWS");
+      const int v = e ? std::atoi(e) : ets::kChainRows;
+      return v < 1 ? 1 : (v > ets::kChainRows ? ets::kChainRows : v);
+    }();
+    const int per_wg = (rows + p.grid_cap - 1) / p.grid_cap;
+    sp.chain_rows = per_wg < chain_rows_max ? per_wg : chain_rows_max;
+    const int units = (rows + sp.chain_rows - 1) / sp.chain_rows;
     static std::atomic<size_t> set_bytes[kMaxDevices];
     st = allow_dynamic_lds(s, reinterpret_cast<const void*>(&ets::split_finish_kernel<DT, true>), s->lds_bytes, set_bytes);
     if (st != ETS_OK) return st;
-    hipLaunchKernelGGL((ets::split_finish_kernel<DT, true>), dim3(p.grid_cap), dim3(ets::kBlock), s->lds_bytes, stream, sp);
+    hipLaunchKernelGGL((ets::split_finish_kernel<DT, true>), dim3(units < p.grid_cap ? units : p.grid_cap), dim3(ets::kBlock),
+                       s->lds_bytes, stream, sp);
   } else {
     static std::atomic<size_t> set_bytes[kMaxDevices];
     st = allow_dynamic_lds(s, reinterpret_cast<const void*>(&ets::split_finish_kernel<DT, false>), s->lds_bytes, set_bytes);

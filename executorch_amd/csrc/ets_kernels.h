@@ -70,20 +70,23 @@ struct RowParams {
 // row a workgroup works on costs one request, so the launch makes p.rows of them, and whoever makes
 // the last one puts the counter back to 0 for the next launch.  A launch with a workgroup per row
 // touches no counter.
-__device__ __forceinline__ void request_row(const RowParams& p, int* lds_slot) {
-  if (static_cast<int>(gridDim.x) < p.rows && threadIdx.x == 0) {
+// (`units`: what is handed out, when it is not single rows)
+__device__ __forceinline__ void request_row(const RowParams& p, int* lds_slot, int units) {
+  if (static_cast<int>(gridDim.x) < units && threadIdx.x == 0) {
     const uint32_t t = atomicAdd(p.ticket, 1u);
-    if (t + 1u == static_cast<uint32_t>(p.rows)) atomicExch(p.ticket, 0u);
+    if (t + 1u == static_cast<uint32_t>(units)) atomicExch(p.ticket, 0u);
     *lds_slot = static_cast<int>(gridDim.x + t);
   }
 }
-__device__ __forceinline__ int take_row(const RowParams& p, const int* lds_slot) {
-  if (static_cast<int>(gridDim.x) >= p.rows) return p.rows;
+__device__ __forceinline__ int take_row(const RowParams& p, const int* lds_slot, int units) {
+  if (static_cast<int>(gridDim.x) >= units) return units;
   __syncthreads();
   const int next = *lds_slot;
   __syncthreads();
   return next;
 }
+__device__ __forceinline__ void request_row(const RowParams& p, int* lds_slot) { request_row(p, lds_slot, p.rows); }
+__device__ __forceinline__ int take_row(const RowParams& p, const int* lds_slot) { return take_row(p, lds_slot, p.rows); }
 
 // A float rounded to the row's element type and back (round to nearest even; a NaN stays a NaN).
 template <int DT>

@@ -139,6 +139,8 @@ struct SplitParams {
   uint64_t* timers;     // phase clocks (profiling), or null
   int32_t list_region;  // entries per region
   int32_t short_lists;  // 1: pass 2 may list only the largest candidates of a peaked row (see RowState::listed_buckets)
+  int32_t chain_rows;   // the looping finish kernel: rows a workgroup takes at a time (1 .. kChainRows); their sums are
+                        //   composed side by side, one wave each
   int32_t row_wgs;      // workgroups of pass 2 per row
   int32_t ns;           // slots per row
   int32_t ns_stride;
@@ -981,7 +983,9 @@ struct FinishShared {
   uint32_t overflow;
   HistPlan plan;
   FusedOps fused;  // (the draw functions are calls: they read the launch's processors from here)
+  float pre_sum[4];  // softmax sums of the rows of a unit (kChainRows), composed before their draws
 };
+constexpr int kChainRows = 4;
 
 // By the whole workgroup, two buckets per lane; `plan_out` is LDS.  Ends with a barrier.
 __device__ __forceinline__ HistPlan split_plan(const uint32_t* hist, float a_total, float topp, float cutoff, int V,
@@ -1552,9 +1556,58 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
   const int wave = tid >> 6;
   const int V = p.row.vocab;
   const int ns = p.ns;
+  // A unit of work is one row, or, in the looping instantiation, p.chain_rows consecutive rows of
+  // the launch: the softmax sum of a row is composed by ONE wave while the others have little to
+  // do, so the sums of a unit's rows are composed side by side, a wave each, before the rows are
+  // drawn one after the other.
+  const int R = LOOP ? p.chain_rows : 1;
+  const int n_units = (p.row.rows + R - 1) / R;
+  const size_t lds_bytes = static_cast<size_t>(p.row.lds_keys) * sizeof(uint64_t);
+  const size_t rec_bytes = (static_cast<size_t>(ns) * sizeof(SlotRec) + 15) / 16 * 16;
+  for (int unit = blockIdx.x; unit < n_units; unit = LOOP ? take_row(p.row, &next_lrow, n_units) : n_units) {
+  if (LOOP) request_row(p.row, &next_lrow, n_units);
+  const int r_first = unit * R;
+  const int r_count = !LOOP ? 1 : (p.row.rows - r_first < R ? p.row.rows - r_first : R);
+  const bool chained = LOOP && R > 1;
+  if (chained) {
+    if (tid < 32) sm.exp2tab[tid] = kExp2Table[tid];
+    // every row gets an equal share of the key buffer for its records and prepared slots
+    const size_t share = lds_bytes / static_cast<size_t>(R) / 16 * 16;
+    const uint32_t fit = share > rec_bytes ? static_cast<uint32_t>((share - rec_bytes) / sizeof(PrepSlot)) : 0u;
+    auto prepared = [&](const RowState& st) -> uint32_t {
+      uint32_t n = st.prep_count < static_cast<uint32_t>(p.prep_cap) ? st.prep_count : static_cast<uint32_t>(p.prep_cap);
+      return n < fit ? n : fit;
+    };
+    for (int k = 0; k < r_count; ++k) {
+      const int row_k = p.row.row_map ? p.row.row_map[r_first + k] : r_first + k;
+      const RowState st = p.row_state[row_k];
+      if (st.nan != 0u) continue;
+      uint4* dst = reinterpret_cast<uint4*>(reinterpret_cast<char*>(lds_keys) + static_cast<size_t>(k) * share);
+      const uint4* rec_src = reinterpret_cast<const uint4*>(p.slot_rec + static_cast<int64_t>(row_k) * p.ns_stride);
+      for (int i = tid; i < ns; i += kBlock) dst[i] = rec_src[i];
+      const uint4* prep_src = reinterpret_cast<const uint4*>(p.prep + static_cast<int64_t>(row_k) * p.prep_cap);
+      const int prep_vecs = static_cast<int>(prepared(st) * (sizeof(PrepSlot) / 16));
+      for (int i = tid; i < prep_vecs; i += kBlock) dst[rec_bytes / 16 + i] = prep_src[i];
+    }
+    __syncthreads();
+    if (wave < r_count) {
+      const int row_k = p.row.row_map ? p.row.row_map[r_first + wave] : r_first + wave;
+      const RowState st = p.row_state[row_k];
+      float sum = __uint_as_float(0x7fc00000u);
+      if (st.nan == 0u) {
+        const float inv_k = p.row.row_cfg ? p.row.row_cfg[row_k].inv_temperature : p.row.inv_temperature;
+        const char* logits_k = static_cast<const char*>(p.row.logits) + static_cast<int64_t>(row_k) * p.row.row_stride * ElemSize<DT>::value;
+        const char* mine = reinterpret_cast<const char*>(lds_keys) + static_cast<size_t>(wave) * share;
+        sum = split_chain<DT>(reinterpret_cast<const SlotRec*>(mine), ns, reinterpret_cast<const PrepSlot*>(mine + rec_bytes),
+                              prepared(st), logits_k, V, inv_k, st.m, sm.exp2tab, p.row.fused,
+                              p.timers ? p.timers + static_cast<int64_t>(row_k) * 8 : nullptr);
+      }
+      if (lane == 0) fs.pre_sum[wave] = sum;
+    }
+    __syncthreads();
+  }
   // lrow, the row of this launch, indexes the buffers whose layout depends on the launch
-  for (int lrow = blockIdx.x; lrow < p.row.rows; lrow = LOOP ? take_row(p.row, &next_lrow) : p.row.rows) {
-  if (LOOP) request_row(p.row, &next_lrow);
+  for (int lrow = r_first; lrow < r_first + r_count; ++lrow) {
   const int row = p.row.row_map ? p.row.row_map[lrow] : lrow;
   const float inv = p.row.row_cfg ? p.row.row_cfg[row].inv_temperature : p.row.inv_temperature;
   const float topp = p.row.row_cfg ? p.row.row_cfg[row].topp : p.row.topp;
@@ -1615,29 +1668,33 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
       for (int q = 0; q < kHistBuckets / kBlock; ++q) fs.hist[q * kBlock + tid] = c[q];
     }
     // ---- LDS: the records, then as many prepared slots as fit (one that does not is redone from
-    //      the logits when its turn comes)
-    const size_t lds_bytes = static_cast<size_t>(p.row.lds_keys) * sizeof(uint64_t);
-    const size_t rec_bytes = (static_cast<size_t>(ns) * sizeof(SlotRec) + 15) / 16 * 16;
+    //      the logits when its turn comes); not when the unit's sums have been composed already
     uint32_t n_prep = rs.prep_count < static_cast<uint32_t>(p.prep_cap) ? rs.prep_count : static_cast<uint32_t>(p.prep_cap);
     const uint32_t fit = static_cast<uint32_t>((lds_bytes - rec_bytes) / sizeof(PrepSlot));
     n_prep = n_prep < fit ? n_prep : fit;
     uint4* lds_vec = reinterpret_cast<uint4*>(lds_keys);
-    const uint4* rec_src = reinterpret_cast<const uint4*>(p.slot_rec + static_cast<int64_t>(row) * p.ns_stride);
-    for (int i = tid; i < ns; i += kBlock) lds_vec[i] = rec_src[i];
-    const uint4* prep_src = reinterpret_cast<const uint4*>(p.prep + static_cast<int64_t>(row) * p.prep_cap);
     uint4* prep_dst = lds_vec + rec_bytes / 16;
-    const int prep_vecs = static_cast<int>(n_prep * (sizeof(PrepSlot) / 16));
-    for (int i = tid; i < prep_vecs; i += kBlock) prep_dst[i] = prep_src[i];
+    if (!chained) {
+      const uint4* rec_src = reinterpret_cast<const uint4*>(p.slot_rec + static_cast<int64_t>(row) * p.ns_stride);
+      for (int i = tid; i < ns; i += kBlock) lds_vec[i] = rec_src[i];
+      const uint4* prep_src = reinterpret_cast<const uint4*>(p.prep + static_cast<int64_t>(row) * p.prep_cap);
+      const int prep_vecs = static_cast<int>(n_prep * (sizeof(PrepSlot) / 16));
+      for (int i = tid; i < prep_vecs; i += kBlock) prep_dst[i] = prep_src[i];
+    }
     __syncthreads();
     n_listed = static_cast<int>(fs.offset[p.row_wgs]);
     lists_ok = fs.overflow == 0u;
     plan = split_plan(fs.hist, rs.a_total, topp, cutoff, V, &fs.plan, sm);
     if (p.timers) t1 = wall_clock64();
     if (wave == 0) {
-      const float sum = split_chain<DT>(reinterpret_cast<const SlotRec*>(lds_keys), ns,
-                                        reinterpret_cast<const PrepSlot*>(prep_dst), n_prep, logits, V, inv, m, sm.exp2tab,
-                                        p.row.fused, p.timers ? p.timers + static_cast<int64_t>(row) * 8 : nullptr);
-      if (lane == 0) sm.bc_sum = sum;
+      if (!chained) {
+        const float sum = split_chain<DT>(reinterpret_cast<const SlotRec*>(lds_keys), ns,
+                                          reinterpret_cast<const PrepSlot*>(prep_dst), n_prep, logits, V, inv, m, sm.exp2tab,
+                                          p.row.fused, p.timers ? p.timers + static_cast<int64_t>(row) * 8 : nullptr);
+        if (lane == 0) sm.bc_sum = sum;
+      } else if (lane == 0) {
+        sm.bc_sum = fs.pre_sum[lrow - r_first];
+      }
     } else if (lists_ok && plan.b_sel >= 0 && plan.n_sel <= 64) {
       // ---- the other waves, meanwhile: one pass over the listed candidates picks out those of the
       //      largest buckets and those that may or may not reach the cutoff
@@ -1799,7 +1856,8 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
       t[4] = static_cast<uint64_t>(path) | (static_cast<uint64_t>(plan.n_sel) << 8) | (static_cast<uint64_t>(fs.band_count) << 32);
     }
   }
-  }  // rows of this workgroup
+  }  // rows of the unit
+  }  // units of this workgroup
 }
 
 }  // namespace ets
