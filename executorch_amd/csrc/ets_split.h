@@ -294,6 +294,7 @@ struct Pass2Shared {
   uint32_t hist[kHistBuckets];
   uint32_t list_count;        // candidates this workgroup has listed
   uint32_t top_mass[32];      // the slots' two largest exps, added up per binade (bin j: [2^-j, 2^(1-j))), in units of 2^-20
+  uint32_t top_all[32];       // the whole mass of the slots, by the binade of their largest exp, in units of 2^-10 (rounded up)
 };
 
 // One wave, one slot: e[] are the lane's 8 entries; `cls` is the slot's entry of Pass2Shared::cls.
@@ -510,7 +511,10 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
   if (p.timers) c0 = wall_clock64();
   if (tid < 32) sm.exp2tab[tid] = kExp2Table[tid];
   if (tid == 0) sh.list_count = 0u;
-  if (TOPP && tid < 32) sh.top_mass[tid] = 0u;
+  if (TOPP && tid < 32) {
+    sh.top_mass[tid] = 0u;
+    sh.top_all[tid] = 0u;
+  }
   // 16-bit rows: entries per bit pattern, behind the expf table
   constexpr bool kPatterns = TOPP && (DT == kDtypeBFloat16 || DT == kDtypeHalf);
   uint32_t* ph = reinterpret_cast<uint32_t*>(lut_mem + (DT == kDtypeBFloat16 ? kLutCountWords : 0));
@@ -592,6 +596,9 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
           const int j = 127 - static_cast<int>(__float_as_uint(below[q]) >> 23);
           if (below[q] > 0.0f && j >= 0 && j < 32) atomicAdd(&sh.top_mass[j], static_cast<uint32_t>(below[q] * 1048576.0f));
         }
+        // the slot's whole mass (at most 512), rounded up: what bounds how many of its entries reach a cut
+        const int j0 = 127 - static_cast<int>(__float_as_uint(below[0]) >> 23);
+        if (j0 >= 0 && j0 < 32) atomicAdd(&sh.top_all[j0], static_cast<uint32_t>(a * 1024.0f) + 1u);
       }
     }
     const float incl = wave_scan_inclusive_f32(a, lane);
@@ -660,11 +667,17 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
     const uint32_t incl = wave_scan_inclusive_u32(mine);
     const float need = topp * a_total * 1.04f * 1048576.0f;
     const uint64_t reach = __ballot(lane < 32 && static_cast<float>(incl) >= need);
+    const uint32_t incl_all = wave_scan_inclusive_u32(lane < 32 ? sh.top_all[lane] : 0u);
     if (reach != 0ull) {
       const uint32_t j = static_cast<uint32_t>(__ffsll(static_cast<long long>(reach)) - 1);  // binades 1 .. j are enough
       // buckets 0 .. 64 j hold every exp from 2^-j up (bucket 64 j starts with 2^-j itself and is listed whole)
       const float whole = __uint_as_float(0x3F800000u - ((64u * j + 1u) << 17) + 1u);
-      if (whole > cut_lo) {
+      // How many entries that can list: an entry that reaches the cut adds at least the cut to its
+      // slot's mass, and only slots whose largest exp is in binades 1 .. j + 1 hold any.  Beyond a
+      // few thousand the full lists (and, for 16-bit rows, the draw by runs) serve better.
+      const float listed_mass = static_cast<float>(readlane_u32(incl_all, j < 30u ? static_cast<int>(j) + 1 : 31)) * (1.0f / 1024.0f);
+      const bool few = listed_mass <= 4096.0f * (whole * 0.97f);
+      if (few && whole > cut_lo) {
         list_cut = whole;
         listed_buckets = 64u * j + 1u;
       }

@@ -145,7 +145,8 @@ def test_short_candidate_lists_do_not_change_tokens(oracle, dev, dtype):
     matters: few to thousands of raised entries (in distinct slots, sharing slots, sharing a lane's
     eight entries, equal to each other), raised by little (the shortcut must not apply) or by much
     (the nucleus is one entry), nuclei of more than 64 entries, a nucleus that ends among equal
-    probabilities.  Tokens and coin states of both calls must be the oracle's."""
+    probabilities, thousands of equal largest entries.  Tokens and coin states of both calls must be
+    the oracle's."""
     rng = np.random.default_rng(21)
     V = 128256 if dtype == W.DTYPE_BFLOAT16 else 70001
     rows = []
@@ -167,9 +168,15 @@ def test_short_candidate_lists_do_not_change_tokens(oracle, dev, dtype):
     x = np.full(V, -30.0, dtype=np.float32)  # almost everything negligible, 100 entries of falling size
     x[rng.choice(V, size=100, replace=False)] = np.linspace(0.0, -6.0, 100, dtype=np.float32)
     rows.append(x)
+    x = np.full(V, -20.0, dtype=np.float32)  # thousands of equal largest entries: too many to list as "the largest"
+    x[rng.choice(V, size=20000, replace=False)] = 6.0
+    rows.append(x)
+    x = rng.standard_normal(V).astype(np.float32)  # the raised entries packed into a few slots
+    x[9000:12000] += 7.0
+    rows.append(x)
     base = W.to_storage(np.stack(rows), dtype)
     B = base.shape[0]
-    for temperature, topp in ((0.6, 0.9), (1.0, 0.5), (1.0, 0.99), (0.3, 0.9), (2.0, 0.95)):
+    for temperature, topp in ((0.6, 0.9), (1.0, 0.5), (1.0, 0.99), (0.3, 0.9), (2.0, 0.95), (1.0, 0.01)):
         for seed in (5, 6, 7):
             states = (np.uint64(seed * 1000) + np.arange(B, dtype=np.uint64)).astype(np.uint64)
             after = states.copy()  # (the oracle advances the states it is given)
