@@ -313,13 +313,14 @@ const char* const kUint16Message =
 // ---- rows spread over several workgroups (ets_split.h) -------------------------------------------
 size_t round_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
-// Workgroups per row of pass 2: about one per CU over the batch, sixteen slots each at least.
+// Workgroups per row of pass 2: as many as keep the launch within one workgroup per CU (a second,
+// partly filled round would cost more than the longer sweeps), sixteen slots each at least.
 int pass2_workgroups(const ets_sampler* s, int32_t rows, int32_t ns) {
   static const int forced = [] {
     const char* e = std::getenv("ETS_SPLIT_WORKGROUPS");
     return e ? std::atoi(e) : 0;
   }();
-  int g = forced > 0 ? forced : ((s->num_cus > 0 ? s->num_cus : 256) + rows - 1) / rows;
+  int g = forced > 0 ? forced : (s->num_cus > 0 ? s->num_cus : 256) / rows;
   const int by_len = (ns + 15) / 16;
   if (g > by_len) g = by_len;
   if (g > ets::kMaxRowWorkgroups) g = ets::kMaxRowWorkgroups;
@@ -427,9 +428,15 @@ ets_status launch_split(ets_sampler* s, const ets::RowParams& p, int32_t rows, h
     return e ? std::atoi(e) : 1;
   }();
   sp.short_lists = short_lists;
-  const int per_block = (ets::kPass1Block / 64) * ets::kPass1SlotsPerWave;
-  hipLaunchKernelGGL((ets::split_pass1_kernel<DT>), dim3((sp.ns + per_block - 1) / per_block, rows), dim3(ets::kPass1Block), 0,
-                     stream, sp);
+  if (rows <= 256) {
+    const int per_block = (ets::kPass1Block / 64) * 2;
+    hipLaunchKernelGGL((ets::split_pass1_kernel<DT, 2>), dim3((sp.ns + per_block - 1) / per_block, rows), dim3(ets::kPass1Block),
+                       0, stream, sp);
+  } else {
+    const int per_block = (ets::kPass1Block / 64) * 4;
+    hipLaunchKernelGGL((ets::split_pass1_kernel<DT, 4>), dim3((sp.ns + per_block - 1) / per_block, rows), dim3(ets::kPass1Block),
+                       0, stream, sp);
+  }
   ETS_HIP(s, hipGetLastError());
   const size_t lut_bytes = (DT == ets::kDtypeBFloat16 ? sizeof(float) * ets::kLutCountWords : 0) + sizeof(uint32_t) * sp.phist_words;
   static std::atomic<size_t> set_bytes2[kMaxDevices];
@@ -547,7 +554,7 @@ size_t layout_static(const ets_sampler* s, int32_t dtype, int32_t rows, char* ba
   sp.ns_stride = static_cast<int32_t>(round_up(static_cast<size_t>(sp.ns), 4));
   sp.prep_cap = ets::kPrepCap;
   wb->max_row_wgs = 4;
-  int g = ((s->num_cus > 0 ? s->num_cus : 256) + rows - 1) / rows;
+  int g = (s->num_cus > 0 ? s->num_cus : 256) / rows;
   const int by_len = (sp.ns + 15) / 16;
   g = g > by_len ? by_len : g;
   g = g > wb->max_row_wgs ? wb->max_row_wgs : (g < 1 ? 1 : g);

@@ -24,7 +24,6 @@ namespace ets {
 
 constexpr int kSlot = 512;        // entries per slot: 64 lanes x 8 consecutive entries
 constexpr int kMaxSlots = 2048;   // rows of up to 1048576 entries take this path
-constexpr int kPass1SlotsPerWave = 4;
 constexpr int kPrepCap = 40;      // prepared slots per row (a row of the usual kind needs 10 to 20)
 
 constexpr uint32_t kSlotStable = 0u;  // even / odd hold the slot's parity summary for binade `kb`
@@ -194,10 +193,12 @@ __device__ __forceinline__ void split_range(int ns, int wgs, int x, int& s_begin
   s_end = min(ns, s_begin + per_wg);
 }
 
-// grid = (ceil(ns / 16), rows), 256 lanes: every wave takes four slots, all loads issued first.
+// grid = (ceil(ns / (4 SLOTS)), rows), 256 lanes: every wave takes SLOTS slots, all loads issued first.
 // (Small workgroups: many are resident per CU, which is what a kernel bound by HBM wants.)
 constexpr int kPass1Block = 256;
-template <int DT>
+// SLOTS: slots per wave (two when the launch is small: more, shorter waves end sooner; four when it
+// fills the chip several times over).
+template <int DT, int SLOTS>
 __global__ void __launch_bounds__(kPass1Block) split_pass1_kernel(SplitParams p) {
   const int row = p.row.row_map ? p.row.row_map[blockIdx.y] : blockIdx.y;
   const int lane = threadIdx.x & 63;
@@ -208,10 +209,10 @@ __global__ void __launch_bounds__(kPass1Block) split_pass1_kernel(SplitParams p)
   const float kInf = __uint_as_float(0x7f800000u);
   const float fill = inv < 0.0f ? kInf : -kInf;  // x = -inf: adds nothing
   const int s_end = p.ns;
-  for (int slot0 = (blockIdx.x * (kPass1Block / 64) + wave) * kPass1SlotsPerWave; slot0 < s_end; slot0 = s_end) {
-    float v[kPass1SlotsPerWave][8];
+  for (int slot0 = (blockIdx.x * (kPass1Block / 64) + wave) * SLOTS; slot0 < s_end; slot0 = s_end) {
+    float v[SLOTS][8];
 #pragma unroll
-    for (int k = 0; k < kPass1SlotsPerWave; ++k) {
+    for (int k = 0; k < SLOTS; ++k) {
       if (slot0 + k < s_end) load_slot_lane<DT>(logits, slot0 + k, lane, V, fill, v[k], p.row.fused);
     }
     // Few instructions per entry (with a workgroup per row the kernel would otherwise be bound by
@@ -223,7 +224,7 @@ __global__ void __launch_bounds__(kPass1Block) split_pass1_kernel(SplitParams p)
     float inv_u = inv;
     if (!(__builtin_fabsf(inv) < kInf)) {
 #pragma unroll
-      for (int k = 0; k < kPass1SlotsPerWave; ++k) {
+      for (int k = 0; k < SLOTS; ++k) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) v[k][e] = v[k][e] * inv;
       }
@@ -231,7 +232,7 @@ __global__ void __launch_bounds__(kPass1Block) split_pass1_kernel(SplitParams p)
     }
     const float c1 = inv_u * kLog2e;
 #pragma unroll
-    for (int k = 0; k < kPass1SlotsPerWave; ++k) {
+    for (int k = 0; k < SLOTS; ++k) {
       const int s = slot0 + k;
       if (s >= s_end) break;
       float ext = inv_u < 0.0f ? kInf : -kInf;
