@@ -1635,6 +1635,8 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
   if (p.timers) t0 = wall_clock64();
   if (tid < 32) sm.exp2tab[tid] = kExp2Table[tid];
   if (tid == 0) fs.fused = p.row.fused;  // (barriers follow before any draw function reads it)
+  uint64_t coin_state = 0ull;  // asked for now, needed once the sum is known
+  if (tid == 0) coin_state = p.row.rng[row];
 
   float S = kNaN;
   int n_listed = 0;
@@ -1736,7 +1738,7 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
 
   // ---- one coin per call (sampler.cpp:237, 210-220)
   if (tid == 0) {
-    uint64_t st = p.row.rng[row];
+    uint64_t st = coin_state;
     st ^= st >> 12;
     st ^= st << 25;
     st ^= st >> 27;
