@@ -1627,6 +1627,24 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
   const float topp = p.row.row_cfg ? p.row.row_cfg[row].topp : p.row.topp;
   const char* logits = static_cast<const char*>(p.row.logits) + static_cast<int64_t>(row) * p.row.row_stride * ElemSize<DT>::value;
   const float kNaN = __uint_as_float(0x7fc00000u);
+  // What the row's state does not decide is requested before the state is looked at (one trip to
+  // memory instead of two in a row): the lane's first slot record, its bucket of the first
+  // workgroups' histograms, the workgroups' list counts.
+  const uint4* rec_src = reinterpret_cast<const uint4*>(p.slot_rec + static_cast<int64_t>(row) * p.ns_stride);
+  const uint4* prep_src = reinterpret_cast<const uint4*>(p.prep + static_cast<int64_t>(row) * p.prep_cap);
+  uint4 early_rec = {0u, 0u, 0u, 0u};
+  uint32_t early_count = 0u;
+  const bool early = !chained;
+  if (early) {
+    if (tid < ns) early_rec = rec_src[tid];
+    if (tid < p.row_wgs) early_count = p.list_count[static_cast<int64_t>(lrow) * kMaxRowWorkgroups + tid];
+  }
+  uint32_t early_hist[4] = {0u, 0u, 0u, 0u};  // bucket `tid` of the first four workgroups' histograms
+  if (early) {
+    const uint32_t* hist_in = p.hist + static_cast<int64_t>(lrow) * p.row_wgs * kHistBuckets;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) early_hist[k] = hist_in[(k < p.row_wgs ? k : 0) * kHistBuckets + tid];
+  }
   const RowState rs = p.row_state[row];
   const float m = rs.m;
   const bool row_nan = rs.nan != 0u;
@@ -1645,7 +1663,7 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
   if (!row_nan) {
     // ---- how many candidates the workgroups of pass 2 listed; their histograms, added up
     if (tid < 64) {
-      const uint32_t c = tid < p.row_wgs ? p.list_count[static_cast<int64_t>(lrow) * kMaxRowWorkgroups + tid] : 0u;
+      const uint32_t c = tid < p.row_wgs ? (early ? early_count : p.list_count[static_cast<int64_t>(lrow) * kMaxRowWorkgroups + tid]) : 0u;
       const uint32_t incl = wave_scan_inclusive_u32(c);
       fs.count[tid] = c;
       fs.offset[tid + 1] = incl;
@@ -1671,7 +1689,11 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
           const int gk = g + k < p.row_wgs ? g + k : g;
 #pragma unroll
           for (int q = 0; q < kHistBuckets / kBlock; ++q) {
-            v[k][q] = q * kBlock + tid < n_hist ? hist_in[gk * kHistBuckets + q * kBlock + tid] : 0u;
+            if (q == 0 && early && g == 0) {
+              v[k][q] = tid < n_hist ? early_hist[k] : 0u;  // (what lies behind the listed buckets is stale)
+            } else {
+              v[k][q] = q * kBlock + tid < n_hist ? hist_in[gk * kHistBuckets + q * kBlock + tid] : 0u;
+            }
           }
         }
 #pragma unroll
@@ -1691,11 +1713,15 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
     uint4* lds_vec = reinterpret_cast<uint4*>(lds_keys);
     uint4* prep_dst = lds_vec + rec_bytes / 16;
     if (!chained) {
-      const uint4* rec_src = reinterpret_cast<const uint4*>(p.slot_rec + static_cast<int64_t>(row) * p.ns_stride);
-      for (int i = tid; i < ns; i += kBlock) lds_vec[i] = rec_src[i];
-      const uint4* prep_src = reinterpret_cast<const uint4*>(p.prep + static_cast<int64_t>(row) * p.prep_cap);
       const int prep_vecs = static_cast<int>(n_prep * (sizeof(PrepSlot) / 16));
-      for (int i = tid; i < prep_vecs; i += kBlock) prep_dst[i] = prep_src[i];
+      if (early) {
+        if (tid < ns) lds_vec[tid] = early_rec;
+        for (int i = tid + kBlock; i < ns; i += kBlock) lds_vec[i] = rec_src[i];
+        for (int i = tid; i < prep_vecs; i += kBlock) prep_dst[i] = prep_src[i];
+      } else {
+        for (int i = tid; i < ns; i += kBlock) lds_vec[i] = rec_src[i];
+        for (int i = tid; i < prep_vecs; i += kBlock) prep_dst[i] = prep_src[i];
+      }
     }
     __syncthreads();
     n_listed = static_cast<int>(fs.offset[p.row_wgs]);
