@@ -1130,10 +1130,11 @@ __device__ bool draw_topp_listed(uint64_t* list, uint64_t* lds_list, int lds_lis
         break;
       }
     }
-    // tighten between tau (enough mass) and 4 * tau (not enough): fewer keys to sort
+    // tighten between tau (enough mass) and 4 * tau (not enough): fewer keys to sort (three steps; up to
+    // eight while the selection does not fit the key buffer)
     if (tau > 0.0f && n_sel > 256) {
       float hi = tau * 4.0f;
-      for (int step = 0; step < 3; ++step) {
+      for (int step = 0; step < 8 && (step < 3 || pow2_ceil(n_sel) > cap); ++step) {
         const float mid = sqrtf(tau * hi);
         float c = 0.0f, m = 0.0f;
         for_each_prob([&](float pj) {

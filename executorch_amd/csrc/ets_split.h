@@ -1866,17 +1866,33 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
         path = 4;
       }
     }
-    if (!done && lists_ok && n_listed > 0 && n_listed <= p.row.lds_keys - kBlock) {
-      // ---- a longer nucleus: the whole list goes to LDS, selection by probability, sort, walks
+    // (a list too long for LDS is worth the passes over it only when the histogram says that the
+    // entries to sort will fit)
+    if (!done && lists_ok && n_listed > 0 && static_cast<int64_t>(n_listed) <= p.row.scratch_stride &&
+        (n_listed <= p.row.lds_keys - kBlock || (plan.b_sel >= 0 && plan.n_sel <= p.row.lds_keys))) {
+      // ---- a longer nucleus: the list goes to LDS as far as it fits and to the workgroup's scratch
+      //      row beyond that (entry j at position j of either), then selection by probability,
+      //      sort of the selected entries, walks
+      const int lds_cap = p.row.lds_keys - kBlock;
+      uint64_t* lds_list = lds_keys + kBlock;
+      uint64_t* far_list = p.row.scratch + static_cast<int64_t>(blockIdx.x) * p.row.scratch_stride;
       for (int g = wave; g < p.row_wgs; g += kWaves) {
         const uint64_t* src = p.list + (static_cast<int64_t>(lrow) * p.row_wgs + g) * p.list_region;
-        uint64_t* dst = lds_keys + kBlock + fs.offset[g];
+        const int first = static_cast<int>(fs.offset[g]);
         const int c = static_cast<int>(fs.count[g]);
-        for (int j = lane; j < c; j += 64) dst[j] = src[j];
+        for (int j = lane; j < c; j += 64) {
+          const uint64_t ent = src[j];
+          if (first + j < lds_cap) {
+            lds_list[first + j] = ent;
+          } else {
+            far_list[first + j] = ent;
+          }
+        }
       }
+      __threadfence_block();  // (the scratch row's entries are read by other lanes of the workgroup)
       __syncthreads();
-      done = draw_topp_listed(nullptr, lds_keys + kBlock, p.row.lds_keys - kBlock, kBlock, n_listed, S, cutoff, topp, coin,
-                              lds_keys, p.row.lds_keys, dbg, token, sm, short_lists);
+      done = draw_topp_listed(far_list, lds_list, lds_cap, kBlock, n_listed, S, cutoff, topp, coin, lds_keys, p.row.lds_keys, dbg,
+                              token, sm, short_lists);
       path = 2;
     }
     if (!done) {

@@ -190,3 +190,31 @@ def test_short_candidate_lists_do_not_change_tokens(oracle, dev, dtype):
                 got = s.sample_batch(to_device(base, dtype, dev), debug_out=dbg).cpu().numpy()
                 assert np.array_equal(got, want), (temperature, topp, seed, with_debug, np.nonzero(got != want)[0])
                 assert np.array_equal(s.get_rng_states(B), after)
+
+
+@pytest.mark.parametrize("dtype", [W.DTYPE_FLOAT, W.DTYPE_HALF])
+def test_candidate_lists_longer_than_lds(oracle, dev, dtype):
+    """Rows with more top-p candidates than the finish kernel's LDS holds (tens of thousands) and a
+    nucleus that still fits its sort: the list continues in the workgroup's scratch row."""
+    rng = np.random.default_rng(31)
+    V = 128256
+    B = 4
+    for scale, temperature, topp in ((2.0, 0.8, 0.5), (3.0, 1.0, 0.9), (2.0, 0.8, 0.9)):
+        x = W.to_storage((rng.standard_normal((B, V)) * scale).astype(np.float32), dtype)
+        for with_debug in (True, False):
+            states = (np.uint64(900) + np.arange(B, dtype=np.uint64)).astype(np.uint64)
+            s = ea.Sampler(V, temperature, topp, 1, max_batch=B)
+            s.set_row_split(SPLIT_ON)
+            s.set_rng_states(states)
+            dbg = torch.zeros((B, 8), dtype=torch.int32, device=dev) if with_debug else None
+            got = s.sample_batch(to_device(x, dtype, dev), debug_out=dbg).cpu().numpy()
+            want, ex = oracle.sample_rows(x, dtype, oracle.inv_temperature(temperature), topp, 0, states, mode=oracle.MODE_UPCAST,
+                                          tie=oracle.TIE_STABLE, threads=4, explain=True)
+            assert np.array_equal(got, want), (scale, temperature, topp, with_debug)
+            assert np.array_equal(s.get_rng_states(B), states)
+            if with_debug:
+                rec = ea.debug_records(dbg)
+                assert min(ex[b].n_candidates for b in range(B)) > 16384  # (the case this test is for)
+                for b in range(B):
+                    assert rec["n_candidates"][b] == ex[b].n_candidates
+                    assert rec["last_idx"][b] == ex[b].last_idx
