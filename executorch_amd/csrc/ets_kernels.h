@@ -334,7 +334,30 @@ typedef __attribute__((address_space(3))) uint64_t* LdsKeys;
 // whose partners lie inside one run (distance < W) are done by that wave alone, without workgroup
 // barriers (a fence that waits for the wave's own accesses separates them), so only the
 // log2(N / W) long-distance sub-stages of each merge pay a barrier.  Ends with a barrier.
+constexpr int kRankSort = 256;
 __device__ void sort_keys_lds(LdsKeys lds, int N) {
+  if (N <= kRankSort) {
+    // A short list: every lane counts the keys below its own (all lanes read the same key at a
+    // time, which LDS broadcasts) and stores its key at that rank.  The keys are distinct but for
+    // the padding (~0) behind the last real key, which stays where it is.
+    const int i = threadIdx.x;
+    uint64_t key = ~0ull;
+    int rank = i;
+    if (i < N) {
+      key = lds[i];
+      if (key != ~0ull) {
+        rank = 0;
+        for (int j = 0; j < N; j += 2) {
+          const uint64_t a = lds[j], b = lds[j + 1];
+          rank += (a < key ? 1 : 0) + (b < key ? 1 : 0);
+        }
+      }
+    }
+    __syncthreads();
+    if (i < N) lds[rank] = key;
+    __syncthreads();
+    return;
+  }
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   int waves = N / 128;  // at least two keys per lane of a participating wave
@@ -406,25 +429,22 @@ __device__ __forceinline__ uint32_t wave_append_slot(bool keep, uint32_t* counte
   return slot0 + static_cast<uint32_t>(__popcll(mask & ((1ull << lane) - 1ull)));
 }
 
-// The CDF walk for short lists (n <= 192; the nucleus of a peaked row is a handful of entries, and
-// a workgroup-wide scan would spend its time in barriers): the first wave loads the probabilities
-// into registers, three per lane, and adds them one by one from there.
+// The CDF walk for short lists (n <= kSmallWalk; the nucleus of a peaked row is a handful of entries,
+// and a workgroup-wide scan would spend its time in barriers): the first wave takes the
+// probabilities sixty-four at a time, one per lane, and adds them in order with the single-wave
+// scheme of the sequential sums (increments under the running sum's ulp; the lane in which the sum
+// changes binade, meets a tie or crosses the threshold adds natively).
+constexpr int kSmallWalk = 512;
 template <typename Keys>
 __device__ SeqSumResult seq_sum_small(Keys keys, int n, float threshold, BlockScratch& sm) {
   if (threadIdx.x < 64) {
     const int lane = threadIdx.x;
-    float p[3];
-#pragma unroll
-    for (int k = 0; k < 3; ++k) p[k] = (lane + 64 * k < n) ? cand_prob(keys[lane + 64 * k]) : 0.0f;
     float s = 0.0f;
     int found = -1;
-#pragma unroll
-    for (int k = 0; k < 3; ++k) {
-      const int hi = min(n - 64 * k, 64);
-      for (int i = 0; i < hi && found < 0; ++i) {
-        s = s + readlane_f32(p[k], i);
-        if (s > threshold) found = 64 * k + i;
-      }
+    for (int base = 0; base < n && found < 0; base += 64) {
+      const uint32_t bits[1] = {base + lane < n ? __float_as_uint(cand_prob(keys[base + lane])) : 0u};
+      // (a sum that is still 0 behind the first group -- every probability 0 -- starts the next one like a row)
+      wave_resolve<1>(s, found, bits, base + lane, n, threshold);
     }
     if (lane == 0) {
       sm.bc_sum = s;
@@ -436,8 +456,6 @@ __device__ SeqSumResult seq_sum_small(Keys keys, int n, float threshold, BlockSc
   __syncthreads();
   return r;
 }
-
-constexpr int kSmallWalk = 192;
 
 // The two CDF walks over candidates sorted by descending probability (sampler.cpp:150-170,
 // :103-119 for top-k).  Returns the sorted position of the draw, or -2 when `n_sorted` entries
@@ -1114,7 +1132,8 @@ __device__ bool draw_topp_listed(uint64_t* list, uint64_t* lds_list, int lds_lis
   const float target = topp * 1.004f + 1e-6f;
   float tau = 0.0f;  // select everything
   int n_sel = n0;
-  if (mass >= target && n0 > 64) {
+  // (a short list of the row's largest entries holds little but the nucleus: sorted as it is)
+  if (mass >= target && n0 > 64 && !(more_exist && n0 <= 1024)) {
     float t = (1.0f / S) * 0.25f;  // the largest probability is fl(1 / S)
     for (int step = 0; step < 24 && t > cutoff; ++step, t *= 0.25f) {
       float c = 0.0f, m = 0.0f;
