@@ -1074,10 +1074,11 @@ __device__ int draw_small_wave(LdsKeys lds, int n, int n_total, float topp, floa
 //   C. only those entries are sorted (in LDS) and the reference's two CDF walks run over them.
 // Returns false when the entries to sort do not fit in LDS or, against expectation, do not reach
 // topp (the caller takes the general path).  more_exist: the list is the row's largest entries,
-// not every candidate.
+// not every candidate.  tau_hint: a threshold the caller expects to do for B (0: none).
 __device__ bool draw_topp_listed(uint64_t* list, uint64_t* lds_list, int lds_list_cap, int list_base, int n_listed,
                                  float S, float cutoff, float topp, float coin, uint64_t* lds_keys, int cap,
-                                 RowDebug& dbg, int32_t& token, BlockScratch& sm, bool more_exist = false) {
+                                 RowDebug& dbg, int32_t& token, BlockScratch& sm, bool more_exist = false,
+                                 float tau_hint = 0.0f) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   uint32_t buf = 0u;
@@ -1133,7 +1134,23 @@ __device__ bool draw_topp_listed(uint64_t* list, uint64_t* lds_list, int lds_lis
   float tau = 0.0f;  // select everything
   int n_sel = n0;
   // (a short list of the row's largest entries holds little but the nucleus: sorted as it is)
-  if (mass >= target && n0 > 64 && !(more_exist && n0 <= 1024)) {
+  bool hinted = false;
+  if (mass >= target && n0 > 64 && !(more_exist && n0 <= 1024) && tau_hint > cutoff) {
+    // the caller knows a threshold that should do (from a histogram of the candidates): one pass to check it
+    float c = 0.0f, m = 0.0f;
+    for_each_prob([&](float pj) {
+      const bool in = pj >= tau_hint;
+      c += in ? 1.0f : 0.0f;
+      m += in ? pj : 0.0f;
+    });
+    block_sum2(c, m, sm, buf);
+    if (m >= target) {
+      tau = tau_hint;
+      n_sel = static_cast<int>(c);
+      hinted = true;
+    }
+  }
+  if (!hinted && mass >= target && n0 > 64 && !(more_exist && n0 <= 1024)) {
     float t = (1.0f / S) * 0.25f;  // the largest probability is fl(1 / S)
     for (int step = 0; step < 24 && t > cutoff; ++step, t *= 0.25f) {
       float c = 0.0f, m = 0.0f;

@@ -1891,8 +1891,10 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
       }
       __threadfence_block();  // (the scratch row's entries are read by other lanes of the workgroup)
       __syncthreads();
+      // (the buckets the plan selected carry more than topp: the probability of their lower edge is the threshold to try)
+      const float tau_hint = plan.b_sel >= 0 ? div_row(hist_edge(plan.b_sel + 1), div) : 0.0f;
       done = draw_topp_listed(far_list, lds_list, lds_cap, kBlock, n_listed, S, cutoff, topp, coin, lds_keys, p.row.lds_keys, dbg,
-                              token, sm, short_lists);
+                              token, sm, short_lists, tau_hint);
       path = 2;
     }
     if (!done) {
