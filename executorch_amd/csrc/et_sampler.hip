@@ -396,8 +396,10 @@ ets_status ensure_phist(ets_sampler* s) {
 }
 
 // Whether a launch of `rows` rows with draw `draw` takes the three-launch path.
-bool use_split(const ets_sampler* s, const void* d_logits, int64_t stride, int32_t dtype, int draw) {
-  if (s->split_mode == ETS_ROW_SPLIT_OFF || draw != ets::kDrawTopP) return false;
+// (Top-p rows, and top-k rows whose k the slots' largest entries can vouch for: two per slot.)
+bool use_split(const ets_sampler* s, const void* d_logits, int64_t stride, int32_t dtype, int draw, int32_t topk) {
+  if (s->split_mode == ETS_ROW_SPLIT_OFF || draw == ets::kDrawMultinomial) return false;
+  if (draw == ets::kDrawTopK && topk > (s->vocab + ets::kSlot - 1) / ets::kSlot) return false;
   const size_t esz = dtype_size(dtype);
   const bool aligned = (reinterpret_cast<uintptr_t>(d_logits) % 16 == 0) && ((static_cast<size_t>(stride) * esz) % 16 == 0);
   if (!aligned || (s->vocab + ets::kSlot - 1) / ets::kSlot > ets::kMaxSlots) return false;
@@ -469,18 +471,21 @@ ets_status launch_split(ets_sampler* s, const ets::RowParams& p, int32_t rows, h
   return ETS_OK;
 }
 
+// The three launches for rows that use_split() accepted (each row's draw follows from its parameters).
+ets_status launch_split_any(ets_sampler* s, const ets::RowParams& p, int32_t dtype, int32_t rows, hipStream_t stream) {
+  switch (dtype) {
+    case ETS_DTYPE_FLOAT:
+      return launch_split<ets::kDtypeFloat>(s, p, rows, stream);
+    case ETS_DTYPE_HALF:
+      return launch_split<ets::kDtypeHalf>(s, p, rows, stream);
+    default:
+      return launch_split<ets::kDtypeBFloat16>(s, p, rows, stream);
+  }
+}
+
 ets_status rows_device(ets_sampler* s, const ets::RowParams& p, int32_t dtype, int32_t rows, hipStream_t stream,
                        int draw) {
-  if (use_split(s, p.logits, p.row_stride, dtype, draw)) {
-    switch (dtype) {
-      case ETS_DTYPE_FLOAT:
-        return launch_split<ets::kDtypeFloat>(s, p, rows, stream);
-      case ETS_DTYPE_HALF:
-        return launch_split<ets::kDtypeHalf>(s, p, rows, stream);
-      default:
-        return launch_split<ets::kDtypeBFloat16>(s, p, rows, stream);
-    }
-  }
+  if (draw != ets::kDrawAny && use_split(s, p.logits, p.row_stride, dtype, draw, p.topk)) return launch_split_any(s, p, dtype, rows, stream);
   switch (dtype) {
     case ETS_DTYPE_FLOAT:
       return launch_rows<ets::kDtypeFloat>(s, p, rows, stream, draw);
@@ -656,7 +661,6 @@ ets_status sample_device_configs(ets_sampler* s, const void* d_logits, int32_t d
   // from its parameters).  maps[g * batch + i]: the i-th row of group g.
   enum { kGreedy = 0, kSplit = 1, kRows = 2 };
   int32_t count[3] = {0, 0, 0};
-  const bool split_ok = use_split(s, d_logits, stride, dtype, ets::kDrawTopP);
   bool any_reseed = false;
   for (int32_t b = 0; b < batch; ++b) {
     const ets_sampling_config& c = configs[b];
@@ -668,7 +672,7 @@ ets_status sample_device_configs(ets_sampler* s, const void* d_logits, int32_t d
     h_reseed[b] = c.seed;
     any_reseed = any_reseed || c.seed != 0;
     int group = kGreedy;
-    if (inv != 0.0f) group = (split_ok && draw_mode(s->vocab, c.top_p, c.top_k) == ets::kDrawTopP) ? kSplit : kRows;
+    if (inv != 0.0f) group = use_split(s, d_logits, stride, dtype, draw_mode(s->vocab, c.top_p, c.top_k), c.top_k) ? kSplit : kRows;
     if (group != kGreedy && dtype == ETS_DTYPE_UINT16) return fail(s, ETS_NOT_SUPPORTED, kUint16Message);
     h_maps[group * batch + count[group]++] = b;
   }
@@ -730,7 +734,7 @@ ets_status sample_device_configs(ets_sampler* s, const void* d_logits, int32_t d
     p.scratch = s->d_scratch + (both_draw ? static_cast<int64_t>(share) * s->scratch_stride : 0);
     p.grid_cap = share;
     p.row_map = d_maps + kSplit * batch;
-    st = rows_device(s, p, dtype, count[kSplit], side, ets::kDrawTopP);
+    st = launch_split_any(s, p, dtype, count[kSplit], side);
     if (st != ETS_OK) return st;
   }
   if (count[kGreedy] > 0) {

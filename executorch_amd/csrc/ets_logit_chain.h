@@ -380,8 +380,8 @@ ets_status ets_sampler_sample_batch_chain(ets_sampler* s, ets_logit_chain* c, vo
   const int32_t n_ops = static_cast<int32_t>(c->ops.size());
   ets::FusedOps fused = {};
   int32_t n_front = n_ops;
-  const bool can_fuse = s->inv_temperature != 0.0f && !s->wb &&
-                        use_split(s, d_logits, row_stride_elems, dtype, draw_mode(s->vocab, s->topp, s->topk));
+  const bool can_fuse = s->inv_temperature != 0.0f && !s->wb && draw_mode(s->vocab, s->topp, s->topk) == ets::kDrawTopP &&
+                        use_split(s, d_logits, row_stride_elems, dtype, ets::kDrawTopP, 0);
   if (can_fuse) {
     while (n_front > 0 && fused.n < ets::kMaxFusedOps &&
            (c->ops[n_front - 1].kind == ets::kOpBias || c->ops[n_front - 1].kind == ets::kOpScale))

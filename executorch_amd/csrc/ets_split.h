@@ -65,8 +65,10 @@ struct RowState {
   int32_t n_bins;       //   how many bins it has (0: no pattern histogram)
   int32_t mag_min;      //   and the KeyMap's first magnitude with a key of its own
   uint32_t listed_buckets;  // 0: every possible candidate is listed; else only those of the histogram's
-                            //   first `listed_buckets` buckets (which carry more than topp of the mass)
+                            //   first `listed_buckets` buckets (which carry more than topp of the mass, or,
+                            //   for a top-k row, hold at least topk entries); kNoLists: nothing usable is listed
 };
+constexpr uint32_t kNoLists = 0xffffffffu;
 
 constexpr int kMaxRowWorkgroups = 64;  // workgroups of pass 2 per row
 constexpr int kListRegion = 16384;     // candidates one workgroup of pass 2 can list
@@ -502,6 +504,8 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
   const int ns = p.ns;
   const float inv = p.row.row_cfg ? p.row.row_cfg[row].inv_temperature : p.row.inv_temperature;
   const float topp = p.row.row_cfg ? p.row.row_cfg[row].topp : p.row.topp;
+  const int32_t topk = p.row.row_cfg ? p.row.row_cfg[row].topk : p.row.topk;
+  const bool row_topk = topk > 0 && topk < p.row.vocab;  // sampler.cpp:239: top-k comes before top-p
   const char* logits = static_cast<const char*>(p.row.logits) + static_cast<int64_t>(row) * p.row.row_stride * ElemSize<DT>::value;
   const float* slot_max = p.slot_max + static_cast<int64_t>(row) * p.ns_stride;
   const float* slot_sum = p.slot_sum + static_cast<int64_t>(row) * p.ns_stride;
@@ -596,6 +600,8 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
         for (int q = 0; q < 2; ++q) {
           const int j = 127 - static_cast<int>(__float_as_uint(below[q]) >> 23);
           if (below[q] > 0.0f && j >= 0 && j < 32) atomicAdd(&sh.top_mass[j], static_cast<uint32_t>(below[q] * 1048576.0f));
+          // a top-k row counts them by histogram bucket (the histogram is not in use yet)
+          if (row_topk && below[q] > 0.0f) atomicAdd(&sh.hist[hist_bucket(__float_as_uint(below[q]))], 1u);
         }
         // the slot's whole mass (at most 512), rounded up: what bounds how many of its entries reach a cut
         const int j0 = 127 - static_cast<int>(__float_as_uint(below[0]) >> 23);
@@ -663,7 +669,35 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
   //      asks for debug records lists everything.
   float list_cut = cut_lo;
   uint32_t listed_buckets = 0u;
-  if (TOPP && p.short_lists != 0 && p.row.debug == nullptr) {
+  if (TOPP && row_topk) {
+    // ---- a top-k row (sampler.cpp:72-120): the k largest entries are among those of the histogram
+    //      buckets in which the slots' two largest exps first number k (lower bounds of the exps of
+    //      distinct entries: at least k entries lie in those buckets), so those buckets are listed, whole.
+    //      (How many more entries they hold is not known here: the finish kernel sorts the row when
+    //      they do not fit its LDS.)  Fewer than k such exps above the last bucket: nothing is listed.
+    static_assert(kHistBuckets == 2 * kBlock, "two buckets per lane");
+    const uint32_t c0 = sh.hist[2 * tid], c1 = sh.hist[2 * tid + 1];
+    const uint32_t incl_c = wave_scan_inclusive_u32(c0 + c1);
+    if (lane == 63) sm.red_u[wave] = incl_c;
+    if (tid == 0) sm.flag = -1;
+    __syncthreads();
+    uint32_t upto = incl_c;
+    for (int w = 0; w < wave; ++w) upto += sm.red_u[w];
+    const uint32_t before = upto - (c0 + c1);
+    const uint32_t k = static_cast<uint32_t>(topk);
+    if (upto >= k && before < k) sm.flag = before + c0 >= k ? 2 * tid : 2 * tid + 1;  // (one lane)
+    __syncthreads();
+    const int b_k = sm.flag;
+    sh.hist[2 * tid] = 0u;  // (the sweep counts the listed candidates here)
+    sh.hist[2 * tid + 1] = 0u;
+    __syncthreads();
+    list_cut = kInf;
+    listed_buckets = kNoLists;
+    if (b_k >= 0 && b_k < kHistBuckets - 1) {
+      list_cut = __uint_as_float(0x3F800000u - (static_cast<uint32_t>(b_k + 1) << 17) + 1u);
+      listed_buckets = static_cast<uint32_t>(b_k) + 1u;
+    }
+  } else if (TOPP && p.short_lists != 0 && p.row.debug == nullptr) {
     const uint32_t mine = lane < 32 ? sh.top_mass[lane] : 0u;
     const uint32_t incl = wave_scan_inclusive_u32(mine);
     const float need = topp * a_total * 1.04f * 1048576.0f;
@@ -690,7 +724,7 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
   //      same two numbers).  Too many bins for the LDS set aside: no pattern histogram.
   KeyMap km = {0, 0, 0};
   // (short lists are drawn from directly: no pattern histogram then)
-  if (kPatterns && listed_buckets == 0u && p.phist_words > 0 && inv > 0.0f && inv < kInf && cut_lo > 0.0f &&
+  if (kPatterns && !row_topk && listed_buckets == 0u && p.phist_words > 0 && inv > 0.0f && inv < kInf && cut_lo > 0.0f &&
       (__float_as_uint(inv) >> 23) != 0u) {
     // magnitudes below 2^(em - ei - 27) vanish against m (em, ei: biased exponents of |m| and inv)
     const uint32_t mb = __float_as_uint(__builtin_fabsf(m));
@@ -757,7 +791,7 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
     if (tid == 0) p.list_count[static_cast<int64_t>(lrow) * kMaxRowWorkgroups + blockIdx.x] = sh.list_count;
     uint32_t* hist_out = p.hist + (static_cast<int64_t>(lrow) * p.row_wgs + blockIdx.x) * kHistBuckets;
     // (short lists: the buckets behind the listed ones are empty, and the finish kernel does not read them)
-    const int n_hist = listed_buckets != 0u ? static_cast<int>(listed_buckets) : kHistBuckets;
+    const int n_hist = listed_buckets == kNoLists ? 0 : (listed_buckets != 0u ? static_cast<int>(listed_buckets) : kHistBuckets);
     for (int b = tid; b < n_hist; b += kBlock) hist_out[b] = sh.hist[b];
     if (kPatterns && km.n_bins > 0) {
       uint32_t* ph_out = p.phist + (static_cast<int64_t>(lrow) * p.row_wgs + blockIdx.x) * p.phist_words;
@@ -1678,7 +1712,7 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
     {
       // (four workgroups' counts are requested at a time: a loop of one load each would wait for each)
       const uint32_t* hist_in = p.hist + static_cast<int64_t>(lrow) * p.row_wgs * kHistBuckets;
-      const int n_hist = rs.listed_buckets != 0u ? static_cast<int>(rs.listed_buckets) : kHistBuckets;  // (the rest was not written)
+      const int n_hist = rs.listed_buckets == kNoLists ? 0 : (rs.listed_buckets != 0u ? static_cast<int>(rs.listed_buckets) : kHistBuckets);  // (the rest was not written)
       uint32_t c[kHistBuckets / kBlock];
 #pragma unroll
       for (int q = 0; q < kHistBuckets / kBlock; ++q) c[q] = 0u;
@@ -1803,7 +1837,35 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
   }
   __syncthreads();
   int path = 0;
-  if (!row_nan) {
+  const int32_t topk = p.row.row_cfg ? p.row.row_cfg[row].topk : p.row.topk;
+  if (topk > 0 && topk < V) {
+    // ---- a top-k row (sampler.cpp:72-120, before top-p: :239): pass 2 listed the entries of the
+    //      histogram's first buckets, at least topk of them; they are sorted and the first topk walked.
+    //      Every probability NaN: every entry ties, the first topk in index order, the last of them drawn.
+    path = 6;
+    if (row_nan) {
+      token = topk - 1;
+    } else {
+      bool done = false;
+      const uint32_t lb = rs.listed_buckets;
+      if (lb != 0u && lb != kNoLists && lists_ok && n_listed >= topk && n_listed <= p.row.lds_keys - kBlock) {
+        for (int g = wave; g < p.row_wgs; g += kWaves) {
+          const uint64_t* src = p.list + (static_cast<int64_t>(lrow) * p.row_wgs + g) * p.list_region;
+          uint64_t* dst = lds_keys + kBlock + fs.offset[g];
+          const int c = static_cast<int>(fs.count[g]);
+          for (int j = lane; j < c; j += 64) dst[j] = src[j];
+        }
+        __syncthreads();
+        const float list_floor = __uint_as_float(0x3F800000u - (lb << 17) + 1u);  // what is not listed is below this
+        done = draw_topk_listed(lds_keys, p.row.lds_keys, kBlock, n_listed, S, list_floor, topk, topp, coin, V, dbg, token, sm);
+      }
+      if (!done) {
+        uint64_t* scratch = p.row.scratch + static_cast<int64_t>(blockIdx.x) * p.row.scratch_stride;
+        token = draw_general<DT>(logits, V, inv, m, S, true, topk, topp, 0.0f, coin, scratch, p.row.scratch_stride, lds_keys,
+                                 p.row.lds_keys, dbg, sm, p.row.fused.n > 0 ? &fs.fused : nullptr);
+      }
+    }
+  } else if (!row_nan) {
     bool done = false;
     const RowDivisor div = row_divisor(S);
     // Short lists (RowState::listed_buckets): the lists hold every entry of the histogram's first

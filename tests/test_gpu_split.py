@@ -218,3 +218,59 @@ def test_candidate_lists_longer_than_lds(oracle, dev, dtype):
                 for b in range(B):
                     assert rec["n_candidates"][b] == ex[b].n_candidates
                     assert rec["last_idx"][b] == ex[b].last_idx
+
+
+def topk_rows(kind, rows, V, rng):
+    if kind == "normal":
+        return rng.standard_normal((rows, V)).astype(np.float32)
+    if kind == "peaked":
+        x = rng.standard_normal((rows, V)).astype(np.float32)
+        for b in range(rows):
+            x[b, rng.choice(V, 20, replace=False)] += 8.0
+        return x
+    if kind == "few":  # a dozen distinct values: every bucket of the largest holds thousands of ties
+        return rng.integers(0, 12, (rows, V)).astype(np.float32) * 0.5
+    if kind == "flat":
+        return (rng.standard_normal((rows, V)) * 0.1).astype(np.float32)
+    if kind == "one":  # one entry carries the whole mass; the k-1 others are ties far below it
+        x = np.full((rows, V), -30.0, dtype=np.float32)
+        x[np.arange(rows), rng.integers(0, V, rows)] = 10.0
+        return x
+    assert kind == "masked"  # fewer finite entries than k in some rows, one NaN row
+    x = np.full((rows, V), -np.inf, dtype=np.float32)
+    for b in range(rows):
+        n = (3, 39, 40, 41, 500, 5000)[b % 6]
+        x[b, rng.choice(V, n, replace=False)] = rng.standard_normal(n).astype(np.float32) * 2.0
+    x[rows - 1, 77] = np.nan
+    return x
+
+
+@pytest.mark.parametrize("dtype", [W.DTYPE_BFLOAT16, W.DTYPE_FLOAT, W.DTYPE_HALF])
+@pytest.mark.parametrize("kind", ["normal", "peaked", "few", "flat", "one", "masked"])
+def test_topk_rows_when_split(oracle, dev, dtype, kind):
+    """Top-k rows (sampler.cpp:72-120) over several workgroups: the histogram buckets in which the
+    slots' two largest exps first number k are listed and the finish kernel keeps the k largest of
+    them.  Against the oracle (tokens, coin states) and against the one-workgroup kernel (debug
+    records as well), for k = 1, 40, 200, the largest k that takes this path and one above it."""
+    V, rows = 128256, 12
+    rng = np.random.default_rng(17)
+    x = W.to_storage(topk_rows(kind, rows, V, rng), dtype)
+    dx = to_device(x, dtype, dev)
+    inv = oracle.inv_temperature(0.8)
+    for k in (1, 40, 200, 251, 252):
+        res = []
+        for mode in (SPLIT_ON, SPLIT_OFF):
+            s = ea.Sampler(V, 0.8, 0.9, 23, max_batch=rows)
+            s.set_topk(k)
+            s.set_row_split(mode)
+            plain = s.sample_batch(dx).cpu().numpy()
+            dbg = torch.zeros((rows, 8), dtype=torch.int32, device=dev)
+            tok = s.sample_batch(dx, debug_out=dbg).cpu().numpy()
+            res.append((tok, ea.debug_records(dbg).copy(), s.get_rng_states(rows), plain))
+        assert_same(res[0], res[1])
+        assert np.array_equal(res[0][3], res[1][3]), k
+        states = (np.uint64(23) + np.arange(rows, dtype=np.uint64)).astype(np.uint64)
+        for step in (3, 0):
+            want, _ = oracle.sample_rows(x, dtype, inv, 0.9, k, states, mode=oracle.MODE_UPCAST, tie=oracle.TIE_STABLE, threads=8)
+            assert np.array_equal(res[0][step], want), (k, step)
+        assert np.array_equal(res[0][2], states), k
