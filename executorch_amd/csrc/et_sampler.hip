@@ -363,6 +363,7 @@ ets_status ensure_split(ets_sampler* s) {
   const size_t o_rec = take(rows * sp.ns_stride * sizeof(ets::SlotRec));
   const size_t o_prep = take(rows * sp.prep_cap * sizeof(ets::PrepSlot));
   const size_t o_state = take(rows * sizeof(ets::RowState));
+  const size_t o_walk = take(rows * sizeof(float2));
   const size_t o_count = take(rows * ets::kMaxRowWorkgroups * sizeof(uint32_t));
   const size_t o_timers = take(rows * 12 * sizeof(uint64_t));
   const size_t o_hist = take(row_wgs * ets::kHistBuckets * sizeof(uint32_t));
@@ -375,6 +376,7 @@ ets_status ensure_split(ets_sampler* s) {
   sp.slot_rec = reinterpret_cast<ets::SlotRec*>(base + o_rec);
   sp.prep = reinterpret_cast<ets::PrepSlot*>(base + o_prep);
   sp.row_state = reinterpret_cast<ets::RowState*>(base + o_state);
+  sp.walk = reinterpret_cast<float2*>(base + o_walk);
   sp.list_count = reinterpret_cast<uint32_t*>(base + o_count);
   sp.hist = reinterpret_cast<uint32_t*>(base + o_hist);
   sp.list = reinterpret_cast<uint64_t*>(base + o_list);
@@ -395,10 +397,13 @@ ets_status ensure_phist(ets_sampler* s) {
   return ETS_OK;
 }
 
-// Whether a launch of `rows` rows with draw `draw` takes the three-launch path.
-// (Top-p rows, and top-k rows whose k the slots' largest entries can vouch for: two per slot.)
-bool use_split(const ets_sampler* s, const void* d_logits, int64_t stride, int32_t dtype, int draw, int32_t topk) {
-  if (s->split_mode == ETS_ROW_SPLIT_OFF || draw == ets::kDrawMultinomial) return false;
+// Whether rows with draw `draw` take the path that spreads a row over several workgroups.
+// (Top-p rows; top-k rows whose k the slots' largest entries can vouch for, two per slot; multinomial
+// rows, by five launches instead of three, unless the caller wants the probabilities written.)
+bool use_split(const ets_sampler* s, const void* d_logits, int64_t stride, int32_t dtype, int draw, int32_t topk,
+               bool probs = false) {
+  if (s->split_mode == ETS_ROW_SPLIT_OFF) return false;
+  if (draw == ets::kDrawMultinomial && probs) return false;
   if (draw == ets::kDrawTopK && topk > (s->vocab + ets::kSlot - 1) / ets::kSlot) return false;
   const size_t esz = dtype_size(dtype);
   const bool aligned = (reinterpret_cast<uintptr_t>(d_logits) % 16 == 0) && ((static_cast<size_t>(stride) * esz) % 16 == 0);
@@ -471,6 +476,65 @@ ets_status launch_split(ets_sampler* s, const ets::RowParams& p, int32_t rows, h
   return ETS_OK;
 }
 
+// Multinomial rows that use_split() accepted: five launches (ets_split.h, split_walk_kernel).
+template <int DT>
+ets_status launch_split_walk(ets_sampler* s, const ets::RowParams& p, int32_t rows, hipStream_t stream) {
+  ets_status st = ETS_OK;
+  if (!s->wb) {
+    st = ensure_split(s);
+    if (st != ETS_OK) return st;
+  }
+  ets::SplitParams sp = s->wb ? s->wb->split : s->split;
+  sp.row = p;
+  sp.row.rows = rows;
+  sp.phist_words = 0;
+  sp.short_lists = 0;
+  sp.row_wgs = pass2_workgroups(s, rows, sp.ns);
+  sp.list_region = 0;
+  if (rows <= 256) {
+    const int per_block = (ets::kPass1Block / 64) * 2;
+    hipLaunchKernelGGL((ets::split_pass1_kernel<DT, 2>), dim3((sp.ns + per_block - 1) / per_block, rows), dim3(ets::kPass1Block),
+                       0, stream, sp);
+  } else {
+    const int per_block = (ets::kPass1Block / 64) * 4;
+    hipLaunchKernelGGL((ets::split_pass1_kernel<DT, 4>), dim3((sp.ns + per_block - 1) / per_block, rows), dim3(ets::kPass1Block),
+                       0, stream, sp);
+  }
+  ETS_HIP(s, hipGetLastError());
+  const size_t lut_bytes = DT == ets::kDtypeBFloat16 ? sizeof(float) * ets::kLutCountWords : 0;
+  // the walk kernel's LDS: the row's records and as many prepared slots as fit beside them
+  const uint32_t walk_lds = static_cast<uint32_t>(round_up(static_cast<size_t>(sp.ns) * sizeof(ets::SlotRec), 16) + 16 * sizeof(ets::PrepSlot));
+  static std::atomic<size_t> set_sum[kMaxDevices], set_walk[kMaxDevices], set_k0[kMaxDevices], set_k1[kMaxDevices];
+  st = allow_dynamic_lds(s, reinterpret_cast<const void*>(&ets::split_pass2_kernel<DT, false, false>), lut_bytes, set_sum);
+  if (st != ETS_OK) return st;
+  st = allow_dynamic_lds(s, reinterpret_cast<const void*>(&ets::split_pass2_kernel<DT, false, true>), lut_bytes, set_walk);
+  if (st != ETS_OK) return st;
+  st = allow_dynamic_lds(s, reinterpret_cast<const void*>(&ets::split_walk_kernel<DT, 0>), walk_lds, set_k0);
+  if (st != ETS_OK) return st;
+  st = allow_dynamic_lds(s, reinterpret_cast<const void*>(&ets::split_walk_kernel<DT, 1>), walk_lds, set_k1);
+  if (st != ETS_OK) return st;
+  hipLaunchKernelGGL((ets::split_pass2_kernel<DT, false, false>), dim3(sp.row_wgs, rows), dim3(ets::kBlock), lut_bytes, stream, sp);
+  ETS_HIP(s, hipGetLastError());
+  hipLaunchKernelGGL((ets::split_walk_kernel<DT, 0>), dim3(rows), dim3(ets::kWalkBlock), walk_lds, stream, sp, walk_lds);
+  ETS_HIP(s, hipGetLastError());
+  hipLaunchKernelGGL((ets::split_pass2_kernel<DT, false, true>), dim3(sp.row_wgs, rows), dim3(ets::kBlock), lut_bytes, stream, sp);
+  ETS_HIP(s, hipGetLastError());
+  hipLaunchKernelGGL((ets::split_walk_kernel<DT, 1>), dim3(rows), dim3(ets::kWalkBlock), walk_lds, stream, sp, walk_lds);
+  ETS_HIP(s, hipGetLastError());
+  return ETS_OK;
+}
+
+ets_status launch_split_walk_any(ets_sampler* s, const ets::RowParams& p, int32_t dtype, int32_t rows, hipStream_t stream) {
+  switch (dtype) {
+    case ETS_DTYPE_FLOAT:
+      return launch_split_walk<ets::kDtypeFloat>(s, p, rows, stream);
+    case ETS_DTYPE_HALF:
+      return launch_split_walk<ets::kDtypeHalf>(s, p, rows, stream);
+    default:
+      return launch_split_walk<ets::kDtypeBFloat16>(s, p, rows, stream);
+  }
+}
+
 // The three launches for rows that use_split() accepted (each row's draw follows from its parameters).
 ets_status launch_split_any(ets_sampler* s, const ets::RowParams& p, int32_t dtype, int32_t rows, hipStream_t stream) {
   switch (dtype) {
@@ -485,7 +549,10 @@ ets_status launch_split_any(ets_sampler* s, const ets::RowParams& p, int32_t dty
 
 ets_status rows_device(ets_sampler* s, const ets::RowParams& p, int32_t dtype, int32_t rows, hipStream_t stream,
                        int draw) {
-  if (draw != ets::kDrawAny && use_split(s, p.logits, p.row_stride, dtype, draw, p.topk)) return launch_split_any(s, p, dtype, rows, stream);
+  if (draw != ets::kDrawAny && use_split(s, p.logits, p.row_stride, dtype, draw, p.topk, p.probs != nullptr)) {
+    if (draw == ets::kDrawMultinomial) return launch_split_walk_any(s, p, dtype, rows, stream);
+    return launch_split_any(s, p, dtype, rows, stream);
+  }
   switch (dtype) {
     case ETS_DTYPE_FLOAT:
       return launch_rows<ets::kDtypeFloat>(s, p, rows, stream, draw);
@@ -578,6 +645,7 @@ size_t layout_static(const ets_sampler* s, int32_t dtype, int32_t rows, char* ba
   sp.slot_rec = reinterpret_cast<ets::SlotRec*>(take(r * sp.ns_stride * sizeof(ets::SlotRec)));
   sp.prep = reinterpret_cast<ets::PrepSlot*>(take(r * sp.prep_cap * sizeof(ets::PrepSlot)));
   sp.row_state = reinterpret_cast<ets::RowState*>(take(r * sizeof(ets::RowState)));
+  sp.walk = reinterpret_cast<float2*>(take(r * sizeof(float2)));
   sp.list_count = reinterpret_cast<uint32_t*>(take(r * ets::kMaxRowWorkgroups * sizeof(uint32_t)));
   sp.hist = reinterpret_cast<uint32_t*>(take(r * g * ets::kHistBuckets * sizeof(uint32_t)));
   sp.phist = reinterpret_cast<uint32_t*>(take(r * g * phist_words * sizeof(uint32_t)));
@@ -656,11 +724,12 @@ ets_status sample_device_configs(ets_sampler* s, const void* d_logits, int32_t d
   uint64_t* h_reseed = reinterpret_cast<uint64_t*>(h + lay.reseed);
   ets::RowConfig* h_cfg = reinterpret_cast<ets::RowConfig*>(h + lay.cfg);
   int32_t* h_maps = reinterpret_cast<int32_t*>(h + lay.maps);
-  // Three groups of rows: arg-max rows, top-p rows that take the three-launch path, and every other
-  // row that draws (one launch of the one-workgroup-per-row kernel, which picks each row's draw
-  // from its parameters).  maps[g * batch + i]: the i-th row of group g.
-  enum { kGreedy = 0, kSplit = 1, kRows = 2 };
-  int32_t count[3] = {0, 0, 0};
+  // Four groups of rows: arg-max rows, top-p and top-k rows that take the three-launch path,
+  // multinomial rows that take the five-launch path, and every other row that draws (one launch of
+  // the one-workgroup-per-row kernel, which picks each row's draw from its parameters).
+  // maps[g * batch + i]: the i-th row of group g.
+  enum { kGreedy = 0, kSplit = 1, kRows = 2, kWalk = 3 };
+  int32_t count[4] = {0, 0, 0, 0};
   bool any_reseed = false;
   for (int32_t b = 0; b < batch; ++b) {
     const ets_sampling_config& c = configs[b];
@@ -672,11 +741,14 @@ ets_status sample_device_configs(ets_sampler* s, const void* d_logits, int32_t d
     h_reseed[b] = c.seed;
     any_reseed = any_reseed || c.seed != 0;
     int group = kGreedy;
-    if (inv != 0.0f) group = use_split(s, d_logits, stride, dtype, draw_mode(s->vocab, c.top_p, c.top_k), c.top_k) ? kSplit : kRows;
+    if (inv != 0.0f) {
+      const int draw = draw_mode(s->vocab, c.top_p, c.top_k);
+      group = !use_split(s, d_logits, stride, dtype, draw, c.top_k) ? kRows : (draw == ets::kDrawMultinomial ? kWalk : kSplit);
+    }
     if (group != kGreedy && dtype == ETS_DTYPE_UINT16) return fail(s, ETS_NOT_SUPPORTED, kUint16Message);
     h_maps[group * batch + count[group]++] = b;
   }
-  if (count[kSplit] + count[kRows] > 0) {
+  if (count[kSplit] + count[kRows] + count[kWalk] > 0) {
     st = ensure_scratch(s);
     if (st != ETS_OK) return st;
   }
@@ -706,11 +778,11 @@ ets_status sample_device_configs(ets_sampler* s, const void* d_logits, int32_t d
   p.lds_keys = s->lds_keys;
   p.row_cfg = reinterpret_cast<const ets::RowConfig*>(d + lay.cfg);
   // The groups touch different rows and different work buffers.  The one-workgroup-per-row launch
-  // is the longest and runs on the caller's stream; when there is one, the other groups run
-  // beside it on a second stream, between a fork and a join (one of each: they cost more on the
+  // and the multinomial rows' five launches are the longest and run on the caller's stream; when
+  // there are any, the other groups run beside them on a second stream, between a fork and a join (one of each: they cost more on the
   // host than the kernels they order).  The two launches that draw share the scratch rows (a
   // workgroup owns the scratch row of its index in its launch).
-  const bool fork = count[kRows] > 0 && count[kSplit] + count[kGreedy] > 0;
+  const bool fork = count[kRows] + count[kWalk] > 0 && count[kSplit] + count[kGreedy] > 0;
   hipStream_t side = stream;
   if (fork) {
     st = ensure_aux_streams(s);
@@ -728,6 +800,11 @@ ets_status sample_device_configs(ets_sampler* s, const void* d_logits, int32_t d
     p.grid_cap = share;
     p.row_map = d_maps + kRows * batch;
     st = rows_device(s, p, dtype, count[kRows], stream, ets::kDrawAny);
+    if (st != ETS_OK) return st;
+  }
+  if (count[kWalk] > 0) {  // (no scratch rows, no tickets)
+    p.row_map = d_maps + kWalk * batch;
+    st = launch_split_walk_any(s, p, dtype, count[kWalk], stream);
     if (st != ETS_OK) return st;
   }
   if (count[kSplit] > 0) {

@@ -137,6 +137,7 @@ struct SplitParams {
   uint32_t* phist;      // [rows, row_wgs, phist_words] 16-bit rows: entries per bit pattern, two 16-bit
                         //   counters per word, from order key RowState::key_cut upwards
   int32_t phist_words;  // words per (row, workgroup) region; 0 disables the pattern histogram
+  float2* walk;         // [rows] multinomial rows: the exact softmax sum and the coin, between the two chains
   uint64_t* timers;     // phase clocks (profiling), or null
   int32_t list_region;  // entries per region
   int32_t short_lists;  // 1: pass 2 may list only the largest candidates of a peaked row (see RowState::listed_buckets)
@@ -490,7 +491,9 @@ __device__ __forceinline__ void split_fold_slot(const SplitParams& p, int row, i
 #ifndef ETS_PASS2_WAVES_PER_EU
 #define ETS_PASS2_WAVES_PER_EU 4
 #endif
-template <int DT, bool TOPP>
+// WALK: the second sum of a multinomial row (sampler.cpp:58-70): the entries are p = fl(e / S) with the exact
+// softmax sum S that the first chain left in SplitParams::walk, and the records describe their running sum.
+template <int DT, bool TOPP, bool WALK = false>
 __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_kernel(SplitParams p) {
   extern __shared__ __align__(16) float lut_mem[];
   __shared__ Pass2Shared sh;
@@ -574,6 +577,13 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
   }
   __syncthreads();
   if (p.timers) c1 = wall_clock64();
+  RowDivisor walk_div = {};
+  float walk_scale = 1.0f;
+  if (WALK) {
+    const float S = p.walk[row].x;
+    walk_div = row_divisor(S);
+    walk_scale = 1.0f / S;  // (the approximate sums only place the running sum in a binade)
+  }
 
   // ---- approximate running sums in front of every slot; from them, the binades the sequential
   //      sum can be in at the two ends of each slot.  A slot that cannot be placed inside one
@@ -589,6 +599,7 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
       const float smax = base == 0 ? first_max : slot_max[s];
       const float f = sum > 0.0f ? fast_exp2((smax - m) * kLog2e) : 0.0f;  // exp of the slot's largest entry
       a = sum > 0.0f ? sum * f : 0.0f;
+      if (WALK) a *= walk_scale;
       if (TOPP) sh.top[s] = f * 1.0001f;  // (the hardware's exp2 is within 1e-5 of the exact exp)
       if (TOPP && f > 0.0f) {
         // lower bounds of the exact exps of the slot's two largest entries, into the bins of their
@@ -655,6 +666,10 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
   int lut_base1 = 0, lut_top = 0, lut_half = 0;
   if constexpr (DT == kDtypeBFloat16) {
     use_lut = build_exp_lut<false>(lut_mem, kLutCountWords, inv, m, sm.exp2tab, lut_base1, lut_top, lut_half);
+    if (WALK && use_lut) {  // one division per bit pattern: the table becomes p = fl(e / S)
+      __syncthreads();
+      for (int idx = tid; idx < 2 * lut_half; idx += kBlock) lut_mem[idx] = div_row(lut_mem[idx], walk_div);
+    }
   }
   __syncthreads();
   if (p.timers) c3 = wall_clock64();
@@ -771,6 +786,7 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
       for (int k = 0; k < 8; ++k) {
         const float d = __builtin_fmaxf(in[k] * inv - m, -104.0f);  // expf is 0 below ln(2^-150); the core gives 0 at -104 too
         e[k] = expf_core(d, tab);
+        if (WALK) e[k] = div_row(e[k], walk_div);
       }
     }
     const bool search = TOPP && __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(sh.top[s]))) >= list_cut;
@@ -904,18 +920,47 @@ __device__ __forceinline__ void resolve_lanes(float& s, const uint32_t (&bits)[8
 // the increment for the sum's parity; a slot pass 2 prepared goes through resolve_lanes(); anything
 // else is redone entry by entry from the logits -- and the walk goes on behind it.  Every step
 // advances by at least one record.
-template <int DT>
+// WALK: the records are those of p = fl(e / S) (`div`), and the walk stops at the first entry behind
+// which the running sum exceeds `threshold` (sampler.cpp:58-70): `*stop` is its index (-1: none), the
+// value returned the sum there.  Sums behind records are exact, so the first record behind which
+// the sum exceeds the threshold holds that entry; it is redone entry by entry from the sum in front of it.
+template <int DT, bool WALK = false>
 __device__ __forceinline__ float split_chain(const SlotRec* recs, int ns, const PrepSlot* prep, uint32_t n_prep,
                                              const char* logits, int V, float inv, float m, const uint64_t* tab,
-                                             const FusedOps& fused, uint64_t* stats = nullptr) {
+                                             const FusedOps& fused, uint64_t* stats = nullptr, const RowDivisor* div = nullptr,
+                                             float threshold = 0.0f, int* stop = nullptr) {
   const int lane = threadIdx.x & 63;
   const float kInf = __uint_as_float(0x7f800000u);
   const float fill = inv < 0.0f ? kInf : -kInf;
   float s = 0.0f;
+  // slot `slot` entry by entry from the logits, from running sum `from` (WALK: with the threshold)
+  auto redo = [&](int slot, float from, int& hit) {
+    float l[8];
+    uint32_t b[8];
+    load_slot_lane<DT>(logits, slot, lane, V, fill, l, fused);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      float e = expf_core(__builtin_fmaxf(l[k] * inv - m, -104.0f), tab);
+      if (WALK) e = div_row(e, *div);
+      b[k] = __float_as_uint(e);
+    }
+    float t = from;
+    wave_resolve<8>(t, hit, b, slot * kSlot + lane * 8, V, WALK ? threshold : kInf);
+    return t;
+  };
+  if (WALK) *stop = -1;
   uint64_t c_start = 0;
   uint32_t n_iter = 0, n_generic = 0, n_prep_used = 0, n_tie = 0, n_inner = 0;
   uint64_t c_prep = 0;
   if (stats) c_start = wall_clock64();
+  auto note = [&]() {
+    if (stats && lane == 0) {
+      stats[4] = wall_clock64() - c_start;
+      stats[6] = static_cast<uint64_t>(n_iter) | (static_cast<uint64_t>(n_generic) << 32);
+      stats[7] = static_cast<uint64_t>(n_prep_used) | (static_cast<uint64_t>(n_tie) << 16) | (static_cast<uint64_t>(n_inner) << 32) |
+                 (c_prep << 48);
+    }
+  };
   for (int base = 0; base < ns; base += 64) {
     SlotRec r = {kSlotZero << 8, 0u, 0u, 0xffffffffu};
     if (base + lane < ns) r = recs[base + lane];
@@ -924,46 +969,107 @@ __device__ __forceinline__ float split_chain(const SlotRec* recs, int ns, const 
     if (base == 0 && readlane_u32(kind, 0) == kSlotExact) {  // pass 2 worked the first slot out
       s = __uint_as_float(readlane_u32(r.even, 0));
       cur = 1;
+      if (WALK && s > threshold) {
+        note();
+        return redo(0, 0.0f, *stop);
+      }
     }
-    int K_scan = -1;
-    uint32_t incl = 0u;
-    uint64_t plain_mask = 0ull;
+    // PARITY: a stable slot with a half-ulp tie inside (one increment for an even sum in front of it,
+    // one for an odd sum) counts as plain, and the prefix is a composition of such pairs (compose()),
+    // which follows the parity through the run; it is redone behind every record worked out
+    // exactly while ties lie ahead.  Otherwise such a slot is worked out on its own, and one plain
+    // prefix sum per binade serves.  (The composition costs several times the plain sum: it pays
+    // where ties are many, as among the probabilities of a 16-bit row, few distinct values of
+    // which some sit on a tie every time they occur.)
+    constexpr bool PARITY = WALK;
+    int K_scan = -1, cur_scan = -1;
+    ParityInc incl = {0u, 0u};
+    uint64_t plain_mask = 0ull, tie_mask = 0ull;
     while (cur < 64) {
       s = uniform_f32(s);
       const SumState ss = sum_state(s);
       const uint32_t K = static_cast<uint32_t>(ss.kb);
-      if (ss.kb != K_scan) {
+      if (PARITY) {
+        if (ss.kb != K_scan || (cur != cur_scan && (tie_mask >> cur) != 0ull)) {
+          const bool plain = kind == kSlotZero || (kind == kSlotStable && kb == K) || (kind == kSlotDual && (kb == K || kb + 1u == K));
+          ParityInc inc = {r.even, r.odd};
+          if (kind == kSlotDual) inc.even = inc.odd = kb != K ? r.odd : r.even;
+          if (kind == kSlotZero || !plain || lane < cur) inc = {0u, 0u};
+          incl = wave_scan_inclusive(inc, lane);  // (saturating at 2^26)
+          plain_mask = __ballot(plain);
+          tie_mask = __ballot(plain && lane >= cur && inc.even != inc.odd);
+          K_scan = ss.kb;
+          cur_scan = cur;
+          if (stats) n_tie += static_cast<uint32_t>(__popcll(tie_mask));
+        }
+      } else if (ss.kb != K_scan) {
         const bool plain = kind == kSlotZero || (kind == kSlotStable && kb == K && r.even == r.odd) ||
                            (kind == kSlotDual && (kb == K || kb + 1u == K));
         const uint32_t inc = kind == kSlotZero ? 0u : ((kind == kSlotDual && kb != K) ? r.odd : r.even);
-        incl = wave_scan_inclusive_u32(plain ? inc : 0u);  // 64 values of at most 2^26 each
+        incl.even = wave_scan_inclusive_u32(plain ? inc : 0u);  // 64 values of at most 2^26 each
         plain_mask = __ballot(plain);
         K_scan = ss.kb;
       }
       const uint64_t from_cur = ~0ull << cur;
       const uint64_t not_plain = ~plain_mask & from_cur;
       const int jn = not_plain ? __ffsll(static_cast<long long>(not_plain)) - 1 : 64;
-      const uint32_t before = cur > 0 ? readlane_u32(incl, cur - 1) : 0u;
-      const uint32_t S_upto = ss.S + (incl - before);
+      const uint32_t incl_p = (PARITY && (ss.S & 1u)) ? incl.odd : incl.even;
+      const uint32_t before = cur > 0 ? readlane_u32(incl_p, cur - 1) : 0u;
+      const uint32_t S_upto = ss.S + (incl_p - before);
       const uint64_t over = __ballot(lane >= cur && lane < jn && S_upto >= (1u << 24));
       const int jo = over ? __ffsll(static_cast<long long>(over)) - 1 : 64;
       const int j = jn < jo ? jn : jo;
+      if (WALK) {
+        // the first plain record of the run behind which the sum exceeds the threshold
+        const uint64_t cross = __ballot(lane >= cur && lane < j && sum_value(S_upto, ss.kb) > threshold);
+        if (cross != 0ull) {
+          const int q = __ffsll(static_cast<long long>(cross)) - 1;
+          if (q > cur) s = sum_value(readlane_u32(S_upto, q - 1), ss.kb);
+          note();
+          return redo(base + q, s, *stop);
+        }
+      }
       if (j > cur) s = sum_value(readlane_u32(S_upto, j - 1), ss.kb);
       if (j == 64) break;
       // ---- record base + j, exactly
       const int slot = base + j;
       const uint32_t kind_j = readlane_u32(kind, j), kb_j = readlane_u32(kb, j);
-      bool resolved = false;
-      if (j == jn && kind_j == kSlotStable && kb_j == K) {  // a tie inside: the increment follows the parity
-        const SumState sj = sum_state(s);
-        const uint32_t inc = (sj.S & 1u) ? readlane_u32(r.odd, j) : readlane_u32(r.even, j);
-        if (sj.S + inc < (1u << 24)) {
-          s = sum_value(sj.S + inc, sj.kb);
-          resolved = true;
+      const float s_front = s;
+      if (!PARITY && j == jn && kind_j == kSlotStable && kb_j == K) {
+        // ---- a tie inside: the increment follows the parity of the sum.  This record, the plain run
+        //      behind it, the next such record and so on, from the prefix sums at hand (a record
+        //      with a tie has none in them), as long as the sum stays inside the binade.
+        uint32_t S_cur = sum_state(s).S;
+        int jj = j, next_cur = -1;
+        while (true) {
+          const uint32_t inc = (S_cur & 1u) ? readlane_u32(r.odd, jj) : readlane_u32(r.even, jj);
+          if (S_cur + inc >= (1u << 24)) {  // leaves the binade inside the record: entry by entry
+            if (jj > j) next_cur = jj;
+            break;
+          }
+          S_cur += inc;
           ++n_tie;
+          next_cur = jj + 1;
+          if (jj == 63) break;
+          const uint64_t np2 = ~plain_mask & (~0ull << (jj + 1));
+          const int jn2 = np2 ? __ffsll(static_cast<long long>(np2)) - 1 : 64;
+          if (jn2 > jj + 1) {
+            const uint32_t S_run = S_cur + (incl.even - readlane_u32(incl.even, jj));
+            if (__ballot(lane > jj && lane < jn2 && S_run >= (1u << 24)) != 0ull) break;  // (the loop finds where)
+            S_cur = readlane_u32(S_run, jn2 - 1);
+          }
+          next_cur = jn2;
+          if (jn2 == 64 || readlane_u32(kind, jn2) != kSlotStable || readlane_u32(kb, jn2) != K) break;
+          jj = jn2;
+        }
+        if (next_cur >= 0) {
+          s = sum_value(S_cur, ss.kb);
+          cur = next_cur;
+          ++n_iter;
+          continue;
         }
       }
-      if (!resolved) {
+      {
         const uint32_t pi = readlane_u32(r.prep, j);
         uint32_t bits[8];
         if (j == jn && kind_j == kSlotSerial && pi < n_prep) {
@@ -986,26 +1092,26 @@ __device__ __forceinline__ float split_chain(const SlotRec* recs, int ns, const 
             ++n_generic;
           }
         } else {
-          float l[8];
-          load_slot_lane<DT>(logits, slot, lane, V, fill, l, fused);
-#pragma unroll
-          for (int k = 0; k < 8; ++k) bits[k] = __float_as_uint(expf_core(__builtin_fmaxf(l[k] * inv - m, -104.0f), tab));
-          int found = -1;
-          wave_resolve<8>(s, found, bits, slot * kSlot + lane * 8, V, kInf);
+          int hit = -1;
+          s = redo(slot, s, hit);
+          if (WALK && hit >= 0) {
+            *stop = hit;
+            note();
+            return s;
+          }
           ++n_generic;
         }
+      }
+      if (WALK && s > threshold) {
+        note();
+        return redo(slot, s_front, *stop);
       }
       cur = j + 1;
       ++n_iter;
     }
     if (stats && base == 0 && lane == 0) stats[5] = wall_clock64() - c_start;
   }
-  if (stats && lane == 0) {
-    stats[4] = 0;
-    stats[6] = static_cast<uint64_t>(n_iter) | (static_cast<uint64_t>(n_generic) << 32);
-    stats[7] = static_cast<uint64_t>(n_prep_used) | (static_cast<uint64_t>(n_tie) << 16) | (static_cast<uint64_t>(n_inner) << 32) |
-               (c_prep << 48);
-  }
+  note();
   return uniform_f32(s);
 }
 
@@ -1980,6 +2086,77 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
   }
   }  // rows of the unit
   }  // units of this workgroup
+}
+
+// ---- multinomial rows (sampler.cpp:58-70, 236-247) -------------------------------------------------
+// Their draw is a second sequential sum over the row, of p = fl(e / S), up to the first entry behind
+// which it exceeds the coin.  Five launches: pass 1; pass 2 (records of the sum of e); this kernel,
+// PHASE 0: the exact S by the chain, the coin; pass 2 again in its WALK instantiation (records of the
+// sum of p); this kernel, PHASE 1: the chain over those, stopped by the coin.
+// grid = rows, kWalkBlock lanes: all of them stage the row's records and prepared slots in LDS
+// (dynamic: `lds_bytes`), the first wave walks.
+constexpr int kWalkBlock = 256;
+template <int DT, int PHASE>
+__global__ void __launch_bounds__(kWalkBlock) split_walk_kernel(SplitParams p, uint32_t lds_bytes) {
+  extern __shared__ __align__(16) uint64_t walk_lds[];
+  __shared__ uint64_t exp2tab[32];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int V = p.row.vocab;
+  const int ns = p.ns;
+  const int row = p.row.row_map ? p.row.row_map[blockIdx.x] : blockIdx.x;
+  const RowState rs = p.row_state[row];
+  if (tid < 32) exp2tab[tid] = kExp2Table[tid];
+  auto toss = [&]() {  // one coin per call (sampler.cpp:237, 210-220)
+    uint64_t st = p.row.rng[row];
+    st ^= st >> 12;
+    st ^= st << 25;
+    st ^= st >> 27;
+    p.row.rng[row] = st;
+    const uint32_t u = static_cast<uint32_t>((st * 0x2545F4914F6CDD1Dull) >> 32);
+    return static_cast<float>(u >> 8) / 16777216.0f;
+  };
+  if (rs.nan != 0u) {
+    // every probability is NaN: the walk never stops and returns the last index
+    if (PHASE == 0 && tid == 0) {
+      const float coin = toss();
+      p.row.tokens[row] = V - 1;
+      if (p.row.debug) p.row.debug[row] = RowDebug{rs.m, __uint_as_float(0x7fc00000u), coin, 0.0f, 0.0f, 0, 0, 0};
+    }
+    return;
+  }
+  const float inv = p.row.row_cfg ? p.row.row_cfg[row].inv_temperature : p.row.inv_temperature;
+  const char* logits = static_cast<const char*>(p.row.logits) + static_cast<int64_t>(row) * p.row.row_stride * ElemSize<DT>::value;
+  const size_t rec_bytes = (static_cast<size_t>(ns) * sizeof(SlotRec) + 15) / 16 * 16;
+  uint32_t n_prep = rs.prep_count < static_cast<uint32_t>(p.prep_cap) ? rs.prep_count : static_cast<uint32_t>(p.prep_cap);
+  const uint32_t fit = lds_bytes > rec_bytes ? static_cast<uint32_t>((lds_bytes - rec_bytes) / sizeof(PrepSlot)) : 0u;
+  n_prep = n_prep < fit ? n_prep : fit;  // (a prepared slot that does not fit is redone from the logits)
+  uint4* lds_vec = reinterpret_cast<uint4*>(walk_lds);
+  const uint4* rec_src = reinterpret_cast<const uint4*>(p.slot_rec + static_cast<int64_t>(row) * p.ns_stride);
+  const uint4* prep_src = reinterpret_cast<const uint4*>(p.prep + static_cast<int64_t>(row) * p.prep_cap);
+  for (int i = tid; i < ns; i += kWalkBlock) lds_vec[i] = rec_src[i];
+  const int prep_vecs = static_cast<int>(n_prep * (sizeof(PrepSlot) / 16));
+  for (int i = tid; i < prep_vecs; i += kWalkBlock) lds_vec[rec_bytes / 16 + i] = prep_src[i];
+  __syncthreads();
+  if (tid >= 64) return;
+  const SlotRec* recs = reinterpret_cast<const SlotRec*>(walk_lds);
+  const PrepSlot* prep = reinterpret_cast<const PrepSlot*>(reinterpret_cast<const char*>(walk_lds) + rec_bytes);
+  if (PHASE == 0) {
+    const float S = split_chain<DT>(recs, ns, prep, n_prep, logits, V, inv, rs.m, exp2tab, p.row.fused,
+                                    p.timers ? p.timers + static_cast<int64_t>(row) * 8 : nullptr);
+    if (lane == 0) p.walk[row] = make_float2(S, toss());
+  } else {
+    const float2 w = p.walk[row];
+    const RowDivisor div = row_divisor(w.x);
+    int stop = -1;
+    const float cdf = split_chain<DT, true>(recs, ns, prep, n_prep, logits, V, inv, rs.m, exp2tab, p.row.fused,
+                                            p.timers ? p.timers + static_cast<int64_t>(gridDim.x) * 8 + static_cast<int64_t>(blockIdx.x) * 4 - 4 : nullptr, &div, w.y, &stop);
+    if (lane == 0) {
+      const int32_t token = stop >= 0 ? stop : V - 1;
+      p.row.tokens[row] = token;
+      if (p.row.debug) p.row.debug[row] = RowDebug{rs.m, w.x, w.y, cdf, 0.0f, 0, 0, token};
+    }
+  }
 }
 
 }  // namespace ets

@@ -274,3 +274,35 @@ def test_topk_rows_when_split(oracle, dev, dtype, kind):
             want, _ = oracle.sample_rows(x, dtype, inv, 0.9, k, states, mode=oracle.MODE_UPCAST, tie=oracle.TIE_STABLE, threads=8)
             assert np.array_equal(res[0][step], want), (k, step)
         assert np.array_equal(res[0][2], states), k
+
+
+@pytest.mark.parametrize("dtype", [W.DTYPE_BFLOAT16, W.DTYPE_FLOAT, W.DTYPE_HALF])
+@pytest.mark.parametrize("kind", ["normal", "peaked", "few", "flat", "one", "masked"])
+def test_multinomial_rows_when_split(oracle, dev, dtype, kind):
+    """Multinomial rows (sampler.cpp:58-70) over several workgroups, five launches: the records of the
+    sum of exp, its chain, the records of the sum of p = exp / sum, and a chain over those that stops
+    where the running sum exceeds the coin.  Against the oracle (tokens, coin states) and against the
+    one-workgroup kernel (debug records as well: the sum, the coin, the running sum at the stop),
+    at three temperatures, four calls each so that the coins land in different parts of the rows."""
+    V, rows = 128256, 12
+    rng = np.random.default_rng(29)
+    x = W.to_storage(topk_rows(kind, rows, V, rng), dtype)
+    dx = to_device(x, dtype, dev)
+    for temperature in (1.0, 0.6, 2.5):
+        inv = oracle.inv_temperature(temperature)
+        samplers = []
+        for mode in (SPLIT_ON, SPLIT_OFF):
+            s = ea.Sampler(V, temperature, 1.0, 31, max_batch=rows)
+            s.set_row_split(mode)
+            samplers.append(s)
+        states = (np.uint64(31) + np.arange(rows, dtype=np.uint64)).astype(np.uint64)
+        for call in range(4):
+            res = []
+            for s in samplers:
+                dbg = torch.zeros((rows, 8), dtype=torch.int32, device=dev)
+                tok = s.sample_batch(dx, debug_out=dbg if call % 2 else None).cpu().numpy()
+                res.append((tok, ea.debug_records(dbg).copy(), s.get_rng_states(rows)))
+            assert_same(res[0], res[1])
+            want, _ = oracle.sample_rows(x, dtype, inv, 1.0, 0, states, mode=oracle.MODE_UPCAST, tie=oracle.TIE_STABLE, threads=8)
+            assert np.array_equal(res[0][0], want), (temperature, call)
+            assert np.array_equal(res[0][2], states), (temperature, call)
