@@ -33,7 +33,7 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 COPY_PROBE_BYTES = 256 << 20
-STEP_KERNELS = ("split_pass1_kernel", "split_pass2_kernel", "split_finish_kernel", "sample_rows_kernel")
+STEP_KERNELS = ("split_pass1_kernel", "split_pass2_kernel", "split_finish_kernel", "split_walk_kernel", "sample_rows_kernel")
 
 
 def synth_logits_device(w, count, torch, dev):
@@ -441,21 +441,34 @@ def parse_pmc(fetch_dir, write_dir, out_path):
            "fetch_factor": probe_kib / copy_f if copy_f else None, "write_factor": probe_kib / copy_w if copy_w else None,
            "kernels": {}}
     total = 0.0
-    for k in STEP_KERNELS:
-        f, nf = mean_of(fetch, k)
-        wv, nw = mean_of(write, k)
-        if f is None and wv is None:
-            continue
-        res["kernels"][k] = {"fetch_kib": f, "write_kib": wv, "dispatches": [nf, nw]}
+    found = {k: (mean_of(fetch, k), mean_of(write, k)) for k in STEP_KERNELS}
+    found = {k: v for k, v in found.items() if v[0][0] is not None or v[1][0] is not None}
+    # a kernel that a step launches twice (multinomial rows: pass 2 and the walk kernel) counts twice
+    steps_f = min((v[0][1] for v in found.values() if v[0][1]), default=0)
+    steps_w = min((v[1][1] for v in found.values() if v[1][1]), default=0)
+    for k, ((f, nf), (wv, nw)) in found.items():
+        per_step = [round(nf / steps_f) if steps_f else 0, round(nw / steps_w) if steps_w else 0]
+        res["kernels"][k] = {"fetch_kib": f, "write_kib": wv, "dispatches": [nf, nw], "launches_per_step": per_step}
         if f is not None and res["fetch_factor"]:
-            total += f * res["fetch_factor"] * 1024
+            total += f * per_step[0] * res["fetch_factor"] * 1024
         if wv is not None and res["write_factor"]:
-            total += wv * res["write_factor"] * 1024
+            total += wv * per_step[1] * res["write_factor"] * 1024
     res["traffic_bytes_per_step"] = total
     with open(out_path, "w") as fo:
         json.dump(res, fo, indent=1)
         fo.write("\n")
     print(json.dumps(res))
+
+
+def step_kernels_text(w):
+    """Which launches make up one step of this workload (what the events of the timed loop bracket)."""
+    if w.temperature == 0.0:
+        return "one step = argmax_partial_kernel + argmax_finish_kernel (two launches)"
+    if not 0.0 < w.topp < 1.0:
+        return ("one step = split_pass1_kernel + split_pass2_kernel + split_walk_kernel + split_pass2_kernel + "
+                "split_walk_kernel (multinomial rows, five launches; their summed duration is what the events bracket)")
+    return ("one step = split_pass1_kernel + split_pass2_kernel + split_finish_kernel (three launches; "
+            "their summed duration is what the events bracket)")
 
 
 def measured_traffic(name):
@@ -567,8 +580,7 @@ def main():
                                f"ring of {ring_len} distinct matrices ({ring_len * step_bytes >> 20} MiB)"},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": traffic, "traffic_source": traffic_source,
-                     "kernel": "one step = split_pass1_kernel + split_pass2_kernel + split_finish_kernel (three launches; "
-                               "their summed duration is what the events bracket)",
+                     "kernel": step_kernels_text(w),
                      "kernel_ms": kernel_ms, "kernel_ms_repeats": repeats_ms, "algorithmic_bytes_per_launch": step_bytes},
     }
     if not args.no_extras:
