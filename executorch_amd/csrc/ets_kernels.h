@@ -1064,6 +1064,82 @@ __device__ int draw_small_wave(LdsKeys lds, int n, int n_total, float topp, floa
   return pos;
 }
 
+// Ascending sort of n distinct candidate keys in LDS by buckets: the keys go into 2048 buckets by
+// the size of their probability (64 per binade below the largest one, like the histogram of the
+// candidates; one counting pass, one scan, one scatter into `work`), then every key counts the keys
+// of its own bucket that are below it (its neighbours read the same keys, which LDS broadcasts) and
+// goes back to `keys` at that rank.  A few passes over the keys instead of the bitonic network's
+// log2(N)^2 / 2, as long as no bucket is long: a nucleus of 4234 fp32 probabilities has about ten
+// keys to a bucket.  `work`: room for n keys and, behind them, 4096 32-bit words.
+// Returns false, with `keys` as they were, when a bucket holds more than kBucketMax keys (many equal
+// probabilities: the caller sorts by the network).  Ends with a barrier.
+constexpr int kSortBuckets = 2048;
+constexpr int kBucketMax = 192;
+__device__ bool sort_keys_bucketed(LdsKeys keys, int n, LdsKeys work, BlockScratch& sm) {
+  static_assert(kSortBuckets == 2 * kBlock, "two buckets per lane");
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  LdsU32 cursor = (LdsU32)(work + n);
+  LdsU32 start = cursor + kSortBuckets;
+  cursor[2 * tid] = 0u;
+  cursor[2 * tid + 1] = 0u;
+  // the largest probability has the smallest key
+  uint32_t top = 0u;
+  for (int i = tid; i < n; i += kBlock) {
+    const uint32_t inv = ~static_cast<uint32_t>(keys[i] >> 32);
+    top = inv > top ? inv : top;
+  }
+  top = wave_max_u32(top);
+  if (lane == 0) sm.red_u[wave] = top;
+  __syncthreads();
+  top = sm.red_u[0];
+  for (int w = 1; w < kWaves; ++w) top = sm.red_u[w] > top ? sm.red_u[w] : top;
+  const uint32_t hi_min = ~top;
+  auto bucket_of = [&](uint64_t key) -> uint32_t {
+    const uint32_t b = (static_cast<uint32_t>(key >> 32) - hi_min) >> 17;
+    return b < static_cast<uint32_t>(kSortBuckets - 1) ? b : static_cast<uint32_t>(kSortBuckets - 1);
+  };
+  for (int i = tid; i < n; i += kBlock)
+    __hip_atomic_fetch_add(&cursor[bucket_of(keys[i])], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+  __syncthreads();
+  const uint32_t c0 = cursor[2 * tid], c1 = cursor[2 * tid + 1];
+  const uint32_t incl = wave_scan_inclusive_u32(c0 + c1);
+  const uint32_t longest = wave_max_u32(c0 > c1 ? c0 : c1);
+  __syncthreads();  // (red_u has been read by everybody)
+  if (lane == 63) sm.red_u[wave] = incl;
+  if (lane == 0) sm.red_f[wave] = __uint_as_float(longest);
+  __syncthreads();
+  uint32_t before = incl - (c0 + c1), worst = 0u;
+  for (int w = 0; w < kWaves; ++w) {
+    if (w < wave) before += sm.red_u[w];
+    const uint32_t l = __float_as_uint(sm.red_f[w]);
+    worst = l > worst ? l : worst;
+  }
+  __syncthreads();  // (red_u and red_f are free again)
+  if (worst > static_cast<uint32_t>(kBucketMax)) return false;
+  start[2 * tid] = before;
+  start[2 * tid + 1] = before + c0;
+  cursor[2 * tid] = before;
+  cursor[2 * tid + 1] = before + c0;
+  __syncthreads();
+  for (int i = tid; i < n; i += kBlock) {
+    const uint64_t key = keys[i];
+    work[__hip_atomic_fetch_add(&cursor[bucket_of(key)], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)] = key;
+  }
+  __syncthreads();  // cursor[b] is now the end of bucket b
+  for (int i = tid; i < n; i += kBlock) {
+    const uint64_t key = work[i];
+    const uint32_t b = bucket_of(key);
+    const int first = static_cast<int>(start[b]), end = static_cast<int>(cursor[b]);
+    int rank = first;
+    for (int j = first; j < end; ++j) rank += work[j] < key ? 1 : 0;
+    keys[rank] = key;
+  }
+  __syncthreads();
+  return true;
+}
+
 // Top-p draw from the listed possible candidates (sampler.cpp:122-171).  Entry j of the list sits
 // in lds_list[j] while j < lds_list_cap and in list[j] (global memory) beyond; lds_list is the
 // upper part of the key buffer lds_keys[0, cap), starting at key index `list_base`.
@@ -1211,7 +1287,10 @@ __device__ bool draw_topp_listed(uint64_t* list, uint64_t* lds_list, int lds_lis
   for (int i = n_sel + tid; i < N; i += kBlock) lds_keys[i] = ~0ull;
   __syncthreads();
   if (n_sel <= 64) return draw_small_wave((LdsKeys)lds_keys, n_sel, n_total, topp, coin, dbg, token, sm) != -2;
-  sort_keys_lds((LdsKeys)lds_keys, N);
+  // (the list is dead from here on: what lies behind the keys is free for the sort by buckets)
+  bool sorted = false;
+  if (n_sel > 512 && N + n_sel + kSortBuckets <= cap) sorted = sort_keys_bucketed((LdsKeys)lds_keys, n_sel, (LdsKeys)lds_keys + N, sm);
+  if (!sorted) sort_keys_lds((LdsKeys)lds_keys, N);
   const int pos = draw_from_sorted((LdsKeys)lds_keys, n_sel, n_total, false, 0, topp, coin, dbg, sm);
   if (pos == -2) return false;  // the pre-selection did not reach topp after all
   token = static_cast<int32_t>(static_cast<uint32_t>(lds_keys[pos]));

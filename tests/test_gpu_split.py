@@ -306,3 +306,35 @@ def test_multinomial_rows_when_split(oracle, dev, dtype, kind):
             want, _ = oracle.sample_rows(x, dtype, inv, 1.0, 0, states, mode=oracle.MODE_UPCAST, tie=oracle.TIE_STABLE, threads=8)
             assert np.array_equal(res[0][0], want), (temperature, call)
             assert np.array_equal(res[0][2], states), (temperature, call)
+
+
+@pytest.mark.parametrize("mode", [SPLIT_ON, SPLIT_OFF])
+def test_nuclei_of_hundreds_to_thousands_of_keys(oracle, dev, mode):
+    """fp32 rows whose nucleus holds from several hundred to several thousand keys: the selected keys
+    are sorted by buckets of their probability (up to about 5000 keys), by the bitonic network beyond
+    that and where a bucket would be long (many equal probabilities: the rows of a dozen distinct
+    values), and the two CDF walks run over them.  Against the oracle: tokens, coin states, the
+    nucleus' last index and mass, the position of the draw."""
+    V, rows = 32000, 8
+    rng = np.random.default_rng(41)
+    kinds = {
+        "normal": (rng.standard_normal((rows, V)) * 2.0).astype(np.float32),
+        "few": rng.integers(0, 12, (rows, V)).astype(np.float32) * 0.5,
+    }
+    for kind, x in kinds.items():
+        dx = to_device(x, W.DTYPE_FLOAT, dev)
+        for temperature, topp in ((0.5, 0.9), (0.8, 0.9), (1.0, 0.95), (1.5, 0.9), (0.8, 0.5)):
+            s = ea.Sampler(V, temperature, topp, 53, max_batch=rows)
+            s.set_row_split(mode)
+            dbg = torch.zeros((rows, 8), dtype=torch.int32, device=dev)
+            got = s.sample_batch(dx, debug_out=dbg).cpu().numpy()
+            rec = ea.debug_records(dbg)
+            states = (np.uint64(53) + np.arange(rows, dtype=np.uint64)).astype(np.uint64)
+            want, ex = oracle.sample_rows(x, W.DTYPE_FLOAT, oracle.inv_temperature(temperature), topp, 0, states,
+                                          mode=oracle.MODE_UPCAST, tie=oracle.TIE_STABLE, explain=True, threads=8)
+            assert np.array_equal(got, want), (kind, temperature, topp)
+            assert np.array_equal(s.get_rng_states(rows), states)
+            for b in range(rows):
+                assert rec["last_idx"][b] == ex[b].last_idx, (kind, temperature, topp, b)
+                assert rec["position"][b] == ex[b].position, (kind, temperature, topp, b)
+                assert f32_bits(np.float32(rec["cumulative"][b])) == f32_bits(np.float32(ex[b].cumulative)), (kind, temperature, topp, b)
