@@ -465,6 +465,7 @@ __device__ int draw_from_sorted(Keys keys, int n_sorted, int n_total, bool use_t
                                 RowDebug& dbg, BlockScratch& sm) {
   const float kInf = __uint_as_float(0x7f800000u);
   auto sorted_prob = [&](int i) -> float { return cand_prob(keys[i]); };
+  auto behind_prefix = [&](int i) -> float { return cand_prob(keys[i + kSmallWalk]); };
   int last_idx;
   float mass;
   if (use_topk) {
@@ -482,14 +483,21 @@ __device__ int draw_from_sorted(Keys keys, int n_sorted, int n_total, bool use_t
       res = seq_sum_small(keys, kSmallWalk, topp, sm);
       decided = res.stop_index >= 0;
     }
-    if (!decided) res = seq_sum_block<4>(sorted_prob, n_sorted, 0.0f, topp, sm);
+    if (!decided) {  // on from where the prefix ended
+      res = seq_sum_block<4>(behind_prefix, n_sorted - kSmallWalk, res.sum, topp, sm);
+      if (res.stop_index >= 0) res.stop_index += kSmallWalk;
+    }
     if (res.stop_index < 0 && n_sorted < n_total) return -2;
     last_idx = res.stop_index >= 0 ? res.stop_index : n_sorted - 1;
     mass = res.sum;
   }
   const float r = coin * mass;  // sampler.cpp:109 / :162
-  const SeqSumResult walk = (last_idx < kSmallWalk) ? seq_sum_small(keys, last_idx + 1, r, sm)
-                                                    : seq_sum_block<4>(sorted_prob, last_idx + 1, 0.0f, r, sm);
+  // (the largest probabilities come first: the walk often ends among them)
+  SeqSumResult walk = seq_sum_small(keys, last_idx + 1 < kSmallWalk ? last_idx + 1 : kSmallWalk, r, sm);
+  if (walk.stop_index < 0 && last_idx + 1 > kSmallWalk) {
+    walk = seq_sum_block<4>(behind_prefix, last_idx + 1 - kSmallWalk, walk.sum, r, sm);
+    if (walk.stop_index >= 0) walk.stop_index += kSmallWalk;
+  }
   const int pos = walk.stop_index >= 0 ? walk.stop_index : last_idx;
   dbg.last_idx = last_idx;
   dbg.cumulative = mass;
