@@ -411,7 +411,8 @@ bool use_split(const ets_sampler* s, const void* d_logits, int64_t stride, int32
   return s->split_mode == ETS_ROW_SPLIT_ON || s->vocab >= 8192;
 }
 
-template <int DT>
+// TOPK: some row may be a top-k row (the kernels of a launch without one leave that case out).
+template <int DT, bool TOPK>
 ets_status launch_split(ets_sampler* s, const ets::RowParams& p, int32_t rows, hipStream_t stream) {
   ets_status st = ETS_OK;
   constexpr bool k16 = DT == ets::kDtypeBFloat16 || DT == ets::kDtypeHalf;
@@ -447,9 +448,9 @@ ets_status launch_split(ets_sampler* s, const ets::RowParams& p, int32_t rows, h
   ETS_HIP(s, hipGetLastError());
   const size_t lut_bytes = (DT == ets::kDtypeBFloat16 ? sizeof(float) * ets::kLutCountWords : 0) + sizeof(uint32_t) * sp.phist_words;
   static std::atomic<size_t> set_bytes2[kMaxDevices];
-  st = allow_dynamic_lds(s, reinterpret_cast<const void*>(&ets::split_pass2_kernel<DT, true>), lut_bytes, set_bytes2);
+  st = allow_dynamic_lds(s, reinterpret_cast<const void*>(&ets::split_pass2_kernel<DT, true, false, TOPK>), lut_bytes, set_bytes2);
   if (st != ETS_OK) return st;
-  hipLaunchKernelGGL((ets::split_pass2_kernel<DT, true>), dim3(sp.row_wgs, rows), dim3(ets::kBlock), lut_bytes, stream, sp);
+  hipLaunchKernelGGL((ets::split_pass2_kernel<DT, true, false, TOPK>), dim3(sp.row_wgs, rows), dim3(ets::kBlock), lut_bytes, stream, sp);
   ETS_HIP(s, hipGetLastError());
   if (rows > p.grid_cap) {
     // more rows than workgroups: a workgroup takes up to kChainRows rows at a time
@@ -462,15 +463,15 @@ ets_status launch_split(ets_sampler* s, const ets::RowParams& p, int32_t rows, h
     sp.chain_rows = per_wg < chain_rows_max ? per_wg : chain_rows_max;
     const int units = (rows + sp.chain_rows - 1) / sp.chain_rows;
     static std::atomic<size_t> set_bytes[kMaxDevices];
-    st = allow_dynamic_lds(s, reinterpret_cast<const void*>(&ets::split_finish_kernel<DT, true>), s->lds_bytes, set_bytes);
+    st = allow_dynamic_lds(s, reinterpret_cast<const void*>(&ets::split_finish_kernel<DT, true, TOPK>), s->lds_bytes, set_bytes);
     if (st != ETS_OK) return st;
-    hipLaunchKernelGGL((ets::split_finish_kernel<DT, true>), dim3(units < p.grid_cap ? units : p.grid_cap), dim3(ets::kBlock),
+    hipLaunchKernelGGL((ets::split_finish_kernel<DT, true, TOPK>), dim3(units < p.grid_cap ? units : p.grid_cap), dim3(ets::kBlock),
                        s->lds_bytes, stream, sp);
   } else {
     static std::atomic<size_t> set_bytes[kMaxDevices];
-    st = allow_dynamic_lds(s, reinterpret_cast<const void*>(&ets::split_finish_kernel<DT, false>), s->lds_bytes, set_bytes);
+    st = allow_dynamic_lds(s, reinterpret_cast<const void*>(&ets::split_finish_kernel<DT, false, TOPK>), s->lds_bytes, set_bytes);
     if (st != ETS_OK) return st;
-    hipLaunchKernelGGL((ets::split_finish_kernel<DT, false>), dim3(rows), dim3(ets::kBlock), s->lds_bytes, stream, sp);
+    hipLaunchKernelGGL((ets::split_finish_kernel<DT, false, TOPK>), dim3(rows), dim3(ets::kBlock), s->lds_bytes, stream, sp);
   }
   ETS_HIP(s, hipGetLastError());
   return ETS_OK;
@@ -536,14 +537,17 @@ ets_status launch_split_walk_any(ets_sampler* s, const ets::RowParams& p, int32_
 }
 
 // The three launches for rows that use_split() accepted (each row's draw follows from its parameters).
-ets_status launch_split_any(ets_sampler* s, const ets::RowParams& p, int32_t dtype, int32_t rows, hipStream_t stream) {
+// topk_rows: some row of the launch has a top-k of its own or the launch-wide one applies.
+ets_status launch_split_any(ets_sampler* s, const ets::RowParams& p, int32_t dtype, int32_t rows, hipStream_t stream,
+                            bool topk_rows) {
   switch (dtype) {
     case ETS_DTYPE_FLOAT:
-      return launch_split<ets::kDtypeFloat>(s, p, rows, stream);
+      return topk_rows ? launch_split<ets::kDtypeFloat, true>(s, p, rows, stream) : launch_split<ets::kDtypeFloat, false>(s, p, rows, stream);
     case ETS_DTYPE_HALF:
-      return launch_split<ets::kDtypeHalf>(s, p, rows, stream);
+      return topk_rows ? launch_split<ets::kDtypeHalf, true>(s, p, rows, stream) : launch_split<ets::kDtypeHalf, false>(s, p, rows, stream);
     default:
-      return launch_split<ets::kDtypeBFloat16>(s, p, rows, stream);
+      return topk_rows ? launch_split<ets::kDtypeBFloat16, true>(s, p, rows, stream)
+                       : launch_split<ets::kDtypeBFloat16, false>(s, p, rows, stream);
   }
 }
 
@@ -551,7 +555,7 @@ ets_status rows_device(ets_sampler* s, const ets::RowParams& p, int32_t dtype, i
                        int draw) {
   if (draw != ets::kDrawAny && use_split(s, p.logits, p.row_stride, dtype, draw, p.topk, p.probs != nullptr)) {
     if (draw == ets::kDrawMultinomial) return launch_split_walk_any(s, p, dtype, rows, stream);
-    return launch_split_any(s, p, dtype, rows, stream);
+    return launch_split_any(s, p, dtype, rows, stream, draw == ets::kDrawTopK);
   }
   switch (dtype) {
     case ETS_DTYPE_FLOAT:
@@ -730,6 +734,7 @@ ets_status sample_device_configs(ets_sampler* s, const void* d_logits, int32_t d
   // maps[g * batch + i]: the i-th row of group g.
   enum { kGreedy = 0, kSplit = 1, kRows = 2, kWalk = 3 };
   int32_t count[4] = {0, 0, 0, 0};
+  bool split_topk = false;  // some row of the three-launch group is a top-k row
   bool any_reseed = false;
   for (int32_t b = 0; b < batch; ++b) {
     const ets_sampling_config& c = configs[b];
@@ -744,6 +749,7 @@ ets_status sample_device_configs(ets_sampler* s, const void* d_logits, int32_t d
     if (inv != 0.0f) {
       const int draw = draw_mode(s->vocab, c.top_p, c.top_k);
       group = !use_split(s, d_logits, stride, dtype, draw, c.top_k) ? kRows : (draw == ets::kDrawMultinomial ? kWalk : kSplit);
+      split_topk = split_topk || (group == kSplit && draw == ets::kDrawTopK);
     }
     if (group != kGreedy && dtype == ETS_DTYPE_UINT16) return fail(s, ETS_NOT_SUPPORTED, kUint16Message);
     h_maps[group * batch + count[group]++] = b;
@@ -811,7 +817,7 @@ ets_status sample_device_configs(ets_sampler* s, const void* d_logits, int32_t d
     p.scratch = s->d_scratch + (both_draw ? static_cast<int64_t>(share) * s->scratch_stride : 0);
     p.grid_cap = share;
     p.row_map = d_maps + kSplit * batch;
-    st = launch_split_any(s, p, dtype, count[kSplit], side);
+    st = launch_split_any(s, p, dtype, count[kSplit], side, split_topk);
     if (st != ETS_OK) return st;
   }
   if (count[kGreedy] > 0) {

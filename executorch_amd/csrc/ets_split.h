@@ -493,7 +493,8 @@ __device__ __forceinline__ void split_fold_slot(const SplitParams& p, int row, i
 #endif
 // WALK: the second sum of a multinomial row (sampler.cpp:58-70): the entries are p = fl(e / S) with the exact
 // softmax sum S that the first chain left in SplitParams::walk, and the records describe their running sum.
-template <int DT, bool TOPP, bool WALK = false>
+// TOPK: some row of the launch may be a top-k row (a launch without one runs the code without that case).
+template <int DT, bool TOPP, bool WALK = false, bool TOPK = false>
 __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_kernel(SplitParams p) {
   extern __shared__ __align__(16) float lut_mem[];
   __shared__ Pass2Shared sh;
@@ -507,8 +508,8 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
   const int ns = p.ns;
   const float inv = p.row.row_cfg ? p.row.row_cfg[row].inv_temperature : p.row.inv_temperature;
   const float topp = p.row.row_cfg ? p.row.row_cfg[row].topp : p.row.topp;
-  const int32_t topk = p.row.row_cfg ? p.row.row_cfg[row].topk : p.row.topk;
-  const bool row_topk = topk > 0 && topk < p.row.vocab;  // sampler.cpp:239: top-k comes before top-p
+  const int32_t topk = !TOPK ? 0 : (p.row.row_cfg ? p.row.row_cfg[row].topk : p.row.topk);
+  const bool row_topk = TOPK && topk > 0 && topk < p.row.vocab;  // sampler.cpp:239: top-k comes before top-p
   const char* logits = static_cast<const char*>(p.row.logits) + static_cast<int64_t>(row) * p.row.row_stride * ElemSize<DT>::value;
   const float* slot_max = p.slot_max + static_cast<int64_t>(row) * p.ns_stride;
   const float* slot_sum = p.slot_sum + static_cast<int64_t>(row) * p.ns_stride;
@@ -920,15 +921,123 @@ __device__ __forceinline__ void resolve_lanes(float& s, const uint32_t (&bits)[8
 // the increment for the sum's parity; a slot pass 2 prepared goes through resolve_lanes(); anything
 // else is redone entry by entry from the logits -- and the walk goes on behind it.  Every step
 // advances by at least one record.
-// WALK: the records are those of p = fl(e / S) (`div`), and the walk stops at the first entry behind
+template <int DT>
+__device__ __forceinline__ float split_chain(const SlotRec* recs, int ns, const PrepSlot* prep, uint32_t n_prep,
+                                             const char* logits, int V, float inv, float m, const uint64_t* tab,
+                                             const FusedOps& fused, uint64_t* stats = nullptr) {
+  const int lane = threadIdx.x & 63;
+  const float kInf = __uint_as_float(0x7f800000u);
+  const float fill = inv < 0.0f ? kInf : -kInf;
+  float s = 0.0f;
+  uint64_t c_start = 0;
+  uint32_t n_iter = 0, n_generic = 0, n_prep_used = 0, n_tie = 0, n_inner = 0;
+  uint64_t c_prep = 0;
+  if (stats) c_start = wall_clock64();
+  for (int base = 0; base < ns; base += 64) {
+    SlotRec r = {kSlotZero << 8, 0u, 0u, 0xffffffffu};
+    if (base + lane < ns) r = recs[base + lane];
+    const uint32_t kind = (r.meta >> 8) & 7u, kb = r.meta & 255u;
+    int cur = 0;
+    if (base == 0 && readlane_u32(kind, 0) == kSlotExact) {  // pass 2 worked the first slot out
+      s = __uint_as_float(readlane_u32(r.even, 0));
+      cur = 1;
+    }
+    int K_scan = -1;
+    uint32_t incl = 0u;
+    uint64_t plain_mask = 0ull;
+    while (cur < 64) {
+      s = uniform_f32(s);
+      const SumState ss = sum_state(s);
+      const uint32_t K = static_cast<uint32_t>(ss.kb);
+      if (ss.kb != K_scan) {
+        const bool plain = kind == kSlotZero || (kind == kSlotStable && kb == K && r.even == r.odd) ||
+                           (kind == kSlotDual && (kb == K || kb + 1u == K));
+        const uint32_t inc = kind == kSlotZero ? 0u : ((kind == kSlotDual && kb != K) ? r.odd : r.even);
+        incl = wave_scan_inclusive_u32(plain ? inc : 0u);  // 64 values of at most 2^26 each
+        plain_mask = __ballot(plain);
+        K_scan = ss.kb;
+      }
+      const uint64_t from_cur = ~0ull << cur;
+      const uint64_t not_plain = ~plain_mask & from_cur;
+      const int jn = not_plain ? __ffsll(static_cast<long long>(not_plain)) - 1 : 64;
+      const uint32_t before = cur > 0 ? readlane_u32(incl, cur - 1) : 0u;
+      const uint32_t S_upto = ss.S + (incl - before);
+      const uint64_t over = __ballot(lane >= cur && lane < jn && S_upto >= (1u << 24));
+      const int jo = over ? __ffsll(static_cast<long long>(over)) - 1 : 64;
+      const int j = jn < jo ? jn : jo;
+      if (j > cur) s = sum_value(readlane_u32(S_upto, j - 1), ss.kb);
+      if (j == 64) break;
+      // ---- record base + j, exactly
+      const int slot = base + j;
+      const uint32_t kind_j = readlane_u32(kind, j), kb_j = readlane_u32(kb, j);
+      bool resolved = false;
+      if (j == jn && kind_j == kSlotStable && kb_j == K) {  // a tie inside: the increment follows the parity
+        const SumState sj = sum_state(s);
+        const uint32_t inc = (sj.S & 1u) ? readlane_u32(r.odd, j) : readlane_u32(r.even, j);
+        if (sj.S + inc < (1u << 24)) {
+          s = sum_value(sj.S + inc, sj.kb);
+          resolved = true;
+          ++n_tie;
+        }
+      }
+      if (!resolved) {
+        const uint32_t pi = readlane_u32(r.prep, j);
+        uint32_t bits[8];
+        if (j == jn && kind_j == kSlotSerial && pi < n_prep) {
+          const PrepSlot& ps = prep[pi];
+          const float4 e0 = *reinterpret_cast<const float4*>(ps.e + lane * 8);
+          const float4 e1 = *reinterpret_cast<const float4*>(ps.e + lane * 8 + 4);
+          bits[0] = __float_as_uint(e0.x); bits[1] = __float_as_uint(e0.y); bits[2] = __float_as_uint(e0.z); bits[3] = __float_as_uint(e0.w);
+          bits[4] = __float_as_uint(e1.x); bits[5] = __float_as_uint(e1.y); bits[6] = __float_as_uint(e1.z); bits[7] = __float_as_uint(e1.w);
+          if (ps.usable) {
+            const uint64_t tie_a = (static_cast<uint64_t>(ps.tie_a_hi) << 32) | ps.tie_a_lo;
+            const uint64_t tie_b = (static_cast<uint64_t>(ps.tie_b_hi) << 32) | ps.tie_b_lo;
+            const uint64_t cb = stats ? wall_clock64() : 0;
+            resolve_lanes(s, bits, ps.pre_a[lane], ps.pre_b[lane], tie_a, tie_b, ps.kb_a, ps.kb_b, slot * kSlot + lane * 8, V,
+                          stats ? &n_inner : nullptr);
+            if (stats) c_prep += wall_clock64() - cb;
+            ++n_prep_used;
+          } else {
+            int found = -1;
+            wave_resolve<8>(s, found, bits, slot * kSlot + lane * 8, V, kInf);
+            ++n_generic;
+          }
+        } else {
+          float l[8];
+          load_slot_lane<DT>(logits, slot, lane, V, fill, l, fused);
+#pragma unroll
+          for (int k = 0; k < 8; ++k) bits[k] = __float_as_uint(expf_core(__builtin_fmaxf(l[k] * inv - m, -104.0f), tab));
+          int found = -1;
+          wave_resolve<8>(s, found, bits, slot * kSlot + lane * 8, V, kInf);
+          ++n_generic;
+        }
+      }
+      cur = j + 1;
+      ++n_iter;
+    }
+    if (stats && base == 0 && lane == 0) stats[5] = wall_clock64() - c_start;
+  }
+  if (stats && lane == 0) {
+    stats[4] = 0;
+    stats[6] = static_cast<uint64_t>(n_iter) | (static_cast<uint64_t>(n_generic) << 32);
+    stats[7] = static_cast<uint64_t>(n_prep_used) | (static_cast<uint64_t>(n_tie) << 16) | (static_cast<uint64_t>(n_inner) << 32) |
+               (c_prep << 48);
+  }
+  return uniform_f32(s);
+}
+
+// The chain of a multinomial row's probabilities (the same walk as split_chain(), which is kept apart
+// so that the finish kernel's code stays what it was): the records are those of p = fl(e / S) (`div`),
+// and the walk stops at the first entry behind
 // which the running sum exceeds `threshold` (sampler.cpp:58-70): `*stop` is its index (-1: none), the
 // value returned the sum there.  Sums behind records are exact, so the first record behind which
 // the sum exceeds the threshold holds that entry; it is redone entry by entry from the sum in front of it.
-template <int DT, bool WALK = false>
-__device__ __forceinline__ float split_chain(const SlotRec* recs, int ns, const PrepSlot* prep, uint32_t n_prep,
-                                             const char* logits, int V, float inv, float m, const uint64_t* tab,
-                                             const FusedOps& fused, uint64_t* stats = nullptr, const RowDivisor* div = nullptr,
-                                             float threshold = 0.0f, int* stop = nullptr) {
+template <int DT>
+__device__ __forceinline__ float split_chain_walk(const SlotRec* recs, int ns, const PrepSlot* prep, uint32_t n_prep,
+                                                  const char* logits, int V, float inv, float m, const uint64_t* tab,
+                                                  const FusedOps& fused, uint64_t* stats, const RowDivisor* div,
+                                                  float threshold, int* stop) {
+  constexpr bool WALK = true;
   const int lane = threadIdx.x & 63;
   const float kInf = __uint_as_float(0x7f800000u);
   const float fill = inv < 0.0f ? kInf : -kInf;
@@ -974,14 +1083,12 @@ __device__ __forceinline__ float split_chain(const SlotRec* recs, int ns, const 
         return redo(0, 0.0f, *stop);
       }
     }
-    // PARITY: a stable slot with a half-ulp tie inside (one increment for an even sum in front of it,
-    // one for an odd sum) counts as plain, and the prefix is a composition of such pairs (compose()),
+    // A stable slot with a half-ulp tie inside (one increment for an even sum in front of it, one for
+    // an odd sum) counts as plain here, and the prefix is a composition of such pairs (compose()),
     // which follows the parity through the run; it is redone behind every record worked out
-    // exactly while ties lie ahead.  Otherwise such a slot is worked out on its own, and one plain
-    // prefix sum per binade serves.  (The composition costs several times the plain sum: it pays
-    // where ties are many, as among the probabilities of a 16-bit row, few distinct values of
-    // which some sit on a tie every time they occur.)
-    constexpr bool PARITY = WALK;
+    // exactly while ties lie ahead.  (The composition costs several times the plain prefix sum of
+    // split_chain(): it pays where ties are many, as among the probabilities of a 16-bit row, few
+    // distinct values of which some sit on a tie every time they occur.)
     int K_scan = -1, cur_scan = -1;
     ParityInc incl = {0u, 0u};
     uint64_t plain_mask = 0ull, tie_mask = 0ull;
@@ -989,7 +1096,7 @@ __device__ __forceinline__ float split_chain(const SlotRec* recs, int ns, const 
       s = uniform_f32(s);
       const SumState ss = sum_state(s);
       const uint32_t K = static_cast<uint32_t>(ss.kb);
-      if (PARITY) {
+      {
         if (ss.kb != K_scan || (cur != cur_scan && (tie_mask >> cur) != 0ull)) {
           const bool plain = kind == kSlotZero || (kind == kSlotStable && kb == K) || (kind == kSlotDual && (kb == K || kb + 1u == K));
           ParityInc inc = {r.even, r.odd};
@@ -1002,18 +1109,11 @@ __device__ __forceinline__ float split_chain(const SlotRec* recs, int ns, const 
           cur_scan = cur;
           if (stats) n_tie += static_cast<uint32_t>(__popcll(tie_mask));
         }
-      } else if (ss.kb != K_scan) {
-        const bool plain = kind == kSlotZero || (kind == kSlotStable && kb == K && r.even == r.odd) ||
-                           (kind == kSlotDual && (kb == K || kb + 1u == K));
-        const uint32_t inc = kind == kSlotZero ? 0u : ((kind == kSlotDual && kb != K) ? r.odd : r.even);
-        incl.even = wave_scan_inclusive_u32(plain ? inc : 0u);  // 64 values of at most 2^26 each
-        plain_mask = __ballot(plain);
-        K_scan = ss.kb;
       }
       const uint64_t from_cur = ~0ull << cur;
       const uint64_t not_plain = ~plain_mask & from_cur;
       const int jn = not_plain ? __ffsll(static_cast<long long>(not_plain)) - 1 : 64;
-      const uint32_t incl_p = (PARITY && (ss.S & 1u)) ? incl.odd : incl.even;
+      const uint32_t incl_p = (ss.S & 1u) ? incl.odd : incl.even;
       const uint32_t before = cur > 0 ? readlane_u32(incl_p, cur - 1) : 0u;
       const uint32_t S_upto = ss.S + (incl_p - before);
       const uint64_t over = __ballot(lane >= cur && lane < jn && S_upto >= (1u << 24));
@@ -1033,42 +1133,8 @@ __device__ __forceinline__ float split_chain(const SlotRec* recs, int ns, const 
       if (j == 64) break;
       // ---- record base + j, exactly
       const int slot = base + j;
-      const uint32_t kind_j = readlane_u32(kind, j), kb_j = readlane_u32(kb, j);
+      const uint32_t kind_j = readlane_u32(kind, j);
       const float s_front = s;
-      if (!PARITY && j == jn && kind_j == kSlotStable && kb_j == K) {
-        // ---- a tie inside: the increment follows the parity of the sum.  This record, the plain run
-        //      behind it, the next such record and so on, from the prefix sums at hand (a record
-        //      with a tie has none in them), as long as the sum stays inside the binade.
-        uint32_t S_cur = sum_state(s).S;
-        int jj = j, next_cur = -1;
-        while (true) {
-          const uint32_t inc = (S_cur & 1u) ? readlane_u32(r.odd, jj) : readlane_u32(r.even, jj);
-          if (S_cur + inc >= (1u << 24)) {  // leaves the binade inside the record: entry by entry
-            if (jj > j) next_cur = jj;
-            break;
-          }
-          S_cur += inc;
-          ++n_tie;
-          next_cur = jj + 1;
-          if (jj == 63) break;
-          const uint64_t np2 = ~plain_mask & (~0ull << (jj + 1));
-          const int jn2 = np2 ? __ffsll(static_cast<long long>(np2)) - 1 : 64;
-          if (jn2 > jj + 1) {
-            const uint32_t S_run = S_cur + (incl.even - readlane_u32(incl.even, jj));
-            if (__ballot(lane > jj && lane < jn2 && S_run >= (1u << 24)) != 0ull) break;  // (the loop finds where)
-            S_cur = readlane_u32(S_run, jn2 - 1);
-          }
-          next_cur = jn2;
-          if (jn2 == 64 || readlane_u32(kind, jn2) != kSlotStable || readlane_u32(kb, jn2) != K) break;
-          jj = jn2;
-        }
-        if (next_cur >= 0) {
-          s = sum_value(S_cur, ss.kb);
-          cur = next_cur;
-          ++n_iter;
-          continue;
-        }
-      }
       {
         const uint32_t pi = readlane_u32(r.prep, j);
         uint32_t bits[8];
@@ -1699,7 +1765,8 @@ __device__ __noinline__ bool draw_topp_runs(RunArgs a, const char* logits, int V
 // slot records and the prepared slots while the sum is composed.
 // LOOP: fewer workgroups than rows, a workgroup takes one row after the other (the loop costs
 // registers, so a launch with a workgroup per row uses the instantiation without it).
-template <int DT, bool LOOP>
+// TOPK: some row of the launch may be a top-k row.
+template <int DT, bool LOOP, bool TOPK = false>
 __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
   extern __shared__ __align__(16) uint64_t lds_keys[];
   __shared__ BlockScratch sm;
@@ -1943,8 +2010,8 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
   }
   __syncthreads();
   int path = 0;
-  const int32_t topk = p.row.row_cfg ? p.row.row_cfg[row].topk : p.row.topk;
-  if (topk > 0 && topk < V) {
+  const int32_t topk = !TOPK ? 0 : (p.row.row_cfg ? p.row.row_cfg[row].topk : p.row.topk);
+  if (TOPK && topk > 0 && topk < V) {
     // ---- a top-k row (sampler.cpp:72-120, before top-p: :239): pass 2 listed the entries of the
     //      histogram's first buckets, at least topk of them; they are sorted and the first topk walked.
     //      Every probability NaN: every entry ties, the first topk in index order, the last of them drawn.
@@ -2149,7 +2216,7 @@ __global__ void __launch_bounds__(kWalkBlock) split_walk_kernel(SplitParams p, u
     const float2 w = p.walk[row];
     const RowDivisor div = row_divisor(w.x);
     int stop = -1;
-    const float cdf = split_chain<DT, true>(recs, ns, prep, n_prep, logits, V, inv, rs.m, exp2tab, p.row.fused,
+    const float cdf = split_chain_walk<DT>(recs, ns, prep, n_prep, logits, V, inv, rs.m, exp2tab, p.row.fused,
                                             p.timers ? p.timers + static_cast<int64_t>(gridDim.x) * 8 + static_cast<int64_t>(blockIdx.x) * 4 - 4 : nullptr, &div, w.y, &stop);
     if (lane == 0) {
       const int32_t token = stop >= 0 ? stop : V - 1;

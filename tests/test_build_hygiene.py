@@ -30,7 +30,7 @@ def test_hot_kernels_keep_nothing_in_private_memory():
                 "gumbel_partial_kernel" in name or "logit_chain_kernel" in name:
             assert v["ScratchSize"] == 0 and v["VGPRs Spill"] == 0, (name, v)
             seen += 1
-        if "split_finish_kernel" in name and "ELb0E" in name:
+        if re.search(r"split_finish_kernelILi\d+ELb0E", name):  # (the instantiations with a workgroup per row)
             # callee-saved registers of the out-of-line draw functions only
             assert v["ScratchSize"] <= 64 and v["VGPRs Spill"] == 0, (name, v)
             seen += 1
