@@ -447,10 +447,21 @@ ets_status launch_split(ets_sampler* s, const ets::RowParams& p, int32_t rows, h
   }
   ETS_HIP(s, hipGetLastError());
   const size_t lut_bytes = (DT == ets::kDtypeBFloat16 ? sizeof(float) * ets::kLutCountWords : 0) + sizeof(uint32_t) * sp.phist_words;
-  static std::atomic<size_t> set_bytes2[kMaxDevices];
-  st = allow_dynamic_lds(s, reinterpret_cast<const void*>(&ets::split_pass2_kernel<DT, true, false, TOPK>), lut_bytes, set_bytes2);
-  if (st != ETS_OK) return st;
-  hipLaunchKernelGGL((ets::split_pass2_kernel<DT, true, false, TOPK>), dim3(sp.row_wgs, rows), dim3(ets::kBlock), lut_bytes, stream, sp);
+  // (a launch that neither writes the probabilities nor fills the phase clocks runs kernels without those branches)
+  const bool extras = sp.timers != nullptr || p.probs != nullptr;
+  if (extras) {
+    static std::atomic<size_t> set_bytes2[kMaxDevices];
+    st = allow_dynamic_lds(s, reinterpret_cast<const void*>(&ets::split_pass2_kernel<DT, true, false, TOPK, true>), lut_bytes, set_bytes2);
+    if (st != ETS_OK) return st;
+    hipLaunchKernelGGL((ets::split_pass2_kernel<DT, true, false, TOPK, true>), dim3(sp.row_wgs, rows), dim3(ets::kBlock), lut_bytes,
+                       stream, sp);
+  } else {
+    static std::atomic<size_t> set_bytes2[kMaxDevices];
+    st = allow_dynamic_lds(s, reinterpret_cast<const void*>(&ets::split_pass2_kernel<DT, true, false, TOPK, false>), lut_bytes, set_bytes2);
+    if (st != ETS_OK) return st;
+    hipLaunchKernelGGL((ets::split_pass2_kernel<DT, true, false, TOPK, false>), dim3(sp.row_wgs, rows), dim3(ets::kBlock), lut_bytes,
+                       stream, sp);
+  }
   ETS_HIP(s, hipGetLastError());
   if (rows > p.grid_cap) {
     // more rows than workgroups: a workgroup takes up to kChainRows rows at a time
@@ -462,16 +473,30 @@ ets_status launch_split(ets_sampler* s, const ets::RowParams& p, int32_t rows, h
     const int per_wg = (rows + p.grid_cap - 1) / p.grid_cap;
     sp.chain_rows = per_wg < chain_rows_max ? per_wg : chain_rows_max;
     const int units = (rows + sp.chain_rows - 1) / sp.chain_rows;
-    static std::atomic<size_t> set_bytes[kMaxDevices];
-    st = allow_dynamic_lds(s, reinterpret_cast<const void*>(&ets::split_finish_kernel<DT, true, TOPK>), s->lds_bytes, set_bytes);
-    if (st != ETS_OK) return st;
-    hipLaunchKernelGGL((ets::split_finish_kernel<DT, true, TOPK>), dim3(units < p.grid_cap ? units : p.grid_cap), dim3(ets::kBlock),
-                       s->lds_bytes, stream, sp);
+    const dim3 grid(units < p.grid_cap ? units : p.grid_cap);
+    if (extras) {
+      static std::atomic<size_t> set_bytes[kMaxDevices];
+      st = allow_dynamic_lds(s, reinterpret_cast<const void*>(&ets::split_finish_kernel<DT, true, TOPK, true>), s->lds_bytes, set_bytes);
+      if (st != ETS_OK) return st;
+      hipLaunchKernelGGL((ets::split_finish_kernel<DT, true, TOPK, true>), grid, dim3(ets::kBlock), s->lds_bytes, stream, sp);
+    } else {
+      static std::atomic<size_t> set_bytes[kMaxDevices];
+      st = allow_dynamic_lds(s, reinterpret_cast<const void*>(&ets::split_finish_kernel<DT, true, TOPK, false>), s->lds_bytes, set_bytes);
+      if (st != ETS_OK) return st;
+      hipLaunchKernelGGL((ets::split_finish_kernel<DT, true, TOPK, false>), grid, dim3(ets::kBlock), s->lds_bytes, stream, sp);
+    }
   } else {
-    static std::atomic<size_t> set_bytes[kMaxDevices];
-    st = allow_dynamic_lds(s, reinterpret_cast<const void*>(&ets::split_finish_kernel<DT, false, TOPK>), s->lds_bytes, set_bytes);
-    if (st != ETS_OK) return st;
-    hipLaunchKernelGGL((ets::split_finish_kernel<DT, false, TOPK>), dim3(rows), dim3(ets::kBlock), s->lds_bytes, stream, sp);
+    if (extras) {
+      static std::atomic<size_t> set_bytes[kMaxDevices];
+      st = allow_dynamic_lds(s, reinterpret_cast<const void*>(&ets::split_finish_kernel<DT, false, TOPK, true>), s->lds_bytes, set_bytes);
+      if (st != ETS_OK) return st;
+      hipLaunchKernelGGL((ets::split_finish_kernel<DT, false, TOPK, true>), dim3(rows), dim3(ets::kBlock), s->lds_bytes, stream, sp);
+    } else {
+      static std::atomic<size_t> set_bytes[kMaxDevices];
+      st = allow_dynamic_lds(s, reinterpret_cast<const void*>(&ets::split_finish_kernel<DT, false, TOPK, false>), s->lds_bytes, set_bytes);
+      if (st != ETS_OK) return st;
+      hipLaunchKernelGGL((ets::split_finish_kernel<DT, false, TOPK, false>), dim3(rows), dim3(ets::kBlock), s->lds_bytes, stream, sp);
+    }
   }
   ETS_HIP(s, hipGetLastError());
   return ETS_OK;

@@ -494,8 +494,9 @@ __device__ __forceinline__ void split_fold_slot(const SplitParams& p, int row, i
 // WALK: the second sum of a multinomial row (sampler.cpp:58-70): the entries are p = fl(e / S) with the exact
 // softmax sum S that the first chain left in SplitParams::walk, and the records describe their running sum.
 // TOPK: some row of the launch may be a top-k row (a launch without one runs the code without that case).
-template <int DT, bool TOPP, bool WALK = false, bool TOPK = false>
+template <int DT, bool TOPP, bool WALK = false, bool TOPK = false, bool EXTRAS = true>
 __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_kernel(SplitParams p) {
+  uint64_t* const timers = EXTRAS ? p.timers : nullptr;  // (EXTRAS: the launch may fill the phase clocks)
   extern __shared__ __align__(16) float lut_mem[];
   __shared__ Pass2Shared sh;
   BlockScratch& sm = sh.sm;
@@ -517,7 +518,7 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
   const float kInf = __uint_as_float(0x7f800000u);
   const float fill = inv < 0.0f ? kInf : -kInf;
   uint64_t c0 = 0, c1 = 0, c2 = 0, c3 = 0;
-  if (p.timers) c0 = wall_clock64();
+  if (timers) c0 = wall_clock64();
   if (tid < 32) sm.exp2tab[tid] = kExp2Table[tid];
   if (tid == 0) sh.list_count = 0u;
   if (TOPP && tid < 32) {
@@ -577,7 +578,7 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
     return;
   }
   __syncthreads();
-  if (p.timers) c1 = wall_clock64();
+  if (timers) c1 = wall_clock64();
   RowDivisor walk_div = {};
   float walk_scale = 1.0f;
   if (WALK) {
@@ -660,7 +661,7 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
     serial_before += chunk_total;
   }
   const float a_total = carry;
-  if (p.timers) c2 = wall_clock64();
+  if (timers) c2 = wall_clock64();
 
   // ---- bf16 rows: expf by bit pattern
   bool use_lut = false;
@@ -673,7 +674,7 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
     }
   }
   __syncthreads();
-  if (p.timers) c3 = wall_clock64();
+  if (timers) c3 = wall_clock64();
   const LutAddr lut_addr = lut_addr_of(lut_mem, lut_base1, lut_top, lut_half);
 
   const float cutoff = TOPP ? (1.0f - topp) / static_cast<float>(V - 1) : 0.0f;  // sampler.cpp:136
@@ -815,8 +816,8 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
       for (int b = tid; b < (km.n_bins + 1) / 2; b += kBlock) ph_out[b] = ph[b];
     }
   }
-  if (p.timers && blockIdx.x == 0 && tid == 0) {
-    uint64_t* t = p.timers + static_cast<int64_t>(gridDim.y) * 8 + static_cast<int64_t>(blockIdx.y) * 4;
+  if (timers && blockIdx.x == 0 && tid == 0) {
+    uint64_t* t = timers + static_cast<int64_t>(gridDim.y) * 8 + static_cast<int64_t>(blockIdx.y) * 4;
     t[0] = c1 - c0;
     t[1] = c2 - c1;
     t[2] = c3 - c2;
@@ -1765,9 +1766,13 @@ __device__ __noinline__ bool draw_topp_runs(RunArgs a, const char* logits, int V
 // slot records and the prepared slots while the sum is composed.
 // LOOP: fewer workgroups than rows, a workgroup takes one row after the other (the loop costs
 // registers, so a launch with a workgroup per row uses the instantiation without it).
-// TOPK: some row of the launch may be a top-k row.
-template <int DT, bool LOOP, bool TOPK = false>
+// TOPK: some row of the launch may be a top-k row.  EXTRAS: the launch may write the probabilities
+// or fill the phase clocks (a launch that does neither runs the code without them: the branches
+// cost a launch of plain top-p rows more than a microsecond in registers and instructions).
+template <int DT, bool LOOP, bool TOPK = false, bool EXTRAS = true>
 __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
+  uint64_t* const timers = EXTRAS ? p.timers : nullptr;
+  float* const probs_out = EXTRAS ? p.row.probs : nullptr;
   extern __shared__ __align__(16) uint64_t lds_keys[];
   __shared__ BlockScratch sm;
   __shared__ FinishShared fs;
@@ -1821,7 +1826,7 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
         const char* mine = reinterpret_cast<const char*>(lds_keys) + static_cast<size_t>(wave) * share;
         sum = split_chain<DT>(reinterpret_cast<const SlotRec*>(mine), ns, reinterpret_cast<const PrepSlot*>(mine + rec_bytes),
                               prepared(st), logits_k, V, inv_k, st.m, sm.exp2tab, p.row.fused,
-                              p.timers ? p.timers + static_cast<int64_t>(row_k) * 8 : nullptr);
+                              timers ? timers + static_cast<int64_t>(row_k) * 8 : nullptr);
       }
       if (lane == 0) fs.pre_sum[wave] = sum;
     }
@@ -1857,7 +1862,7 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
   const bool row_nan = rs.nan != 0u;
   const float cutoff = (1.0f - topp) / static_cast<float>(V - 1);  // sampler.cpp:136
   uint64_t t0 = 0, t1 = 0, t2 = 0;
-  if (p.timers) t0 = wall_clock64();
+  if (timers) t0 = wall_clock64();
   if (tid < 32) sm.exp2tab[tid] = kExp2Table[tid];
   if (tid == 0) fs.fused = p.row.fused;  // (barriers follow before any draw function reads it)
   uint64_t coin_state = 0ull;  // asked for now, needed once the sum is known
@@ -1934,12 +1939,12 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
     n_listed = static_cast<int>(fs.offset[p.row_wgs]);
     lists_ok = fs.overflow == 0u;
     plan = split_plan(fs.hist, rs.a_total, topp, cutoff, V, &fs.plan, sm);
-    if (p.timers) t1 = wall_clock64();
+    if (timers) t1 = wall_clock64();
     if (wave == 0) {
       if (!chained) {
         const float sum = split_chain<DT>(reinterpret_cast<const SlotRec*>(lds_keys), ns,
                                           reinterpret_cast<const PrepSlot*>(prep_dst), n_prep, logits, V, inv, m, sm.exp2tab,
-                                          p.row.fused, p.timers ? p.timers + static_cast<int64_t>(row) * 8 : nullptr);
+                                          p.row.fused, timers ? timers + static_cast<int64_t>(row) * 8 : nullptr);
         if (lane == 0) sm.bc_sum = sum;
       } else if (lane == 0) {
         sm.bc_sum = fs.pre_sum[lrow - r_first];
@@ -1966,7 +1971,7 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
     }
     __syncthreads();
     S = sm.bc_sum;
-    if (p.timers) t2 = wall_clock64();
+    if (timers) t2 = wall_clock64();
   }
 
   // ---- one coin per call (sampler.cpp:237, 210-220)
@@ -1983,8 +1988,8 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
   const float coin = sm.red_f[0];
   __syncthreads();
 
-  if (p.row.probs) {
-    float* probs = p.row.probs + static_cast<int64_t>(row) * V;
+  if (probs_out) {
+    float* probs = probs_out + static_cast<int64_t>(row) * V;
     if (row_nan) {
       for (int i = tid; i < V; i += kBlock) {
         const float x = load_logit<DT>(logits, i, p.row.fused) * inv;
@@ -2142,8 +2147,8 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
   if (tid == 0) {
     p.row.tokens[row] = token;
     if (p.row.debug) p.row.debug[row] = dbg;
-    if (p.timers) {
-      uint64_t* t = p.timers + static_cast<int64_t>(row) * 8;
+    if (timers) {
+      uint64_t* t = timers + static_cast<int64_t>(row) * 8;
       t[0] = t1 - t0;
       t[1] = t2 - t1;
       t[2] = wall_clock64() - t2;
