@@ -371,7 +371,7 @@ def bench_floors(w, ring, torch, dev):
 
     from executorch_amd import _capi
 
-    L = _capi.lib()
+    L = _capi.hooks()
     stream = torch.cuda.current_stream(dev).cuda_stream
     sink = torch.zeros(4, dtype=torch.int32, device=dev)
     empty_us = timed_us(lambda: L.ets_test_empty_launch(stream), 200, torch, repeats=5)
@@ -385,6 +385,17 @@ def bench_floors(w, ring, torch, dev):
         us = timed_us(step, 100, torch, repeats=5)
         res[f"read_{wgs}_workgroups_us"] = us
         res[f"read_{wgs}_workgroups_gbs"] = w.bytes_per_step / (us * 1e-6) / 1e9
+    # a hand-over between two workgroups through a word in device memory (release by one, bounded
+    # polling by the other): microseconds per one-way signal, on another die and on the same one
+    hops = 2000
+    for label, partner in (("other_xcd", 1), ("same_xcd", 8)):
+        words = torch.zeros(64, dtype=torch.int32, device=dev)
+        res_w = torch.zeros(4, dtype=torch.int32, device=dev)
+        st = L.ets_test_signal_floor(words.data_ptr(), hops, 1 << 16, partner, res_w.data_ptr(), stream)
+        torch.cuda.synchronize()
+        ticks = res_w.cpu().numpy().astype("uint32")
+        ok = st == 0 and int(ticks[0]) == 0
+        res[f"signal_{label}_us"] = float(ticks[1]) * 0.01 / (2 * hops) if ok else None  # (100 MHz clock)
     return res
 
 
@@ -533,7 +544,7 @@ def main():
         dst = torch.empty_like(src)
         for _ in range(5):
             from executorch_amd import _capi
-            st = _capi.lib().ets_test_copy_probe(src.data_ptr(), dst.data_ptr(), COPY_PROBE_BYTES, torch.cuda.current_stream().cuda_stream)
+            st = _capi.hooks().ets_test_copy_probe(src.data_ptr(), dst.data_ptr(), COPY_PROBE_BYTES, torch.cuda.current_stream().cuda_stream)
             assert st == 0
         torch.cuda.synchronize()
         del src, dst

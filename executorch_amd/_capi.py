@@ -10,6 +10,7 @@ import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libet_sampler.so")
+HOOKS_PATH = os.path.join(HERE, "libet_sampler_hooks.so")  # csrc/ets_test_hooks.h: tests and the benchmark only
 
 OK, INTERNAL, INVALID_STATE, NOT_SUPPORTED, INVALID_ARGUMENT, MEMORY_ALLOCATION_FAILED = 0x00, 0x01, 0x02, 0x10, 0x12, 0x21
 DTYPE_HALF, DTYPE_FLOAT, DTYPE_BFLOAT16, DTYPE_UINT16 = 5, 6, 15, 27
@@ -81,8 +82,10 @@ CHAIN_SIGNATURES = {
     "ets_logit_chain_last_error": (C.c_char_p, [C.c_void_p]),
 }
 
-# csrc/ets_test_hooks.h
+# csrc/ets_test_hooks.h (libet_sampler_hooks.so)
 TEST_HOOKS = {
+    "ets_test_signal_floor": (C.c_int32, [C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p]),
+    "ets_test_last_error": (C.c_char_p, []),
     "ets_test_expf": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p]),
     "ets_test_seq_sum": (C.c_int32, [C.c_void_p, C.c_int32, C.c_float, C.c_float, C.c_void_p, C.c_void_p, C.c_void_p]),
     "ets_test_split_timers": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int32]),
@@ -92,20 +95,33 @@ TEST_HOOKS = {
 }
 
 _lib = None
+_hooks = None
+
+
+def _load(path: str, tables) -> C.CDLL:
+    if not os.path.exists(path):
+        raise RuntimeError(
+            f"{path} is missing: build it with `python -m executorch_amd.build` "
+            "(there is no CPU fallback for the sampler)")
+    L = C.CDLL(path)
+    for table in tables:
+        for name, (res, args) in table.items():
+            f = getattr(L, name)
+            f.restype = res
+            f.argtypes = args
+    return L
 
 
 def lib() -> C.CDLL:
     global _lib
     if _lib is None:
-        if not os.path.exists(LIB_PATH):
-            raise RuntimeError(
-                f"{LIB_PATH} is missing: build it with `python -m executorch_amd.build` "
-                "(there is no CPU fallback for the sampler)")
-        L = C.CDLL(LIB_PATH)
-        for table in (SIGNATURES, CHAIN_SIGNATURES, TEST_HOOKS):
-            for name, (res, args) in table.items():
-                f = getattr(L, name)
-                f.restype = res
-                f.argtypes = args
-        _lib = L
+        _lib = _load(LIB_PATH, (SIGNATURES, CHAIN_SIGNATURES))
     return _lib
+
+
+def hooks() -> C.CDLL:
+    """The test and measurement hooks: a library of their own, not part of the product."""
+    global _hooks
+    if _hooks is None:
+        _hooks = _load(HOOKS_PATH, (TEST_HOOKS,))
+    return _hooks

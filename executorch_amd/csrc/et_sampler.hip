@@ -15,9 +15,8 @@
 
 #include <cstdlib>
 
-#include "ets_kernels.h"
-#include "ets_split.h"
-#include "ets_test_hooks.h"
+#include "ets_host.h"
+
 
 namespace {
 
@@ -29,77 +28,7 @@ struct ErrorSink {
 
 }  // namespace
 
-// Device memory a call works in beyond its inputs and outputs, when it is not the handle's own:
-// the entry point that allocates nothing lays it out inside the library's static array.
-struct WorkBuffers {
-  ets::SplitParams split = {};
-  uint64_t* scratch = nullptr;  // [rows, scratch_stride] keys of the general draw
-  uint32_t* tickets = nullptr;
-  int32_t scratch_rows = 0;
-  int64_t scratch_stride = 0;
-  uint64_t* partials = nullptr;  // [rows, kMaxSplits] arg-max partial results
-  int max_row_wgs = 0;           // workgroups of pass 2 per row, at most
-};
-
-struct ets_sampler {
-  const WorkBuffers* wb = nullptr;  // set for the duration of a call that brings its own buffers
-  int32_t vocab = 0;
-  float inv_temperature = 0.0f;
-  float topp = 0.9f;
-  int32_t topk = 0;
-  int32_t max_batch = 0;
-  int device = 0;
-  int lds_keys = 0;            // keys that fit in the dynamic LDS sort buffer (power of two)
-  size_t lds_bytes = 0;
-  int64_t scratch_stride = 0;  // keys per row of candidate scratch (twice the vocabulary, rounded up)
-  uint64_t* d_rng = nullptr;       // [max_batch]
-  uint32_t* d_tickets = nullptr;   // row counters of the row kernels' launches (0 between launches), one per draw
-  int32_t scratch_rows = 0;        // rows of candidate scratch: one per workgroup that can be resident, not one per row
-  uint64_t* d_scratch = nullptr;   // [max_batch, scratch_stride], allocated on first stochastic use
-  uint64_t* d_partials = nullptr;  // [max_batch, kMaxSplits] argmax partial results
-  void* d_row = nullptr;           // staging for one host row (vocab * 4 bytes)
-  int32_t* d_token = nullptr;      // staging for one token
-  // work buffers of the path that spreads a row over several workgroups (ets_split.h): one
-  // allocation, made on first use
-  size_t split_row_wgs = 0;  // (row, workgroup) pairs of the largest launch
-  int split_mode = 0;  // ETS_ROW_SPLIT_AUTO
-  int num_cus = 0;
-  void* d_split = nullptr;
-  void* d_phist = nullptr;  // pattern histograms of 16-bit rows, allocated on their first use
-  ets::SplitParams split = {};
-  // per-row sampling parameters of ets_sampler_sample_batch_configs(): pinned host staging, its
-  // device copy, and the event that says the last upload has left the staging buffer
-  void* h_stage = nullptr;
-  void* d_stage = nullptr;
-  hipEvent_t stage_event = nullptr;
-  bool stage_pending = false;
-  // the last stream a call that uses the staging copy ran on, and the event behind its launches: a
-  // call on another stream waits for it before it overwrites the device copy
-  hipEvent_t stage_done = nullptr;
-  hipStream_t stage_stream = nullptr;
-  bool stage_used = false;
-  // ets_sampler_sample_batch_configs(): rows that take different launches run side by side, one
-  // group on the call's stream and the others on a second stream (default priority) that starts
-  // behind the call's stream and is joined again before the call returns
-  hipStream_t aux_stream = nullptr;
-  hipEvent_t fork_event = nullptr;
-  hipEvent_t join_event = nullptr;
-  // opt-in device timing (ets_sampler_set_timing): a ring of event pairs around the launches of a
-  // call, harvested when a slot is reused or the totals are read
-  bool timing = false;
-  static constexpr int kTimingSlots = 32;
-  hipEvent_t t_begin[kTimingSlots] = {};
-  hipEvent_t t_end[kTimingSlots] = {};
-  int32_t t_rows[kTimingSlots] = {};
-  bool t_busy[kTimingSlots] = {};
-  uint64_t t_next = 0;
-  ets_sampler_stats stats = {};
-  std::string last_error;
-};
-
-namespace {
-
-constexpr int kMaxSplits = 64;
+namespace ets_host {
 
 ets_status fail(ets_sampler* s, ets_status code, const std::string& msg) {
   if (s) {
@@ -115,11 +44,106 @@ ets_status hip_fail(ets_sampler* s, hipError_t e, const char* what) {
               std::string(what) + ": " + hipGetErrorString(e));
 }
 
-#define ETS_HIP(s, call)                                  \
-  do {                                                    \
-    hipError_t e_ = (call);                               \
-    if (e_ != hipSuccess) return hip_fail(s, e_, #call);  \
-  } while (0)
+// Raises a kernel's dynamic-LDS limit to `bytes` on the handle's device.  The limit is kept per
+// kernel and device, so it is set again only when a handle asks for more than was set before.
+ets_status allow_dynamic_lds(ets_sampler* s, const void* kernel, size_t bytes, std::atomic<size_t>* set_bytes) {
+  const int dev = s->device >= 0 && s->device < kMaxDevices ? s->device : 0;
+  if (set_bytes[dev].load(std::memory_order_acquire) >= bytes) return ETS_OK;
+  ETS_HIP(s, hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(bytes)));
+  set_bytes[dev].store(bytes, std::memory_order_release);
+  return ETS_OK;
+}
+
+// ---- rows spread over several workgroups (ets_split.h) -------------------------------------------
+
+// Workgroups per row of pass 2: as many as keep the launch within one workgroup per CU (a second,
+// partly filled round would cost more than the longer sweeps), sixteen slots each at least.
+// (ETS_SPLIT_WORKGROUPS forces a number; not for a call that brings its own work buffers, whose
+// layout was made for the automatic choice.)
+int pass2_workgroups(const ets_sampler* s, int32_t rows, int32_t ns) {
+  static const int forced = [] {
+    const char* e = std::getenv("ETS_SPLIT_WORKGROUPS");
+    return e ? std::atoi(e) : 0;
+  }();
+  int g = (forced > 0 && !s->wb) ? forced : (s->num_cus > 0 ? s->num_cus : 256) / rows;
+  const int by_len = (ns + 15) / 16;
+  if (g > by_len) g = by_len;
+  if (g > ets::kMaxRowWorkgroups) g = ets::kMaxRowWorkgroups;
+  if (s->wb && g > s->wb->max_row_wgs) g = s->wb->max_row_wgs;
+  return g < 1 ? 1 : g;
+}
+
+// Candidates one workgroup of pass 2 can list when `g` of them share a row: all of its entries,
+// up to kListRegion.
+int32_t list_region(int32_t ns, int g) {
+  const int per_wg = ((ns + g - 1) / g + 15) / 16 * 16;
+  const int64_t entries = static_cast<int64_t>(per_wg) * ets::kSlot;
+  return static_cast<int32_t>(entries < ets::kListRegion ? entries : ets::kListRegion);
+}
+
+ets_status ensure_split(ets_sampler* s) {
+  if (s->d_split) return ETS_OK;
+  ets::SplitParams& sp = s->split;
+  const size_t rows = static_cast<size_t>(s->max_batch);
+  sp.ns = (s->vocab + ets::kSlot - 1) / ets::kSlot;
+  sp.ns_stride = static_cast<int32_t>(round_up(static_cast<size_t>(sp.ns), 4));
+  sp.prep_cap = ets::kPrepCap;
+  // the candidate lists of the largest launch: rows x workgroups per row x region
+  size_t list_entries = 0, row_wgs = 0;
+  for (int32_t r = 1; r <= s->max_batch; ++r) {
+    const int g = pass2_workgroups(s, r, sp.ns);
+    const size_t need = static_cast<size_t>(r) * g * list_region(sp.ns, g);
+    if (need > list_entries) list_entries = need;
+    if (static_cast<size_t>(r) * g > row_wgs) row_wgs = static_cast<size_t>(r) * g;
+  }
+  size_t at = 0;
+  auto take = [&](size_t bytes) {
+    const size_t here = at;
+    at = round_up(at + bytes, 256);
+    return here;
+  };
+  const size_t o_max = take(rows * sp.ns_stride * sizeof(float));
+  const size_t o_max2 = take(rows * sp.ns_stride * sizeof(float));
+  const size_t o_sum = take(rows * sp.ns_stride * sizeof(float));
+  const size_t o_rec = take(rows * sp.ns_stride * sizeof(ets::SlotRec));
+  const size_t o_prep = take(rows * sp.prep_cap * sizeof(ets::PrepSlot));
+  const size_t o_state = take(rows * sizeof(ets::RowState));
+  const size_t o_walk = take(rows * sizeof(float2));
+  const size_t o_count = take(rows * ets::kMaxRowWorkgroups * sizeof(uint32_t));
+  const size_t o_timers = take(rows * 12 * sizeof(uint64_t));
+  const size_t o_hist = take(row_wgs * ets::kHistBuckets * sizeof(uint32_t));
+  const size_t o_list = take(list_entries * sizeof(uint64_t));
+  ETS_HIP(s, hipMalloc(&s->d_split, at));
+  char* base = static_cast<char*>(s->d_split);
+  sp.slot_max = reinterpret_cast<float*>(base + o_max);
+  sp.slot_max2 = reinterpret_cast<float*>(base + o_max2);
+  sp.slot_sum = reinterpret_cast<float*>(base + o_sum);
+  sp.slot_rec = reinterpret_cast<ets::SlotRec*>(base + o_rec);
+  sp.prep = reinterpret_cast<ets::PrepSlot*>(base + o_prep);
+  sp.row_state = reinterpret_cast<ets::RowState*>(base + o_state);
+  sp.walk = reinterpret_cast<float2*>(base + o_walk);
+  sp.list_count = reinterpret_cast<uint32_t*>(base + o_count);
+  sp.hist = reinterpret_cast<uint32_t*>(base + o_hist);
+  sp.list = reinterpret_cast<uint64_t*>(base + o_list);
+  sp.timers = (ETS_PHASE_CLOCKS && std::getenv("ETS_SPLIT_TIMERS")) ? reinterpret_cast<uint64_t*>(base + o_timers) : nullptr;  // (profiling builds only)
+  s->split_row_wgs = row_wgs;
+  return ETS_OK;
+}
+
+
+ets_status ensure_phist(ets_sampler* s) {
+  if (s->d_phist) return ETS_OK;
+  const size_t bytes = round_up(s->split_row_wgs * kPhistWordsHalf * sizeof(uint32_t), 256);
+  ETS_HIP(s, hipMalloc(&s->d_phist, bytes));
+  s->split.phist = static_cast<uint32_t*>(s->d_phist);
+  return ETS_OK;
+}
+
+}  // namespace ets_host
+
+using namespace ets_host;
+
+namespace {
 
 bool dtype_ok(int32_t dtype) {
   return dtype == ETS_DTYPE_FLOAT || dtype == ETS_DTYPE_HALF || dtype == ETS_DTYPE_BFLOAT16 ||
@@ -211,72 +235,11 @@ ets_status launch_argmax(ets_sampler* s, const void* d_logits, int32_t batch, in
   return ETS_OK;
 }
 
-// Raises a kernel's dynamic-LDS limit to `bytes` on the handle's device.  The limit is kept per
-// kernel and device, so it is set again only when a handle asks for more than was set before.
-constexpr int kMaxDevices = 64;
-ets_status allow_dynamic_lds(ets_sampler* s, const void* kernel, size_t bytes, std::atomic<size_t>* set_bytes) {
-  const int dev = s->device >= 0 && s->device < kMaxDevices ? s->device : 0;
-  if (set_bytes[dev].load(std::memory_order_acquire) >= bytes) return ETS_OK;
-  ETS_HIP(s, hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(bytes)));
-  set_bytes[dev].store(bytes, std::memory_order_release);
-  return ETS_OK;
-}
-
-template <int DT, bool ALIGNED, int DRAW, bool LOOP>
-ets_status launch_rows_looped(ets_sampler* s, const ets::RowParams& p, int grid, hipStream_t stream) {
-  static std::atomic<size_t> set_bytes[kMaxDevices];
-  const size_t lds = s->lds_bytes;
-  ets_status st = allow_dynamic_lds(s, reinterpret_cast<const void*>(&ets::sample_rows_kernel<DT, ALIGNED, DRAW, LOOP>), lds, set_bytes);
-  if (st != ETS_OK) return st;
-  hipLaunchKernelGGL((ets::sample_rows_kernel<DT, ALIGNED, DRAW, LOOP>), dim3(grid), dim3(ets::kBlock), lds, stream, p);
-  ETS_HIP(s, hipGetLastError());
-  return ETS_OK;
-}
-
-template <int DT, bool ALIGNED, int DRAW>
-ets_status launch_rows_impl(ets_sampler* s, const ets::RowParams& p_in, int32_t batch, hipStream_t stream) {
-  ets::RowParams p = p_in;
-  p.rows = batch;
-  p.ticket = (s->wb ? s->wb->tickets : s->d_tickets) + DRAW;
-  // a workgroup per row while the scratch rows last; beyond that the rows are handed out by ticket
-  return batch > p.grid_cap ? launch_rows_looped<DT, ALIGNED, DRAW, true>(s, p, p.grid_cap, stream)
-                            : launch_rows_looped<DT, ALIGNED, DRAW, false>(s, p, batch, stream);
-}
-
 // Which draw follows the softmax (sampler.cpp:238-249).
 int draw_mode(int32_t vocab, float topp, int32_t topk) {
   if (topk > 0 && topk < vocab) return ets::kDrawTopK;
   if (topp <= 0.0f || topp >= 1.0f) return ets::kDrawMultinomial;
   return ets::kDrawTopP;
-}
-
-template <int DT>
-ets_status launch_rows(ets_sampler* s, const ets::RowParams& p, int32_t batch, hipStream_t stream, int draw) {
-  // 128-bit loads need a 16-byte aligned base and row pitch
-  const size_t esz = ets::ElemSize<DT>::value;
-  const bool aligned = (reinterpret_cast<uintptr_t>(p.logits) % 16 == 0) && ((static_cast<size_t>(p.row_stride) * esz) % 16 == 0);
-  // one kernel instantiation per draw
-  const bool use_topk = draw == ets::kDrawTopK;
-  const bool use_mult = draw == ets::kDrawMultinomial;
-  if (draw == ets::kDrawAny) {
-    // rows of different draws in one launch (the looping instantiation serves every batch size)
-    ets::RowParams q = p;
-    q.rows = batch;
-    q.ticket = (s->wb ? s->wb->tickets : s->d_tickets) + 4;  // (0 .. 2: the launches of one draw, 3: the finish kernel)
-    const int grid = batch < q.grid_cap ? batch : q.grid_cap;
-    return aligned ? launch_rows_looped<DT, true, ets::kDrawAny, true>(s, q, grid, stream)
-                   : launch_rows_looped<DT, false, ets::kDrawAny, true>(s, q, grid, stream);
-  }
-  if (use_topk) {
-    return aligned ? launch_rows_impl<DT, true, ets::kDrawTopK>(s, p, batch, stream)
-                   : launch_rows_impl<DT, false, ets::kDrawTopK>(s, p, batch, stream);
-  }
-  if (use_mult) {
-    return aligned ? launch_rows_impl<DT, true, ets::kDrawMultinomial>(s, p, batch, stream)
-                   : launch_rows_impl<DT, false, ets::kDrawMultinomial>(s, p, batch, stream);
-  }
-  return aligned ? launch_rows_impl<DT, true, ets::kDrawTopP>(s, p, batch, stream)
-                 : launch_rows_impl<DT, false, ets::kDrawTopP>(s, p, batch, stream);
 }
 
 float inverse_temperature_ctor(float temperature) {
@@ -310,93 +273,6 @@ const char* const kUint16Message =
     "0/1 weights); use temperature 0 or dequantise first";
 
 
-// ---- rows spread over several workgroups (ets_split.h) -------------------------------------------
-size_t round_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
-
-// Workgroups per row of pass 2: as many as keep the launch within one workgroup per CU (a second,
-// partly filled round would cost more than the longer sweeps), sixteen slots each at least.
-int pass2_workgroups(const ets_sampler* s, int32_t rows, int32_t ns) {
-  static const int forced = [] {
-    const char* e = std::getenv("ETS_SPLIT_WORKGROUPS");
-    return e ? std::atoi(e) : 0;
-  }();
-  int g = forced > 0 ? forced : (s->num_cus > 0 ? s->num_cus : 256) / rows;
-  const int by_len = (ns + 15) / 16;
-  if (g > by_len) g = by_len;
-  if (g > ets::kMaxRowWorkgroups) g = ets::kMaxRowWorkgroups;
-  if (s->wb && g > s->wb->max_row_wgs) g = s->wb->max_row_wgs;
-  return g < 1 ? 1 : g;
-}
-
-// Candidates one workgroup of pass 2 can list when `g` of them share a row: all of its entries,
-// up to kListRegion.
-int32_t list_region(int32_t ns, int g) {
-  const int per_wg = ((ns + g - 1) / g + 15) / 16 * 16;
-  const int64_t entries = static_cast<int64_t>(per_wg) * ets::kSlot;
-  return static_cast<int32_t>(entries < ets::kListRegion ? entries : ets::kListRegion);
-}
-
-ets_status ensure_split(ets_sampler* s) {
-  if (s->d_split) return ETS_OK;
-  ets::SplitParams& sp = s->split;
-  const size_t rows = static_cast<size_t>(s->max_batch);
-  sp.ns = (s->vocab + ets::kSlot - 1) / ets::kSlot;
-  sp.ns_stride = static_cast<int32_t>(round_up(static_cast<size_t>(sp.ns), 4));
-  sp.prep_cap = ets::kPrepCap;
-  // the candidate lists of the largest launch: rows x workgroups per row x region
-  size_t list_entries = 0, row_wgs = 0;
-  for (int32_t r = 1; r <= s->max_batch; ++r) {
-    const int g = pass2_workgroups(s, r, sp.ns);
-    const size_t need = static_cast<size_t>(r) * g * list_region(sp.ns, g);
-    if (need > list_entries) list_entries = need;
-    if (static_cast<size_t>(r) * g > row_wgs) row_wgs = static_cast<size_t>(r) * g;
-  }
-  size_t at = 0;
-  auto take = [&](size_t bytes) {
-    const size_t here = at;
-    at = round_up(at + bytes, 256);
-    return here;
-  };
-  const size_t o_max = take(rows * sp.ns_stride * sizeof(float));
-  const size_t o_max2 = take(rows * sp.ns_stride * sizeof(float));
-  const size_t o_sum = take(rows * sp.ns_stride * sizeof(float));
-  const size_t o_rec = take(rows * sp.ns_stride * sizeof(ets::SlotRec));
-  const size_t o_prep = take(rows * sp.prep_cap * sizeof(ets::PrepSlot));
-  const size_t o_state = take(rows * sizeof(ets::RowState));
-  const size_t o_walk = take(rows * sizeof(float2));
-  const size_t o_count = take(rows * ets::kMaxRowWorkgroups * sizeof(uint32_t));
-  const size_t o_timers = take(rows * 12 * sizeof(uint64_t));
-  const size_t o_hist = take(row_wgs * ets::kHistBuckets * sizeof(uint32_t));
-  const size_t o_list = take(list_entries * sizeof(uint64_t));
-  ETS_HIP(s, hipMalloc(&s->d_split, at));
-  char* base = static_cast<char*>(s->d_split);
-  sp.slot_max = reinterpret_cast<float*>(base + o_max);
-  sp.slot_max2 = reinterpret_cast<float*>(base + o_max2);
-  sp.slot_sum = reinterpret_cast<float*>(base + o_sum);
-  sp.slot_rec = reinterpret_cast<ets::SlotRec*>(base + o_rec);
-  sp.prep = reinterpret_cast<ets::PrepSlot*>(base + o_prep);
-  sp.row_state = reinterpret_cast<ets::RowState*>(base + o_state);
-  sp.walk = reinterpret_cast<float2*>(base + o_walk);
-  sp.list_count = reinterpret_cast<uint32_t*>(base + o_count);
-  sp.hist = reinterpret_cast<uint32_t*>(base + o_hist);
-  sp.list = reinterpret_cast<uint64_t*>(base + o_list);
-  sp.timers = std::getenv("ETS_SPLIT_TIMERS") ? reinterpret_cast<uint64_t*>(base + o_timers) : nullptr;
-  s->split_row_wgs = row_wgs;
-  return ETS_OK;
-}
-
-// Words of packed 16-bit counters per (row, workgroup) of the pattern histogram: what fits in
-// pass 2's LDS next to the expf table.
-constexpr int kPhistWordsHalf = 24576, kPhistWordsBFloat16 = 8192;
-
-ets_status ensure_phist(ets_sampler* s) {
-  if (s->d_phist) return ETS_OK;
-  const size_t bytes = round_up(s->split_row_wgs * kPhistWordsHalf * sizeof(uint32_t), 256);
-  ETS_HIP(s, hipMalloc(&s->d_phist, bytes));
-  s->split.phist = static_cast<uint32_t*>(s->d_phist);
-  return ETS_OK;
-}
-
 // Whether rows with draw `draw` take the path that spreads a row over several workgroups.
 // (Top-p rows; top-k rows whose k the slots' largest entries can vouch for, two per slot; multinomial
 // rows, by five launches instead of three, unless the caller wants the probabilities written.)
@@ -411,153 +287,14 @@ bool use_split(const ets_sampler* s, const void* d_logits, int64_t stride, int32
   return s->split_mode == ETS_ROW_SPLIT_ON || s->vocab >= 8192;
 }
 
-// TOPK: some row may be a top-k row (the kernels of a launch without one leave that case out).
-template <int DT, bool TOPK>
-ets_status launch_split(ets_sampler* s, const ets::RowParams& p, int32_t rows, hipStream_t stream) {
-  ets_status st = ETS_OK;
-  constexpr bool k16 = DT == ets::kDtypeBFloat16 || DT == ets::kDtypeHalf;
-  if (!s->wb) {
-    st = ensure_split(s);
-    if (st != ETS_OK) return st;
-    if (k16) {
-      st = ensure_phist(s);
-      if (st != ETS_OK) return st;
-    }
-  }
-  ets::SplitParams sp = s->wb ? s->wb->split : s->split;
-  sp.row = p;
-  sp.row.rows = rows;
-  sp.row.ticket = (s->wb ? s->wb->tickets : s->d_tickets) + 3;  // (0 .. 2 are the one-workgroup-per-row kernel's, by draw)
-  sp.phist_words = DT == ets::kDtypeBFloat16 ? kPhistWordsBFloat16 : (DT == ets::kDtypeHalf ? kPhistWordsHalf : 0);
-  sp.row_wgs = pass2_workgroups(s, rows, sp.ns);
-  sp.list_region = list_region(sp.ns, sp.row_wgs);
-  static const int short_lists = [] {
-    const char* e = std::getenv("ETS_SHORT_LISTS");  // 0: pass 2 lists every possible candidate, always
-    return e ? std::atoi(e) : 1;
-  }();
-  sp.short_lists = short_lists;
-  if (rows <= 256) {
-    const int per_block = (ets::kPass1Block / 64) * 2;
-    hipLaunchKernelGGL((ets::split_pass1_kernel<DT, 2>), dim3((sp.ns + per_block - 1) / per_block, rows), dim3(ets::kPass1Block),
-                       0, stream, sp);
-  } else {
-    const int per_block = (ets::kPass1Block / 64) * 4;
-    hipLaunchKernelGGL((ets::split_pass1_kernel<DT, 4>), dim3((sp.ns + per_block - 1) / per_block, rows), dim3(ets::kPass1Block),
-                       0, stream, sp);
-  }
-  ETS_HIP(s, hipGetLastError());
-  const size_t lut_bytes = (DT == ets::kDtypeBFloat16 ? sizeof(float) * ets::kLutCountWords : 0) + sizeof(uint32_t) * sp.phist_words;
-  // (a launch that neither writes the probabilities nor fills the phase clocks runs kernels without those branches)
-  const bool extras = sp.timers != nullptr || p.probs != nullptr;
-  if (extras) {
-    static std::atomic<size_t> set_bytes2[kMaxDevices];
-    st = allow_dynamic_lds(s, reinterpret_cast<const void*>(&ets::split_pass2_kernel<DT, true, false, TOPK, true>), lut_bytes, set_bytes2);
-    if (st != ETS_OK) return st;
-    hipLaunchKernelGGL((ets::split_pass2_kernel<DT, true, false, TOPK, true>), dim3(sp.row_wgs, rows), dim3(ets::kBlock), lut_bytes,
-                       stream, sp);
-  } else {
-    static std::atomic<size_t> set_bytes2[kMaxDevices];
-    st = allow_dynamic_lds(s, reinterpret_cast<const void*>(&ets::split_pass2_kernel<DT, true, false, TOPK, false>), lut_bytes, set_bytes2);
-    if (st != ETS_OK) return st;
-    hipLaunchKernelGGL((ets::split_pass2_kernel<DT, true, false, TOPK, false>), dim3(sp.row_wgs, rows), dim3(ets::kBlock), lut_bytes,
-                       stream, sp);
-  }
-  ETS_HIP(s, hipGetLastError());
-  if (rows > p.grid_cap) {
-    // more rows than workgroups: a workgroup takes up to kChainRows rows at a time
-    static const int chain_rows_max = [] {
-      const char* e = std::getenv("ETS_CHAIN_ROWS");
-      const int v = e ? std::atoi(e) : ets::kChainRows;
-      return v < 1 ? 1 : (v > ets::kChainRows ? ets::kChainRows : v);
-    }();
-    const int per_wg = (rows + p.grid_cap - 1) / p.grid_cap;
-    sp.chain_rows = per_wg < chain_rows_max ? per_wg : chain_rows_max;
-    const int units = (rows + sp.chain_rows - 1) / sp.chain_rows;
-    const dim3 grid(units < p.grid_cap ? units : p.grid_cap);
-    if (extras) {
-      static std::atomic<size_t> set_bytes[kMaxDevices];
-      st = allow_dynamic_lds(s, reinterpret_cast<const void*>(&ets::split_finish_kernel<DT, true, TOPK, true>), s->lds_bytes, set_bytes);
-      if (st != ETS_OK) return st;
-      hipLaunchKernelGGL((ets::split_finish_kernel<DT, true, TOPK, true>), grid, dim3(ets::kBlock), s->lds_bytes, stream, sp);
-    } else {
-      static std::atomic<size_t> set_bytes[kMaxDevices];
-      st = allow_dynamic_lds(s, reinterpret_cast<const void*>(&ets::split_finish_kernel<DT, true, TOPK, false>), s->lds_bytes, set_bytes);
-      if (st != ETS_OK) return st;
-      hipLaunchKernelGGL((ets::split_finish_kernel<DT, true, TOPK, false>), grid, dim3(ets::kBlock), s->lds_bytes, stream, sp);
-    }
-  } else {
-    if (extras) {
-      static std::atomic<size_t> set_bytes[kMaxDevices];
-      st = allow_dynamic_lds(s, reinterpret_cast<const void*>(&ets::split_finish_kernel<DT, false, TOPK, true>), s->lds_bytes, set_bytes);
-      if (st != ETS_OK) return st;
-      hipLaunchKernelGGL((ets::split_finish_kernel<DT, false, TOPK, true>), dim3(rows), dim3(ets::kBlock), s->lds_bytes, stream, sp);
-    } else {
-      static std::atomic<size_t> set_bytes[kMaxDevices];
-      st = allow_dynamic_lds(s, reinterpret_cast<const void*>(&ets::split_finish_kernel<DT, false, TOPK, false>), s->lds_bytes, set_bytes);
-      if (st != ETS_OK) return st;
-      hipLaunchKernelGGL((ets::split_finish_kernel<DT, false, TOPK, false>), dim3(rows), dim3(ets::kBlock), s->lds_bytes, stream, sp);
-    }
-  }
-  ETS_HIP(s, hipGetLastError());
-  return ETS_OK;
-}
-
-// Multinomial rows that use_split() accepted: five launches (ets_split.h, split_walk_kernel).
-template <int DT>
-ets_status launch_split_walk(ets_sampler* s, const ets::RowParams& p, int32_t rows, hipStream_t stream) {
-  ets_status st = ETS_OK;
-  if (!s->wb) {
-    st = ensure_split(s);
-    if (st != ETS_OK) return st;
-  }
-  ets::SplitParams sp = s->wb ? s->wb->split : s->split;
-  sp.row = p;
-  sp.row.rows = rows;
-  sp.phist_words = 0;
-  sp.short_lists = 0;
-  sp.row_wgs = pass2_workgroups(s, rows, sp.ns);
-  sp.list_region = 0;
-  if (rows <= 256) {
-    const int per_block = (ets::kPass1Block / 64) * 2;
-    hipLaunchKernelGGL((ets::split_pass1_kernel<DT, 2>), dim3((sp.ns + per_block - 1) / per_block, rows), dim3(ets::kPass1Block),
-                       0, stream, sp);
-  } else {
-    const int per_block = (ets::kPass1Block / 64) * 4;
-    hipLaunchKernelGGL((ets::split_pass1_kernel<DT, 4>), dim3((sp.ns + per_block - 1) / per_block, rows), dim3(ets::kPass1Block),
-                       0, stream, sp);
-  }
-  ETS_HIP(s, hipGetLastError());
-  const size_t lut_bytes = DT == ets::kDtypeBFloat16 ? sizeof(float) * ets::kLutCountWords : 0;
-  // the walk kernel's LDS: the row's records and as many prepared slots as fit beside them
-  const uint32_t walk_lds = static_cast<uint32_t>(round_up(static_cast<size_t>(sp.ns) * sizeof(ets::SlotRec), 16) + 16 * sizeof(ets::PrepSlot));
-  static std::atomic<size_t> set_sum[kMaxDevices], set_walk[kMaxDevices], set_k0[kMaxDevices], set_k1[kMaxDevices];
-  st = allow_dynamic_lds(s, reinterpret_cast<const void*>(&ets::split_pass2_kernel<DT, false, false>), lut_bytes, set_sum);
-  if (st != ETS_OK) return st;
-  st = allow_dynamic_lds(s, reinterpret_cast<const void*>(&ets::split_pass2_kernel<DT, false, true>), lut_bytes, set_walk);
-  if (st != ETS_OK) return st;
-  st = allow_dynamic_lds(s, reinterpret_cast<const void*>(&ets::split_walk_kernel<DT, 0>), walk_lds, set_k0);
-  if (st != ETS_OK) return st;
-  st = allow_dynamic_lds(s, reinterpret_cast<const void*>(&ets::split_walk_kernel<DT, 1>), walk_lds, set_k1);
-  if (st != ETS_OK) return st;
-  hipLaunchKernelGGL((ets::split_pass2_kernel<DT, false, false>), dim3(sp.row_wgs, rows), dim3(ets::kBlock), lut_bytes, stream, sp);
-  ETS_HIP(s, hipGetLastError());
-  hipLaunchKernelGGL((ets::split_walk_kernel<DT, 0>), dim3(rows), dim3(ets::kWalkBlock), walk_lds, stream, sp, walk_lds);
-  ETS_HIP(s, hipGetLastError());
-  hipLaunchKernelGGL((ets::split_pass2_kernel<DT, false, true>), dim3(sp.row_wgs, rows), dim3(ets::kBlock), lut_bytes, stream, sp);
-  ETS_HIP(s, hipGetLastError());
-  hipLaunchKernelGGL((ets::split_walk_kernel<DT, 1>), dim3(rows), dim3(ets::kWalkBlock), walk_lds, stream, sp, walk_lds);
-  ETS_HIP(s, hipGetLastError());
-  return ETS_OK;
-}
-
 ets_status launch_split_walk_any(ets_sampler* s, const ets::RowParams& p, int32_t dtype, int32_t rows, hipStream_t stream) {
   switch (dtype) {
     case ETS_DTYPE_FLOAT:
-      return launch_split_walk<ets::kDtypeFloat>(s, p, rows, stream);
+      return launch_split_walk_f32(s, p, rows, stream);
     case ETS_DTYPE_HALF:
-      return launch_split_walk<ets::kDtypeHalf>(s, p, rows, stream);
+      return launch_split_walk_f16(s, p, rows, stream);
     default:
-      return launch_split_walk<ets::kDtypeBFloat16>(s, p, rows, stream);
+      return launch_split_walk_bf16(s, p, rows, stream);
   }
 }
 
@@ -567,12 +304,11 @@ ets_status launch_split_any(ets_sampler* s, const ets::RowParams& p, int32_t dty
                             bool topk_rows) {
   switch (dtype) {
     case ETS_DTYPE_FLOAT:
-      return topk_rows ? launch_split<ets::kDtypeFloat, true>(s, p, rows, stream) : launch_split<ets::kDtypeFloat, false>(s, p, rows, stream);
+      return launch_split_f32(s, p, rows, stream, topk_rows);
     case ETS_DTYPE_HALF:
-      return topk_rows ? launch_split<ets::kDtypeHalf, true>(s, p, rows, stream) : launch_split<ets::kDtypeHalf, false>(s, p, rows, stream);
+      return launch_split_f16(s, p, rows, stream, topk_rows);
     default:
-      return topk_rows ? launch_split<ets::kDtypeBFloat16, true>(s, p, rows, stream)
-                       : launch_split<ets::kDtypeBFloat16, false>(s, p, rows, stream);
+      return launch_split_bf16(s, p, rows, stream, topk_rows);
   }
 }
 
@@ -584,11 +320,11 @@ ets_status rows_device(ets_sampler* s, const ets::RowParams& p, int32_t dtype, i
   }
   switch (dtype) {
     case ETS_DTYPE_FLOAT:
-      return launch_rows<ets::kDtypeFloat>(s, p, rows, stream, draw);
+      return launch_rows_f32(s, p, rows, stream, draw);
     case ETS_DTYPE_HALF:
-      return launch_rows<ets::kDtypeHalf>(s, p, rows, stream, draw);
+      return launch_rows_f16(s, p, rows, stream, draw);
     default:
-      return launch_rows<ets::kDtypeBFloat16>(s, p, rows, stream, draw);
+      return launch_rows_bf16(s, p, rows, stream, draw);
   }
 }
 
@@ -1319,60 +1055,6 @@ float ets_random_f32(uint64_t* state) { return static_cast<float>(ets_random_u32
 const char* ets_sampler_last_error(const ets_sampler* s) { return s ? s->last_error.c_str() : g_thread_error.c_str(); }
 
 const char* ets_version(void) { return "et_sampler 0.1 (gfx950)"; }
-
-// ---- test hooks (not part of the drop-in surface; declared in csrc/ets_test_hooks.h) ----------
-ets_status ets_test_expf(const float* d_x, float* d_y, int64_t n, void* hip_stream) {
-  if (!d_x || !d_y || n < 0) return fail(nullptr, ETS_INVALID_ARGUMENT, "ets_test_expf: bad arguments");
-  if (n == 0) return ETS_OK;
-  int64_t blocks = (n + 255) / 256;
-  if (blocks > 65536) blocks = 65536;
-  hipLaunchKernelGGL(ets::expf_exact_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0,
-                     static_cast<hipStream_t>(hip_stream), d_x, d_y, n);
-  ETS_HIP(nullptr, hipGetLastError());
-  return ETS_OK;
-}
-
-ets_status ets_test_seq_sum(const float* d_a, int32_t n, float s0, float threshold, float* d_sum, int32_t* d_stop,
-                            void* hip_stream) {
-  if (!d_a || !d_sum || !d_stop || n < 0) return fail(nullptr, ETS_INVALID_ARGUMENT, "ets_test_seq_sum: bad arguments");
-  hipLaunchKernelGGL(ets::seq_sum_kernel, dim3(1), dim3(ets::kBlock), 0, static_cast<hipStream_t>(hip_stream), d_a, n,
-                     s0, threshold, d_sum, d_stop);
-  ETS_HIP(nullptr, hipGetLastError());
-  return ETS_OK;
-}
-
-ets_status ets_test_empty_launch(void* hip_stream) {
-  hipLaunchKernelGGL(ets::empty_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(hip_stream));
-  ETS_HIP(nullptr, hipGetLastError());
-  return ETS_OK;
-}
-
-ets_status ets_test_read_floor(const void* d_data, int64_t bytes, int32_t workgroups, uint32_t* d_out, void* hip_stream) {
-  if (!d_data || !d_out || bytes < 16 || workgroups < 1 || reinterpret_cast<uintptr_t>(d_data) % 16 != 0)
-    return fail(nullptr, ETS_INVALID_ARGUMENT, "ets_test_read_floor: bad arguments");
-  hipLaunchKernelGGL(ets::read_floor_kernel, dim3(workgroups), dim3(256), 0, static_cast<hipStream_t>(hip_stream),
-                     static_cast<const uint4*>(d_data), bytes / 16, d_out);
-  ETS_HIP(nullptr, hipGetLastError());
-  return ETS_OK;
-}
-
-ets_status ets_test_copy_probe(const void* d_src, void* d_dst, int64_t bytes, void* hip_stream) {
-  if (!d_src || !d_dst || bytes < 16 || reinterpret_cast<uintptr_t>(d_src) % 16 != 0 || reinterpret_cast<uintptr_t>(d_dst) % 16 != 0)
-    return fail(nullptr, ETS_INVALID_ARGUMENT, "ets_test_copy_probe: bad arguments");
-  hipLaunchKernelGGL(ets::copy_probe_kernel, dim3(4096), dim3(256), 0, static_cast<hipStream_t>(hip_stream),
-                     static_cast<const uint4*>(d_src), static_cast<uint4*>(d_dst), bytes / 16);
-  ETS_HIP(nullptr, hipGetLastError());
-  return ETS_OK;
-}
-
-ets_status ets_test_split_timers(ets_sampler* s, uint64_t* out, int32_t rows) {
-  if (!s || !out || rows < 0 || rows > s->max_batch) return fail(s, ETS_INVALID_ARGUMENT, "ets_test_split_timers: bad arguments");
-  if (!s->d_split || !s->split.timers)
-    return fail(s, ETS_INVALID_STATE, "ets_test_split_timers: set ETS_SPLIT_TIMERS before the handle's first stochastic call");
-  DeviceGuard g(s->device);
-  ETS_HIP(s, hipMemcpy(out, s->split.timers, sizeof(uint64_t) * 12 * rows, hipMemcpyDeviceToHost));
-  return ETS_OK;
-}
 
 }  // extern "C"
 

@@ -104,7 +104,7 @@ __device__ __forceinline__ void load_run(const void* row, int first, int n, floa
 // doubles, 2^(r/32) from a cubic in r, all in double with one final rounding to float.  The
 // reference sampler calls libm expf once per vocabulary entry (sampler.cpp:201); matching its
 // last bit is what makes the sequential softmax sum reproducible.
-__device__ __constant__ uint64_t kExp2Table[32] = {
+static __device__ __constant__ uint64_t kExp2Table[32] = {
     0x3ff0000000000000ull, 0x3fefd9b0d3158574ull, 0x3fefb5586cf9890full, 0x3fef9301d0125b51ull,
     0x3fef72b83c7d517bull, 0x3fef54873168b9aaull, 0x3fef387a6e756238ull, 0x3fef1e9df51fdee1ull,
     0x3fef06fe0a31b715ull, 0x3feef1a7373aa9cbull, 0x3feedea64c123422ull, 0x3feece086061892dull,

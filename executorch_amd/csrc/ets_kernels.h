@@ -306,7 +306,7 @@ gumbel_partial_kernel(const void* logits_all, int64_t row_stride, int32_t vocab,
   store_block_best(best, &partials[static_cast<int64_t>(row) * splits + blockIdx.x]);
 }
 
-__global__ void __launch_bounds__(64)
+static __global__ void __launch_bounds__(64)
 gumbel_finish_kernel(const uint64_t* partials, int32_t splits, int32_t advance_rng, uint64_t* rng, int32_t* tokens) {
   const int row = blockIdx.x;
   const int lane = threadIdx.x;
@@ -2021,90 +2021,6 @@ __global__ void __launch_bounds__(kBlock) sample_rows_kernel(RowParams p) {
     if (p.debug) p.debug[row] = dbg;
   }
   }  // rows of this workgroup
-}
-
-// ---- measurement floors (hooks for the benchmark: what a launch and a plain read cost here) ------
-__global__ void empty_kernel() {}
-
-// dst = src, 16 bytes per lane and access as in the row kernels: the transfer of known size that the
-// hardware's fetch and write counters are scaled by.
-__global__ void __launch_bounds__(256) copy_probe_kernel(const uint4* src, uint4* dst, int64_t n_vec) {
-  for (int64_t j = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; j < n_vec; j += static_cast<int64_t>(gridDim.x) * 256)
-    dst[j] = src[j];
-}
-
-// Every workgroup reads its share of `n_vec` 16-byte vectors (eight loads in flight per lane) and
-// keeps an XOR of them: nothing but the read.
-__global__ void __launch_bounds__(256) read_floor_kernel(const uint4* data, int64_t n_vec, uint32_t* out) {
-  const int64_t per = (n_vec + gridDim.x - 1) / gridDim.x;
-  const int64_t lo = per * blockIdx.x, hi = lo + per < n_vec ? lo + per : n_vec;
-  uint32_t acc = 0u;
-  for (int64_t j = lo + threadIdx.x; j < hi; j += 8 * 256) {
-    uint4 r[8];
-#pragma unroll
-    for (int k = 0; k < 8; ++k) {
-      const int64_t jk = j + k * 256;
-      r[k] = data[jk < hi ? jk : j];
-    }
-#pragma unroll
-    for (int k = 0; k < 8; ++k) acc ^= r[k].x ^ r[k].y ^ r[k].z ^ r[k].w;
-  }
-  if (acc == 0x9e3779b9u) out[0] = acc;  // (keeps the loads alive; practically never taken)
-}
-
-// Evaluates expf_exact over an array (test hook for the exhaustive comparison with libm).
-__global__ void __launch_bounds__(256) expf_exact_kernel(const float* x, float* y, int64_t n) {
-  __shared__ uint64_t tab[32];
-  if (threadIdx.x < 32) tab[threadIdx.x] = kExp2Table[threadIdx.x];
-  __syncthreads();
-  for (int64_t i = blockIdx.x * 256ll + threadIdx.x; i < n; i += 256ll * gridDim.x) {
-    const float v = x[i];
-    // non-positive arguments go through the branch-free form the sampler uses
-    y[i] = (v <= 0.0f) ? expf_nonpositive(v, tab) : expf_exact(v, tab);
-  }
-}
-
-// Sequential float sum of an array by one workgroup (test hook).  Same loop structure as
-// scan_row: groups of kGroup chunks of 4 elements per lane through seq_sum_group, the remainder
-// through seq_sum_chunk.
-__global__ void __launch_bounds__(kBlock)
-seq_sum_kernel(const float* a, int32_t n, float s0, float threshold, float* sum_out, int32_t* stop_out) {
-  __shared__ BlockScratch sm;
-  constexpr int R = 4;
-  const int tid = threadIdx.x;
-  SeqSum st = {s0, -1, 0u};
-  bool stopped = false;
-  int base = 0;
-  for (; !stopped && base + kGroup * kBlock * R <= n; base += kGroup * kBlock * R) {
-    const float scale = fast_scale(st.s);
-    FastAcc acc[kGroup];
-#pragma unroll
-    for (int u = 0; u < kGroup; ++u) acc[u] = {0.0f, 0.0f};
-    uint32_t bits[kGroup][R];
-    int first[kGroup];
-#pragma unroll
-    for (int u = 0; u < kGroup; ++u) {
-      first[u] = base + (u * kBlock + tid) * R;
-#pragma unroll
-      for (int e = 0; e < R; ++e) {
-        const float v = a[first[u] + e];
-        bits[u][e] = __float_as_uint(v);
-        fast_fold(acc[u], v, scale);
-      }
-    }
-    stopped = seq_sum_group<kGroup, R>(st, bits, acc, scale, first, n, threshold, sm);
-  }
-  for (; !stopped && base < n; base += kBlock * R) {
-    uint32_t bits[R];
-    const int first = base + tid * R;
-#pragma unroll
-    for (int e = 0; e < R; ++e) bits[e] = (first + e < n) ? __float_as_uint(a[first + e]) : 0u;
-    stopped = seq_sum_chunk<R>(st, bits, first, n, threshold, sm);
-  }
-  if (threadIdx.x == 0) {
-    *sum_out = st.s;
-    *stop_out = st.stop_index;
-  }
 }
 
 }  // namespace ets

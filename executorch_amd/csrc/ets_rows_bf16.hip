@@ -1,0 +1,10 @@
+// sample_rows_kernel for one element type (a translation unit per type: they compile side by side).
+#include "ets_rows_launch.h"
+
+namespace ets_host {
+
+ets_status launch_rows_bf16(ets_sampler* s, const ets::RowParams& p, int32_t batch, hipStream_t stream, int draw) {
+  return launch_rows<ets::kDtypeBFloat16>(s, p, batch, stream, draw);
+}
+
+}  // namespace ets_host

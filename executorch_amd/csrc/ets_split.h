@@ -22,6 +22,12 @@
 
 namespace ets {
 
+// Phase clocks inside the kernels (device wall-clock reads around the phases of pass 2, of the
+// finish kernel and of the chain) exist only in a profiling build: -DETS_PHASE_CLOCKS=1.
+#ifndef ETS_PHASE_CLOCKS
+#define ETS_PHASE_CLOCKS 0
+#endif
+
 constexpr int kSlot = 512;        // entries per slot: 64 lanes x 8 consecutive entries
 constexpr int kMaxSlots = 2048;   // rows of up to 1048576 entries take this path
 constexpr int kPrepCap = 40;      // prepared slots per row (a row of the usual kind needs 10 to 20)
@@ -496,7 +502,7 @@ __device__ __forceinline__ void split_fold_slot(const SplitParams& p, int row, i
 // TOPK: some row of the launch may be a top-k row (a launch without one runs the code without that case).
 template <int DT, bool TOPP, bool WALK = false, bool TOPK = false, bool EXTRAS = true>
 __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_kernel(SplitParams p) {
-  uint64_t* const timers = EXTRAS ? p.timers : nullptr;  // (EXTRAS: the launch may fill the phase clocks)
+  uint64_t* const timers = (ETS_PHASE_CLOCKS && EXTRAS) ? p.timers : nullptr;  // (EXTRAS: the launch may fill the phase clocks)
   extern __shared__ __align__(16) float lut_mem[];
   __shared__ Pass2Shared sh;
   BlockScratch& sm = sh.sm;
@@ -1771,7 +1777,7 @@ __device__ __noinline__ bool draw_topp_runs(RunArgs a, const char* logits, int V
 // cost a launch of plain top-p rows more than a microsecond in registers and instructions).
 template <int DT, bool LOOP, bool TOPK = false, bool EXTRAS = true>
 __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
-  uint64_t* const timers = EXTRAS ? p.timers : nullptr;
+  uint64_t* const timers = (ETS_PHASE_CLOCKS && EXTRAS) ? p.timers : nullptr;
   float* const probs_out = EXTRAS ? p.row.probs : nullptr;
   extern __shared__ __align__(16) uint64_t lds_keys[];
   __shared__ BlockScratch sm;
@@ -2172,6 +2178,7 @@ template <int DT, int PHASE>
 __global__ void __launch_bounds__(kWalkBlock) split_walk_kernel(SplitParams p, uint32_t lds_bytes) {
   extern __shared__ __align__(16) uint64_t walk_lds[];
   __shared__ uint64_t exp2tab[32];
+  uint64_t* const walk_timers = ETS_PHASE_CLOCKS ? p.timers : nullptr;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int V = p.row.vocab;
@@ -2215,14 +2222,14 @@ __global__ void __launch_bounds__(kWalkBlock) split_walk_kernel(SplitParams p, u
   const PrepSlot* prep = reinterpret_cast<const PrepSlot*>(reinterpret_cast<const char*>(walk_lds) + rec_bytes);
   if (PHASE == 0) {
     const float S = split_chain<DT>(recs, ns, prep, n_prep, logits, V, inv, rs.m, exp2tab, p.row.fused,
-                                    p.timers ? p.timers + static_cast<int64_t>(row) * 8 : nullptr);
+                                    walk_timers ? walk_timers + static_cast<int64_t>(row) * 8 : nullptr);
     if (lane == 0) p.walk[row] = make_float2(S, toss());
   } else {
     const float2 w = p.walk[row];
     const RowDivisor div = row_divisor(w.x);
     int stop = -1;
     const float cdf = split_chain_walk<DT>(recs, ns, prep, n_prep, logits, V, inv, rs.m, exp2tab, p.row.fused,
-                                            p.timers ? p.timers + static_cast<int64_t>(gridDim.x) * 8 + static_cast<int64_t>(blockIdx.x) * 4 - 4 : nullptr, &div, w.y, &stop);
+                                            walk_timers ? walk_timers + static_cast<int64_t>(gridDim.x) * 8 + static_cast<int64_t>(blockIdx.x) * 4 - 4 : nullptr, &div, w.y, &stop);
     if (lane == 0) {
       const int32_t token = stop >= 0 ? stop : V - 1;
       p.row.tokens[row] = token;

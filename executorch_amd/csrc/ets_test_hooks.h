@@ -1,7 +1,9 @@
 /* TEST AND MEASUREMENT HOOKS, not part of the drop-in surface (no reference counterpart): they exist
  * so that tests can exercise two device building blocks in isolation (the bit-faithful expf and the
- * sequential-sum emulation) and so that the benchmark can time what a launch and a plain read cost.
- * A product build may leave them out: nothing in include/ declares them. */
+ * sequential-sum emulation) and so that the benchmark can time what a launch, a plain read and a
+ * hand-over between workgroups cost.  They are built into a library of their own,
+ * libet_sampler_hooks.so (csrc/ets_test_hooks.hip); libet_sampler.so does not export them and
+ * nothing in include/ declares them. */
 #ifndef ETS_TEST_HOOKS_H_
 #define ETS_TEST_HOOKS_H_
 
@@ -29,10 +31,21 @@ ETS_API ets_status ets_test_read_floor(const void* d_data, int64_t bytes, int32_
  * transfer of known size that fetch and write counters of a profiler run are scaled by. */
 ETS_API ets_status ets_test_copy_probe(const void* d_src, void* d_dst, int64_t bytes, void* hip_stream);
 
+/* Round trips between workgroup 0 and workgroup `partner` (1 .. 15) of a 16-workgroup launch through
+ * two words in device memory (`d_words`: 64 words, zeroed by the caller), every wait bounded by
+ * `spin_limit` polls.  d_out[0] (zeroed by the caller): waits that ran out; d_out[1]: ticks of the
+ * 100 MHz clock that workgroup 0 spent on `hops` round trips.  DEVICE pointers. */
+ETS_API ets_status ets_test_signal_floor(uint32_t* d_words, int32_t hops, int32_t spin_limit, int32_t partner,
+                                         uint32_t* d_out, void* hip_stream);
+
+/* The message of the calling thread's last failed hook. */
+ETS_API const char* ets_test_last_error(void);
+
 /* Phase clocks of the finish kernel of the several-workgroups-per-row path, four 64-bit words per
  * row (staging, ordered sum, draw, in ticks of the 100 MHz wall clock; then the candidate and
- * prepared-slot counts), filled when ETS_SPLIT_TIMERS was set before the handle's first stochastic
- * call.  HOST pointer. */
+ * prepared-slot counts), filled when libet_sampler.so was built with -DETS_PHASE_CLOCKS=1 (a
+ * profiling build; the product build has no clocks in its kernels) and ETS_SPLIT_TIMERS was set before
+ * the handle's first stochastic call.  HOST pointer. */
 ETS_API ets_status ets_test_split_timers(ets_sampler* s, uint64_t* out, int32_t rows);
 
 #ifdef __cplusplus

@@ -12,8 +12,8 @@ to the host and sampled by the oracle (test infrastructure, never the thing meas
   * against the reference's native 16-bit arithmetic (sample<BFloat16> / sample<Half>): agreement is
     counted and reported, not required (every intermediate is rounded to 8 / 11 bits there).
 
-Prints one JSON line.  Not collected by pytest (a long run); the GPU tests cover the same
-comparisons on fewer rows.
+Prints one JSON line.  tests/test_gpu_parity_sweep.py runs the same function inside the GPU suite
+(100 000 rows of cfg2, a few thousand of the other workloads).
 """
 import argparse
 import json
@@ -96,8 +96,8 @@ def run(workload="cfg2", rows=100000, chunk=1024, threads=16, seed=20240607):
         sums = np.ascontiguousarray(ea.debug_records(ddbg)["sum"], dtype=np.float32)
         want_sums = np.array([ex[b].sum for b in range(n)], dtype=np.float32)
         sum_mismatches += int((sums.view(np.uint32) != want_sums.view(np.uint32)).sum())
-        ref, _ = O.sample_rows(host, w.dtype, inv, w.topp, 0, seeds.copy(), mode=O.MODE_UPCAST, tie=O.TIE_LIBSTDCXX,
-                               threads=args.threads)
+        ref, ref_ex = O.sample_rows(host, w.dtype, inv, w.topp, 0, seeds.copy(), mode=O.MODE_UPCAST, tie=O.TIE_LIBSTDCXX,
+                                    threads=args.threads, explain=True)
         native, _ = O.sample_rows(host, w.dtype, inv, w.topp, 0, seeds.copy(), mode=O.MODE_NATIVE, tie=O.TIE_LIBSTDCXX,
                                   threads=args.threads)
         mismatches += int((got != want).sum())
@@ -105,10 +105,15 @@ def run(workload="cfg2", rows=100000, chunk=1024, threads=16, seed=20240607):
         native_agree += int((got == native).sum())
         for b in np.nonzero(ref != want)[0]:
             tie_rows += 1
-            po = np.empty(w.vocab, dtype=np.float32)
-            o = O.Sampler(w.vocab, w.temperature, w.topp, 1, mode=O.MODE_UPCAST)
-            o.sample(host[b].copy(), w.dtype, probs_out=po)
-            if po[ref[b]] != po[want[b]]:
+            if ex[b].branch in (O.BRANCH_TOPP, O.BRANCH_TOPK):
+                # both runs report the probability of the token they returned
+                equal = np.float32(ex[b].p_token).view(np.uint32) == np.float32(ref_ex[b].p_token).view(np.uint32)
+            else:
+                po = np.empty(w.vocab, dtype=np.float32)
+                o = O.Sampler(w.vocab, w.temperature, w.topp, 1, mode=O.MODE_UPCAST)
+                o.sample(host[b].copy(), w.dtype, probs_out=po)
+                equal = po[ref[b]] == po[want[b]]
+            if not equal:
                 tie_not_equal += 1
         done += n
         print(f"parity_report: {done} rows, {mismatches} + {plain_mismatches} mismatches, {time.time() - t0:.0f} s", file=sys.stderr,

@@ -50,10 +50,20 @@ def test_no_packed_fp32_instructions_in_the_device_code(tmp_path):
         pytest.skip("needs ROCm's clang-offload-bundler / llvm-objdump and objcopy")
     fat = tmp_path / "fatbin"
     subprocess.check_call(["objcopy", "-O", "binary", "--only-section=.hip_fatbin", _capi.LIB_PATH, str(fat)])
-    co = tmp_path / "gfx950.co"
-    subprocess.check_call([bundler, "--unbundle", "--type=o", f"--input={fat}", f"--output={co}",
-                           "--targets=hipv4-amdgcn-amd-amdhsa--gfx950"])
-    asm = subprocess.run([objdump, "-d", str(co)], stdout=subprocess.PIPE, text=True, check=True).stdout
-    assert asm.count("s_endpgm") >= 40  # the kernels are in there
-    packed = re.findall(r"\bv_pk_(?:add|mul|fma)_f32\b", asm)
+    # one bundle per translation unit, one after the other in the section
+    magic = b"__CLANG_OFFLOAD_BUNDLE__"
+    data = fat.read_bytes()
+    starts = [m.start() for m in re.finditer(re.escape(magic), data)]
+    assert len(starts) >= len(build.LIB_UNITS)
+    ends, packed = 0, []
+    for k, at in enumerate(starts):
+        piece = tmp_path / f"bundle{k}"
+        piece.write_bytes(data[at:starts[k + 1] if k + 1 < len(starts) else len(data)])
+        co = tmp_path / f"gfx950_{k}.co"
+        subprocess.check_call([bundler, "--unbundle", "--type=o", f"--input={piece}", f"--output={co}",
+                               "--targets=hipv4-amdgcn-amd-amdhsa--gfx950"])
+        asm = subprocess.run([objdump, "-d", str(co)], stdout=subprocess.PIPE, text=True, check=True).stdout
+        ends += asm.count("s_endpgm")
+        packed += re.findall(r"\bv_pk_(?:add|mul|fma)_f32\b", asm)
+    assert ends >= 40  # the kernels are in there
     assert not packed, f"{len(packed)} packed fp32 instructions in the device code"

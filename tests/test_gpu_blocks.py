@@ -13,7 +13,7 @@ pytestmark = pytest.mark.gpu
 def gpu_expf(x, dev):
     dx = torch.from_numpy(np.ascontiguousarray(x, dtype=np.float32)).to(dev)
     dy = torch.empty_like(dx)
-    assert _capi.lib().ets_test_expf(dx.data_ptr(), dy.data_ptr(), dx.numel(), None) == _capi.OK
+    assert _capi.hooks().ets_test_expf(dx.data_ptr(), dy.data_ptr(), dx.numel(), None) == _capi.OK
     torch.cuda.synchronize()
     return dy.cpu().numpy()
 
@@ -53,7 +53,7 @@ def gpu_seq_sum(a, s0, thr, dev):
     da = torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).to(dev)
     ds = torch.zeros(1, device=dev)
     dstop = torch.zeros(1, dtype=torch.int32, device=dev)
-    st = _capi.lib().ets_test_seq_sum(da.data_ptr(), da.numel(), float(s0), float(thr), ds.data_ptr(), dstop.data_ptr(), None)
+    st = _capi.hooks().ets_test_seq_sum(da.data_ptr(), da.numel(), float(s0), float(thr), ds.data_ptr(), dstop.data_ptr(), None)
     assert st == _capi.OK
     torch.cuda.synchronize()
     return np.float32(ds.item()), int(dstop.item())

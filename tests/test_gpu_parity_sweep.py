@@ -1,7 +1,8 @@
 """Parity at a scale the fixed cases do not reach, as part of the GPU suite: the randomised cases of
 fuzz_parity.py in the three settings of the row split (automatic, forced, off) and with per-row
-parameters, and a few thousand rows of the headline workload's distribution against the oracle
-(tokens, the softmax normaliser bit for bit, the reference's own tie order).  The same code runs
+parameters, and 100 000 rows of the headline workload's distribution and a few thousand of the others against the
+oracle (tokens, the softmax normaliser bit for bit, the reference's own tie order, agreement with the
+native 16-bit instantiations).  The same code runs
 longer from the command line: `python tests/fuzz_parity.py --cases N`, `python tests/parity_report.py`."""
 import pytest
 
@@ -25,11 +26,19 @@ def test_randomised_cases_with_per_row_parameters(monkeypatch):
     assert res["failures"] == 0, res["first_failures"]
 
 
-@pytest.mark.parametrize("workload,rows", [("cfg2", 4096), ("cfg1", 1024)])
-def test_rows_of_a_workload_at_scale(workload, rows):
-    res = parity_report.run(workload=workload, rows=rows, chunk=1024, threads=8, seed=7)
+# 100 000 seeded rows of the headline workload (what the benchmark contract asks identical tokens
+# on), 2 000 rows each of the other batched workloads and 1 024 of the reference's own batch-1 case.
+@pytest.mark.parametrize("workload,rows", [("cfg2", 100_000), ("cfg1", 1024), ("cfg3", 2000), ("cfg4", 2000), ("cfg5", 2000)])
+def test_rows_of_a_workload_at_scale(workload, rows, capsys):
+    res = parity_report.run(workload=workload, rows=rows, chunk=1024, threads=16, seed=7)
+    with capsys.disabled():  # the classified report, in the suite's own output
+        print(f"\nparity at scale: {res}", flush=True)
     assert res["rows"] == rows
     assert res["token_mismatches_vs_oracle_fp32_index_ties"] == 0, res
     assert res["token_mismatches_without_debug_records"] == 0, res
     assert res["normaliser_bit_mismatches_vs_oracle"] == 0, res
+    # rows on which the reference's own (unstable) sort order gives another token: only ever between
+    # two tokens of exactly equal probability
     assert res["of_which_not_between_equal_probabilities"] == 0, res
+    # (agreement with the reference's native 16-bit arithmetic is reported, not required)
+    assert 0 <= res["rows_equal_to_native_16bit_reference_arithmetic"] <= rows
