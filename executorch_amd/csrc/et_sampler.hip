@@ -560,36 +560,43 @@ ets_status sample_device_configs(ets_sampler* s, const void* d_logits, int32_t d
   }
   const bool both_draw = count[kRows] > 0 && count[kSplit] > 0;
   const int32_t share = both_draw ? s->scratch_rows / 2 : s->scratch_rows;
+  // Every exit from here on goes through the join and the release below: a launch that fails must
+  // not leave the side stream running unjoined, nor the staging copy unguarded, while kernels that
+  // were launched before it still read the row maps and parameters.
+  ets_status first = ETS_OK;
   if (count[kSplit] + count[kRows] > 0 && share < 1)
-    return fail(s, ETS_INTERNAL, "ets_sampler_sample_batch_configs: no scratch rows");
-  if (count[kRows] > 0) {
+    first = fail(s, ETS_INTERNAL, "ets_sampler_sample_batch_configs: no scratch rows");
+  if (first == ETS_OK && count[kRows] > 0) {
     p.scratch = s->d_scratch;
     p.grid_cap = share;
     p.row_map = d_maps + kRows * batch;
-    st = rows_device(s, p, dtype, count[kRows], stream, ets::kDrawAny);
-    if (st != ETS_OK) return st;
+    first = rows_device(s, p, dtype, count[kRows], stream, ets::kDrawAny);
   }
-  if (count[kWalk] > 0) {  // (no scratch rows, no tickets)
+  if (first == ETS_OK && count[kWalk] > 0) {  // (no scratch rows, no tickets)
     p.row_map = d_maps + kWalk * batch;
-    st = launch_split_walk_any(s, p, dtype, count[kWalk], stream);
-    if (st != ETS_OK) return st;
+    first = launch_split_walk_any(s, p, dtype, count[kWalk], stream);
   }
-  if (count[kSplit] > 0) {
+  if (first == ETS_OK && count[kSplit] > 0) {
     p.scratch = s->d_scratch + (both_draw ? static_cast<int64_t>(share) * s->scratch_stride : 0);
     p.grid_cap = share;
     p.row_map = d_maps + kSplit * batch;
-    st = launch_split_any(s, p, dtype, count[kSplit], side, split_topk);
-    if (st != ETS_OK) return st;
+    first = launch_split_any(s, p, dtype, count[kSplit], side, split_topk);
   }
-  if (count[kGreedy] > 0) {
-    st = argmax_device(s, d_logits, dtype, count[kGreedy], stride, d_tokens, side, d_maps + kGreedy * batch);
-    if (st != ETS_OK) return st;
-  }
+  if (first == ETS_OK && count[kGreedy] > 0)
+    first = argmax_device(s, d_logits, dtype, count[kGreedy], stride, d_tokens, side, d_maps + kGreedy * batch);
+  const std::string first_message = s->last_error;
+  ets_status closing = ETS_OK;
   if (fork) {
-    ETS_HIP(s, hipEventRecord(s->join_event, side));
-    ETS_HIP(s, hipStreamWaitEvent(stream, s->join_event, 0));
+    hipError_t e = hipEventRecord(s->join_event, side);
+    if (e == hipSuccess) e = hipStreamWaitEvent(stream, s->join_event, 0);
+    if (e != hipSuccess) closing = hip_fail(s, e, "joining the side stream");
   }
-  return stage_release(s, stream);
+  const ets_status released = stage_release(s, stream);
+  if (first != ETS_OK) {
+    s->last_error = first_message;
+    return first;
+  }
+  return closing != ETS_OK ? closing : released;
 }
 
 }  // namespace

@@ -40,7 +40,10 @@ constexpr uint32_t kSlotDual = 3u;    // no entry ties under the ulp of binade k
 constexpr uint32_t kSlotExact = 4u;   // slot 0 only: `even` holds the bits of the exact sum behind the slot
 
 struct SlotRec {
-  uint32_t meta;  // bits 0-7: biased exponent the summary was folded for; bits 8-10: kind
+  uint32_t meta;  // bits 0-7: biased exponent the summary was folded for; bits 8-10: kind; bits 16-23: the biased
+                  //   exponent the sum is predicted to have when it reaches the slot (a serial slot: behind the
+                  //   slot); serial slots, bit 24: "prepared, both binades in the range of the float shortcut" (the
+                  //   chain's short form can serve it)
   uint32_t even, odd;
   uint32_t prep;  // index of the slot's PrepSlot, or 0xffffffff
 };
@@ -49,7 +52,7 @@ struct SlotRec {
 // over the lanes of the increments rne(e / ulp) of each lane's 8 entries, under the ulp of the
 // binade the running sum is expected to enter the slot in (a) and of the one it is expected to
 // leave it in (b), with the lanes in which an entry sits on a half-ulp tie (their increment
-// depends on the order of the adds).  A lane's increment is capped at 2^25 (far beyond what any
+// depends on the order of the adds).  A lane's increment is capped at 2^24 (at least what any
 // binade has room for), so the sums are exact integers wherever they matter and never wrap.
 struct PrepSlot {
   float e[kSlot];
@@ -60,6 +63,8 @@ struct PrepSlot {
   uint32_t usable;  // both binades are in the range of the float shortcut
   uint32_t pad;
 };
+constexpr uint32_t kPrepTie = 0x80000000u;   // bit 31 of pre_a[l] / pre_b[l]: an entry of lane l ties under that binade's ulp
+constexpr uint32_t kPrepSum = 0x7fffffffu;   //   (the prefix sums stay below 2^31: 64 lanes of at most 2^24)
 static_assert(sizeof(PrepSlot) % 16 == 0, "prepared slots are copied as 16-byte vectors");
 
 struct RowState {
@@ -299,7 +304,8 @@ __global__ void __launch_bounds__(kPass1Block) split_pass1_kernel(SplitParams p)
 struct Pass2Shared {
   BlockScratch sm;
   float upto[kMaxSlots + 1];  // approximate running sum in front of every slot, in units of exp(-m)
-  uint32_t cls[kMaxSlots];    // per slot: kb_lo | kb_hi << 8 | kind << 16 | prepared-slot index << 19
+  uint32_t cls[kMaxSlots];    // per slot: kb_lo | kb_hi << 8 | kind << 16 | prepared-slot index << 19 (11 bits) | bit 30: the
+                              //   binade predicted at the slot's entry is the upper one
   float top[kMaxSlots];       // per slot: an upper bound of its largest exp (top-p: a slot below the listing cut is not searched)
   uint32_t hist[kHistBuckets];
   uint32_t list_count;        // candidates this workgroup has listed
@@ -407,12 +413,14 @@ __device__ __forceinline__ void split_fold_slot(const SplitParams& p, int row, i
   }
   // ---- every entry 0: no effect on any running sum
   const uint32_t any_bits = bits[0] | bits[1] | bits[2] | bits[3] | bits[4] | bits[5] | bits[6] | bits[7];  // (no -0 among exps)
-  if (__ballot(any_bits != 0u) == 0ull) {
-    if (lane == 0) p.slot_rec[rec_at] = {kSlotZero << 8, 0u, 0u, 0xffffffffu};
-    return;
-  }
   const uint32_t kb_lo = cls & 255u, kb_hi = (cls >> 8) & 255u;
   const uint32_t kind = (cls >> 16) & 7u;
+  // the binade the sum is predicted to be in when it reaches the slot (bits 16-23 of the record)
+  const uint32_t kb_in = ((kb_lo + ((cls >> 30) & 1u)) & 255u) << 16;
+  if (__ballot(any_bits != 0u) == 0ull) {
+    if (lane == 0) p.slot_rec[rec_at] = {(kSlotZero << 8) | kb_in, 0u, 0u, 0xffffffffu};
+    return;
+  }
   if (kind == kSlotStable) {
     // ---- the sum stays in binade kb_lo throughout the slot
     const float scale = __uint_as_float((277u - kb_lo) << 23);  // 2^(150 - kb)
@@ -430,7 +438,7 @@ __device__ __forceinline__ void split_fold_slot(const SplitParams& p, int row, i
       slot.even = readlane_u32(upto.even, 63);
       slot.odd = readlane_u32(upto.odd, 63);
     }
-    if (lane == 0) p.slot_rec[rec_at] = {kb_lo | (kSlotStable << 8), slot.even, slot.odd, 0xffffffffu};
+    if (lane == 0) p.slot_rec[rec_at] = {kb_lo | (kSlotStable << 8) | (kb_lo << 16), slot.even, slot.odd, 0xffffffffu};
     return;
   }
   if (kind == kSlotDual) {
@@ -446,17 +454,18 @@ __device__ __forceinline__ void split_fold_slot(const SplitParams& p, int row, i
     const float inc_a = wave_sum_f32(fa.inc), inc_b = wave_sum_f32(fb.inc);
     if (lane == 0) {
       if (ties) {  // (rare) the finish kernel works the slot out from the logits
-        p.slot_rec[rec_at] = {kb_lo | (kSlotSerial << 8), 0u, 0u, 0xffffffffu};
+        p.slot_rec[rec_at] = {kb_lo | (kSlotSerial << 8) | ((kb_lo + 1u) << 16), 0u, 0u, 0xffffffffu};
       } else {
-        p.slot_rec[rec_at] = {kb_lo | (kSlotDual << 8), inc_a < 67108864.0f ? static_cast<uint32_t>(inc_a) : kSat,
+        p.slot_rec[rec_at] = {kb_lo | (kSlotDual << 8) | kb_in, inc_a < 67108864.0f ? static_cast<uint32_t>(inc_a) : kSat,
                               inc_b < 67108864.0f ? static_cast<uint32_t>(inc_b) : kSat, 0xffffffffu};
       }
     }
     return;
   }
   // ---- to be resolved in order: keep the entries and the lanes' increments under both candidate ulps
-  const uint32_t idx = cls >> 19;
+  const uint32_t idx = (cls >> 19) & 0x7ffu;
   const uint32_t kb_a = kb_lo, kb_b = kb_hi > kb_lo ? kb_hi : kb_lo + 1u;
+  bool clean = false;  // prepared, both binades in the range of the float shortcut
   if (idx < static_cast<uint32_t>(p.prep_cap)) {
     PrepSlot& ps = p.prep[static_cast<int64_t>(row) * p.prep_cap + idx];
     float4* pe = reinterpret_cast<float4*>(ps.e + lane * 8);
@@ -472,10 +481,11 @@ __device__ __forceinline__ void split_fold_slot(const SplitParams& p, int row, i
         fast_fold(fb, e[k], scale_b);
       }
     }
-    const float kCap = 33554432.0f;  // 2^25
-    ps.pre_a[lane] = wave_scan_inclusive_u32(static_cast<uint32_t>(__builtin_fminf(fa.inc, kCap)));
-    ps.pre_b[lane] = wave_scan_inclusive_u32(static_cast<uint32_t>(__builtin_fminf(fb.inc, kCap)));
+    const float kCap = 16777216.0f;  // 2^24
+    ps.pre_a[lane] = wave_scan_inclusive_u32(static_cast<uint32_t>(__builtin_fminf(fa.inc, kCap))) | (fa.tie == 0.5f ? kPrepTie : 0u);
+    ps.pre_b[lane] = wave_scan_inclusive_u32(static_cast<uint32_t>(__builtin_fminf(fb.inc, kCap))) | (fb.tie == 0.5f ? kPrepTie : 0u);
     const uint64_t tie_a = __ballot(fa.tie == 0.5f), tie_b = __ballot(fb.tie == 0.5f);
+    clean = usable && kb_b <= 255u;
     if (lane == 0) {
       ps.kb_a = kb_a;
       ps.kb_b = kb_b;
@@ -488,7 +498,7 @@ __device__ __forceinline__ void split_fold_slot(const SplitParams& p, int row, i
     }
   }
   if (lane == 0) {
-    p.slot_rec[rec_at] = {kb_a | (kSlotSerial << 8), 0u, 0u,
+    p.slot_rec[rec_at] = {kb_a | (kSlotSerial << 8) | ((kb_b & 255u) << 16) | (clean ? 1u << 24 : 0u), 0u, 0u,
                           idx < static_cast<uint32_t>(p.prep_cap) ? idx : 0xffffffffu};
   }
 }
@@ -663,7 +673,9 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
       chunk_total += sm.red_u[w];
     }
     rank += static_cast<uint32_t>(__popcll(serial_ballot & ((1ull << lane) - 1ull)));
-    if (s < ns) sh.cls[s] = (kb_lo & 255u) | ((kb_hi > 255u ? 255u : kb_hi) << 8) | (kind << 16) | (rank << 19);
+    // (bit 30: the approximate sum in front of the slot lies in the upper of the two binades)
+    const uint32_t in_hi = (__float_as_uint(a_in) >> 23) > kb_lo ? 1u << 30 : 0u;
+    if (s < ns) sh.cls[s] = (kb_lo & 255u) | ((kb_hi > 255u ? 255u : kb_hi) << 8) | (kind << 16) | ((rank & 0x7ffu) << 19) | in_hi;
     serial_before += chunk_total;
   }
   const float a_total = carry;
@@ -917,6 +929,72 @@ __device__ __forceinline__ void resolve_lanes(float& s, const uint32_t (&bits)[8
   }
 }
 
+// A value every lane holds alike (loaded from one address, say), as a scalar: what is decided by it
+// then runs on the scalar unit, and branches on it do not touch the execution mask.
+__device__ __forceinline__ uint32_t uniform_u32(uint32_t v) { return __builtin_amdgcn_readfirstlane(v); }
+
+// LDS of a row while its sum is composed: the slot records, then one (even, odd) pair per record --
+// the increment of the run of plain records that ends with the record, for either parity of the
+// sum that enters the run (split_chain_prepare) --, then the prepared slots.
+__host__ __device__ __forceinline__ size_t chain_pairs_offset(int ns) { return (static_cast<size_t>(ns) * sizeof(SlotRec) + 15) / 16 * 16; }
+__host__ __device__ __forceinline__ size_t chain_rec_bytes(int ns) {
+  return chain_pairs_offset(ns) + (static_cast<size_t>(ns) * sizeof(uint2) + 15) / 16 * 16;
+}
+
+// What the chain needs of a chunk of 64 records that does not depend on the running sum, worked
+// out by any wave before the chain starts (sixteen waves do the chunks of a row side by side, where
+// the chain's one wave would take them one after the other).  Every record is read under the
+// binade pass 2 predicted for its slot.  A run is a stretch of plain records read under one
+// binade: zero slots, stable slots (with or without a half-ulp tie inside), dual slots; it ends in
+// front of a serial record, where the predicted binade changes, and with the chunk.  pairs[i] is
+// the composition of the records of i's run up to and including i (a serial record adds nothing:
+// it holds the total of the run in front of it).
+__device__ __forceinline__ void split_chain_prepare(const SlotRec* recs, int ns, uint2* pairs, int first_chunk, int chunk_step) {
+  const int lane = threadIdx.x & 63;
+  for (int base = first_chunk * 64; base < ns; base += chunk_step * 64) {
+    const int n = ns - base < 64 ? ns - base : 64;
+    SlotRec r = {kSlotZero << 8, 0u, 0u, 0xffffffffu};
+    if (lane < n) r = recs[base + lane];
+    const uint32_t kind = (r.meta >> 8) & 7u, kb = r.meta & 255u, kb_in = (r.meta >> 16) & 255u;
+    const bool runs = lane < n && (kind == kSlotZero || (kind == kSlotStable && kb == kb_in) ||
+                                   (kind == kSlotDual && (kb == kb_in || kb + 1u == kb_in)));
+    ParityInc v = {0u, 0u};
+    if (runs && kind == kSlotStable) v = {r.even, r.odd};
+    if (runs && kind == kSlotDual) v.even = v.odd = (kb == kb_in ? r.even : r.odd);
+    v.even = v.even < (1u << 25) ? v.even : (1u << 25);  // (64 of them cannot wrap; 2^24 and up fails the chain's check)
+    v.odd = v.odd < (1u << 25) ? v.odd : (1u << 25);
+    // a lane starts a run when it is the chunk's first, when the lane in front of it is no part of a
+    // run, or when it is read under another binade than the lane in front of it
+    const uint64_t run_mask = __ballot(runs);
+    const uint32_t kb_front = __builtin_amdgcn_update_dpp(0u, kb_in, 0x138, 0xf, 0xf, false);  // wave_shr:1
+    const bool front_runs = lane > 0 && ((run_mask >> (lane - 1)) & 1ull) != 0ull;
+    const bool head = lane == 0 || !front_runs || (runs && kb_in != kb_front);
+    const uint64_t heads = __ballot(head);
+    const int head_at = 63 - __clzll(static_cast<long long>(heads & ((2ull << lane) - 1ull)));  // (lane 0 is one)
+    if (__ballot(v.even != v.odd) == 0ull) {
+      // no tie in the chunk: one prefix sum, less what lies in front of the lane's run
+      const uint32_t incl = wave_scan_inclusive_u32(v.even);
+      const uint32_t front = static_cast<uint32_t>(__shfl(static_cast<int>(incl), head_at > 0 ? head_at - 1 : 0));
+      v.even = v.odd = incl - (head_at > 0 ? front : 0u);
+    } else {
+      const ParityInc id = {0u, 0u};
+#define ETS_SEG_STEP(CTRL, MASK, SRC)                              \
+  {                                                                \
+    const ParityInc o = dpp_parity_or_identity<CTRL, MASK>(v);     \
+    v = compose((SRC) >= head_at ? o : id, v);                     \
+  }
+      ETS_SEG_STEP(0x111, 0xf, lane - 1)
+      ETS_SEG_STEP(0x112, 0xf, lane - 2)
+      ETS_SEG_STEP(0x114, 0xf, lane - 4)
+      ETS_SEG_STEP(0x118, 0xf, lane - 8)
+      ETS_SEG_STEP(0x142, 0xa, (lane & ~15) - 1)
+      ETS_SEG_STEP(0x143, 0xc, 31)
+#undef ETS_SEG_STEP
+    }
+    if (lane < n) pairs[base + lane] = make_uint2(v.even, v.odd);
+  }
+}
+
 // The sequential softmax sum of one row (sampler.cpp:199-203) from the slot records, by ONE wave.
 // `recs` (ns records) and `prep` (the first `n_prep` prepared slots) are in LDS.  Sixty-four
 // records at a time, one per lane.  Under the binade K of the exact running sum a record is
@@ -929,18 +1007,21 @@ __device__ __forceinline__ void resolve_lanes(float& s, const uint32_t (&bits)[8
 // else is redone entry by entry from the logits -- and the walk goes on behind it.  Every step
 // advances by at least one record.
 template <int DT>
-__device__ __forceinline__ float split_chain(const SlotRec* recs, int ns, const PrepSlot* prep, uint32_t n_prep,
+__device__ __forceinline__ float split_chain(const SlotRec* recs, const uint2* pairs, int ns, const PrepSlot* prep, uint32_t n_prep,
                                              const char* logits, int V, float inv, float m, const uint64_t* tab,
                                              const FusedOps& fused, uint64_t* stats = nullptr) {
   const int lane = threadIdx.x & 63;
   const float kInf = __uint_as_float(0x7f800000u);
   const float fill = inv < 0.0f ? kInf : -kInf;
+  n_prep = uniform_u32(n_prep);
   float s = 0.0f;
   uint64_t c_start = 0;
   uint32_t n_iter = 0, n_generic = 0, n_prep_used = 0, n_tie = 0, n_inner = 0;
   uint64_t c_prep = 0;
   if (stats) c_start = wall_clock64();
+  uint64_t ph_load = 0, ph_scan = 0, ph_walk = 0, ph_t = 0;
   for (int base = 0; base < ns; base += 64) {
+    if (stats) ph_t = wall_clock64();
     SlotRec r = {kSlotZero << 8, 0u, 0u, 0xffffffffu};
     if (base + lane < ns) r = recs[base + lane];
     const uint32_t kind = (r.meta >> 8) & 7u, kb = r.meta & 255u;
@@ -949,6 +1030,160 @@ __device__ __forceinline__ float split_chain(const SlotRec* recs, int ns, const 
       s = __uint_as_float(readlane_u32(r.even, 0));
       cur = 1;
     }
+    if (stats) {
+      const uint64_t now = wall_clock64();
+      ph_load += now - ph_t;
+      ph_t = now;
+    }
+    // ---- the usual chunk, with as few instructions on this one wave's path as it takes (a wave on its
+    //      own issues an instruction every few nanoseconds, whatever the instruction is).  The runs of
+    //      plain records were added up beforehand (split_chain_prepare), each under the binade predicted
+    //      for it and for either parity of the sum that enters it, so the walk goes from stop to stop
+    //      on the scalar unit, the sum kept as (binade, integer).  A stop is a record that is no part
+    //      of a run (a serial one), the last record in front of a change of the predicted binade, or
+    //      the chunk's last.  At a stop the run that ends there is committed after checking that the
+    //      sum entered it in the binade it was read under and stays inside it (increments are not
+    //      negative, so the total decides for every prefix); a prepared slot without ties then takes
+    //      the short form of resolve_lanes() below, any other serial record the general code.  A run
+    //      that fails a check goes to the record-by-record loop further down, with the rest of the chunk.
+    bool fast_ok = true;
+    {
+      const int n = ns - base < 64 ? ns - base : 64;
+      const uint2 pr = lane < n ? pairs[base + lane] : make_uint2(0u, 0u);
+      const uint32_t kb_in = (r.meta >> 16) & 255u;  // (a serial record: the binade predicted behind it)
+      const bool runs = lane < n && (kind == kSlotZero || (kind == kSlotStable && kb == kb_in) ||
+                                     (kind == kSlotDual && (kb == kb_in || kb + 1u == kb_in)));
+      const uint64_t run_mask = __ballot(runs);
+      const uint32_t kb_front = __builtin_amdgcn_update_dpp(0u, kb_in, 0x138, 0xf, 0xf, false);  // wave_shr:1
+      const bool turn = lane > 0 && runs && ((run_mask >> (lane - 1)) & 1ull) != 0ull && kb_in != kb_front;  // a run starts here, behind another
+      const uint64_t in_chunk = n < 64 ? (1ull << n) - 1ull : ~0ull;
+      const uint64_t stop_mask = ((~run_mask) | (__ballot(turn) >> 1) | (1ull << (n - 1))) & in_chunk;
+      // what kind of stop a lane is: kind | "prepared, in the float shortcut's range" << 3 (0 for a record that is part of a run)
+      const uint32_t stop_info = runs ? 0u : (kind | (((r.meta >> 24) & 1u) << 3));
+      uint32_t sb = uniform_u32(__float_as_uint(s));
+      uint32_t K = sb >> 23 ? sb >> 23 : 1u;                          // sum_state()
+      uint32_t S = sb >> 23 ? ((sb & 0x7fffffu) | 0x800000u) : sb;
+      if (stats) {
+        const uint64_t now = wall_clock64();
+        ph_scan += now - ph_t;
+        ph_t = now;
+      }
+      while (cur < n) {
+        cur = static_cast<int>(uniform_u32(static_cast<uint32_t>(cur)));
+        const int t = static_cast<int>(uniform_u32(static_cast<uint32_t>(__builtin_ctzll(stop_mask & (~0ull << cur)))));  // (lane n - 1 is a stop)
+        const uint32_t info_t = readlane_u32(stop_info, t);
+        if (info_t == 0u) {
+          // ---- a run ends with record t and nothing else happens there
+          const uint32_t S_run = S + readlane_u32((S & 1u) ? pr.y : pr.x, t);
+          if (K != readlane_u32(kb_in, cur) || S_run >= (1u << 24)) {
+            fast_ok = false;
+            break;
+          }
+          S = S_run;
+          cur = t + 1;
+          continue;
+        }
+        const uint32_t pi = readlane_u32(r.prep, t);
+        // what a prepared slot needs is asked for before the run in front of it is committed
+        const bool short_form = info_t == (kSlotSerial | 8u) && pi < n_prep;
+        const PrepSlot& ps = prep[short_form ? pi : 0u];
+        const float4 e0 = *reinterpret_cast<const float4*>(ps.e + lane * 8);
+        const float4 e1 = *reinterpret_cast<const float4*>(ps.e + lane * 8 + 4);
+        const uint32_t raw_a = ps.pre_a[lane], raw_b = ps.pre_b[lane];
+        const uint32_t pre_a = raw_a & kPrepSum, pre_b = raw_b & kPrepSum;
+        // ---- the run that ends in front of t (empty when lane cur is no part of a run: then t == cur)
+        if ((run_mask >> cur) & 1ull) {
+          const uint32_t S_run = S + readlane_u32((S & 1u) ? pr.y : pr.x, t);
+          if (K != readlane_u32(kb_in, cur) || S_run >= (1u << 24)) {
+            fast_ok = false;
+            break;
+          }
+          S = S_run;
+        }
+        cur = t;
+        {
+          // ---- record base + t, no part of a run
+          bool done = false;
+          if (short_form && K == (readlane_u32(r.meta, t) & 255u)) {
+            // resolve_lanes() for a slot entered in the binade it was prepared for: the lanes in front
+            // of the one in which the sum leaves the binade by their prefix sum (none of them may hold
+            // a tie under that binade's ulp), that lane's eight entries natively (every lane adds; one
+            // result is read), the lanes behind it by the prefix sums under the next binade (no tie
+            // under its ulp among them)
+            const uint32_t room = (1u << 24) - S;
+            const uint64_t over = __ballot(pre_a >= room);
+            const uint64_t tie_a = __ballot((raw_a & kPrepTie) != 0u), tie_b = __ballot((raw_b & kPrepTie) != 0u);
+            if (over == 0ull) {
+              if (tie_a == 0ull) {
+                S += readlane_u32(pre_a, 63);
+                done = true;
+              }
+            } else if ((tie_a & ((over & (0ull - over)) - 1ull)) == 0ull && (tie_b & ((~0ull << __builtin_ctzll(over)) << 1)) == 0ull) {
+              const int jl = __builtin_ctzll(over);
+              const uint32_t excl_a = __builtin_amdgcn_update_dpp(0u, pre_a, 0x138, 0xf, 0xf, false);  // wave_shr:1
+              const uint32_t rest_b = readlane_u32(pre_b, 63) - pre_b;
+              const uint32_t S_j = S + readlane_u32(excl_a, jl);
+              float v = __uint_as_float(((K - 1u) << 23) + S_j);
+              v = v + e0.x; v = v + e0.y; v = v + e0.z; v = v + e0.w;
+              v = v + e1.x; v = v + e1.y; v = v + e1.z; v = v + e1.w;
+              const uint32_t vb = readlane_u32(__float_as_uint(v), jl);
+              const uint32_t S_b = ((vb & 0x7fffffu) | 0x800000u) + readlane_u32(rest_b, jl);
+              if ((vb >> 23) == readlane_u32(kb_in, t) && S_b < (1u << 24)) {
+                K = vb >> 23;
+                S = S_b;
+                done = true;
+              }
+            }
+            if (done) ++n_prep_used;
+          }
+          if (!done) {
+            // ---- the general code, from the exact sum in front of the record
+            s = sum_value(S, static_cast<int>(K));
+            const int slot = base + t;
+            uint32_t bits[8];
+            if (readlane_u32(kind, t) == kSlotSerial && pi < n_prep) {
+              const PrepSlot& pg = prep[pi];
+              const float4 g0 = *reinterpret_cast<const float4*>(pg.e + lane * 8);
+              const float4 g1 = *reinterpret_cast<const float4*>(pg.e + lane * 8 + 4);
+              bits[0] = __float_as_uint(g0.x); bits[1] = __float_as_uint(g0.y); bits[2] = __float_as_uint(g0.z); bits[3] = __float_as_uint(g0.w);
+              bits[4] = __float_as_uint(g1.x); bits[5] = __float_as_uint(g1.y); bits[6] = __float_as_uint(g1.z); bits[7] = __float_as_uint(g1.w);
+              if (uniform_u32(pg.usable)) {
+                const uint64_t tie_a = (static_cast<uint64_t>(uniform_u32(pg.tie_a_hi)) << 32) | uniform_u32(pg.tie_a_lo);
+                const uint64_t tie_b = (static_cast<uint64_t>(uniform_u32(pg.tie_b_hi)) << 32) | uniform_u32(pg.tie_b_lo);
+                resolve_lanes(s, bits, pg.pre_a[lane] & kPrepSum, pg.pre_b[lane] & kPrepSum, tie_a, tie_b, uniform_u32(pg.kb_a), uniform_u32(pg.kb_b),
+                              slot * kSlot + lane * 8, V, stats ? &n_inner : nullptr);
+                ++n_prep_used;
+              } else {
+                int found = -1;
+                wave_resolve<8>(s, found, bits, slot * kSlot + lane * 8, V, kInf);
+                ++n_generic;
+              }
+            } else {
+              float l[8];
+              load_slot_lane<DT>(logits, slot, lane, V, fill, l, fused);
+#pragma unroll
+              for (int k = 0; k < 8; ++k) bits[k] = __float_as_uint(expf_core(__builtin_fmaxf(l[k] * inv - m, -104.0f), tab));
+              int found = -1;
+              wave_resolve<8>(s, found, bits, slot * kSlot + lane * 8, V, kInf);
+              ++n_generic;
+            }
+            sb = uniform_u32(__float_as_uint(s));
+            K = sb >> 23 ? sb >> 23 : 1u;
+            S = sb >> 23 ? ((sb & 0x7fffffu) | 0x800000u) : sb;
+          }
+          ++n_iter;
+        }
+        cur = t + 1;
+      }
+      s = sum_value(S, static_cast<int>(K));
+      if (fast_ok) cur = 64;
+    }
+    if (stats) {
+      const uint64_t now = wall_clock64();
+      ph_walk += now - ph_t;
+      ph_t = now;
+    }
+    // ---- record by record (a run in which the sum leaves its binade)
     int K_scan = -1;
     uint32_t incl = 0u;
     uint64_t plain_mask = 0ull;
@@ -996,11 +1231,11 @@ __device__ __forceinline__ float split_chain(const SlotRec* recs, int ns, const 
           const float4 e1 = *reinterpret_cast<const float4*>(ps.e + lane * 8 + 4);
           bits[0] = __float_as_uint(e0.x); bits[1] = __float_as_uint(e0.y); bits[2] = __float_as_uint(e0.z); bits[3] = __float_as_uint(e0.w);
           bits[4] = __float_as_uint(e1.x); bits[5] = __float_as_uint(e1.y); bits[6] = __float_as_uint(e1.z); bits[7] = __float_as_uint(e1.w);
-          if (ps.usable) {
-            const uint64_t tie_a = (static_cast<uint64_t>(ps.tie_a_hi) << 32) | ps.tie_a_lo;
-            const uint64_t tie_b = (static_cast<uint64_t>(ps.tie_b_hi) << 32) | ps.tie_b_lo;
+          if (uniform_u32(ps.usable)) {
+            const uint64_t tie_a = (static_cast<uint64_t>(uniform_u32(ps.tie_a_hi)) << 32) | uniform_u32(ps.tie_a_lo);
+            const uint64_t tie_b = (static_cast<uint64_t>(uniform_u32(ps.tie_b_hi)) << 32) | uniform_u32(ps.tie_b_lo);
             const uint64_t cb = stats ? wall_clock64() : 0;
-            resolve_lanes(s, bits, ps.pre_a[lane], ps.pre_b[lane], tie_a, tie_b, ps.kb_a, ps.kb_b, slot * kSlot + lane * 8, V,
+            resolve_lanes(s, bits, ps.pre_a[lane] & kPrepSum, ps.pre_b[lane] & kPrepSum, tie_a, tie_b, uniform_u32(ps.kb_a), uniform_u32(ps.kb_b), slot * kSlot + lane * 8, V,
                           stats ? &n_inner : nullptr);
             if (stats) c_prep += wall_clock64() - cb;
             ++n_prep_used;
@@ -1026,7 +1261,8 @@ __device__ __forceinline__ float split_chain(const SlotRec* recs, int ns, const 
   }
   if (stats && lane == 0) {
     stats[4] = 0;
-    stats[6] = static_cast<uint64_t>(n_iter) | (static_cast<uint64_t>(n_generic) << 32);
+    stats[6] = static_cast<uint64_t>(n_iter & 255u) | (static_cast<uint64_t>(n_generic & 255u) << 8) | ((ph_load & 0xffff) << 16) |
+               ((ph_scan & 0xffff) << 32) | ((ph_walk & 0xffff) << 48);
     stats[7] = static_cast<uint64_t>(n_prep_used) | (static_cast<uint64_t>(n_tie) << 16) | (static_cast<uint64_t>(n_inner) << 32) |
                (c_prep << 48);
   }
@@ -1045,6 +1281,7 @@ __device__ __forceinline__ float split_chain_walk(const SlotRec* recs, int ns, c
                                                   const FusedOps& fused, uint64_t* stats, const RowDivisor* div,
                                                   float threshold, int* stop) {
   constexpr bool WALK = true;
+  n_prep = uniform_u32(n_prep);
   const int lane = threadIdx.x & 63;
   const float kInf = __uint_as_float(0x7f800000u);
   const float fill = inv < 0.0f ? kInf : -kInf;
@@ -1151,11 +1388,11 @@ __device__ __forceinline__ float split_chain_walk(const SlotRec* recs, int ns, c
           const float4 e1 = *reinterpret_cast<const float4*>(ps.e + lane * 8 + 4);
           bits[0] = __float_as_uint(e0.x); bits[1] = __float_as_uint(e0.y); bits[2] = __float_as_uint(e0.z); bits[3] = __float_as_uint(e0.w);
           bits[4] = __float_as_uint(e1.x); bits[5] = __float_as_uint(e1.y); bits[6] = __float_as_uint(e1.z); bits[7] = __float_as_uint(e1.w);
-          if (ps.usable) {
-            const uint64_t tie_a = (static_cast<uint64_t>(ps.tie_a_hi) << 32) | ps.tie_a_lo;
-            const uint64_t tie_b = (static_cast<uint64_t>(ps.tie_b_hi) << 32) | ps.tie_b_lo;
+          if (uniform_u32(ps.usable)) {
+            const uint64_t tie_a = (static_cast<uint64_t>(uniform_u32(ps.tie_a_hi)) << 32) | uniform_u32(ps.tie_a_lo);
+            const uint64_t tie_b = (static_cast<uint64_t>(uniform_u32(ps.tie_b_hi)) << 32) | uniform_u32(ps.tie_b_lo);
             const uint64_t cb = stats ? wall_clock64() : 0;
-            resolve_lanes(s, bits, ps.pre_a[lane], ps.pre_b[lane], tie_a, tie_b, ps.kb_a, ps.kb_b, slot * kSlot + lane * 8, V,
+            resolve_lanes(s, bits, ps.pre_a[lane] & kPrepSum, ps.pre_b[lane] & kPrepSum, tie_a, tie_b, uniform_u32(ps.kb_a), uniform_u32(ps.kb_b), slot * kSlot + lane * 8, V,
                           stats ? &n_inner : nullptr);
             if (stats) c_prep += wall_clock64() - cb;
             ++n_prep_used;
@@ -1795,7 +2032,8 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
   const int R = LOOP ? p.chain_rows : 1;
   const int n_units = (p.row.rows + R - 1) / R;
   const size_t lds_bytes = static_cast<size_t>(p.row.lds_keys) * sizeof(uint64_t);
-  const size_t rec_bytes = (static_cast<size_t>(ns) * sizeof(SlotRec) + 15) / 16 * 16;
+  const size_t rec_bytes = chain_rec_bytes(ns);  // the records and, behind them, the pairs of split_chain_prepare()
+  const size_t pairs_at = chain_pairs_offset(ns);
   for (int unit = blockIdx.x; unit < n_units; unit = LOOP ? take_row(p.row, &next_lrow, n_units) : n_units) {
   if (LOOP) request_row(p.row, &next_lrow, n_units);
   const int r_first = unit * R;
@@ -1822,6 +2060,16 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
       for (int i = tid; i < prep_vecs; i += kBlock) dst[rec_bytes / 16 + i] = prep_src[i];
     }
     __syncthreads();
+    {
+      // the runs of every row's records, the rows' chunks spread over the waves (a NaN row's share
+      // holds stale records: nothing reads what comes of them)
+      const int k = wave % r_count, per_row = kWaves / r_count;
+      if (wave / r_count < per_row) {
+        char* mine = reinterpret_cast<char*>(lds_keys) + static_cast<size_t>(k) * share;
+        split_chain_prepare(reinterpret_cast<const SlotRec*>(mine), ns, reinterpret_cast<uint2*>(mine + pairs_at), wave / r_count, per_row);
+      }
+    }
+    __syncthreads();
     if (wave < r_count) {
       const int row_k = p.row.row_map ? p.row.row_map[r_first + wave] : r_first + wave;
       const RowState st = p.row_state[row_k];
@@ -1830,7 +2078,8 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
         const float inv_k = p.row.row_cfg ? p.row.row_cfg[row_k].inv_temperature : p.row.inv_temperature;
         const char* logits_k = static_cast<const char*>(p.row.logits) + static_cast<int64_t>(row_k) * p.row.row_stride * ElemSize<DT>::value;
         const char* mine = reinterpret_cast<const char*>(lds_keys) + static_cast<size_t>(wave) * share;
-        sum = split_chain<DT>(reinterpret_cast<const SlotRec*>(mine), ns, reinterpret_cast<const PrepSlot*>(mine + rec_bytes),
+        sum = split_chain<DT>(reinterpret_cast<const SlotRec*>(mine), reinterpret_cast<const uint2*>(mine + pairs_at), ns,
+                              reinterpret_cast<const PrepSlot*>(mine + rec_bytes),
                               prepared(st), logits_k, V, inv_k, st.m, sm.exp2tab, p.row.fused,
                               timers ? timers + static_cast<int64_t>(row_k) * 8 : nullptr);
       }
@@ -1942,16 +2191,32 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
       }
     }
     __syncthreads();
+    // the runs of the row's records, a chunk of 64 per wave (the barriers of split_plan() lie between this and the chain)
+    if (!chained)
+      split_chain_prepare(reinterpret_cast<const SlotRec*>(lds_keys), ns,
+                          reinterpret_cast<uint2*>(reinterpret_cast<char*>(lds_keys) + pairs_at), wave, kWaves);
     n_listed = static_cast<int>(fs.offset[p.row_wgs]);
     lists_ok = fs.overflow == 0u;
     plan = split_plan(fs.hist, rs.a_total, topp, cutoff, V, &fs.plan, sm);
     if (timers) t1 = wall_clock64();
     if (wave == 0) {
       if (!chained) {
-        const float sum = split_chain<DT>(reinterpret_cast<const SlotRec*>(lds_keys), ns,
+        const float sum = split_chain<DT>(reinterpret_cast<const SlotRec*>(lds_keys),
+                                          reinterpret_cast<const uint2*>(reinterpret_cast<const char*>(lds_keys) + pairs_at), ns,
                                           reinterpret_cast<const PrepSlot*>(prep_dst), n_prep, logits, V, inv, m, sm.exp2tab,
                                           p.row.fused, timers ? timers + static_cast<int64_t>(row) * 8 : nullptr);
         if (lane == 0) sm.bc_sum = sum;
+#if ETS_PHASE_CLOCKS
+        if (timers) {  // the same chain once more, its code now in the instruction cache and no clocks inside
+          const uint64_t ta = wall_clock64();
+          const float again = split_chain<DT>(reinterpret_cast<const SlotRec*>(lds_keys),
+                                              reinterpret_cast<const uint2*>(reinterpret_cast<const char*>(lds_keys) + pairs_at), ns,
+                                              reinterpret_cast<const PrepSlot*>(prep_dst), n_prep, logits, V, inv, m, sm.exp2tab,
+                                              p.row.fused, nullptr);
+          const uint64_t tb = wall_clock64();
+          if (lane == 0) timers[static_cast<int64_t>(row) * 8 + 5] = (tb - ta) | (again == sum ? 0ull : 1ull << 40);
+        }
+#endif
       } else if (lane == 0) {
         sm.bc_sum = fs.pre_sum[lrow - r_first];
       }
@@ -2206,7 +2471,7 @@ __global__ void __launch_bounds__(kWalkBlock) split_walk_kernel(SplitParams p, u
   }
   const float inv = p.row.row_cfg ? p.row.row_cfg[row].inv_temperature : p.row.inv_temperature;
   const char* logits = static_cast<const char*>(p.row.logits) + static_cast<int64_t>(row) * p.row.row_stride * ElemSize<DT>::value;
-  const size_t rec_bytes = (static_cast<size_t>(ns) * sizeof(SlotRec) + 15) / 16 * 16;
+  const size_t rec_bytes = chain_rec_bytes(ns);
   uint32_t n_prep = rs.prep_count < static_cast<uint32_t>(p.prep_cap) ? rs.prep_count : static_cast<uint32_t>(p.prep_cap);
   const uint32_t fit = lds_bytes > rec_bytes ? static_cast<uint32_t>((lds_bytes - rec_bytes) / sizeof(PrepSlot)) : 0u;
   n_prep = n_prep < fit ? n_prep : fit;  // (a prepared slot that does not fit is redone from the logits)
@@ -2217,11 +2482,16 @@ __global__ void __launch_bounds__(kWalkBlock) split_walk_kernel(SplitParams p, u
   const int prep_vecs = static_cast<int>(n_prep * (sizeof(PrepSlot) / 16));
   for (int i = tid; i < prep_vecs; i += kWalkBlock) lds_vec[rec_bytes / 16 + i] = prep_src[i];
   __syncthreads();
+  uint2* pairs = reinterpret_cast<uint2*>(reinterpret_cast<char*>(walk_lds) + chain_pairs_offset(ns));
+  if (PHASE == 0) {  // the runs of the row's records, a chunk of 64 per wave
+    split_chain_prepare(reinterpret_cast<const SlotRec*>(walk_lds), ns, pairs, tid >> 6, kWalkBlock / 64);
+    __syncthreads();
+  }
   if (tid >= 64) return;
   const SlotRec* recs = reinterpret_cast<const SlotRec*>(walk_lds);
   const PrepSlot* prep = reinterpret_cast<const PrepSlot*>(reinterpret_cast<const char*>(walk_lds) + rec_bytes);
   if (PHASE == 0) {
-    const float S = split_chain<DT>(recs, ns, prep, n_prep, logits, V, inv, rs.m, exp2tab, p.row.fused,
+    const float S = split_chain<DT>(recs, pairs, ns, prep, n_prep, logits, V, inv, rs.m, exp2tab, p.row.fused,
                                     walk_timers ? walk_timers + static_cast<int64_t>(row) * 8 : nullptr);
     if (lane == 0) p.walk[row] = make_float2(S, toss());
   } else {

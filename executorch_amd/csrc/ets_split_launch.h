@@ -89,6 +89,9 @@ ets_status launch_split(ets_sampler* s, const ets::RowParams& p, int32_t rows, h
     }();
     const int per_wg = (rows + p.grid_cap - 1) / p.grid_cap;
     sp.chain_rows = per_wg < chain_rows_max ? per_wg : chain_rows_max;
+    // every row of a unit needs room for its records and at least one prepared slot in its share of the key buffer
+    const int by_lds = static_cast<int>(s->lds_bytes / (ets::chain_rec_bytes(sp.ns) + sizeof(ets::PrepSlot)));
+    if (sp.chain_rows > by_lds) sp.chain_rows = by_lds < 1 ? 1 : by_lds;
     const int units = (rows + sp.chain_rows - 1) / sp.chain_rows;
     const dim3 grid(units < p.grid_cap ? units : p.grid_cap);
     if (extras) {
@@ -140,7 +143,7 @@ ets_status launch_split_walk(ets_sampler* s, const ets::RowParams& p, int32_t ro
   ETS_HIP(s, hipGetLastError());
   const size_t lut_bytes = DT == ets::kDtypeBFloat16 ? sizeof(float) * ets::kLutCountWords : 0;
   // the walk kernel's LDS: the row's records and as many prepared slots as fit beside them
-  const uint32_t walk_lds = static_cast<uint32_t>(round_up(static_cast<size_t>(sp.ns) * sizeof(ets::SlotRec), 16) + 16 * sizeof(ets::PrepSlot));
+  const uint32_t walk_lds = static_cast<uint32_t>(ets::chain_rec_bytes(sp.ns) + 16 * sizeof(ets::PrepSlot));
   static std::atomic<size_t> set_sum[kMaxDevices], set_walk[kMaxDevices], set_k0[kMaxDevices], set_k1[kMaxDevices];
   st = allow_dynamic_lds(s, reinterpret_cast<const void*>(&ets::split_pass2_kernel<DT, false, false>), lut_bytes, set_sum);
   if (st != ETS_OK) return st;

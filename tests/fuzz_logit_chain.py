@@ -10,7 +10,8 @@ penalties over histories with repeats, out-of-range ids and zero lengths.  The c
 the device and the restatement (test infrastructure, never the thing measured) processor by
 processor on the host; every element must be equal bit for bit (NaN with NaN), and the sequence
 positions before the last one of a rank-3 tensor must be untouched.  Prints one JSON line; exits
-non-zero on a mismatch and names the case.  Not collected by pytest.
+non-zero on a mismatch and names the case.  tests/test_gpu_logit_processor.py runs a few hundred
+cases of it with every GPU suite.
 """
 import argparse
 import json
@@ -35,12 +36,9 @@ def make_values(rng, shape, kind, lpo):
     return lpo.storage_round(x, kind)
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--cases", type=int, default=1000)
-    ap.add_argument("--seed", type=int, default=1)
-    ap.add_argument("--max-vocab", type=int, default=200000)
-    args = ap.parse_args()
+def run(cases=1000, seed=1, max_vocab=200000, stop_after=10):
+    """The comparison; returns the report as a dict (stops after `stop_after` mismatches)."""
+    args = argparse.Namespace(cases=cases, seed=seed, max_vocab=max_vocab)
 
     import torch
 
@@ -123,13 +121,23 @@ def main():
         if not ok:
             failures.append(label)
             print("fuzz_logit_chain: MISMATCH", json.dumps(label), file=sys.stderr, flush=True)
-            if len(failures) >= 10:
+            if len(failures) >= stop_after:
                 break
         if case % 100 == 99:
             print(f"fuzz_logit_chain: {case + 1} cases, {len(failures)} failures, {time.time() - t0:.0f} s", file=sys.stderr,
                   flush=True)
-    print(json.dumps({"cases": case + 1, "failures": len(failures), "first_failures": failures[:3], "seconds": round(time.time() - t0, 1)}))
-    sys.exit(1 if failures else 0)
+    return {"cases": case + 1, "failures": len(failures), "first_failures": failures[:3], "seconds": round(time.time() - t0, 1)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--cases", type=int, default=1000)
+    ap.add_argument("--seed", type=int, default=1)
+    ap.add_argument("--max-vocab", type=int, default=200000)
+    args = ap.parse_args()
+    res = run(args.cases, args.seed, args.max_vocab)
+    print(json.dumps(res))
+    sys.exit(1 if res["failures"] else 0)
 
 
 if __name__ == "__main__":

@@ -223,3 +223,13 @@ def test_chain_fused_falls_back_in_place(dev):
         got = s2.sample_batch_chain(b, c2).cpu().numpy()
         assert np.array_equal(got, want)
         assert torch.equal(a, b)
+
+
+def test_randomised_chains_against_the_restatement():
+    """A few hundred random chains over random tensors (tests/fuzz_logit_chain.py), every element
+    compared bit for bit with the CPU restatement; stops at the first mismatch."""
+    import fuzz_logit_chain
+
+    res = fuzz_logit_chain.run(cases=300, seed=5, stop_after=1)
+    assert res["failures"] == 0, res["first_failures"]
+    assert res["cases"] == 300
