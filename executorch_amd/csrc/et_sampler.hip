@@ -110,11 +110,16 @@ ets_status ensure_split(ets_sampler* s) {
   const size_t o_state = take(rows * sizeof(ets::RowState));
   const size_t o_walk = take(rows * sizeof(float2));
   const size_t o_count = take(rows * ets::kMaxRowWorkgroups * sizeof(uint32_t));
+  const size_t o_arrive = take(rows * 2 * sizeof(uint32_t));
+  const size_t o_part = take(rows * ets::kMaxRowWorkgroups * sizeof(float));
   const size_t o_timers = take(rows * 12 * sizeof(uint64_t));
   const size_t o_hist = take(row_wgs * ets::kHistBuckets * sizeof(uint32_t));
   const size_t o_list = take(list_entries * sizeof(uint64_t));
   ETS_HIP(s, hipMalloc(&s->d_split, at));
   char* base = static_cast<char*>(s->d_split);
+  ETS_HIP(s, hipMemset(base + o_arrive, 0, rows * 2 * sizeof(uint32_t)));  // (0 between launches)
+  sp.arrive = reinterpret_cast<uint32_t*>(base + o_arrive);
+  sp.part_max = reinterpret_cast<float*>(base + o_part);
   sp.slot_max = reinterpret_cast<float*>(base + o_max);
   sp.slot_max2 = reinterpret_cast<float*>(base + o_max2);
   sp.slot_sum = reinterpret_cast<float*>(base + o_sum);
@@ -137,6 +142,15 @@ ets_status ensure_phist(ets_sampler* s) {
   ETS_HIP(s, hipMalloc(&s->d_phist, bytes));
   s->split.phist = static_cast<uint32_t*>(s->d_phist);
   return ETS_OK;
+}
+
+namespace {
+bool g_static_arrive_dirty[kMaxDevices] = {};
+}
+
+bool* arrive_dirty_flag(ets_sampler* s) {
+  if (!s->wb) return &s->arrive_dirty;
+  return &g_static_arrive_dirty[s->device >= 0 && s->device < kMaxDevices ? s->device : 0];
 }
 
 }  // namespace ets_host
@@ -364,6 +378,7 @@ ets_status sample_device(ets_sampler* s, const void* d_logits, int32_t dtype, in
 // process ends.  Host code never uses the array's name as an address: the device address is looked
 // up once per device (at the first handle created there) and kept.
 constexpr size_t kStaticScratchBytes = size_t{32} << 20;
+constexpr int kStaticArriveRows = 1024;
 static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 std::mutex g_static_mutex;
@@ -404,6 +419,10 @@ size_t layout_static(const ets_sampler* s, int32_t dtype, int32_t rows, char* ba
     return base + here;
   };
   wb->tickets = reinterpret_cast<uint32_t*>(take(16 * sizeof(uint32_t)));  // always the array's first bytes: 0 between launches
+  // (the same bytes whatever the call's sizes: 0 between launches, like the tickets.  A call of more
+  // rows than this holds does not use the fused launch.)
+  sp.arrive = reinterpret_cast<uint32_t*>(take(kStaticArriveRows * 2 * sizeof(uint32_t)));
+  wb->arrive_rows = kStaticArriveRows;
   sp.slot_max = reinterpret_cast<float*>(take(r * sp.ns_stride * sizeof(float)));
   sp.slot_max2 = reinterpret_cast<float*>(take(r * sp.ns_stride * sizeof(float)));
   sp.slot_sum = reinterpret_cast<float*>(take(r * sp.ns_stride * sizeof(float)));
@@ -412,6 +431,7 @@ size_t layout_static(const ets_sampler* s, int32_t dtype, int32_t rows, char* ba
   sp.row_state = reinterpret_cast<ets::RowState*>(take(r * sizeof(ets::RowState)));
   sp.walk = reinterpret_cast<float2*>(take(r * sizeof(float2)));
   sp.list_count = reinterpret_cast<uint32_t*>(take(r * ets::kMaxRowWorkgroups * sizeof(uint32_t)));
+  sp.part_max = reinterpret_cast<float*>(take(r * ets::kMaxRowWorkgroups * sizeof(float)));
   sp.hist = reinterpret_cast<uint32_t*>(take(r * g * ets::kHistBuckets * sizeof(uint32_t)));
   sp.phist = reinterpret_cast<uint32_t*>(take(r * g * phist_words * sizeof(uint32_t)));
   sp.list = reinterpret_cast<uint64_t*>(take(r * g * list_region(sp.ns, g) * sizeof(uint64_t)));

@@ -25,6 +25,7 @@ struct WorkBuffers {
   int64_t scratch_stride = 0;
   uint64_t* partials = nullptr;  // [rows, kMaxSplits] arg-max partial results
   int max_row_wgs = 0;           // workgroups of pass 2 per row, at most
+  int arrive_rows = 0;           // rows the fused launch's counters are laid out for
 };
 
 struct ets_sampler {
@@ -52,6 +53,7 @@ struct ets_sampler {
   int num_cus = 0;
   void* d_split = nullptr;
   void* d_phist = nullptr;  // pattern histograms of 16-bit rows, allocated on their first use
+  bool arrive_dirty = false;  // a fused launch was not followed by its finish kernel: the counters are cleared before the next one
   ets::SplitParams split = {};
   // per-row sampling parameters of ets_sampler_sample_batch_configs(): pinned host staging, its
   // device copy, and the event that says the last upload has left the staging buffer
@@ -113,6 +115,10 @@ ets_status allow_dynamic_lds(ets_sampler* s, const void* kernel, size_t bytes, s
 ets_status ensure_split(ets_sampler* s);
 ets_status ensure_phist(ets_sampler* s);
 int pass2_workgroups(const ets_sampler* s, int32_t rows, int32_t ns);
+// Whether the arrival counters of the fused launch may hold something other than 0 (a fused launch
+// whose finish kernel was never launched): the handle's own flag, or, for a call that works in the
+// library's static array, that device's.
+bool* arrive_dirty_flag(ets_sampler* s);
 int32_t list_region(int32_t ns, int g);
 
 // ---- launchers, one translation unit per element type -------------------------------------------

@@ -149,6 +149,10 @@ struct SplitParams {
                         //   counters per word, from order key RowState::key_cut upwards
   int32_t phist_words;  // words per (row, workgroup) region; 0 disables the pattern histogram
   float2* walk;         // [rows] multinomial rows: the exact softmax sum and the coin, between the two chains
+  uint32_t* arrive;     // [rows, 2] the fused launch: workgroups of the row that have stored their largest x, and their
+                        //   slots' maxima and sums (0 before a launch; the finish kernel puts them back)
+  float* part_max;      // [rows, kMaxRowWorkgroups] the fused launch: every workgroup's largest x
+  int32_t spin_limit;   // the fused launch: polls of `arrive` after which a workgroup stops waiting for the others
   uint64_t* timers;     // phase clocks (profiling), or null
   int32_t list_region;  // entries per region
   int32_t short_lists;  // 1: pass 2 may list only the largest candidates of a peaked row (see RowState::listed_buckets)
@@ -207,6 +211,94 @@ __device__ __forceinline__ void split_range(int ns, int wgs, int x, int& s_begin
   s_end = min(ns, s_begin + per_wg);
 }
 
+// Pass 1 for one slot, by one wave: `v` are the lane's 8 entries (logits; products with an
+// infinite inv_temperature when `inv_u` is 1 for that reason).  Stores the slot's maximum of
+// x = logit * inv_temperature (NaN when the slot holds one), the largest x of the other 63 lanes and
+// the approximate sum of exp(x - slot maximum).
+// Few instructions per entry (with a workgroup per row the kernel would otherwise be bound by
+// them, not by HBM): the maximum is taken over the raw logits -- rounding is monotone, so the
+// largest product l * inv is the product of the largest (smallest, for a negative inv) logit --
+// and the exponent comes from one fused multiply-add per entry.
+// COHERENT: the three values are read by other workgroups of the same launch (the fused kernel): they
+// are stored with device-scope accesses that go through to memory, one by one, so that no workgroup
+// has to write its die's whole L2 back (a release fence does, and costs microseconds per workgroup
+// when every workgroup of a die issues one).
+__device__ __forceinline__ void coherent_store(float* ptr, float v) {
+  __hip_atomic_store(reinterpret_cast<uint32_t*>(ptr), __float_as_uint(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float coherent_load(const float* ptr) {
+  return __uint_as_float(__hip_atomic_load(reinterpret_cast<const uint32_t*>(ptr), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+}
+struct SlotMax {
+  float M, M2;  // the slot's largest x = logit * inv_temperature (NaN entries ignored), and the largest of the other 63 lanes
+};
+__device__ __forceinline__ SlotMax split_pass1_max(const float (&v)[8], float inv_u) {
+  const int lane = threadIdx.x & 63;
+  const float kInf = __uint_as_float(0x7f800000u);
+  float ext = inv_u < 0.0f ? kInf : -kInf;
+  if (inv_u < 0.0f) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ext = __builtin_fminf(ext, v[e]);  // ignores NaN
+  } else {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ext = __builtin_fmaxf(ext, v[e]);
+  }
+  // (a lane whose entries all lie past the row's end holds the fill value, whose product is -inf)
+  // (reduced as integer keys: one instruction per step.  A NaN product -- the row is one then --
+  // may come out as the maximum: the slot's maximum is stored as NaN in that case anyway.)
+  const uint32_t xk = float_max_key(ext * inv_u);
+  const uint32_t Mk = wave_max_u32(xk);
+  // the largest entry of the other lanes (pass 2 bounds the mass of the row's largest entries
+  // from below with the two)
+  const uint64_t holds = __ballot(xk == Mk);
+  const int holder = __ffsll(static_cast<long long>(holds)) - 1;  // (some lane holds the maximum)
+  return {float_of_max_key(Mk), float_of_max_key(wave_max_u32(lane == holder ? float_max_key(-kInf) : xk))};
+}
+template <bool COHERENT = false>
+__device__ __forceinline__ void split_pass1_sum(const SplitParams& p, int row, int s, const float (&v)[8], float inv_u, SlotMax x) {
+  const int lane = threadIdx.x & 63;
+  const float kInf = __uint_as_float(0x7f800000u);
+  const float c1 = inv_u * kLog2e;
+  const float M = x.M;
+  // With a finite maximum of ordinary size every entry's exponent below is finite or -inf unless
+  // the entry is NaN, so the sum itself tells whether the slot holds a NaN; otherwise the
+  // entries are tested one by one.
+  const bool ordinary = M > -kInf && __builtin_fabsf(M) < 1e38f;
+  float sum = 0.0f;
+  bool nan = false;
+  if (ordinary) {
+    const float c2 = -M * kLog2e;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) sum += fast_exp2(__builtin_fmaf(v[e], c1, c2));
+  } else {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) nan = nan || (v[e] != v[e]);
+    if (M > -kInf) {
+      const float c2 = -M * kLog2e;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) sum += fast_exp2(__builtin_fmaf(v[e], c1, c2));  // (a NaN here: the row is one)
+    }
+  }
+  sum = wave_sum_f32(sum);
+  const bool any_nan = ordinary ? sum != sum : __ballot(nan) != 0ull;
+  if (lane == 0) {
+    const int64_t at = static_cast<int64_t>(row) * p.ns_stride + s;
+    if (COHERENT) {
+      coherent_store(p.slot_max + at, any_nan ? __uint_as_float(0x7fc00000u) : M);
+      coherent_store(p.slot_max2 + at, x.M2);
+      coherent_store(p.slot_sum + at, sum);
+    } else {
+      p.slot_max[at] = any_nan ? __uint_as_float(0x7fc00000u) : M;
+      p.slot_max2[at] = x.M2;
+      p.slot_sum[at] = sum;
+    }
+  }
+}
+template <bool COHERENT = false>
+__device__ __forceinline__ void split_pass1_slot(const SplitParams& p, int row, int s, const float (&v)[8], float inv_u) {
+  split_pass1_sum<COHERENT>(p, row, s, v, inv_u, split_pass1_max(v, inv_u));
+}
+
 // grid = (ceil(ns / (4 SLOTS)), rows), 256 lanes: every wave takes SLOTS slots, all loads issued first.
 // (Small workgroups: many are resident per CU, which is what a kernel bound by HBM wants.)
 constexpr int kPass1Block = 256;
@@ -229,12 +321,6 @@ __global__ void __launch_bounds__(kPass1Block) split_pass1_kernel(SplitParams p)
     for (int k = 0; k < SLOTS; ++k) {
       if (slot0 + k < s_end) load_slot_lane<DT>(logits, slot0 + k, lane, V, fill, v[k], p.row.fused);
     }
-    // Few instructions per entry (with a workgroup per row the kernel would otherwise be bound by
-    // them, not by HBM): the maximum is taken over the raw logits -- rounding is monotone, so the
-    // largest product l * inv is the product of the largest (smallest, for a negative inv) logit --
-    // and the exponent comes from one fused multiply-add per entry.
-    // (An infinite inv can turn a finite logit into a NaN product: then the products themselves
-    // are reduced, with a factor of 1.)
     float inv_u = inv;
     if (!(__builtin_fabsf(inv) < kInf)) {
 #pragma unroll
@@ -244,57 +330,11 @@ __global__ void __launch_bounds__(kPass1Block) split_pass1_kernel(SplitParams p)
       }
       inv_u = 1.0f;
     }
-    const float c1 = inv_u * kLog2e;
 #pragma unroll
     for (int k = 0; k < SLOTS; ++k) {
       const int s = slot0 + k;
       if (s >= s_end) break;
-      float ext = inv_u < 0.0f ? kInf : -kInf;
-      if (inv_u < 0.0f) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) ext = __builtin_fminf(ext, v[k][e]);  // ignores NaN
-      } else {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) ext = __builtin_fmaxf(ext, v[k][e]);
-      }
-      // (a lane whose entries all lie past the row's end holds the fill value, whose product is -inf)
-      // (reduced as integer keys: one instruction per step.  A NaN product -- the row is one then --
-      // may come out as the maximum: the slot's maximum is stored as NaN in that case anyway.)
-      const uint32_t xk = float_max_key(ext * inv_u);
-      const uint32_t Mk = wave_max_u32(xk);
-      const float M = float_of_max_key(Mk);
-      // the largest entry of the other lanes (pass 2 bounds the mass of the row's largest entries
-      // from below with the two)
-      const uint64_t holds = __ballot(xk == Mk);
-      const int holder = __ffsll(static_cast<long long>(holds)) - 1;  // (some lane holds the maximum)
-      const float M2 = float_of_max_key(wave_max_u32(lane == holder ? float_max_key(-kInf) : xk));
-      // With a finite maximum of ordinary size every entry's exponent below is finite or -inf unless
-      // the entry is NaN, so the sum itself tells whether the slot holds a NaN; otherwise the
-      // entries are tested one by one.
-      const bool ordinary = M > -kInf && __builtin_fabsf(M) < 1e38f;
-      float sum = 0.0f;
-      bool nan = false;
-      if (ordinary) {
-        const float c2 = -M * kLog2e;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) sum += fast_exp2(__builtin_fmaf(v[k][e], c1, c2));
-      } else {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) nan = nan || (v[k][e] != v[k][e]);
-        if (M > -kInf) {
-          const float c2 = -M * kLog2e;
-#pragma unroll
-          for (int e = 0; e < 8; ++e) sum += fast_exp2(__builtin_fmaf(v[k][e], c1, c2));  // (a NaN here: the row is one)
-        }
-      }
-      sum = wave_sum_f32(sum);
-      const bool any_nan = ordinary ? sum != sum : __ballot(nan) != 0ull;
-      if (lane == 0) {
-        const int64_t at = static_cast<int64_t>(row) * p.ns_stride + s;
-        p.slot_max[at] = any_nan ? __uint_as_float(0x7fc00000u) : M;
-        p.slot_max2[at] = M2;
-        p.slot_sum[at] = sum;
-      }
+      split_pass1_slot(p, row, s, v[k], inv_u);
     }
   }
 }
@@ -510,14 +550,36 @@ __device__ __forceinline__ void split_fold_slot(const SplitParams& p, int row, i
 // WALK: the second sum of a multinomial row (sampler.cpp:58-70): the entries are p = fl(e / S) with the exact
 // softmax sum S that the first chain left in SplitParams::walk, and the records describe their running sum.
 // TOPK: some row of the launch may be a top-k row (a launch without one runs the code without that case).
-template <int DT, bool TOPP, bool WALK = false, bool TOPK = false, bool EXTRAS = true>
+// FUSED: pass 1 inside this kernel, for launches whose workgroups are all resident at once (at most one per
+// compute unit) and hold at most kFusedSlots slots per wave: a workgroup loads its slots ONCE, keeps them in
+// registers, stores their maxima and approximate sums, and meets the other workgroups of its row at a counter
+// in device memory before it goes on with what pass 2 does.  The wait is bounded: a workgroup that has polled
+// `spin_limit` times works the other workgroups' slots out itself from the logits (the same values: whoever
+// stores them stores the same bits), so every workgroup ends whatever the others do.  The grid is one-
+// dimensional and the workgroups of a row are dealt so that they share a die (XCD) and its L2 when the number
+// of rows is a multiple of eight (workgroups go to the eight dies in turn by their index).
+constexpr int kFusedSlots = 4;
+template <int DT, bool TOPP, bool WALK = false, bool TOPK = false, bool EXTRAS = true, bool FUSED = false>
 __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_kernel(SplitParams p) {
   uint64_t* const timers = (ETS_PHASE_CLOCKS && EXTRAS) ? p.timers : nullptr;  // (EXTRAS: the launch may fill the phase clocks)
   extern __shared__ __align__(16) float lut_mem[];
   __shared__ Pass2Shared sh;
   BlockScratch& sm = sh.sm;
-  const int lrow = blockIdx.y;  // row of this launch: indexes the buffers whose layout depends on the launch
-  const int row = p.row.row_map ? p.row.row_map[blockIdx.y] : blockIdx.y;
+  int part = blockIdx.x, n_parts = gridDim.x;
+  int lrow = blockIdx.y;  // row of this launch: indexes the buffers whose layout depends on the launch
+  if (FUSED) {
+    n_parts = p.row_wgs;
+    const int rows = p.row.rows;
+    if ((rows & 7) == 0) {
+      const int die = blockIdx.x & 7, k = blockIdx.x >> 3;  // rows die, die + 8, ... on one die
+      lrow = (k / n_parts) * 8 + die;
+      part = k % n_parts;
+    } else {
+      lrow = blockIdx.x / n_parts;
+      part = blockIdx.x % n_parts;
+    }
+  }
+  const int row = p.row.row_map ? p.row.row_map[lrow] : lrow;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
@@ -533,7 +595,7 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
   const float* slot_max2 = p.slot_max2 + static_cast<int64_t>(row) * p.ns_stride;
   const float kInf = __uint_as_float(0x7f800000u);
   const float fill = inv < 0.0f ? kInf : -kInf;
-  uint64_t c0 = 0, c1 = 0, c2 = 0, c3 = 0;
+  uint64_t c0 = 0, c1 = 0, c2 = 0, c3 = 0, cf0 = 0, cf1 = 0, cf2 = 0;
   if (timers) c0 = wall_clock64();
   if (tid < 32) sm.exp2tab[tid] = kExp2Table[tid];
   if (tid == 0) sh.list_count = 0u;
@@ -554,21 +616,121 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
   // ---- this workgroup's slots: wave w takes s_begin + w, s_begin + w + 16, ...; the first one's
   //      entries are requested before anything else
   int s_begin, s_end;
-  split_range(ns, gridDim.x, blockIdx.x, s_begin, s_end);
+  split_range(ns, n_parts, part, s_begin, s_end);
   float l[8];
   int s_mine = s_begin + wave;
-  if (s_mine < s_end) load_slot_lane<DT>(logits, s_mine, lane, V, fill, l, p.row.fused);
+  static_assert(kFusedSlots == 4, "four named register sets below");
+  int lut_base1 = 0, lut_top = 0, lut_half = 0;
+  int early_lut = -1;      // FUSED: the expf table was built for early_m already (1: usable, 0: not)
+  float early_m = 0.0f;
+  float held0[8], held1[8], held2[8], held3[8];  // FUSED: the wave's slots, read once (named one by one: they stay in registers)
+  if constexpr (FUSED) {
+    if (s_mine < s_end) load_slot_lane<DT>(logits, s_mine, lane, V, fill, held0, p.row.fused);
+    if (s_mine + kWaves < s_end) load_slot_lane<DT>(logits, s_mine + kWaves, lane, V, fill, held1, p.row.fused);
+    if (s_mine + 2 * kWaves < s_end) load_slot_lane<DT>(logits, s_mine + 2 * kWaves, lane, V, fill, held2, p.row.fused);
+    if (s_mine + 3 * kWaves < s_end) load_slot_lane<DT>(logits, s_mine + 3 * kWaves, lane, V, fill, held3, p.row.fused);
+    // ---- pass 1 for these slots (the host sends no launch with an infinite inverse temperature here),
+    //      in two steps, each handed to the row's other workgroups as soon as it is done: the
+    //      workgroup's largest x first -- the row maximum is all the expf table needs, and the table is
+    //      built while the second step's values are still on their way --, then every slot's maximum
+    //      and approximate sum.  What the workgroups exchange is stored and read with device-scope
+    //      accesses that go through to memory one by one, complete (the wait below) before lane 0
+    //      counts the workgroup in; no fence of device scope, which would write back or discard the
+    //      die's whole L2 (microseconds, when every workgroup of the die does it).
+    const float kNegInf = -kInf;
+    SlotMax x0m = {kNegInf, kNegInf}, x1m = x0m, x2m = x0m, x3m = x0m;
+    if (s_mine < s_end) x0m = split_pass1_max(held0, inv);
+    if (s_mine + kWaves < s_end) x1m = split_pass1_max(held1, inv);
+    if (s_mine + 2 * kWaves < s_end) x2m = split_pass1_max(held2, inv);
+    if (s_mine + 3 * kWaves < s_end) x3m = split_pass1_max(held3, inv);
+    if (lane == 0) sm.red_f[wave] = __builtin_fmaxf(__builtin_fmaxf(x0m.M, x1m.M), __builtin_fmaxf(x2m.M, x3m.M));
+    __syncthreads();
+    uint32_t* const arrive_max = p.arrive + 2 * lrow;
+    uint32_t* const arrive_sum = arrive_max + 1;
+    float* const part_max = p.part_max + static_cast<int64_t>(lrow) * kMaxRowWorkgroups;
+    if (tid == 0) {
+      float mw = sm.red_f[0];
+      for (int w = 1; w < kWaves; ++w) mw = __builtin_fmaxf(mw, sm.red_f[w]);
+      coherent_store(part_max + part, mw);
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __hip_atomic_fetch_add(arrive_max, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    if (s_mine < s_end) split_pass1_sum<true>(p, row, s_mine, held0, inv, x0m);
+    if (s_mine + kWaves < s_end) split_pass1_sum<true>(p, row, s_mine + kWaves, held1, inv, x1m);
+    if (s_mine + 2 * kWaves < s_end) split_pass1_sum<true>(p, row, s_mine + 2 * kWaves, held2, inv, x2m);
+    if (s_mine + 3 * kWaves < s_end) split_pass1_sum<true>(p, row, s_mine + 3 * kWaves, held3, inv, x3m);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (timers) cf0 = wall_clock64();
+    __syncthreads();
+    if (tid == 0) __hip_atomic_fetch_add(arrive_sum, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    // One lane polls a counter, a bounded number of times; every lane learns the outcome.
+    auto all_there = [&](uint32_t* counter) -> bool {
+      if (tid == 0) {
+        int met = 0;
+        for (int spin = 0; spin < p.spin_limit; ++spin) {
+          if (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= static_cast<uint32_t>(n_parts)) {
+            met = 1;
+            break;
+          }
+          __builtin_amdgcn_s_sleep(2);
+        }
+        sm.flag = met;
+      }
+      __syncthreads();
+      const bool met = sm.flag != 0;
+      __syncthreads();
+      return met;
+    };
+    // Given up on the others: their slots from the logits (whoever stores a slot's three values stores the same bits).
+    auto alone = [&]() {
+      for (int s = wave; s < ns; s += kWaves) {
+        if (s >= s_begin && s < s_end) continue;
+        float v[8];
+        load_slot_lane<DT>(logits, s, lane, V, fill, v, p.row.fused);
+        split_pass1_slot<true>(p, row, s, v, inv);
+      }
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();
+    };
+    bool on_my_own = !all_there(arrive_max);
+    if (timers) cf1 = wall_clock64();
+    float m_early;
+    if (on_my_own) {
+      alone();
+      m_early = kNegInf;
+      for (int s = lane; s < ns; s += 64) m_early = __builtin_fmaxf(m_early, coherent_load(slot_max + s));  // (ignores NaN)
+      m_early = wave_max_ignoring_nan(m_early);
+    } else {
+      m_early = lane < n_parts ? coherent_load(part_max + lane) : kNegInf;
+      m_early = wave_max_ignoring_nan(m_early);
+    }
+    {
+      const float x_first = load_logit<DT>(logits, 0, p.row.fused) * inv;
+      if (x_first != x_first) m_early = x_first;
+    }
+    if constexpr (DT == kDtypeBFloat16) {
+      if (m_early > kNegInf && m_early < kInf)
+        early_lut = build_exp_lut<false>(lut_mem, kLutCountWords, inv, m_early, sm.exp2tab, lut_base1, lut_top, lut_half) ? 1 : 0;
+      early_m = m_early;
+    }
+    if (!on_my_own && !all_there(arrive_sum)) alone();
+    if (timers) cf2 = wall_clock64();
+  } else {
+    if (s_mine < s_end) load_slot_lane<DT>(logits, s_mine, lane, V, fill, l, p.row.fused);
+  }
 
   // ---- row maximum (sampler.cpp:191-197) from the slots' maxima
   float m = -kInf;
   bool any_nan = false;
   float first_max = 0.0f, first_sum = 0.0f, first_max2 = -kInf;  // the scan below starts with the same slots
+  // (FUSED: other workgroups of this launch stored these)
+  auto slot_value = [&](const float* a, int s) { return FUSED ? coherent_load(a + s) : a[s]; };
   for (int s = tid; s < ns; s += kBlock) {
-    const float v = slot_max[s];
+    const float v = slot_value(slot_max, s);
     if (s == tid) {
       first_max = v;
-      first_sum = slot_sum[s];
-      if (TOPP) first_max2 = slot_max2[s];
+      first_sum = slot_value(slot_sum, s);
+      if (TOPP) first_max2 = slot_value(slot_max2, s);
     }
     any_nan = any_nan || (v != v);
     m = __builtin_fmaxf(m, v);
@@ -590,7 +752,7 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
   if (x0 != x0) m = x0;  // max_val starts at x[0]; nothing compares greater than NaN
   const bool row_nan = nan_any != 0u || !(m > -kInf && m < kInf);
   if (row_nan) {  // one NaN addend poisons the sum: the finish kernel needs nothing else
-    if (blockIdx.x == 0 && tid == 0) p.row_state[row] = {0u, m, 1u, 0.0f, 0, 0, 0, 0u};
+    if (part == 0 && tid == 0) p.row_state[row] = {0u, m, 1u, 0.0f, 0, 0, 0, 0u};
     return;
   }
   __syncthreads();
@@ -613,8 +775,8 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
     const int s = base + tid;
     float a = 0.0f;
     if (s < ns) {
-      const float sum = base == 0 ? first_sum : slot_sum[s];
-      const float smax = base == 0 ? first_max : slot_max[s];
+      const float sum = base == 0 ? first_sum : slot_value(slot_sum, s);
+      const float smax = base == 0 ? first_max : slot_value(slot_max, s);
       const float f = sum > 0.0f ? fast_exp2((smax - m) * kLog2e) : 0.0f;  // exp of the slot's largest entry
       a = sum > 0.0f ? sum * f : 0.0f;
       if (WALK) a *= walk_scale;
@@ -622,7 +784,7 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
       if (TOPP && f > 0.0f) {
         // lower bounds of the exact exps of the slot's two largest entries, into the bins of their
         // binades (integers: every workgroup of the row arrives at the same totals)
-        const float smax2 = base == 0 ? first_max2 : slot_max2[s];
+        const float smax2 = base == 0 ? first_max2 : slot_value(slot_max2, s);
         const float f2 = smax2 > -kInf ? fast_exp2((smax2 - m) * kLog2e) : 0.0f;
         const float below[2] = {f * 0.9999f, f2 * 0.9999f};
 #pragma unroll
@@ -683,9 +845,12 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
 
   // ---- bf16 rows: expf by bit pattern
   bool use_lut = false;
-  int lut_base1 = 0, lut_top = 0, lut_half = 0;
   if constexpr (DT == kDtypeBFloat16) {
-    use_lut = build_exp_lut<false>(lut_mem, kLutCountWords, inv, m, sm.exp2tab, lut_base1, lut_top, lut_half);
+    if (FUSED && early_lut >= 0 && __float_as_uint(early_m) == __float_as_uint(m)) {
+      use_lut = early_lut != 0;  // (built while the slots' sums were on their way)
+    } else {
+      use_lut = build_exp_lut<false>(lut_mem, kLutCountWords, inv, m, sm.exp2tab, lut_base1, lut_top, lut_half);
+    }
     if (WALK && use_lut) {  // one division per bit pattern: the table becomes p = fl(e / S)
       __syncthreads();
       for (int idx = tid; idx < 2 * lut_half; idx += kBlock) lut_mem[idx] = div_row(lut_mem[idx], walk_div);
@@ -753,7 +918,7 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
       }
     }
   }
-  uint64_t* region = p.list + (static_cast<int64_t>(lrow) * p.row_wgs + blockIdx.x) * p.list_region;
+  uint64_t* region = p.list + (static_cast<int64_t>(lrow) * p.row_wgs + part) * p.list_region;
   // ---- the pattern histogram's range of order keys: from safely below the smallest logit whose exp
   //      can reach cut_lo up to the row's largest logit (every workgroup of the row arrives at the
   //      same two numbers).  Too many bins for the LDS set aside: no pattern histogram.
@@ -779,7 +944,7 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
     km.n_bins = key_top - km.key_cut + 1;
     if (km.n_bins < 1 || km.n_bins > 2 * p.phist_words) km.n_bins = 0;
   }
-  if (blockIdx.x == 0 && tid == 0) p.row_state[row] = {serial_before, m, 0u, a_total, km.key_cut, km.n_bins, km.mag_min, listed_buckets};
+  if (part == 0 && tid == 0) p.row_state[row] = {serial_before, m, 0u, a_total, km.key_cut, km.n_bins, km.mag_min, listed_buckets};
 
   // ---- the slots, no barriers.  Two buffers take turns, so that the entries of the slot after this
   //      one are on their way while this one is worked on (a copy from one buffer to the other
@@ -812,31 +977,38 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
     const bool search = TOPP && __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(sh.top[s]))) >= list_cut;
     split_fold_slot<TOPP, DT>(p, row, s, e, in, sh.cls[s], list_cut, search, V, region, sh, km, ph);
   };
-  float l2[8];
-  while (s_mine < s_end) {
-    if (s_mine + kWaves < s_end) load_slot_lane<DT>(logits, s_mine + kWaves, lane, V, fill, l2, p.row.fused);
-    work(s_mine, l);
-    s_mine += kWaves;
-    if (s_mine >= s_end) break;
-    if (s_mine + kWaves < s_end) load_slot_lane<DT>(logits, s_mine + kWaves, lane, V, fill, l, p.row.fused);
-    work(s_mine, l2);
-    s_mine += kWaves;
+  if constexpr (FUSED) {
+    if (s_mine < s_end) work(s_mine, held0);
+    if (s_mine + kWaves < s_end) work(s_mine + kWaves, held1);
+    if (s_mine + 2 * kWaves < s_end) work(s_mine + 2 * kWaves, held2);
+    if (s_mine + 3 * kWaves < s_end) work(s_mine + 3 * kWaves, held3);
+  } else {
+    float l2[8];
+    while (s_mine < s_end) {
+      if (s_mine + kWaves < s_end) load_slot_lane<DT>(logits, s_mine + kWaves, lane, V, fill, l2, p.row.fused);
+      work(s_mine, l);
+      s_mine += kWaves;
+      if (s_mine >= s_end) break;
+      if (s_mine + kWaves < s_end) load_slot_lane<DT>(logits, s_mine + kWaves, lane, V, fill, l, p.row.fused);
+      work(s_mine, l2);
+      s_mine += kWaves;
+    }
   }
   if (TOPP) {
     __syncthreads();
-    if (tid == 0) p.list_count[static_cast<int64_t>(lrow) * kMaxRowWorkgroups + blockIdx.x] = sh.list_count;
-    uint32_t* hist_out = p.hist + (static_cast<int64_t>(lrow) * p.row_wgs + blockIdx.x) * kHistBuckets;
+    if (tid == 0) p.list_count[static_cast<int64_t>(lrow) * kMaxRowWorkgroups + part] = sh.list_count;
+    uint32_t* hist_out = p.hist + (static_cast<int64_t>(lrow) * p.row_wgs + part) * kHistBuckets;
     // (short lists: the buckets behind the listed ones are empty, and the finish kernel does not read them)
     const int n_hist = listed_buckets == kNoLists ? 0 : (listed_buckets != 0u ? static_cast<int>(listed_buckets) : kHistBuckets);
     for (int b = tid; b < n_hist; b += kBlock) hist_out[b] = sh.hist[b];
     if (kPatterns && km.n_bins > 0) {
-      uint32_t* ph_out = p.phist + (static_cast<int64_t>(lrow) * p.row_wgs + blockIdx.x) * p.phist_words;
+      uint32_t* ph_out = p.phist + (static_cast<int64_t>(lrow) * p.row_wgs + part) * p.phist_words;
       for (int b = tid; b < (km.n_bins + 1) / 2; b += kBlock) ph_out[b] = ph[b];
     }
   }
-  if (timers && blockIdx.x == 0 && tid == 0) {
-    uint64_t* t = timers + static_cast<int64_t>(gridDim.y) * 8 + static_cast<int64_t>(blockIdx.y) * 4;
-    t[0] = c1 - c0;
+  if (timers && part == 0 && tid == 0) {
+    uint64_t* t = timers + static_cast<int64_t>(p.row.rows) * 8 + static_cast<int64_t>(lrow) * 4;
+    t[0] = (c1 - c0) | (FUSED ? ((cf0 - c0) << 16) | ((cf1 - cf0) << 32) | ((cf2 - cf1) << 48) : 0ull);
     t[1] = c2 - c1;
     t[2] = c3 - c2;
     t[3] = wall_clock64() - c3;
@@ -2113,6 +2285,7 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
     for (int k = 0; k < 4; ++k) early_hist[k] = hist_in[(k < p.row_wgs ? k : 0) * kHistBuckets + tid];
   }
   const RowState rs = p.row_state[row];
+  if (tid < 2 && p.arrive) p.arrive[2 * lrow + tid] = 0u;  // (the fused launch's counters, for the next launch)
   const float m = rs.m;
   const bool row_nan = rs.nan != 0u;
   const float cutoff = (1.0f - topp) / static_cast<float>(V - 1);  // sampler.cpp:136

@@ -61,12 +61,42 @@ ets_status launch_split(ets_sampler* s, const ets::RowParams& p, int32_t rows, h
     return e ? std::atoi(e) : 1;
   }();
   sp.short_lists = short_lists;
-  launch_split_pass1<DT>(sp, rows, stream);
-  ETS_HIP(s, hipGetLastError());
   const size_t lut_bytes = (DT == ets::kDtypeBFloat16 ? sizeof(float) * ets::kLutCountWords : 0) + sizeof(uint32_t) * sp.phist_words;
   // (a launch that neither writes the probabilities nor fills the phase clocks runs kernels without those branches)
   const bool extras = sp.timers != nullptr || p.probs != nullptr;
-  if (extras) {
+  // Pass 1 inside pass 2 (one read of the logits, one launch fewer) when every workgroup of the launch
+  // is resident at once and a wave's slots fit its registers: plain top-p launches with one
+  // temperature, a finite one.  ETS_FUSE=0 switches it off; ETS_FUSE_SPIN_LIMIT sets how often a
+  // workgroup polls for the others of its row before it works their slots out itself (0: at once).
+  // (read at every launch, so that a test can switch between them inside one process)
+  const char* const fuse_text = std::getenv("ETS_FUSE");
+  const int fuse_env = fuse_text ? std::atoi(fuse_text) : 1;
+  const char* const spin_text = std::getenv("ETS_FUSE_SPIN_LIMIT");
+  const int spin_env = spin_text ? std::atoi(spin_text) : (1 << 16);
+  const int per_wg_slots = ((sp.ns + sp.row_wgs - 1) / sp.row_wgs + ets::kWaves - 1) / ets::kWaves * ets::kWaves;
+  const float abs_inv = p.inv_temperature < 0.0f ? -p.inv_temperature : p.inv_temperature;
+  const bool fused = !TOPK && (!extras || (ETS_PHASE_CLOCKS && p.probs == nullptr)) && fuse_env != 0 && p.row_cfg == nullptr && abs_inv < 3.0e38f && sp.arrive != nullptr &&
+                     static_cast<int64_t>(rows) * sp.row_wgs <= (s->num_cus > 0 ? s->num_cus : 0) &&
+                     per_wg_slots <= ets::kFusedSlots * ets::kWaves && (!s->wb || rows <= s->wb->arrive_rows);
+  bool* dirty = arrive_dirty_flag(s);
+  if (fused) {
+    if constexpr (!TOPK) {
+      if (*dirty) ETS_HIP(s, hipMemsetAsync(sp.arrive, 0, 2 * sizeof(uint32_t) * static_cast<size_t>(s->wb ? s->wb->arrive_rows : s->max_batch), stream));
+      *dirty = true;  // (until this call's finish kernel, which clears the counters, has been launched)
+      sp.spin_limit = spin_env < 0 ? 0 : spin_env;
+      static std::atomic<size_t> set_bytes_f[kMaxDevices];
+      constexpr bool kClocks = ETS_PHASE_CLOCKS != 0;  // (a profiling build: the fused kernel with its phase clocks)
+      st = allow_dynamic_lds(s, reinterpret_cast<const void*>(&ets::split_pass2_kernel<DT, true, false, false, kClocks, true>), lut_bytes, set_bytes_f);
+      if (st != ETS_OK) return st;
+      hipLaunchKernelGGL((ets::split_pass2_kernel<DT, true, false, false, kClocks, true>), dim3(sp.row_wgs * rows), dim3(ets::kBlock), lut_bytes,
+                         stream, sp);
+    }
+  } else {
+    launch_split_pass1<DT>(sp, rows, stream);
+    ETS_HIP(s, hipGetLastError());
+  }
+  if (fused) {
+  } else if (extras) {
     static std::atomic<size_t> set_bytes2[kMaxDevices];
     st = allow_dynamic_lds(s, reinterpret_cast<const void*>(&ets::split_pass2_kernel<DT, true, false, TOPK, true>), lut_bytes, set_bytes2);
     if (st != ETS_OK) return st;
@@ -119,6 +149,7 @@ ets_status launch_split(ets_sampler* s, const ets::RowParams& p, int32_t rows, h
     }
   }
   ETS_HIP(s, hipGetLastError());
+  if (fused) *dirty = false;
   return ETS_OK;
 }
 
