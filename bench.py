@@ -141,10 +141,12 @@ def cpu_baseline(w, gpu_tokens, seconds_budget=12.0):
     t0 = time.perf_counter()
     one_row(1 % rows, 5)
     one_core = 5 / (time.perf_counter() - t0)
+    both = cpu_baseline_config(w, seconds=1.5)
     return {
         "value": rows * reps / dt,
         "unit": "rows/s",
         "cores": cores,
+        "native_and_upcast": {k: both[k] for k in ("native", "upcast_fp32") if k in both},
         "kind": "reference" if use_ref else "port",
         "sample": f"{rows} rows of {w.name} step 0, each sampled {reps} times by its own Sampler, native "
                   f"{W.DTYPE_NAMES[w.dtype]} sample<T>, {cores} threads ({dt:.1f} s)",
@@ -155,6 +157,58 @@ def cpu_baseline(w, gpu_tokens, seconds_budget=12.0):
         "compiler": "g++ -std=c++17 -O2 (sampler.cpp as the reference builds it)" if use_ref else "g++ -std=c++17 -O2 (restatement)",
         "parity": {"rows_checked": rows, "token_mismatches_vs_oracle": mismatches},
     }
+
+
+def cpu_baseline_config(w, seconds=1.2):
+    """The reference sampler on this box's host cores for one workload of the contract, on a bounded
+    sample of its rows (step 0): one core, one Sampler, rows one after the other (the literal
+    reference usage); and every thread of this job's share of the host, a Sampler each.  16-bit
+    workloads are timed twice: the native sample<T> instantiation, and sample<float> on the rows
+    converted to fp32 beforehand (the arithmetic the GPU path reproduces; the conversion itself is
+    not timed).  `sampler.cpp` itself (oracle/_ref) when it was built, else the oracle's restatement."""
+    import numpy as np
+
+    from executorch_amd import workloads as W
+    from oracle import oracle as O
+
+    cores = max(1, min(16, os.cpu_count() or 1))
+    use_ref = O.have_ref()
+    rows = cores
+    if w.batch >= rows:
+        x = W.logits(w, 0, rows)
+    else:  # (a workload of one row per step: the rows of as many steps)
+        x = np.concatenate([W.logits(w, step, w.batch) for step in range(-(-rows // w.batch))])[:rows]
+    modes = [("native", x, w.dtype, O.MODE_NATIVE)]
+    if w.dtype != W.DTYPE_FLOAT:
+        modes.append(("upcast_fp32", np.ascontiguousarray(W.to_f32(x, w.dtype), dtype=np.float32), W.DTYPE_FLOAT, O.MODE_NATIVE))
+    res = {"kind": "reference" if use_ref else "port", "cores": cores, "unit": "rows/s",
+           "sample": f"{rows} rows of {w.name} (step 0; the first steps of a one-row workload), each sampled repeatedly by its own "
+                     f"Sampler ({seconds:.1f} s per figure)"}
+
+    def make(b):
+        if use_ref:
+            return O.RefSampler(w.vocab, w.temperature, w.topp, w.coin_seed + b)
+        return O.Sampler(w.vocab, w.temperature, w.topp, w.coin_seed + b, mode=O.MODE_NATIVE)
+
+    for label, data, dtype, _ in modes:
+        def run(b, reps):
+            smp = make(b)
+            for _ in range(reps):
+                smp.sample(data[b].copy(), dtype)  # (the sampler overwrites its input: a fresh copy per call)
+
+        t0 = time.perf_counter()
+        run(0, 2)
+        per_row = max((time.perf_counter() - t0) / 2, 1e-6)
+        reps = max(1, min(20000, int(seconds / per_row)))
+        t0 = time.perf_counter()
+        run(0, reps)
+        one = reps / (time.perf_counter() - t0)
+        t0 = time.perf_counter()
+        with ThreadPoolExecutor(cores) as pool:
+            list(pool.map(lambda b: run(b, reps), range(rows)))
+        many = rows * reps / (time.perf_counter() - t0)
+        res[label] = {"rows_per_s_one_core": one, "rows_per_s_all_threads": many, "threads": rows}
+    return res
 
 
 def timed_us(fn, reps, torch, repeats=1):
@@ -328,7 +382,7 @@ def bench_batch_sweep(w, torch, dev):
     return res
 
 
-def bench_all_configs(torch, dev):
+def bench_all_configs(torch, dev, with_cpu=True):
     """Every workload of the benchmark contract at its own batch, element type and parameters:
     microseconds per step (median of five repeats, device time), rows/s, and the step's algorithmic
     bytes (B x V x element size, read once) against the HBM peak.  Small rings (at least two
@@ -358,6 +412,11 @@ def bench_all_configs(torch, dev):
                      "top_p": w.topp, "us_per_step": us, "rows_per_s": w.batch / (us * 1e-6),
                      "algorithmic_bytes": w.bytes_per_step, "gbs": gbs, "frac_of_hbm_peak": gbs / HBM_PEAK_GBS,
                      "ring_matrices": n_ring, "steps_per_repeat": reps, "repeats": 5}
+        if w.batch == 1:
+            res[name]["note"] = ("one row per step: the ring's matrices stay in the caches, and a step is bound by the latency of "
+                                 "its launches, not by bytes: read us_per_step, not the fraction of the HBM peak")
+        if with_cpu:
+            res[name]["cpu_baseline"] = cpu_baseline_config(w)
         del ring, s
         torch.cuda.empty_cache()
     return res
@@ -607,7 +666,7 @@ def main():
             line["batch_sweep"] = bench_batch_sweep(w, torch, dev)
         del ring
         torch.cuda.empty_cache()
-        line["configs"] = bench_all_configs(torch, dev)
+        line["configs"] = bench_all_configs(torch, dev, with_cpu=not args.no_cpu_baseline)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(w, got)
     print(json.dumps(line))

@@ -1041,12 +1041,26 @@ ets_status ets_logits_to_token(const void* data, int32_t dtype, int32_t rank, co
   // 2-argument constructor's parameters and a clock seed -- is set again on every call.
   struct Cached {
     ets_sampler* handle = nullptr;
-    ~Cached() { ets_sampler_destroy(handle); }
+    // (at thread or process exit the HIP runtime may be gone already: then nothing is freed)
+    ~Cached() {
+      int n = 0;
+      if (handle && hipGetDeviceCount(&n) == hipSuccess && n > 0) ets_sampler_destroy(handle);
+    }
   };
   thread_local Cached cache;
   int device = -1;
   if (hipGetDevice(&device) != hipSuccess) device = -1;
   ets_sampler* s = cache.handle;
+  if (s) {
+    // a device reset since the last call leaves the handle's buffers dangling: it is dropped, not freed
+    hipPointerAttribute_t attr;
+    if (hipPointerGetAttributes(&attr, s->d_rng) != hipSuccess) {
+      (void)hipGetLastError();
+      delete s;
+      cache.handle = nullptr;
+      s = nullptr;
+    }
+  }
   if (!s || s->vocab != vocab || s->device != device) {
     ets_sampler_destroy(cache.handle);
     cache.handle = nullptr;

@@ -38,6 +38,12 @@ ETS_API ets_status ets_test_copy_probe(const void* d_src, void* d_dst, int64_t b
 ETS_API ets_status ets_test_signal_floor(uint32_t* d_words, int32_t hops, int32_t spin_limit, int32_t partner,
                                          uint32_t* d_out, void* hip_stream);
 
+/* Which of the handle's lazily allocated device buffers exist: out[0] candidate scratch, out[1] the
+ * work buffers of the several-workgroups-per-row path, out[2] the pattern histograms, out[3] the
+ * per-row parameter staging (1: allocated).  A handle that has only served calls of
+ * ets_sampler_sample_batch_static() has none of them.  HOST pointer to four int32. */
+ETS_API ets_status ets_test_handle_buffers(const ets_sampler* s, int32_t* out);
+
 /* The message of the calling thread's last failed hook. */
 ETS_API const char* ets_test_last_error(void);
 

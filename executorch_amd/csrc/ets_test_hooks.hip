@@ -216,6 +216,15 @@ ets_status ets_test_split_timers(ets_sampler* s, uint64_t* out, int32_t rows) {
   return ETS_OK;
 }
 
+ets_status ets_test_handle_buffers(const ets_sampler* s, int32_t* out) {
+  if (!s || !out) return hook_fail(ETS_INVALID_ARGUMENT, "ets_test_handle_buffers: null pointer");
+  out[0] = s->d_scratch != nullptr;
+  out[1] = s->d_split != nullptr;
+  out[2] = s->d_phist != nullptr;
+  out[3] = s->d_stage != nullptr;
+  return ETS_OK;
+}
+
 const char* ets_test_last_error(void) { return g_hook_error.c_str(); }
 
 }  // extern "C"

@@ -102,11 +102,23 @@ ETS_API ets_status ets_sampler_set_topk(ets_sampler* s, int32_t topk);
 ETS_API ets_status ets_sampler_set_topp(ets_sampler* s, float topp);
 
 /* No counterpart (the reference is one scalar loop).  How the stochastic path uses the GPU:
- *   ETS_ROW_SPLIT_AUTO  rows of 8192 entries and more take three launches in which many
- *                       workgroups share a row (16-byte aligned rows, top-p draw); smaller ones,
- *                       other draws and unaligned rows take one launch, one workgroup per row;
- *   ETS_ROW_SPLIT_ON    the three launches wherever they apply, whatever the vocabulary size;
+ *   ETS_ROW_SPLIT_AUTO  rows of 8192 entries and more, 16-byte aligned, take the launches in which
+ *                       several workgroups share a row; everything else takes one launch with one
+ *                       workgroup per row;
+ *   ETS_ROW_SPLIT_ON    several workgroups per row wherever that path applies, whatever the
+ *                       vocabulary size;
  *   ETS_ROW_SPLIT_OFF   always one workgroup per row.
+ * Several workgroups per row, by draw: top-p rows three launches (two when every workgroup of
+ * the launch is resident at once, about batch x workgroups-per-row <= compute units, and the
+ * launch has one finite temperature and no debug output: the first two are then one kernel);
+ * top-k rows with k <= ceil(vocab / 512) the same three launches, larger k one workgroup per row;
+ * multinomial rows (top_p <= 0 or >= 1) FIVE launches, or one workgroup per row when the
+ * probabilities are asked for.  All launches of a call go to the call's stream, in order.
+ * Work buffers of that path are allocated at the first call that needs them and kept: per row of
+ * max_batch about 16 bytes x ceil(vocab / 512) slots x 2 + 40 prepared slots of 2.6 KB, plus per
+ * (row, workgroup) of the largest launch a 2048-bucket histogram, a candidate list of up to
+ * 16384 x 8 bytes and, for 16-bit rows, a pattern histogram of up to 96 KB -- about 240 MB at
+ * max_batch 1024 and vocab 151936.
  * The tokens, coin states and debug records are the same on every setting. */
 #define ETS_ROW_SPLIT_AUTO 0
 #define ETS_ROW_SPLIT_ON 1
@@ -235,7 +247,12 @@ ETS_API ets_status ets_sample_from_logits_batch(ets_sampler* s, const void* d_da
                                                 const int64_t* sizes, int32_t* d_tokens, void* hip_stream);
 
 /* logits_to_token(const Tensor&, float temperature = 0)  -- util.h:64-71: a temporary
- * 2-argument Sampler over the tensor's last dimension. */
+ * 2-argument Sampler over the tensor's last dimension.  The reference builds that object per
+ * call, which costs it nothing; a handle here owns device buffers, so every calling THREAD keeps
+ * the handle of its last call (about vocab x 4 bytes of row staging plus the work buffers of the
+ * draw, held until the thread ends) and reuses it while device and vocabulary stay the same; the
+ * 2-argument constructor's parameters and a clock seed are set again on every call.  The cached
+ * handle is dropped without freeing when the HIP runtime has been torn down or the device reset. */
 ETS_API ets_status ets_logits_to_token(const void* data, int32_t dtype, int32_t rank, const int64_t* sizes,
                                        float temperature, int32_t* token_out);
 

@@ -52,3 +52,59 @@ def test_static_entry_refuses_what_does_not_fit(dev):
     # the handle is still usable, and a problem that fits goes through
     small = ea.Sampler(V, 0.6, 0.9, 1, max_batch=8)
     assert small.sample_batch_static(x[:8]).shape == (8,)
+
+
+def handle_buffers(s):
+    out = np.zeros(4, dtype=np.int32)
+    assert _capi.hooks().ets_test_handle_buffers(s._h, out.ctypes.data) == _capi.OK
+    return out.tolist()
+
+
+def test_static_calls_allocate_nothing(dev):
+    """What the entry point exists for: after the handle is created, calls allocate no device memory.
+    The free memory the driver reports is the same before and after a run of calls of several shapes
+    and element types (inputs and outputs are made beforehand), and the handle's own lazily allocated
+    work buffers still do not exist afterwards."""
+    V = 50264
+    cases = []
+    for dtype, rows, peaked in ((W.DTYPE_BFLOAT16, 8, True), (W.DTYPE_HALF, 5, False), (W.DTYPE_FLOAT, 3, True), (W.DTYPE_BFLOAT16, 1, False)):
+        x = to_device(rows_of(V, rows, dtype, 10 + rows, peaked), dtype, dev)
+        cases.append((x, torch.empty(rows, dtype=torch.int32, device=dev)))
+    s = ea.Sampler(V, 0.7, 0.9, 99, max_batch=8)
+    greedy = ea.Sampler(V, 0.0, 0.9, 99, max_batch=8)
+    multinomial = ea.Sampler(V, 1.0, 1.0, 99, max_batch=8)
+    assert handle_buffers(s) == [0, 0, 0, 0]
+    x0, out0 = cases[0]
+    s.sample_batch_static(x0, out=out0)  # (first call: kernel attributes are set, code objects loaded)
+    greedy.sample_batch_static(x0, out=out0)
+    multinomial.sample_batch_static(x0, out=out0)
+    torch.cuda.synchronize()
+    free_before, _ = torch.cuda.mem_get_info()
+    for _ in range(5):
+        for x, out in cases:
+            s.sample_batch_static(x, out=out)
+            greedy.sample_batch_static(x, out=out)
+            multinomial.sample_batch_static(x, out=out)
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info()
+    assert free_after == free_before, (free_before, free_after)
+    for h in (s, greedy, multinomial):
+        assert handle_buffers(h) == [0, 0, 0, 0]
+    # ... while the allocating entry point does allocate them (the comparison is not vacuous)
+    s.sample_batch(x0, out=out0)
+    assert handle_buffers(s)[:2] == [1, 1]
+
+
+def test_two_handles_take_turns_on_one_stream(dev):
+    """Every handle on a GPU works in the same static array: used one after the other on one stream
+    they must not disturb each other."""
+    V = 50264
+    a_ref, b_ref = ea.Sampler(V, 0.7, 0.9, 7, max_batch=8), ea.Sampler(V, 0.9, 0.8, 8, max_batch=8)
+    a, b = ea.Sampler(V, 0.7, 0.9, 7, max_batch=8), ea.Sampler(V, 0.9, 0.8, 8, max_batch=8)
+    for step in range(3):
+        xa = to_device(rows_of(V, 8, W.DTYPE_BFLOAT16, 30 + step, True), W.DTYPE_BFLOAT16, dev)
+        xb = to_device(rows_of(V, 6, W.DTYPE_HALF, 40 + step, False), W.DTYPE_HALF, dev)
+        got_a = a.sample_batch_static(xa)
+        got_b = b.sample_batch_static(xb)  # (queued behind a's launches, before they have run)
+        assert np.array_equal(got_a.cpu().numpy(), a_ref.sample_batch(xa).cpu().numpy())
+        assert np.array_equal(got_b.cpu().numpy(), b_ref.sample_batch(xb).cpu().numpy())
