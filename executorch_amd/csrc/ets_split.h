@@ -1179,14 +1179,44 @@ __device__ __forceinline__ void split_chain_prepare(const SlotRec* recs, int ns,
 // else is redone entry by entry from the logits -- and the walk goes on behind it.  Every step
 // advances by at least one record.
 template <int DT>
+__device__ __forceinline__ float split_chain_walk(const SlotRec* recs, int ns, const PrepSlot* prep, uint32_t n_prep,
+                                                  const char* logits, int V, float inv, float m, const uint64_t* tab,
+                                                  const FusedOps& fused, uint64_t* stats, const RowDivisor* div,
+                                                  float threshold, int* stop, int base0, int cur0, float s0);
+
+// Slot `slot` of a multinomial row's probabilities p = fl(e / S) entry by entry from the logits, from
+// running sum `from`, up to the first entry behind which the sum exceeds `threshold` (`hit`: its index).
+template <int DT>
+__device__ __forceinline__ float walk_redo(const char* logits, int slot, int V, float inv, float m, const uint64_t* tab,
+                                           const FusedOps& fused, const RowDivisor& div, float threshold, float from, int& hit) {
+  const int lane = threadIdx.x & 63;
+  const float kInf = __uint_as_float(0x7f800000u);
+  float l[8];
+  uint32_t b[8];
+  load_slot_lane<DT>(logits, slot, lane, V, inv < 0.0f ? kInf : -kInf, l, fused);
+#pragma unroll
+  for (int k = 0; k < 8; ++k) b[k] = __float_as_uint(div_row(expf_core(__builtin_fmaxf(l[k] * inv - m, -104.0f), tab), div));
+  float t = from;
+  wave_resolve<8>(t, hit, b, slot * kSlot + lane * 8, V, threshold);
+  return t;
+}
+
+// WALKING: the records are those of a multinomial row's probabilities p = fl(e / S) (`div`), and the
+// walk ends at the first entry behind which the running sum exceeds `threshold` (sampler.cpp:58-70):
+// `*stop` is its index (-1: none), the value returned the sum there.  Increments are not negative, so
+// the sum is compared with the threshold at the stops only; the record at which it is first exceeded
+// is then looked up among the run's prefixes and redone entry by entry from the sum in front of it.
+template <int DT, bool WALKING = false>
 __device__ __forceinline__ float split_chain(const SlotRec* recs, const uint2* pairs, int ns, const PrepSlot* prep, uint32_t n_prep,
                                              const char* logits, int V, float inv, float m, const uint64_t* tab,
-                                             const FusedOps& fused, uint64_t* stats = nullptr) {
+                                             const FusedOps& fused, uint64_t* stats = nullptr, const RowDivisor* div = nullptr,
+                                             float threshold = 0.0f, int* stop = nullptr) {
   const int lane = threadIdx.x & 63;
   const float kInf = __uint_as_float(0x7f800000u);
   const float fill = inv < 0.0f ? kInf : -kInf;
   n_prep = uniform_u32(n_prep);
   float s = 0.0f;
+  if (WALKING) *stop = -1;
   uint64_t c_start = 0;
   uint32_t n_iter = 0, n_generic = 0, n_prep_used = 0, n_tie = 0, n_inner = 0;
   uint64_t c_prep = 0;
@@ -1201,6 +1231,7 @@ __device__ __forceinline__ float split_chain(const SlotRec* recs, const uint2* p
     if (base == 0 && readlane_u32(kind, 0) == kSlotExact) {  // pass 2 worked the first slot out
       s = __uint_as_float(readlane_u32(r.even, 0));
       cur = 1;
+      if (WALKING && s > threshold) return walk_redo<DT>(logits, 0, V, inv, m, tab, fused, *div, threshold, 0.0f, *stop);
     }
     if (stats) {
       const uint64_t now = wall_clock64();
@@ -1240,6 +1271,14 @@ __device__ __forceinline__ float split_chain(const SlotRec* recs, const uint2* p
         ph_scan += now - ph_t;
         ph_t = now;
       }
+      // WALKING: the sum exceeds the threshold behind one of the records first .. last of a run entered with (K, S)
+      auto in_run = [&](int first, int last, uint32_t K_in, uint32_t S_in) {
+        const uint32_t S_upto = S_in + ((S_in & 1u) ? pr.y : pr.x);
+        const uint64_t cross = __ballot(lane >= first && lane <= last && sum_value(S_upto, static_cast<int>(K_in)) > threshold);
+        const int q = static_cast<int>(uniform_u32(static_cast<uint32_t>(__builtin_ctzll(cross))));
+        const float front = sum_value(q > first ? readlane_u32(S_upto, q - 1) : S_in, static_cast<int>(K_in));
+        return walk_redo<DT>(logits, base + q, V, inv, m, tab, fused, *div, threshold, front, *stop);
+      };
       while (cur < n) {
         cur = static_cast<int>(uniform_u32(static_cast<uint32_t>(cur)));
         const int t = static_cast<int>(uniform_u32(static_cast<uint32_t>(__builtin_ctzll(stop_mask & (~0ull << cur)))));  // (lane n - 1 is a stop)
@@ -1251,6 +1290,7 @@ __device__ __forceinline__ float split_chain(const SlotRec* recs, const uint2* p
             fast_ok = false;
             break;
           }
+          if (WALKING && sum_value(S_run, static_cast<int>(K)) > threshold) return in_run(cur, t, K, S);
           S = S_run;
           cur = t + 1;
           continue;
@@ -1270,11 +1310,13 @@ __device__ __forceinline__ float split_chain(const SlotRec* recs, const uint2* p
             fast_ok = false;
             break;
           }
+          if (WALKING && sum_value(S_run, static_cast<int>(K)) > threshold) return in_run(cur, t - 1, K, S);
           S = S_run;
         }
         cur = t;
         {
           // ---- record base + t, no part of a run
+          const uint32_t K_front = K, S_front = S;
           bool done = false;
           if (short_form && K == (readlane_u32(r.meta, t) & 255u)) {
             // resolve_lanes() for a slot entered in the binade it was prepared for: the lanes in front
@@ -1334,7 +1376,11 @@ __device__ __forceinline__ float split_chain(const SlotRec* recs, const uint2* p
               float l[8];
               load_slot_lane<DT>(logits, slot, lane, V, fill, l, fused);
 #pragma unroll
-              for (int k = 0; k < 8; ++k) bits[k] = __float_as_uint(expf_core(__builtin_fmaxf(l[k] * inv - m, -104.0f), tab));
+              for (int k = 0; k < 8; ++k) {
+                float e = expf_core(__builtin_fmaxf(l[k] * inv - m, -104.0f), tab);
+                if (WALKING) e = div_row(e, *div);
+                bits[k] = __float_as_uint(e);
+              }
               int found = -1;
               wave_resolve<8>(s, found, bits, slot * kSlot + lane * 8, V, kInf);
               ++n_generic;
@@ -1344,6 +1390,9 @@ __device__ __forceinline__ float split_chain(const SlotRec* recs, const uint2* p
             S = sb >> 23 ? ((sb & 0x7fffffu) | 0x800000u) : sb;
           }
           ++n_iter;
+          if (WALKING && sum_value(S, static_cast<int>(K)) > threshold) {
+            return walk_redo<DT>(logits, base + t, V, inv, m, tab, fused, *div, threshold, sum_value(S_front, static_cast<int>(K_front)), *stop);
+          }
         }
         cur = t + 1;
       }
@@ -1356,6 +1405,9 @@ __device__ __forceinline__ float split_chain(const SlotRec* recs, const uint2* p
       ph_t = now;
     }
     // ---- record by record (a run in which the sum leaves its binade)
+    if (WALKING && cur < 64) {
+      return split_chain_walk<DT>(recs, ns, prep, n_prep, logits, V, inv, m, tab, fused, nullptr, div, threshold, stop, base, cur, s);
+    }
     int K_scan = -1;
     uint32_t incl = 0u;
     uint64_t plain_mask = 0ull;
@@ -1441,39 +1493,26 @@ __device__ __forceinline__ float split_chain(const SlotRec* recs, const uint2* p
   return uniform_f32(s);
 }
 
-// The chain of a multinomial row's probabilities (the same walk as split_chain(), which is kept apart
-// so that the finish kernel's code stays what it was): the records are those of p = fl(e / S) (`div`),
-// and the walk stops at the first entry behind
-// which the running sum exceeds `threshold` (sampler.cpp:58-70): `*stop` is its index (-1: none), the
+// The chain of a multinomial row's probabilities record by record, from record `cur0` of the chunk
+// at `base0` and the exact sum `s0` in front of it: where split_chain<DT, true>() goes on when a run
+// does not stay in the binade predicted for it.  The walk stops at the first entry behind which the
+// running sum exceeds `threshold` (sampler.cpp:58-70): `*stop` is its index (-1: none), the
 // value returned the sum there.  Sums behind records are exact, so the first record behind which
 // the sum exceeds the threshold holds that entry; it is redone entry by entry from the sum in front of it.
 template <int DT>
 __device__ __forceinline__ float split_chain_walk(const SlotRec* recs, int ns, const PrepSlot* prep, uint32_t n_prep,
                                                   const char* logits, int V, float inv, float m, const uint64_t* tab,
                                                   const FusedOps& fused, uint64_t* stats, const RowDivisor* div,
-                                                  float threshold, int* stop) {
+                                                  float threshold, int* stop, int base0, int cur0, float s0) {
   constexpr bool WALK = true;
   n_prep = uniform_u32(n_prep);
   const int lane = threadIdx.x & 63;
   const float kInf = __uint_as_float(0x7f800000u);
-  const float fill = inv < 0.0f ? kInf : -kInf;
-  float s = 0.0f;
-  // slot `slot` entry by entry from the logits, from running sum `from` (WALK: with the threshold)
+  float s = s0;
   auto redo = [&](int slot, float from, int& hit) {
-    float l[8];
-    uint32_t b[8];
-    load_slot_lane<DT>(logits, slot, lane, V, fill, l, fused);
-#pragma unroll
-    for (int k = 0; k < 8; ++k) {
-      float e = expf_core(__builtin_fmaxf(l[k] * inv - m, -104.0f), tab);
-      if (WALK) e = div_row(e, *div);
-      b[k] = __float_as_uint(e);
-    }
-    float t = from;
-    wave_resolve<8>(t, hit, b, slot * kSlot + lane * 8, V, WALK ? threshold : kInf);
-    return t;
+    return walk_redo<DT>(logits, slot, V, inv, m, tab, fused, *div, threshold, from, hit);
   };
-  if (WALK) *stop = -1;
+  *stop = -1;
   uint64_t c_start = 0;
   uint32_t n_iter = 0, n_generic = 0, n_prep_used = 0, n_tie = 0, n_inner = 0;
   uint64_t c_prep = 0;
@@ -1486,19 +1525,11 @@ __device__ __forceinline__ float split_chain_walk(const SlotRec* recs, int ns, c
                  (c_prep << 48);
     }
   };
-  for (int base = 0; base < ns; base += 64) {
+  for (int base = base0; base < ns; base += 64) {
     SlotRec r = {kSlotZero << 8, 0u, 0u, 0xffffffffu};
     if (base + lane < ns) r = recs[base + lane];
     const uint32_t kind = (r.meta >> 8) & 7u, kb = r.meta & 255u;
-    int cur = 0;
-    if (base == 0 && readlane_u32(kind, 0) == kSlotExact) {  // pass 2 worked the first slot out
-      s = __uint_as_float(readlane_u32(r.even, 0));
-      cur = 1;
-      if (WALK && s > threshold) {
-        note();
-        return redo(0, 0.0f, *stop);
-      }
-    }
+    int cur = base == base0 ? cur0 : 0;  // (a first slot that pass 2 worked out lies in front of cur0)
     // A stable slot with a half-ulp tie inside (one increment for an even sum in front of it, one for
     // an odd sum) counts as plain here, and the prefix is a composition of such pairs (compose()),
     // which follows the parity through the run; it is redone behind every record worked out
@@ -2656,10 +2687,9 @@ __global__ void __launch_bounds__(kWalkBlock) split_walk_kernel(SplitParams p, u
   for (int i = tid; i < prep_vecs; i += kWalkBlock) lds_vec[rec_bytes / 16 + i] = prep_src[i];
   __syncthreads();
   uint2* pairs = reinterpret_cast<uint2*>(reinterpret_cast<char*>(walk_lds) + chain_pairs_offset(ns));
-  if (PHASE == 0) {  // the runs of the row's records, a chunk of 64 per wave
-    split_chain_prepare(reinterpret_cast<const SlotRec*>(walk_lds), ns, pairs, tid >> 6, kWalkBlock / 64);
-    __syncthreads();
-  }
+  // the runs of the row's records, a chunk of 64 per wave
+  split_chain_prepare(reinterpret_cast<const SlotRec*>(walk_lds), ns, pairs, tid >> 6, kWalkBlock / 64);
+  __syncthreads();
   if (tid >= 64) return;
   const SlotRec* recs = reinterpret_cast<const SlotRec*>(walk_lds);
   const PrepSlot* prep = reinterpret_cast<const PrepSlot*>(reinterpret_cast<const char*>(walk_lds) + rec_bytes);
@@ -2671,8 +2701,7 @@ __global__ void __launch_bounds__(kWalkBlock) split_walk_kernel(SplitParams p, u
     const float2 w = p.walk[row];
     const RowDivisor div = row_divisor(w.x);
     int stop = -1;
-    const float cdf = split_chain_walk<DT>(recs, ns, prep, n_prep, logits, V, inv, rs.m, exp2tab, p.row.fused,
-                                            walk_timers ? walk_timers + static_cast<int64_t>(gridDim.x) * 8 + static_cast<int64_t>(blockIdx.x) * 4 - 4 : nullptr, &div, w.y, &stop);
+    const float cdf = split_chain<DT, true>(recs, pairs, ns, prep, n_prep, logits, V, inv, rs.m, exp2tab, p.row.fused, nullptr, &div, w.y, &stop);
     if (lane == 0) {
       const int32_t token = stop >= 0 ? stop : V - 1;
       p.row.tokens[row] = token;
