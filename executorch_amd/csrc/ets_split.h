@@ -398,10 +398,32 @@ __device__ __forceinline__ void split_fold_slot(const SplitParams& p, int row, i
         uint32_t base = 0u;
         if (lane == 0) base = atomicAdd(&sh.list_count, total);
         base = readlane_u32(base, 0);
-        at = base + incl - mine;
+        if (base >= static_cast<uint32_t>(p.list_region)) {
+          // The workgroup's list is full already, so the finish kernel will find that the row's
+          // lists do not hold every candidate and use neither them nor the histogram by size
+          // (every use of the two is behind that check): only the count above and the count per
+          // bit pattern, by which a 16-bit row with a long nucleus is drawn, are still needed.
+          if constexpr (DT == kDtypeBFloat16 || DT == kDtypeHalf) {
+            if (km.n_bins > 0) {
+              const int shift = 0x8000 - km.key_cut, first_mag = km.mag_min - 1;
 #pragma unroll
-        for (int k = 0; k < 8; ++k) {
-          if ((cmask >> k) & 1u) note(e[k], logit[k], k);
+              for (int k = 0; k < 8; ++k) {
+                // pattern_key() - key_cut (a negative value's key 0x7fff - cm is 0x8000 + ~cm)
+                const uint32_t pat = value_pattern<DT>(logit[k]);
+                const int mag = static_cast<int>(pat & 0x7fffu) - first_mag;
+                const int cm = mag > 0 ? mag : 0;
+                const int bin = (cm ^ (static_cast<int>(pat << 16) >> 31)) + shift;
+                if (((cmask >> k) & 1u) && static_cast<uint32_t>(bin) < static_cast<uint32_t>(km.n_bins))
+                  atomicAdd(&ph[bin >> 1], 1u << ((bin & 1) << 4));
+              }
+            }
+          }
+        } else {
+          at = base + incl - mine;
+#pragma unroll
+          for (int k = 0; k < 8; ++k) {
+            if ((cmask >> k) & 1u) note(e[k], logit[k], k);
+          }
         }
       } else {
         // sparse (the usual row: a few candidates in a slot, at most two in a lane): two rounds,
@@ -1720,10 +1742,14 @@ struct RunSlotRec {
   uint32_t pad;
 };
 
+// Where counter word w lies in LDS: a pad word behind every 32, so that lanes that each walk a
+// stretch of bins of their own (32 bins are 16 words) do not all read from the same two banks.
+__device__ __forceinline__ int run_word(int w) { return w + (w >> 5); }
+
 // Probability and count of the bin at sorted position q (bins in falling key order).
 template <int DT>
 struct RunBins {
-  const uint32_t* cnt;  // LDS: two 16-bit counters per word
+  const uint32_t* cnt;  // LDS: two 16-bit counters per word, at run_word()
   int key_cut, n_bins, mag_min;
   float inv, m, cutoff;
   RowDivisor div;
@@ -1736,7 +1762,7 @@ struct RunBins {
       const float l = pattern_value<DT>(key_pattern(key_cut + bin, mag_min));
       const float e = expf_core(__builtin_fmaxf(l * inv - m, -104.0f), tab);
       prob = div_row(e, div);
-      const uint32_t c = (cnt[bin >> 1] >> ((bin & 1) << 4)) & 0xffffu;
+      const uint32_t c = (cnt[run_word(bin >> 1)] >> ((bin & 1) << 4)) & 0xffffu;
       count = (prob >= cutoff) ? c : 0u;  // sampler.cpp:137-143
     }
   }
@@ -1748,7 +1774,7 @@ struct RunBins {
     count = 0u;
     if (q < n_bins) {
       const int bin = n_bins - 1 - q;
-      const uint32_t c = (cnt[bin >> 1] >> ((bin & 1) << 4)) & 0xffffu;
+      const uint32_t c = (cnt[run_word(bin >> 1)] >> ((bin & 1) << 4)) & 0xffffu;
       if (c != 0u) {
         const float l = pattern_value<DT>(key_pattern(key_cut + bin, mag_min));
         const float x = __builtin_fmaxf(l * inv - m, -104.0f);
@@ -1847,19 +1873,43 @@ __device__ __noinline__ bool draw_topp_runs(RunArgs a, const char* logits, int V
   // ---- LDS: counters | group records | exact sums at group boundaries | candidates in front of
   //      each group | approximate masses in front of each group
   uint32_t* cnt = reinterpret_cast<uint32_t*>(lds);
-  RunSlotRec* recs = reinterpret_cast<RunSlotRec*>(cnt + (words + 3) / 4 * 4);
+  RunSlotRec* recs = reinterpret_cast<RunSlotRec*>(cnt + (run_word(words) + 4) / 4 * 4);
   float* sbound = reinterpret_cast<float*>(recs + n_groups);
   uint32_t* cbound = reinterpret_cast<uint32_t*>(sbound + n_groups + 1);
   float* mbound = reinterpret_cast<float*>(cbound + n_groups + 1);
   float* gfirst = mbound + n_groups + 1;  // probability of a group's first and last candidate bin (-1: none)
   float* glast = gfirst + n_groups;
-  if (reinterpret_cast<char*>(glast + n_groups) > reinterpret_cast<char*>(lds) + static_cast<size_t>(a.lds_keys) * 8)
-    return false;
+  char* const lds_end = reinterpret_cast<char*>(lds) + static_cast<size_t>(a.lds_keys) * 8;
+  if (reinterpret_cast<char*>(glast + n_groups) > lds_end) return false;
+  // ... | groups in which the sum is expected to change binade, prepared for the walk (kSideGroups
+  //      of them, if that much is left: the number taken, the groups, per bin the prefix sums of the
+  //      increments under the two ulps and the probability)
+  constexpr int kSideGroups = 24;
+  uint32_t* side_n = reinterpret_cast<uint32_t*>(glast + n_groups);
+  uint32_t* side_group = side_n + 1;
+  uint32_t* side_a = side_group + kSideGroups;
+  uint32_t* side_b = side_a + kSideGroups * 64;
+  float* side_p = reinterpret_cast<float*>(side_b + kSideGroups * 64);
+  const int side_cap = reinterpret_cast<char*>(side_p + kSideGroups * 64) <= lds_end ? kSideGroups : 0;
+  if (side_cap > 0 && tid == 0) *side_n = 0u;  // (barriers follow before pass B counts)
   // ---- the workgroups' counters, added up (16-bit halves add without carries unless one overflows,
   //      which the totals give away)
   {
     const uint32_t* in = a.phist;
     uint32_t sum16 = 0u;
+    if (a.row_wgs == 1) {
+      // one workgroup's counters: a copy, eight words of a lane requested at a time
+      for (int w0 = tid; w0 < words; w0 += 8 * kBlock) {
+        uint32_t v[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) v[k] = w0 + k * kBlock < words ? in[w0 + k * kBlock] : 0u;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+          if (w0 + k * kBlock < words) cnt[run_word(w0 + k * kBlock)] = v[k];
+          sum16 += (v[k] & 0xffffu) + (v[k] >> 16);
+        }
+      }
+    } else
     for (int w = tid; w < words; w += kBlock) {
       uint32_t lo = 0u, hi = 0u;
       for (int g = 0; g < a.row_wgs; g += 4) {
@@ -1875,7 +1925,7 @@ __device__ __noinline__ bool draw_topp_runs(RunArgs a, const char* logits, int V
         }
       }
       const bool fits = lo <= 0xffffu && hi <= 0xffffu;
-      cnt[w] = fits ? (lo | (hi << 16)) : 0u;
+      cnt[run_word(w)] = fits ? (lo | (hi << 16)) : 0u;
       sum16 += fits ? lo + hi : 0x40000000u;  // (spoils the total)
     }
     sum16 = wave_sum_u32(sum16);
@@ -1888,13 +1938,32 @@ __device__ __noinline__ bool draw_topp_runs(RunArgs a, const char* logits, int V
   }
   const RunBins<DT> bins = {cnt, a.key_cut, n_bins, a.mag_min, inv, a.m, cutoff, row_divisor(S), sm.exp2tab};
   // ---- pass A: per group the candidates (exactly) and their approximate mass
-  for (int t = wave; t < n_groups; t += kWaves) {
-    float prob;
-    uint32_t count;
-    bins.at_approx(64 * t + lane, prob, count);
-    const float mass = wave_sum_f32(static_cast<float>(count) * prob);
-    const uint32_t c = wave_sum_u32(count);
-    if (lane == 0) {
+  //      Eight lanes take a group, eight bins each, one bin after the other: no sums over a whole wave
+  //      (a wave to a group would spend most of its instructions on them), and the groups go round
+  //      the workgroup's lanes evenly.
+  constexpr int kPer = 8;  // bins of a lane; 64 / kPer lanes to a group
+  const int n_units = n_groups * (64 / kPer);
+  for (int u0 = 0; u0 < n_units; u0 += kBlock) {
+    const int u = u0 + tid;
+    const int t = u / (64 / kPer);
+    float mass = 0.0f;
+    uint32_t c = 0u;
+    if (u < n_units) {
+#pragma unroll 2
+      for (int i = 0; i < kPer; ++i) {
+        float prob;
+        uint32_t count;
+        bins.at_approx(kPer * u + i, prob, count);
+        mass += static_cast<float>(count) * prob;
+        c += count;
+      }
+    }
+#pragma unroll
+    for (int d = 1; d < 64 / kPer; d <<= 1) {
+      mass += __shfl_xor(mass, d);
+      c += static_cast<uint32_t>(__shfl_xor(static_cast<int>(c), d));
+    }
+    if (u < n_units && (lane & (64 / kPer - 1)) == 0) {
       mbound[t + 1] = mass;
       cbound[t + 1] = c;
     }
@@ -1941,54 +2010,87 @@ __device__ __noinline__ bool draw_topp_runs(RunArgs a, const char* logits, int V
   //      under the ulp(s) of the binade(s) the cumulative sum can be in while it passes the group;
   //      one that may hold the place where the sum exceeds topp, that spans more than two binades
   //      or in which an entry ties is left to the ordered walk.
+  //      As in pass A eight lanes take a group, eight bins each in order, and put their parts together.
   bool rising = false;
-  for (int t = wave; t < n_groups; t += kWaves) {
-    const uint32_t c_in = cbound[t], c_out = cbound[t + 1];
+  for (int u0 = 0; u0 < n_units; u0 += kBlock) {
+    const int u = u0 + tid;
+    const int t = u / (64 / kPer);
+    const bool valid = u < n_units;
+    const uint32_t c_in = valid ? cbound[t] : 0u, c_out = valid ? cbound[t + 1] : 0u;
     RunSlotRec rec = {kSlotZero << 8, 0u, 0u, 0u};
-    float first_p = -1.0f, last_p = -1.0f;
+    bool walked = false, folded = false;
+    uint32_t kb_lo = 0u, kb_hi = 0u;
     if (c_out != c_in) {
       const float eps_in = static_cast<float>(c_in) * (1.02f / 16777216.0f) + 6e-5f;
       const float eps_out = static_cast<float>(c_out) * (1.02f / 16777216.0f) + 6e-5f;
       const float lo = mbound[t] * (1.0f - eps_in), hi = mbound[t + 1] * (1.0f + eps_out);
-      const uint32_t kb_lo = __float_as_uint(lo > 0.0f ? lo : 0.0f) >> 23, kb_hi = __float_as_uint(hi) >> 23;
+      kb_lo = __float_as_uint(lo > 0.0f ? lo : 0.0f) >> 23;
+      kb_hi = __float_as_uint(hi) >> 23;
       const bool near_topp = !(hi < topp * 0.9999f);  // (the walk ends there: nothing behind it is needed)
       rec.meta = (kSlotSerial << 8) | (kb_lo & 255u);
-      if (!(lo > topp * 1.001f)) {  // (a group the walk cannot reach stays "serial": worked out exactly if reached after all)
+      walked = !(lo > topp * 1.001f);  // (a group the walk cannot reach stays "serial": worked out exactly if reached after all)
+      folded = walked && !near_topp && lo > 0.0f && kb_lo >= 70u && kb_hi <= 250u && kb_hi <= kb_lo + 1u;
+    }
+    // this lane's part of the group: its first and last candidate bin, whether the probabilities
+    // rise from one candidate bin to the next, the increments under the two ulps
+    float first_p = -1.0f, last_p = -1.0f;
+    bool up = false, tie = false;
+    uint32_t ia = 0u, ib = 0u;
+    if (walked) {
+      const float scale_a = __uint_as_float((277u - kb_lo) << 23), scale_b = __uint_as_float((276u - kb_lo) << 23);
+      for (int i = 0; i < kPer; ++i) {
         float prob;
         uint32_t count;
-        bins.at(64 * t + lane, prob, count);
-        // among the group's candidate bins: each against the next one
-        const uint64_t occ = __ballot(count != 0u);
-        const uint64_t above = lane == 63 ? 0ull : occ >> (lane + 1);
-        const int next = above ? lane + __ffsll(static_cast<long long>(above)) : lane;
-        const float next_prob = __shfl(prob, next);
-        if (count != 0u && above != 0ull && next_prob > prob) rising = true;
-        if (occ != 0ull) {
-          first_p = readlane_f32(prob, __ffsll(static_cast<long long>(occ)) - 1);
-          last_p = readlane_f32(prob, 63 - __clzll(static_cast<long long>(occ)));
-        }
-        if (!near_topp && lo > 0.0f && kb_lo >= 70u && kb_hi <= 250u && kb_hi <= kb_lo + 1u) {
-          const float scale_a = __uint_as_float((277u - kb_lo) << 23), scale_b = __uint_as_float((276u - kb_lo) << 23);
-          const float ta = prob * scale_a, tb = prob * scale_b;
-          const float ra = __builtin_rintf(ta), rb = __builtin_rintf(tb);
-          const bool tie = count != 0u && (__builtin_fabsf(ta - ra) == 0.5f || (kb_hi != kb_lo && __builtin_fabsf(tb - rb) == 0.5f));
-          const float fc = static_cast<float>(count);
-          const uint32_t ia = static_cast<uint32_t>(__builtin_fminf(ra * fc, 33554432.0f));
-          const uint32_t ib = static_cast<uint32_t>(__builtin_fminf(rb * fc, 33554432.0f));
-          const uint32_t inc_a = wave_sum_u32(ia), inc_b = wave_sum_u32(ib);
-          if (__ballot(tie) == 0ull) {
-            rec.meta = ((kb_hi == kb_lo ? kSlotStable : kSlotDual) << 8) | kb_lo;
-            rec.inc_a = inc_a < kSat ? inc_a : kSat;
-            rec.inc_b = inc_b < kSat ? inc_b : kSat;
+        bins.at(kPer * u + i, prob, count);
+        if (count != 0u) {
+          if (first_p < 0.0f) first_p = prob;
+          if (last_p >= 0.0f && prob > last_p) up = true;
+          last_p = prob;
+          if (folded) {
+            const float ta = prob * scale_a, tb = prob * scale_b;
+            const float ra = __builtin_rintf(ta), rb = __builtin_rintf(tb);
+            tie = tie || __builtin_fabsf(ta - ra) == 0.5f || (kb_hi != kb_lo && __builtin_fabsf(tb - rb) == 0.5f);
+            const float fc = static_cast<float>(count);
+            ia += static_cast<uint32_t>(__builtin_fminf(ra * fc, 33554432.0f));  // (64 of them to a group: below 2^31)
+            ib += static_cast<uint32_t>(__builtin_fminf(rb * fc, 33554432.0f));
           }
         }
       }
     }
-    if (lane == 0) {
+    // the parts of a group, put together pair by pair (of two partners the one with the lower lane
+    // holds the earlier bins); every lane of the group ends up with the whole
+#pragma unroll
+    for (int d = 1; d < 64 / kPer; d <<= 1) {
+      const float o_first = __shfl_xor(first_p, d), o_last = __shfl_xor(last_p, d);
+      const bool o_up = __shfl_xor(up ? 1 : 0, d) != 0, o_tie = __shfl_xor(tie ? 1 : 0, d) != 0;
+      ia += static_cast<uint32_t>(__shfl_xor(static_cast<int>(ia), d));
+      ib += static_cast<uint32_t>(__shfl_xor(static_cast<int>(ib), d));
+      const bool left = (lane & d) == 0;
+      const float l_first = left ? first_p : o_first, l_last = left ? last_p : o_last;
+      const float r_first = left ? o_first : first_p, r_last = left ? o_last : last_p;
+      up = up || o_up || (l_last >= 0.0f && r_first >= 0.0f && r_first > l_last);
+      tie = tie || o_tie;
+      first_p = l_first >= 0.0f ? l_first : r_first;
+      last_p = r_last >= 0.0f ? r_last : l_last;
+    }
+    if (valid && (lane & (64 / kPer - 1)) == 0) {
+      if (folded && !tie) {
+        rec.meta = ((kb_hi == kb_lo ? kSlotStable : kSlotDual) << 8) | kb_lo;
+        rec.inc_a = ia < kSat ? ia : kSat;
+        rec.inc_b = ib < kSat ? ib : kSat;
+        if (kb_hi != kb_lo && side_cap > 0) {  // the sum is expected to change binade inside: prepared below
+          const uint32_t d = atomicAdd(side_n, 1u);
+          if (d < static_cast<uint32_t>(side_cap)) {
+            side_group[d] = static_cast<uint32_t>(t);
+            rec.pad = d + 1u;
+          }
+        }
+      }
       recs[t] = rec;
       gfirst[t] = first_p;
       glast[t] = last_p;
     }
+    if (up) rising = true;
   }
   {
     const uint64_t any = __ballot(rising);
@@ -2021,6 +2123,33 @@ __device__ __noinline__ bool draw_topp_runs(RunArgs a, const char* logits, int V
     bad |= static_cast<uint32_t>(sm.flag);
     __syncthreads();
     if (bad != 0u) return false;
+  }
+  // ---- the groups in which the sum is expected to change binade (kb -> kb + 1), a wave each: per bin
+  //      the exact probability and the prefix sums of the increments under either ulp.  The walk
+  //      then finds the bin in which the sum leaves binade kb from the first prefix sums, adds that
+  //      bin's copies in closed form and the bins behind it from the second.  (No bin of a folded
+  //      group ties under either ulp.)  A group with a bin whose increment is not below 2^25 is not
+  //      prepared.
+  if (side_cap > 0) {
+    const int n_side = static_cast<int>(*side_n < static_cast<uint32_t>(side_cap) ? *side_n : static_cast<uint32_t>(side_cap));
+    for (int d = wave; d < n_side; d += kWaves) {
+      const int t = static_cast<int>(side_group[d]);
+      const uint32_t kb = recs[t].meta & 255u;
+      float prob;
+      uint32_t count;
+      bins.at(64 * t + lane, prob, count);
+      const float fc = static_cast<float>(count);
+      const float va = __builtin_rintf(prob * __uint_as_float((277u - kb) << 23)) * fc;
+      const float vb = __builtin_rintf(prob * __uint_as_float((276u - kb) << 23)) * fc;
+      const bool big = !(va < 33554432.0f) || !(vb < 33554432.0f);
+      const uint32_t pre_a = wave_scan_inclusive_u32(big ? 0u : static_cast<uint32_t>(va));
+      const uint32_t pre_b = wave_scan_inclusive_u32(big ? 0u : static_cast<uint32_t>(vb));
+      side_a[d * 64 + lane] = pre_a;
+      side_b[d * 64 + lane] = pre_b;
+      side_p[d * 64 + lane] = count != 0u ? prob : 0.0f;
+      if (__ballot(big) != 0ull && lane == 0) recs[t].pad = 0u;
+    }
+    __syncthreads();
   }
   // ---- walk 1 (sampler.cpp:150-158): the groups in order until the sum exceeds topp.  One wave.
   if (wave == 0) {
@@ -2068,6 +2197,54 @@ __device__ __noinline__ bool draw_topp_runs(RunArgs a, const char* logits, int V
         if (j == 64) break;
         const int t = base + j;
         if (t >= n_groups) break;
+        // ---- a prepared group folded for this binade that the sum leaves inside it, topp far away
+        const uint32_t side = readlane_u32(r.pad, j);
+        if (j == jo && side != 0u && readlane_u32(kb, j) == K && limit == (1u << 24) && K < 250u) {
+          const int d = static_cast<int>(side) - 1;
+          const uint32_t pre_a = side_a[d * 64 + lane], pre_b = side_b[d * 64 + lane];
+          const SumState sj = sum_state(uniform_f32(s));
+          const uint32_t room = (1u << 24) - sj.S;
+          const uint64_t out = __ballot(pre_a >= room);
+          if (out != 0ull && sj.kb == ss.kb) {
+            const int jl = static_cast<int>(uniform_u32(static_cast<uint32_t>(__builtin_ctzll(out))));
+            const uint32_t front_a = jl > 0 ? readlane_u32(pre_a, jl - 1) : 0u;
+            const uint32_t S_j = sj.S + front_a;  // below 2^24
+            const float pl = side_p[d * 64 + jl];
+            // bin jl: c copies of pl, each n_a under this ulp (their product is the bin's increment)
+            const float scale_a = __uint_as_float((277u - K) << 23), scale_b = __uint_as_float((276u - K) << 23);
+            const float n_af = __builtin_rintf(pl * scale_a);
+            const uint32_t n_a = static_cast<uint32_t>(n_af), n_b = static_cast<uint32_t>(__builtin_rintf(pl * scale_b));
+            const uint32_t inc_l = readlane_u32(pre_a, jl) - front_a;  // c * n_a, at least the room left: n_a is not 0
+            // copies after which the sum is still below 2^24 ulps: floor((2^24 - S_j - 1) / n_a), fewer than c
+            const uint32_t x = (1u << 24) - S_j - 1u;
+            uint32_t stay = static_cast<uint32_t>(static_cast<float>(x) / n_af);
+            if (stay * n_a > x) --stay;
+            if ((stay + 1u) * n_a <= x) ++stay;
+            // the next copy goes natively and takes the sum into binade K + 1; the rest and the
+            // bins behind jl add under its ulp
+            const float crossed = sum_value(S_j + stay * n_a, static_cast<int>(K)) + pl;
+            const uint32_t cb = __float_as_uint(crossed);
+            const int bin_l = n_bins - 1 - (64 * t + jl);  // (a candidate bin: its increment is not 0)
+            const uint32_t c_l = uniform_u32((cnt[run_word(bin_l >> 1)] >> ((bin_l & 1) << 4)) & 0xffffu);
+            const uint32_t rest = readlane_u32(pre_b, 63) - readlane_u32(pre_b, jl);
+            uint32_t limit_b = 1u << 24;
+            {
+              const float tt = topp * scale_b;
+              if (tt < 16777216.0f) {
+                const uint32_t Tn = static_cast<uint32_t>(__builtin_floorf(tt)) + 1u;
+                limit_b = Tn < limit_b ? Tn : limit_b;
+              }
+            }
+            const uint64_t S_b = static_cast<uint64_t>((cb & 0x7fffffu) | 0x800000u) +
+                                 static_cast<uint64_t>(c_l - stay - 1u) * n_b + rest;
+            if (n_a != 0u && c_l * n_a == inc_l && stay < c_l && (cb >> 23) == K + 1u && S_b < limit_b) {
+              s = sum_value(static_cast<uint32_t>(S_b), static_cast<int>(K + 1u));
+              if (lane == 0) sbound[t + 1] = s;
+              cur = j + 1;
+              continue;
+            }
+          }
+        }
         found = resolve_run_group<DT>(s, t, cbound[t], topp, bins);
         if (lane == 0) sbound[t + 1] = s;
         if (found >= 0) last_group = t;
@@ -2158,20 +2335,72 @@ __device__ __noinline__ bool draw_topp_runs(RunArgs a, const char* logits, int V
   const int ns = a.ns;
   uint32_t* occ = reinterpret_cast<uint32_t*>(lds);  // (the counters are dead) ns + 1 words
   const float kInf = __uint_as_float(0x7f800000u);
+  // Keys rise with the values, and a key above 0x8001 or below 0x7ffe belongs to one pattern that is
+  // not a zero: a range of such keys of one sign is a range of values, and an entry is compared as a
+  // number (two comparisons instead of its key; the zeros of the two signs compare equal and have
+  // different keys, which is why they stay with the keys).
+  const bool by_value = key_lo > 0x8001 || key_hi < 0x7ffe;
+  const float v_lo = pattern_value<DT>(key_pattern(key_lo, a.mag_min)), v_hi = pattern_value<DT>(key_pattern(key_hi, a.mag_min));
+  auto matching = [&](const float (&l)[8], int s_, int lane_) -> uint32_t {
+    uint32_t mask = 0u;
+    if (by_value) {
+#pragma unroll
+      for (int k = 0; k < 8; ++k) mask |= (l[k] >= v_lo && l[k] <= v_hi) ? (1u << k) : 0u;
+    } else {
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        const int key = pattern_key(value_pattern<DT>(l[k]), a.mag_min);
+        mask |= (key >= key_lo && key <= key_hi) ? (1u << k) : 0u;
+      }
+    }
+    const int left = V - (s_ * kSlot + lane_ * 8);  // (entries past the row's end)
+    return mask & (left >= 8 ? 0xffu : (left > 0 ? (1u << left) - 1u : 0u));
+  };
   auto matches = [&](int s_, int lane_) -> uint32_t {
     float l[8];
     load_slot_lane<DT>(logits, s_, lane_, V, -kInf, l, *a.fused);
-    uint32_t mask = 0u;
-#pragma unroll
-    for (int k = 0; k < 8; ++k) {
-      const int key = pattern_key(value_pattern<DT>(l[k]), a.mag_min);
-      mask |= (key >= key_lo && key <= key_hi && s_ * kSlot + lane_ * 8 + k < V) ? (1u << k) : 0u;
-    }
-    return mask;
+    return matching(l, s_, lane_);
   };
-  for (int s_ = wave; s_ < ns; s_ += kWaves) {
-    const uint32_t c = wave_sum_u32(static_cast<uint32_t>(__popc(matches(s_, lane))));
-    if (lane == 0) occ[s_] = c;
+  {
+    // (five slots of a wave requested at a time: a slot is 16 bytes per lane of a 16-bit row)
+    constexpr int kAhead = 5;
+    static_assert(VecElems<DT>::value == 8, "a lane's eight entries are one 16-byte load");
+    const bool plain = by_value && a.fused->n == 0;
+    for (int s0 = wave; s0 < ns; s0 += kAhead * kWaves) {
+      uint4 raw[kAhead];
+#pragma unroll
+      for (int j = 0; j < kAhead; ++j) {
+        const int s_ = s0 + j * kWaves;
+        raw[j] = {0u, 0u, 0u, 0u};
+        if (s_ < ns && (s_ + 1) * kSlot <= V)
+          raw[j] = *reinterpret_cast<const uint4*>(logits + static_cast<int64_t>(s_ * kSlot + lane * 8) * ElemSize<DT>::value);
+      }
+#pragma unroll
+      for (int j = 0; j < kAhead; ++j) {
+        const int s_ = s0 + j * kWaves;
+        if (s_ < ns) {
+          float l[8];
+          uint32_t c;
+          if (plain && (s_ + 1) * kSlot <= V) {
+            // the usual slot: two comparisons per entry, their outcomes over the wave counted on
+            // the scalar unit (no mask per lane, no sum over the lanes)
+            decode_vec<DT>(raw[j], l);
+            c = 0u;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) c += static_cast<uint32_t>(__popcll(__ballot(l[k] >= v_lo && l[k] <= v_hi)));
+          } else {
+            if ((s_ + 1) * kSlot <= V) {
+              decode_vec<DT>(raw[j], l);
+              if (a.fused->n > 0) apply_fused<DT, 8>(l, *a.fused);
+            } else {
+              load_slot_lane<DT>(logits, s_, lane, V, -kInf, l, *a.fused);
+            }
+            c = wave_sum_u32(static_cast<uint32_t>(__popc(matching(l, s_, lane))));
+          }
+          if (lane == 0) occ[s_] = c;
+        }
+      }
+    }
   }
   __syncthreads();
   if (wave == 0) {
