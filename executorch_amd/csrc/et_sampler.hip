@@ -7,6 +7,7 @@
 #include <algorithm>
 #include <atomic>
 #include <cstdio>
+#include <cmath>
 #include <cstring>
 #include <ctime>
 #include <mutex>
@@ -65,7 +66,9 @@ int pass2_workgroups(const ets_sampler* s, int32_t rows, int32_t ns) {
     const char* e = std::getenv("ETS_SPLIT_WORKGROUPS");
     return e ? std::atoi(e) : 0;
   }();
-  int g = (forced > 0 && !s->wb) ? forced : (s->num_cus > 0 ? s->num_cus : 256) / rows;
+  // (launches that run side by side share the compute units: each takes its share of them, so that
+  // the workgroups of both are resident at once)
+  int g = (forced > 0 && !s->wb) ? forced : (s->num_cus > 0 ? s->num_cus : 256) / (rows + s->beside_rows);
   const int by_len = (ns + 15) / 16;
   if (g > by_len) g = by_len;
   if (g > ets::kMaxRowWorkgroups) g = ets::kMaxRowWorkgroups;
@@ -457,6 +460,22 @@ struct StageLayout {
   }
 };
 
+// The upload of a staging buffer: a kernel that reads the pinned host buffer and writes the device
+// copy.  (An asynchronous copy of a few kilobytes enqueued behind a kernel held the calling thread
+// until that kernel had run -- tens of microseconds per call, serialising host and GPU; a launch
+// does not.)
+__global__ void stage_upload_kernel(const uint4* host, uint4* device, int32_t n) {
+  const int32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) device[i] = host[i];
+}
+ets_status stage_upload(ets_sampler* s, const void* h, void* d, size_t bytes, hipStream_t stream) {
+  const int32_t n = static_cast<int32_t>((bytes + 15) / 16);  // (both buffers are allocated in multiples of 256 bytes)
+  hipLaunchKernelGGL(stage_upload_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, static_cast<const uint4*>(h),
+                     static_cast<uint4*>(d), n);
+  ETS_HIP(s, hipGetLastError());
+  return ETS_OK;
+}
+
 __global__ void reseed_kernel(uint64_t* rng, const uint64_t* reseed, int32_t rows) {
   const int32_t b = blockIdx.x * blockDim.x + threadIdx.x;
   if (b < rows && reseed[b] != 0ull) rng[b] = reseed[b];
@@ -465,10 +484,30 @@ __global__ void reseed_kernel(uint64_t* rng, const uint64_t* reseed, int32_t row
 ets_status ensure_stage(ets_sampler* s) {
   if (s->h_stage) return ETS_OK;
   const StageLayout full(s->max_batch);
-  ETS_HIP(s, hipHostMalloc(&s->h_stage, full.bytes, hipHostMallocDefault));
-  ETS_HIP(s, hipMalloc(&s->d_stage, full.bytes));
-  ETS_HIP(s, hipEventCreateWithFlags(&s->stage_event, hipEventDisableTiming));
+  s->stage_bytes = round_up(full.bytes, 256);
+  ETS_HIP(s, hipHostMalloc(&s->h_stage, s->stage_bytes * ets_sampler::kStageSlots, hipHostMallocDefault));
+  ETS_HIP(s, hipMalloc(&s->d_stage, s->stage_bytes));
+  for (int i = 0; i < ets_sampler::kStageSlots; ++i) ETS_HIP(s, hipEventCreateWithFlags(&s->stage_event[i], hipEventDisableTiming));
   ETS_HIP(s, hipEventCreateWithFlags(&s->stage_done, hipEventDisableTiming));
+  return ETS_OK;
+}
+
+// The pinned buffer this call fills: the next of the ring, once the upload last made from it has left it.
+ets_status stage_host_buffer(ets_sampler* s, char** out) {
+  const int slot = s->stage_next;
+  if (s->stage_pending[slot]) {
+    ETS_HIP(s, hipEventSynchronize(s->stage_event[slot]));
+    s->stage_pending[slot] = false;
+  }
+  *out = static_cast<char*>(s->h_stage) + static_cast<size_t>(slot) * s->stage_bytes;
+  return ETS_OK;
+}
+// Behind the upload from that buffer.
+ets_status stage_uploaded(ets_sampler* s, hipStream_t stream) {
+  const int slot = s->stage_next;
+  ETS_HIP(s, hipEventRecord(s->stage_event[slot], stream));
+  s->stage_pending[slot] = true;
+  s->stage_next = (slot + 1) % ets_sampler::kStageSlots;
   return ETS_OK;
 }
 
@@ -499,16 +538,15 @@ ets_status sample_device_configs(ets_sampler* s, const void* d_logits, int32_t d
                                  hipStream_t stream) {
   ets_status st = ensure_stage(s);
   if (st != ETS_OK) return st;
-  if (s->stage_pending) {
-    ETS_HIP(s, hipEventSynchronize(s->stage_event));  // the previous upload has left the staging buffer
-    s->stage_pending = false;
-  }
   const StageLayout lay(batch);
-  char* h = static_cast<char*>(s->h_stage);
+  char* h = nullptr;
+  st = stage_host_buffer(s, &h);
+  if (st != ETS_OK) return st;
   char* d = static_cast<char*>(s->d_stage);
   uint64_t* h_reseed = reinterpret_cast<uint64_t*>(h + lay.reseed);
   ets::RowConfig* h_cfg = reinterpret_cast<ets::RowConfig*>(h + lay.cfg);
   int32_t* h_maps = reinterpret_cast<int32_t*>(h + lay.maps);
+  std::memset(h, 0, lay.bytes);  // (what this call does not fill must not differ from call to call: see the comparison below)
   // Four groups of rows: arg-max rows, top-p and top-k rows that take the three-launch path,
   // multinomial rows that take the five-launch path, and every other row that draws (one launch of
   // the one-workgroup-per-row kernel, which picks each row's draw from its parameters).
@@ -517,10 +555,12 @@ ets_status sample_device_configs(ets_sampler* s, const void* d_logits, int32_t d
   int32_t count[4] = {0, 0, 0, 0};
   bool split_topk = false;  // some row of the three-launch group is a top-k row
   bool any_reseed = false;
+  bool inv_ordinary = true;
   for (int32_t b = 0; b < batch; ++b) {
     const ets_sampling_config& c = configs[b];
     // temperature < 0: the handle's own (SamplingConfig: "-1 temperature means implementation default")
     const float inv = c.temperature < 0.0f ? s->inv_temperature : inverse_temperature_ctor(c.temperature);
+    inv_ordinary = inv_ordinary && std::fabs(inv) < 3.0e38f;
     h_cfg[b].inv_temperature = inv;
     h_cfg[b].topp = c.top_p;
     h_cfg[b].topk = c.top_k;
@@ -541,9 +581,15 @@ ets_status sample_device_configs(ets_sampler* s, const void* d_logits, int32_t d
   }
   st = stage_acquire(s, stream);
   if (st != ETS_OK) return st;
-  ETS_HIP(s, hipMemcpyAsync(d, h, lay.bytes, hipMemcpyHostToDevice, stream));
-  ETS_HIP(s, hipEventRecord(s->stage_event, stream));
-  s->stage_pending = true;
+  if (!(s->stage_shadow_valid && s->stage_shadow.size() == lay.bytes && std::memcmp(s->stage_shadow.data(), h, lay.bytes) == 0)) {
+    s->stage_shadow_valid = false;
+    st = stage_upload(s, h, d, lay.bytes, stream);
+    if (st != ETS_OK) return st;
+    st = stage_uploaded(s, stream);
+    if (st != ETS_OK) return st;
+    s->stage_shadow.assign(h, lay.bytes);
+    s->stage_shadow_valid = true;
+  }
   if (any_reseed) {
     hipLaunchKernelGGL(reseed_kernel, dim3((batch + 255) / 256), dim3(256), 0, stream, s->d_rng,
                        reinterpret_cast<const uint64_t*>(d + lay.reseed), batch);
@@ -592,16 +638,21 @@ ets_status sample_device_configs(ets_sampler* s, const void* d_logits, int32_t d
     p.row_map = d_maps + kRows * batch;
     first = rows_device(s, p, dtype, count[kRows], stream, ets::kDrawAny);
   }
+  // (the multinomial rows' launches and the three launches of the top-p and top-k rows run side by side)
+  s->cfg_inv_ordinary = inv_ordinary;
   if (first == ETS_OK && count[kWalk] > 0) {  // (no scratch rows, no tickets)
     p.row_map = d_maps + kWalk * batch;
+    s->beside_rows = fork ? count[kSplit] : 0;
     first = launch_split_walk_any(s, p, dtype, count[kWalk], stream);
   }
   if (first == ETS_OK && count[kSplit] > 0) {
     p.scratch = s->d_scratch + (both_draw ? static_cast<int64_t>(share) * s->scratch_stride : 0);
     p.grid_cap = share;
     p.row_map = d_maps + kSplit * batch;
+    s->beside_rows = fork ? count[kWalk] + count[kRows] : 0;  // (what the caller's stream runs meanwhile)
     first = launch_split_any(s, p, dtype, count[kSplit], side, split_topk);
   }
+  s->beside_rows = 0;
   if (first == ETS_OK && count[kGreedy] > 0)
     first = argmax_device(s, d_logits, dtype, count[kGreedy], stride, d_tokens, side, d_maps + kGreedy * batch);
   const std::string first_message = s->last_error;
@@ -728,7 +779,9 @@ ets_status ets_sampler_destroy(ets_sampler* s) {
     if (s->aux_stream) (void)hipStreamDestroy(s->aux_stream);
     if (s->join_event) (void)hipEventDestroy(s->join_event);
     if (s->fork_event) (void)hipEventDestroy(s->fork_event);
-    if (s->stage_event) (void)hipEventDestroy(s->stage_event);
+    for (int i = 0; i < ets_sampler::kStageSlots; ++i) {
+      if (s->stage_event[i]) (void)hipEventDestroy(s->stage_event[i]);
+    }
     if (s->stage_done) (void)hipEventDestroy(s->stage_done);
     for (int i = 0; i < ets_sampler::kTimingSlots; ++i) {
       if (s->t_begin[i]) (void)hipEventDestroy(s->t_begin[i]);
@@ -871,16 +924,17 @@ ets_status ets_sampler_gumbel_max_batch(ets_sampler* s, const void* d_logits, in
   if (n_temperatures > 1) {
     st = ensure_stage(s);
     if (st != ETS_OK) return st;
-    if (s->stage_pending) {
-      ETS_HIP(s, hipEventSynchronize(s->stage_event));
-      s->stage_pending = false;
-    }
-    std::memcpy(s->h_stage, temperatures, sizeof(float) * n_temperatures);
+    char* h = nullptr;
+    st = stage_host_buffer(s, &h);
+    if (st != ETS_OK) return st;
+    std::memcpy(h, temperatures, sizeof(float) * n_temperatures);
     st = stage_acquire(s, stream);
     if (st != ETS_OK) return st;
-    ETS_HIP(s, hipMemcpyAsync(s->d_stage, s->h_stage, sizeof(float) * n_temperatures, hipMemcpyHostToDevice, stream));
-    ETS_HIP(s, hipEventRecord(s->stage_event, stream));
-    s->stage_pending = true;
+    s->stage_shadow_valid = false;  // (the device copy holds temperatures from here on)
+    st = stage_upload(s, h, s->d_stage, sizeof(float) * n_temperatures, stream);
+    if (st != ETS_OK) return st;
+    st = stage_uploaded(s, stream);
+    if (st != ETS_OK) return st;
     d_row_temperatures = static_cast<const float*>(s->d_stage);
   }
   const float temperature = temperatures[0];

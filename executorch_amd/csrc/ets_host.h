@@ -53,14 +53,25 @@ struct ets_sampler {
   int num_cus = 0;
   void* d_split = nullptr;
   void* d_phist = nullptr;  // pattern histograms of 16-bit rows, allocated on their first use
+  bool cfg_inv_ordinary = false;  // per-row parameters of the call in progress: every inverse temperature is finite
+  int32_t beside_rows = 0;  // rows of other launches that run beside this one on another stream (set for the duration of a call)
   bool arrive_dirty = false;  // a fused launch was not followed by its finish kernel: the counters are cleared before the next one
   ets::SplitParams split = {};
-  // per-row sampling parameters of ets_sampler_sample_batch_configs(): pinned host staging, its
-  // device copy, and the event that says the last upload has left the staging buffer
-  void* h_stage = nullptr;
+  // per-row sampling parameters of ets_sampler_sample_batch_configs(): pinned host staging buffers
+  // that take turns (a call fills the next one and waits only if the upload made from it
+  // kStageSlots calls ago has not left it yet, so the host runs ahead of the GPU), the device copy,
+  // and per buffer the event that says its last upload has left it
+  static constexpr int kStageSlots = 4;
+  void* h_stage = nullptr;  // kStageSlots buffers of stage_bytes each, one after the other
+  size_t stage_bytes = 0;
   void* d_stage = nullptr;
-  hipEvent_t stage_event = nullptr;
-  bool stage_pending = false;
+  hipEvent_t stage_event[kStageSlots] = {};
+  bool stage_pending[kStageSlots] = {};
+  int stage_next = 0;
+  // what the device copy holds (a call whose staging data equals it uploads nothing: the parameters
+  // of a serving loop's rows rarely change from one step to the next)
+  std::string stage_shadow;
+  bool stage_shadow_valid = false;
   // the last stream a call that uses the staging copy ran on, and the event behind its launches: a
   // call on another stream waits for it before it overwrites the device copy
   hipEvent_t stage_done = nullptr;

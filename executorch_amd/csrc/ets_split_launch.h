@@ -75,7 +75,10 @@ ets_status launch_split(ets_sampler* s, const ets::RowParams& p, int32_t rows, h
   const int spin_env = spin_text ? std::atoi(spin_text) : (1 << 16);
   const int per_wg_slots = ((sp.ns + sp.row_wgs - 1) / sp.row_wgs + ets::kWaves - 1) / ets::kWaves * ets::kWaves;
   const float abs_inv = p.inv_temperature < 0.0f ? -p.inv_temperature : p.inv_temperature;
-  const bool fused = !TOPK && (!extras || (ETS_PHASE_CLOCKS && p.probs == nullptr)) && fuse_env != 0 && p.row_cfg == nullptr && abs_inv < 3.0e38f && sp.arrive != nullptr &&
+  // (rows with parameters of their own: the caller has looked at their temperatures; a launch that
+  // shares the compute units with one on another stream may not have all its workgroups resident)
+  const bool inv_ordinary = p.row_cfg ? s->cfg_inv_ordinary : abs_inv < 3.0e38f;
+  const bool fused = !TOPK && (!extras || (ETS_PHASE_CLOCKS && p.probs == nullptr)) && fuse_env != 0 && inv_ordinary && s->beside_rows == 0 && sp.arrive != nullptr &&
                      static_cast<int64_t>(rows) * sp.row_wgs <= (s->num_cus > 0 ? s->num_cus : 0) &&
                      per_wg_slots <= ets::kFusedSlots * ets::kWaves && (!s->wb || rows <= s->wb->arrive_rows);
   bool* dirty = arrive_dirty_flag(s);

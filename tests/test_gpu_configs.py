@@ -56,6 +56,33 @@ def test_mixed_batch_matches_per_row_samplers(oracle, dev, name, rows):
                 assert dbg["position"][b] == ex[b].position
 
 
+@pytest.mark.parametrize("rows,greedy_every", [(16, 0), (64, 0), (24, 3)])
+def test_top_p_rows_with_parameters_of_their_own(oracle, dev, rows, greedy_every):
+    """Only top-p rows (and, in one case, greedy ones between them, so that the drawing rows are reached
+    through the row map): the launch in which the workgroups of a row exchange their maxima and sums
+    inside one kernel reads every row's own temperature and top-p."""
+    w = W.WORKLOADS["cfg2"]
+    cfgs = []
+    for b in range(rows):
+        if greedy_every and b % greedy_every == 1:
+            cfgs.append((0.0, 0.9, 0, 0))
+        else:
+            cfgs.append((0.5 + 0.05 * (b % 9), 0.7 + 0.03 * (b % 8), 0, 0))
+    s = ea.Sampler(w.vocab, 0.33, 0.5, 900, max_batch=rows)
+    states = (np.uint64(900) + np.arange(rows, dtype=np.uint64)).astype(np.uint64)
+    for step in range(2):
+        x = W.logits(w, step, rows)
+        ddbg = torch.zeros((rows, 8), dtype=torch.int32, device=dev)
+        got = s.sample_batch_configs(to_device(x, w.dtype, dev), cfgs, debug_out=ddbg).cpu().numpy()
+        want, ex = oracle_rows(oracle, x, w.dtype, cfgs, 0.33, states)
+        assert np.array_equal(got, want), (rows, step, np.nonzero(got != want)[0])
+        assert np.array_equal(s.get_rng_states(rows), states)
+        dbg = ea.debug_records(ddbg)
+        for b in range(rows):
+            if ex[b].branch == oracle.BRANCH_TOPP:
+                assert f32_bits(dbg["sum"][b]) == f32_bits(ex[b].sum)
+
+
 def test_uniform_configs_equal_the_plain_batch(dev):
     w = W.WORKLOADS["cfg2"]
     rows = 16
