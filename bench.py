@@ -537,6 +537,12 @@ def step_kernels_text(w):
     if not 0.0 < w.topp < 1.0:
         return ("one step = split_pass1_kernel + split_pass2_kernel + split_walk_kernel + split_pass2_kernel + "
                 "split_walk_kernel (multinomial rows, five launches; their summed duration is what the events bracket)")
+    ns = (w.vocab + 511) // 512
+    g = max(1, min(256 // w.batch if w.batch <= 256 else 1, (ns + 15) // 16, 64))
+    fused = os.environ.get("ETS_FUSE", "1") != "0" and w.batch * g <= 256 and -(-ns // g) <= 64
+    if fused:
+        return ("one step = split_pass2_kernel with pass 1 inside (the workgroups of a row exchange maxima and sums "
+                "through memory) + split_finish_kernel (two launches; their summed duration is what the events bracket)")
     return ("one step = split_pass1_kernel + split_pass2_kernel + split_finish_kernel (three launches; "
             "their summed duration is what the events bracket)")
 
