@@ -2437,6 +2437,16 @@ __device__ __noinline__ bool draw_topp_runs(RunArgs a, const char* logits, int V
   return token >= 0;
 }
 
+// split_chain() as a call, for the looping finish kernel: the chain's registers are then the
+// callee's own and do not add to what the loop over the rows keeps alive.  (`fused` points into LDS: a
+// reference into the kernel's argument block would move that block to private memory.)
+template <int DT>
+__device__ __noinline__ float split_chain_call(const SlotRec* recs, const uint2* pairs, int ns, const PrepSlot* prep, uint32_t n_prep,
+                                               const char* logits, int V, float inv, float m, const uint64_t* tab,
+                                               const FusedOps* fused) {
+  return split_chain<DT>(recs, pairs, ns, prep, n_prep, logits, V, inv, m, tab, *fused, nullptr);
+}
+
 // grid = rows; dynamic LDS: the key buffer of the draw (p.row.lds_keys keys), which holds the
 // slot records and the prepared slots while the sum is composed.
 // LOOP: fewer workgroups than rows, a workgroup takes one row after the other (the loop costs
@@ -2473,6 +2483,7 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
   const bool chained = LOOP && R > 1;
   if (chained) {
     if (tid < 32) sm.exp2tab[tid] = kExp2Table[tid];
+    if (tid == 0) fs.fused = p.row.fused;  // (the barrier behind the staging comes before the chains)
     // every row gets an equal share of the key buffer for its records and prepared slots
     const size_t share = lds_bytes / static_cast<size_t>(R) / 16 * 16;
     const uint32_t fit = share > rec_bytes ? static_cast<uint32_t>((share - rec_bytes) / sizeof(PrepSlot)) : 0u;
@@ -2510,10 +2521,9 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
         const float inv_k = p.row.row_cfg ? p.row.row_cfg[row_k].inv_temperature : p.row.inv_temperature;
         const char* logits_k = static_cast<const char*>(p.row.logits) + static_cast<int64_t>(row_k) * p.row.row_stride * ElemSize<DT>::value;
         const char* mine = reinterpret_cast<const char*>(lds_keys) + static_cast<size_t>(wave) * share;
-        sum = split_chain<DT>(reinterpret_cast<const SlotRec*>(mine), reinterpret_cast<const uint2*>(mine + pairs_at), ns,
-                              reinterpret_cast<const PrepSlot*>(mine + rec_bytes),
-                              prepared(st), logits_k, V, inv_k, st.m, sm.exp2tab, p.row.fused,
-                              timers ? timers + static_cast<int64_t>(row_k) * 8 : nullptr);
+        sum = split_chain_call<DT>(reinterpret_cast<const SlotRec*>(mine), reinterpret_cast<const uint2*>(mine + pairs_at), ns,
+                                   reinterpret_cast<const PrepSlot*>(mine + rec_bytes),
+                                   prepared(st), logits_k, V, inv_k, st.m, sm.exp2tab, &fs.fused);
       }
       if (lane == 0) fs.pre_sum[wave] = sum;
     }
@@ -2634,10 +2644,17 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
     if (timers) t1 = wall_clock64();
     if (wave == 0) {
       if (!chained) {
-        const float sum = split_chain<DT>(reinterpret_cast<const SlotRec*>(lds_keys),
-                                          reinterpret_cast<const uint2*>(reinterpret_cast<const char*>(lds_keys) + pairs_at), ns,
-                                          reinterpret_cast<const PrepSlot*>(prep_dst), n_prep, logits, V, inv, m, sm.exp2tab,
-                                          p.row.fused, timers ? timers + static_cast<int64_t>(row) * 8 : nullptr);
+        float sum;
+        if constexpr (LOOP) {  // (fs.fused was stored before the barrier behind the staging)
+          sum = split_chain_call<DT>(reinterpret_cast<const SlotRec*>(lds_keys),
+                                     reinterpret_cast<const uint2*>(reinterpret_cast<const char*>(lds_keys) + pairs_at), ns,
+                                     reinterpret_cast<const PrepSlot*>(prep_dst), n_prep, logits, V, inv, m, sm.exp2tab, &fs.fused);
+        } else {
+          sum = split_chain<DT>(reinterpret_cast<const SlotRec*>(lds_keys),
+                                reinterpret_cast<const uint2*>(reinterpret_cast<const char*>(lds_keys) + pairs_at), ns,
+                                reinterpret_cast<const PrepSlot*>(prep_dst), n_prep, logits, V, inv, m, sm.exp2tab,
+                                p.row.fused, timers ? timers + static_cast<int64_t>(row) * 8 : nullptr);
+        }
         if (lane == 0) sm.bc_sum = sum;
 #if ETS_PHASE_CLOCKS
         if (timers) {  // the same chain once more, its code now in the instruction cache and no clocks inside

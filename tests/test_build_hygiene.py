@@ -37,8 +37,9 @@ def test_hot_kernels_keep_nothing_in_private_memory():
             seen += 1
         if re.search(r"split_finish_kernelILi\d+ELb1E", name):  # (a workgroup takes one row after the other)
             # The loop over the rows costs registers: these instantiations do spill (launches with
-            # more rows than compute units only).  The bound keeps that from growing unnoticed.
-            assert v["ScratchSize"] <= 384 and v["VGPRs Spill"] <= 80, (name, v)
+            # more rows than compute units only).  The bound keeps that from growing unnoticed.  (The
+            # private memory includes the frames of the functions the kernel calls, the chain among them.)
+            assert v["ScratchSize"] <= 448 and v["VGPRs Spill"] <= 56, (name, v)
             seen += 1
     assert seen >= 24
 
