@@ -39,7 +39,7 @@ def test_hot_kernels_keep_nothing_in_private_memory():
             # The loop over the rows costs registers: these instantiations do spill (launches with
             # more rows than compute units only).  The bound keeps that from growing unnoticed.  (The
             # private memory includes the frames of the functions the kernel calls, the chain among them.)
-            assert v["ScratchSize"] <= 448 and v["VGPRs Spill"] <= 56, (name, v)
+            assert v["ScratchSize"] <= 448 and v["VGPRs Spill"] <= 64, (name, v)
             seen += 1
     assert seen >= 24
 
