@@ -83,6 +83,41 @@ def test_top_p_rows_with_parameters_of_their_own(oracle, dev, rows, greedy_every
                 assert f32_bits(dbg["sum"][b]) == f32_bits(ex[b].sum)
 
 
+def test_unchanged_parameters_are_not_uploaded_again_but_changed_ones_are(oracle, dev):
+    """A call whose parameters equal the previous call's reuses the device copy.  That copy is also what a
+    Gumbel-max call with one temperature per row writes to, and a call on another stream reads it: in both
+    cases, and whenever a parameter changes, the rows must still be sampled with their own parameters."""
+    w = W.WORKLOADS["cfg2"]
+    rows = 12
+    cfgs = [(0.5 + 0.1 * (b % 5), 0.8 + 0.02 * (b % 4), 0, 0) for b in range(rows)]
+    s = ea.Sampler(w.vocab, 0.9, 0.5, 4100, max_batch=rows)
+    states = (np.uint64(4100) + np.arange(rows, dtype=np.uint64)).astype(np.uint64)
+    other = torch.cuda.Stream()
+
+    def check(step, c):
+        x = W.logits(w, step, rows)
+        got = s.sample_batch_configs(to_device(x, w.dtype, dev), c).cpu().numpy()
+        want, _ = oracle_rows(oracle, x, w.dtype, c, 0.9, states)
+        assert np.array_equal(got, want), (step, np.nonzero(got != want)[0])
+        assert np.array_equal(s.get_rng_states(rows), states)
+
+    check(0, cfgs)
+    check(1, cfgs)  # (nothing to upload)
+    x = to_device(W.logits(w, 2, rows), w.dtype, dev)
+    s.gumbel_max_batch(x, np.linspace(0.3, 1.4, rows, dtype=np.float32))  # (overwrites the device copy)
+    states[:] = s.get_rng_states(rows)  # (its noise is keyed by the rows' coin states and moves them on)
+    check(2, cfgs)
+    changed = list(cfgs)
+    changed[5] = (0.0, 0.9, 0, 0)  # one row turns greedy: another grouping, other row maps
+    check(3, changed)
+    check(4, cfgs)
+    torch.cuda.synchronize()
+    with torch.cuda.stream(other):
+        check(5, cfgs)  # (the same parameters, on another stream)
+        check(6, changed)
+    torch.cuda.synchronize()
+
+
 def test_uniform_configs_equal_the_plain_batch(dev):
     w = W.WORKLOADS["cfg2"]
     rows = 16
