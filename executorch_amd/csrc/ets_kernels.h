@@ -1008,56 +1008,74 @@ __device__ __forceinline__ void block_sum2(float& x, float& y, BlockScratch& sm,
 // With topk > 0 (n >= topk) the walks are top-k's (sampler.cpp:103-119): the mass of the first topk
 // keys, no threshold.  `p_floor`: entries that are not among the keys may have probabilities up to
 // p_floor; the last key walked must have a larger one for the prefix to be the reference's (else -2).
+// The wave's part of draw_small_wave(): `key` is the lane's candidate key (all ones in lanes from n on).
+// Returns the sorted position (-2: undecided) and, with it, the last index walked, the mass, r and the token.
+__device__ __forceinline__ int small_wave_core(uint64_t key, int n, int n_total, float topp, float coin, int topk, float p_floor,
+                                               int& last_idx_out, float& mass_out, float& r_out, uint32_t& token_out) {
+  int rank = 0;
+  const int lane = threadIdx.x & 63;
+  const uint32_t key_hi = static_cast<uint32_t>(key >> 32), key_lo = static_cast<uint32_t>(key);
+  for (int j = 0; j < n; ++j) {
+    const uint64_t other = (static_cast<uint64_t>(readlane_u32(key_hi, j)) << 32) | readlane_u32(key_lo, j);
+    rank += other < key ? 1 : 0;
+  }
+  if (lane >= n) rank = lane;  // padding stays where it is; ranks of real keys are < n
+  const uint32_t hi = __builtin_amdgcn_ds_permute(rank * 4, static_cast<int>(key >> 32));
+  const uint32_t lo = __builtin_amdgcn_ds_permute(rank * 4, static_cast<int>(static_cast<uint32_t>(key)));
+  const float prob = __uint_as_float(0xffffffffu - hi);  // cand_prob
+  float s = 0.0f;
+  int found = -1;
+  if (topk > 0) {
+    for (int i = 0; i < topk; ++i) s = s + readlane_f32(prob, i);
+    found = topk - 1;
+  } else {
+    for (int i = 0; i < n; ++i) {
+      s = s + readlane_f32(prob, i);
+      if (s > topp) {
+        found = i;
+        break;
+      }
+    }
+  }
+  int pos = -2;
+  if ((found >= 0 || n == n_total) && readlane_f32(prob, found >= 0 ? found : n - 1) > p_floor) {
+    const int last_idx = found >= 0 ? found : n - 1;
+    const float r = coin * s;  // sampler.cpp:162
+    float c = 0.0f;
+    pos = last_idx;
+    for (int i = 0; i <= last_idx; ++i) {
+      c = c + readlane_f32(prob, i);
+      if (c > r) {
+        pos = i;
+        break;
+      }
+    }
+    last_idx_out = last_idx;
+    mass_out = s;
+    r_out = r;
+    token_out = readlane_u32(lo, pos);
+  }
+  return pos;
+}
+
 __device__ int draw_small_wave(LdsKeys lds, int n, int n_total, float topp, float coin, RowDebug& dbg,
                                int32_t& token, BlockScratch& sm, int topk = 0, float p_floor = -1.0f) {
   if (threadIdx.x < 64) {
     const int lane = threadIdx.x;
     const uint64_t key = lane < n ? lds[lane] : ~0ull;
-    int rank = 0;
-    const uint32_t key_hi = static_cast<uint32_t>(key >> 32), key_lo = static_cast<uint32_t>(key);
-    for (int j = 0; j < n; ++j) {
-      const uint64_t other = (static_cast<uint64_t>(readlane_u32(key_hi, j)) << 32) | readlane_u32(key_lo, j);
-      rank += other < key ? 1 : 0;
-    }
-    if (lane >= n) rank = lane;  // padding stays where it is; ranks of real keys are < n
-    const uint32_t hi = __builtin_amdgcn_ds_permute(rank * 4, static_cast<int>(key >> 32));
-    const uint32_t lo = __builtin_amdgcn_ds_permute(rank * 4, static_cast<int>(static_cast<uint32_t>(key)));
-    const float prob = __uint_as_float(0xffffffffu - hi);  // cand_prob
-    float s = 0.0f;
-    int found = -1;
-    if (topk > 0) {
-      for (int i = 0; i < topk; ++i) s = s + readlane_f32(prob, i);
-      found = topk - 1;
-    } else {
-      for (int i = 0; i < n; ++i) {
-        s = s + readlane_f32(prob, i);
-        if (s > topp) {
-          found = i;
-          break;
-        }
-      }
-    }
-    int pos = -2;
-    if ((found >= 0 || n == n_total) && readlane_f32(prob, found >= 0 ? found : n - 1) > p_floor) {
-      const int last_idx = found >= 0 ? found : n - 1;
-      const float r = coin * s;  // sampler.cpp:162
-      float c = 0.0f;
-      pos = last_idx;
-      for (int i = 0; i <= last_idx; ++i) {
-        c = c + readlane_f32(prob, i);
-        if (c > r) {
-          pos = i;
-          break;
-        }
-      }
-      if (lane == 0) {
+    int last_idx = 0;
+    float mass = 0.0f, r = 0.0f;
+    uint32_t tok = 0u;
+    const int pos = small_wave_core(key, n, n_total, topp, coin, topk, p_floor, last_idx, mass, r, tok);
+    if (lane == 0) {
+      if (pos != -2) {
         sm.flag = last_idx;
-        sm.bc_sum = s;
+        sm.bc_sum = mass;
         sm.red_f[1] = r;
-        sm.counter = readlane_u32(lo, pos);
+        sm.counter = tok;
       }
+      sm.bc_found = pos;
     }
-    if (lane == 0) sm.bc_found = pos;
   }
   __syncthreads();
   const int pos = sm.bc_found;

@@ -2695,6 +2695,57 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
     if (timers) t2 = wall_clock64();
   }
 
+  // ---- The usual row of a launch that asks for nothing but tokens -- short lists, a selection of at
+  //      most 64 entries, all of them picked out while the chain ran -- is finished by the first wave
+  //      alone: coin, keys, rank, the two walks and the token in registers, no barrier between them
+  //      (the steps below, for any row, hand every intermediate result round the workgroup through
+  //      LDS: eight barriers).  If the selection turns out not to decide the draw the wave leaves
+  //      everything as it was, coin state included, and the row takes the steps below.
+  if constexpr (!EXTRAS) {
+    const int32_t row_topk = !TOPK ? 0 : (p.row.row_cfg ? p.row.row_cfg[row].topk : p.row.topk);
+    const bool small_tail = !row_nan && p.row.debug == nullptr && !(TOPK && row_topk > 0 && row_topk < V) && lists_ok &&
+                            rs.listed_buckets != 0u && plan.b_sel >= 0 && plan.n_sel >= 1 && plan.n_sel <= 64 &&
+                            fs.sel_count == static_cast<uint32_t>(plan.n_sel) && plan.b_sel < static_cast<int>(rs.listed_buckets);
+    if (small_tail) {
+      if (wave == 0) {
+        uint64_t st = (static_cast<uint64_t>(readlane_u32(static_cast<uint32_t>(coin_state >> 32), 0)) << 32) |
+                      readlane_u32(static_cast<uint32_t>(coin_state), 0);
+        st ^= st >> 12;
+        st ^= st << 25;
+        st ^= st >> 27;
+        const uint32_t u = static_cast<uint32_t>((st * 0x2545F4914F6CDD1Dull) >> 32);
+        const float coin1 = static_cast<float>(u >> 8) / 16777216.0f;
+        const RowDivisor div = row_divisor(S);
+        const int n_sel = plan.n_sel;
+        bool is_in = true;
+        uint64_t key = ~0ull;
+        if (lane < n_sel) {
+          const uint64_t ent = fs.sel[lane];
+          const float pj = div_row(__uint_as_float(static_cast<uint32_t>(ent >> 32)), div);
+          is_in = pj >= cutoff;  // sampler.cpp:137-143
+          key = cand_key(pj, static_cast<int>(static_cast<uint32_t>(ent)));
+        }
+        int pos = -2, last_idx = 0;
+        float mass = 0.0f, r = 0.0f;
+        uint32_t tok = 0u;
+        if (__ballot(!is_in) == 0ull) {
+          // (more candidates exist than the lists hold; entries outside the selection have exps up to the edge of the next bucket)
+          pos = small_wave_core(key, n_sel, 0x7fffffff, topp, coin1, 0, div_row(hist_edge(plan.b_sel + 1), div), last_idx, mass, r, tok);
+        }
+        if (lane == 0) {
+          if (pos != -2) {
+            p.row.rng[row] = st;
+            p.row.tokens[row] = static_cast<int32_t>(tok);
+          }
+          sm.flag = pos != -2 ? 1 : 0;
+        }
+      }
+      __syncthreads();
+      const bool tail_done = sm.flag != 0;
+      __syncthreads();
+      if (tail_done) continue;  // (the next row of the unit, if any)
+    }
+  }
   // ---- one coin per call (sampler.cpp:237, 210-220)
   if (tid == 0) {
     uint64_t st = coin_state;
