@@ -61,14 +61,14 @@ ets_status allow_dynamic_lds(ets_sampler* s, const void* kernel, size_t bytes, s
 // partly filled round would cost more than the longer sweeps), sixteen slots each at least.
 // (ETS_SPLIT_WORKGROUPS forces a number; not for a call that brings its own work buffers, whose
 // layout was made for the automatic choice.)
-int pass2_workgroups(const ets_sampler* s, int32_t rows, int32_t ns) {
+int pass2_workgroups(const ets_sampler* s, int32_t rows, int32_t ns, int32_t beside) {
   static const int forced = [] {
     const char* e = std::getenv("ETS_SPLIT_WORKGROUPS");
     return e ? std::atoi(e) : 0;
   }();
   // (launches that run side by side share the compute units: each takes its share of them, so that
   // the workgroups of both are resident at once)
-  int g = (forced > 0 && !s->wb) ? forced : (s->num_cus > 0 ? s->num_cus : 256) / (rows + s->beside_rows);
+  int g = (forced > 0 && !s->wb) ? forced : (s->num_cus > 0 ? s->num_cus : 256) / (rows + beside);
   const int by_len = (ns + 15) / 16;
   if (g > by_len) g = by_len;
   if (g > ets::kMaxRowWorkgroups) g = ets::kMaxRowWorkgroups;
@@ -93,8 +93,10 @@ ets_status ensure_split(ets_sampler* s) {
   sp.prep_cap = ets::kPrepCap;
   // the candidate lists of the largest launch: rows x workgroups per row x region
   size_t list_entries = 0, row_wgs = 0;
+  // (with nothing beside the launch: a launch of r rows beside b others gets the workgroups per row
+  // of a launch of r + b rows, which this loop covers)
   for (int32_t r = 1; r <= s->max_batch; ++r) {
-    const int g = pass2_workgroups(s, r, sp.ns);
+    const int g = pass2_workgroups(s, r, sp.ns, 0);
     const size_t need = static_cast<size_t>(r) * g * list_region(sp.ns, g);
     if (need > list_entries) list_entries = need;
     if (static_cast<size_t>(r) * g > row_wgs) row_wgs = static_cast<size_t>(r) * g;

@@ -125,7 +125,9 @@ ets_status allow_dynamic_lds(ets_sampler* s, const void* kernel, size_t bytes, s
 // that brings its own).
 ets_status ensure_split(ets_sampler* s);
 ets_status ensure_phist(ets_sampler* s);
-int pass2_workgroups(const ets_sampler* s, int32_t rows, int32_t ns);
+// Workgroups of pass 2 per row for a launch of `rows` rows that shares the compute units with `beside`
+// rows of other launches.  (The work buffers are sized for beside = 0, which covers every other case.)
+int pass2_workgroups(const ets_sampler* s, int32_t rows, int32_t ns, int32_t beside);
 // Whether the arrival counters of the fused launch may hold something other than 0 (a fused launch
 // whose finish kernel was never launched): the handle's own flag, or, for a call that works in the
 // library's static array, that device's.

@@ -52,7 +52,7 @@ ets_status launch_split(ets_sampler* s, const ets::RowParams& p, int32_t rows, h
   sp.row.rows = rows;
   sp.row.ticket = (s->wb ? s->wb->tickets : s->d_tickets) + 3;  // (0 .. 2 are the one-workgroup-per-row kernel's, by draw)
   sp.phist_words = DT == ets::kDtypeBFloat16 ? kPhistWordsBFloat16 : (DT == ets::kDtypeHalf ? kPhistWordsHalf : 0);
-  sp.row_wgs = pass2_workgroups(s, rows, sp.ns);
+  sp.row_wgs = pass2_workgroups(s, rows, sp.ns, s->beside_rows);
   st = check_row_wgs(s, sp.row_wgs);
   if (st != ETS_OK) return st;
   sp.list_region = list_region(sp.ns, sp.row_wgs);
@@ -169,7 +169,7 @@ ets_status launch_split_walk(ets_sampler* s, const ets::RowParams& p, int32_t ro
   sp.row.rows = rows;
   sp.phist_words = 0;
   sp.short_lists = 0;
-  sp.row_wgs = pass2_workgroups(s, rows, sp.ns);
+  sp.row_wgs = pass2_workgroups(s, rows, sp.ns, s->beside_rows);
   st = check_row_wgs(s, sp.row_wgs);
   if (st != ETS_OK) return st;
   sp.list_region = 0;

@@ -118,6 +118,28 @@ def test_unchanged_parameters_are_not_uploaded_again_but_changed_ones_are(oracle
     torch.cuda.synchronize()
 
 
+def test_work_buffers_do_not_depend_on_the_first_call(oracle, dev):
+    """The work buffers of the several-workgroups-per-row path are allocated by the first call that needs
+    them.  When that call runs two groups of rows side by side, each group gets fewer workgroups per row
+    than it would alone; the buffers must still be sized for any later call (and for the second group of
+    the same call, which runs beside fewer rows than the first).  A vocabulary large enough for the number
+    of workgroups per row to depend on the number of rows (more than 16 x 32 slots)."""
+    vocab, rows = 290000, 8
+    rng = np.random.default_rng(77)
+    x = (rng.standard_normal((rows, vocab)) * 2.0).astype(np.float32)
+    s = ea.Sampler(vocab, 0.8, 0.9, 321, max_batch=rows)
+    states = (np.uint64(321) + np.arange(rows, dtype=np.uint64)).astype(np.uint64)
+    dx = to_device(W.to_storage(x, W.DTYPE_BFLOAT16), W.DTYPE_BFLOAT16, dev)
+    xs = W.to_storage(x, W.DTYPE_BFLOAT16)
+    mixed = [(1.0, 1.0, 0, 0)] * 3 + [(0.7, 0.9, 0, 0)] * 5  # three multinomial rows beside five top-p rows
+    alone = [(0.7, 0.9, 0, 0)] * rows
+    for cfgs in (mixed, alone, mixed):
+        got = s.sample_batch_configs(dx, cfgs).cpu().numpy()
+        want, _ = oracle_rows(oracle, xs, W.DTYPE_BFLOAT16, cfgs, 0.8, states)
+        assert np.array_equal(got, want), (np.nonzero(got != want)[0], got, want)
+        assert np.array_equal(s.get_rng_states(rows), states)
+
+
 def test_uniform_configs_equal_the_plain_batch(dev):
     w = W.WORKLOADS["cfg2"]
     rows = 16
