@@ -84,6 +84,9 @@ def run(cases=2000, seed=1, max_vocab=300000, configs=False):
         dtype = int(rng.choice(dtypes))
         kind = str(rng.choice(kinds))
         rows = int(rng.integers(1, 9 if args.configs else 5))
+        if args.configs and rng.random() < 0.05:
+            # now and then enough rows for the groups of a call to share the compute units unevenly
+            rows = int(rng.integers(9, 41))
         temperature = float(rng.choice([0.05, 0.3, 0.6, 0.8, 1.0, 1.5, 7.0, 50.0, -1.0, 0.0]))
         topp = float(rng.choice([0.0, 0.02, 0.5, 0.8, 0.9, 0.95, 0.999, 1.0]))
         topk = int(rng.choice([0, 0, 0, 1, 2, 40, 64, 65, 256, 257, 1000, vocab - 1, vocab, vocab + 5]))
