@@ -109,8 +109,10 @@ ETS_API ets_status ets_sampler_set_topp(ets_sampler* s, float topp);
  *                       vocabulary size;
  *   ETS_ROW_SPLIT_OFF   always one workgroup per row.
  * Several workgroups per row, by draw: top-p rows three launches (two when every workgroup of
- * the launch is resident at once, about batch x workgroups-per-row <= compute units, and the
- * launch has one finite temperature and no debug output: the first two are then one kernel);
+ * the launch is resident at once, about batch x workgroups-per-row <= compute units, every
+ * temperature of the launch is finite, no probabilities are asked for and no other launch of
+ * the call runs beside it: the first two are then one kernel, whose workgroups hand each
+ * other their results with bounded waits);
  * top-k rows with k <= ceil(vocab / 512) the same three launches, larger k one workgroup per row;
  * multinomial rows (top_p <= 0 or >= 1) FIVE launches, or one workgroup per row when the
  * probabilities are asked for.  All launches of a call go to the call's stream, in order.
