@@ -72,7 +72,7 @@ ets_status launch_split(ets_sampler* s, const ets::RowParams& p, int32_t rows, h
   const char* const fuse_text = std::getenv("ETS_FUSE");
   const int fuse_env = fuse_text ? std::atoi(fuse_text) : 1;
   const char* const spin_text = std::getenv("ETS_FUSE_SPIN_LIMIT");
-  const int spin_env = spin_text ? std::atoi(spin_text) : (1 << 16);
+  const int spin_env = spin_text ? std::atoi(spin_text) : (1 << 13);  // (about ten milliseconds; the usual wait is a few polls)
   const int per_wg_slots = ((sp.ns + sp.row_wgs - 1) / sp.row_wgs + ets::kWaves - 1) / ets::kWaves * ets::kWaves;
   const float abs_inv = p.inv_temperature < 0.0f ? -p.inv_temperature : p.inv_temperature;
   // (rows with parameters of their own: the caller has looked at their temperatures; a launch that
