@@ -117,6 +117,7 @@ ets_status ensure_split(ets_sampler* s) {
   const size_t o_count = take(rows * ets::kMaxRowWorkgroups * sizeof(uint32_t));
   const size_t o_arrive = take(rows * 2 * sizeof(uint32_t));
   const size_t o_part = take(rows * ets::kMaxRowWorkgroups * sizeof(float));
+  const size_t o_pack = take(rows * sp.ns_stride * sizeof(float4));
   const size_t o_timers = take(rows * 12 * sizeof(uint64_t));
   const size_t o_hist = take(row_wgs * ets::kHistBuckets * sizeof(uint32_t));
   const size_t o_list = take(list_entries * sizeof(uint64_t));
@@ -125,6 +126,7 @@ ets_status ensure_split(ets_sampler* s) {
   ETS_HIP(s, hipMemset(base + o_arrive, 0, rows * 2 * sizeof(uint32_t)));  // (0 between launches)
   sp.arrive = reinterpret_cast<uint32_t*>(base + o_arrive);
   sp.part_max = reinterpret_cast<float*>(base + o_part);
+  sp.slot_pack = reinterpret_cast<float4*>(base + o_pack);
   sp.slot_max = reinterpret_cast<float*>(base + o_max);
   sp.slot_max2 = reinterpret_cast<float*>(base + o_max2);
   sp.slot_sum = reinterpret_cast<float*>(base + o_sum);
@@ -437,6 +439,7 @@ size_t layout_static(const ets_sampler* s, int32_t dtype, int32_t rows, char* ba
   sp.walk = reinterpret_cast<float2*>(take(r * sizeof(float2)));
   sp.list_count = reinterpret_cast<uint32_t*>(take(r * ets::kMaxRowWorkgroups * sizeof(uint32_t)));
   sp.part_max = reinterpret_cast<float*>(take(r * ets::kMaxRowWorkgroups * sizeof(float)));
+  sp.slot_pack = reinterpret_cast<float4*>(take(r * sp.ns_stride * sizeof(float4)));
   sp.hist = reinterpret_cast<uint32_t*>(take(r * g * ets::kHistBuckets * sizeof(uint32_t)));
   sp.phist = reinterpret_cast<uint32_t*>(take(r * g * phist_words * sizeof(uint32_t)));
   sp.list = reinterpret_cast<uint64_t*>(take(r * g * list_region(sp.ns, g) * sizeof(uint64_t)));

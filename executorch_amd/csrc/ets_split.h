@@ -138,6 +138,7 @@ struct SplitParams {
   float* slot_max;      // [rows, ns_stride] largest x = logit * inv_temperature of the slot (NaN: the slot holds one)
   float* slot_max2;     // [rows, ns_stride] largest x among the other 63 lanes' entries
   float* slot_sum;      // [rows, ns_stride] sum of exp(x - slot_max), approximate
+  float4* slot_pack;    // [rows, ns_stride] (slot_max, slot_max2, slot_sum, -) of a launch with pass 1 inside pass 2
   SlotRec* slot_rec;    // [rows, ns_stride]
   PrepSlot* prep;       // [rows, prep_cap]
   RowState* row_state;  // [rows]
@@ -229,6 +230,19 @@ __device__ __forceinline__ void coherent_store(float* ptr, float v) {
 __device__ __forceinline__ float coherent_load(const float* ptr) {
   return __uint_as_float(__hip_atomic_load(reinterpret_cast<const uint32_t*>(ptr), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
 }
+// The same for a slot's three values at once: one 16-byte request through to memory instead of three
+// of four bytes (every such store is charged a partial line behind L2).  The compiler does not count
+// these accesses: the load waits for its own result, the stores are waited for where the others are.
+typedef float ets_f32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void coherent_store4(float4* ptr, float a, float b, float c) {
+  const ets_f32x4 v = {a, b, c, 0.0f};
+  asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(ptr), "v"(v) : "memory");
+}
+__device__ __forceinline__ ets_f32x4 coherent_load4(const float4* ptr) {
+  ets_f32x4 v;
+  asm volatile("global_load_dwordx4 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=v"(v) : "v"(ptr) : "memory");
+  return v;
+}
 struct SlotMax {
   float M, M2;  // the slot's largest x = logit * inv_temperature (NaN entries ignored), and the largest of the other 63 lanes
 };
@@ -284,9 +298,7 @@ __device__ __forceinline__ void split_pass1_sum(const SplitParams& p, int row, i
   if (lane == 0) {
     const int64_t at = static_cast<int64_t>(row) * p.ns_stride + s;
     if (COHERENT) {
-      coherent_store(p.slot_max + at, any_nan ? __uint_as_float(0x7fc00000u) : M);
-      coherent_store(p.slot_max2 + at, x.M2);
-      coherent_store(p.slot_sum + at, sum);
+      coherent_store4(p.slot_pack + at, any_nan ? __uint_as_float(0x7fc00000u) : M, x.M2, sum);
     } else {
       p.slot_max[at] = any_nan ? __uint_as_float(0x7fc00000u) : M;
       p.slot_max2[at] = x.M2;
@@ -615,6 +627,7 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
   const float* slot_max = p.slot_max + static_cast<int64_t>(row) * p.ns_stride;
   const float* slot_sum = p.slot_sum + static_cast<int64_t>(row) * p.ns_stride;
   const float* slot_max2 = p.slot_max2 + static_cast<int64_t>(row) * p.ns_stride;
+  const float4* slot_pack = p.slot_pack + static_cast<int64_t>(row) * p.ns_stride;  // (FUSED)
   const float kInf = __uint_as_float(0x7f800000u);
   const float fill = inv < 0.0f ? kInf : -kInf;
   uint64_t c0 = 0, c1 = 0, c2 = 0, c3 = 0, cf0 = 0, cf1 = 0, cf2 = 0;
@@ -720,7 +733,7 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
     if (on_my_own) {
       alone();
       m_early = kNegInf;
-      for (int s = lane; s < ns; s += 64) m_early = __builtin_fmaxf(m_early, coherent_load(slot_max + s));  // (ignores NaN)
+      for (int s = lane; s < ns; s += 64) m_early = __builtin_fmaxf(m_early, coherent_load4(slot_pack + s).x);  // (ignores NaN)
       m_early = wave_max_ignoring_nan(m_early);
     } else {
       m_early = lane < n_parts ? coherent_load(part_max + lane) : kNegInf;
@@ -746,13 +759,26 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
   bool any_nan = false;
   float first_max = 0.0f, first_sum = 0.0f, first_max2 = -kInf;  // the scan below starts with the same slots
   // (FUSED: other workgroups of this launch stored these)
-  auto slot_value = [&](const float* a, int s) { return FUSED ? coherent_load(a + s) : a[s]; };
+  // a slot's maximum, second maximum and sum
+  auto slot_values = [&](int s, float& mx, float& mx2, float& sum) {
+    if constexpr (FUSED) {
+      const ets_f32x4 v = coherent_load4(slot_pack + s);
+      mx = v.x;
+      mx2 = v.y;
+      sum = v.z;
+    } else {
+      mx = slot_max[s];
+      sum = slot_sum[s];
+      mx2 = TOPP ? slot_max2[s] : -kInf;
+    }
+  };
   for (int s = tid; s < ns; s += kBlock) {
-    const float v = slot_value(slot_max, s);
+    float v, v2, vs;
+    slot_values(s, v, v2, vs);
     if (s == tid) {
       first_max = v;
-      first_sum = slot_value(slot_sum, s);
-      if (TOPP) first_max2 = slot_value(slot_max2, s);
+      first_sum = vs;
+      first_max2 = v2;
     }
     any_nan = any_nan || (v != v);
     m = __builtin_fmaxf(m, v);
@@ -797,8 +823,8 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
     const int s = base + tid;
     float a = 0.0f;
     if (s < ns) {
-      const float sum = base == 0 ? first_sum : slot_value(slot_sum, s);
-      const float smax = base == 0 ? first_max : slot_value(slot_max, s);
+      float sum = first_sum, smax = first_max, smax2_in = first_max2;
+      if (base != 0) slot_values(s, smax, smax2_in, sum);
       const float f = sum > 0.0f ? fast_exp2((smax - m) * kLog2e) : 0.0f;  // exp of the slot's largest entry
       a = sum > 0.0f ? sum * f : 0.0f;
       if (WALK) a *= walk_scale;
@@ -806,7 +832,7 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
       if (TOPP && f > 0.0f) {
         // lower bounds of the exact exps of the slot's two largest entries, into the bins of their
         // binades (integers: every workgroup of the row arrives at the same totals)
-        const float smax2 = base == 0 ? first_max2 : slot_value(slot_max2, s);
+        const float smax2 = smax2_in;
         const float f2 = smax2 > -kInf ? fast_exp2((smax2 - m) * kLog2e) : 0.0f;
         const float below[2] = {f * 0.9999f, f2 * 0.9999f};
 #pragma unroll
