@@ -563,9 +563,10 @@ constexpr int kLutCountWords = 12288;  // a table entry's counter sits 48 KiB ab
 // Returns false (no table; the caller evaluates expf per entry) when inv or max are not positive
 // finite in the way the bounds need, or when the table would not fit in `cap` floats.
 // COUNTERS = false builds the table alone (`cap` then only has to hold its 2 * half floats).
+// The threads from `first_thread` on share the entries; the ones before it only learn where the table lies.
 template <bool COUNTERS = true>
 __device__ bool build_exp_lut(float* lut, int cap, float inv, float m, const uint64_t* tab, int& base1, int& top,
-                              int& half) {
+                              int& half, int first_thread = 0) {
   const float kInf = __uint_as_float(0x7f800000u);
   if (!(inv > 0.0f && inv < kInf && m > -kInf && m < kInf)) return false;
   const uint32_t ib = __float_as_uint(inv);
@@ -588,7 +589,8 @@ __device__ bool build_exp_lut(float* lut, int cap, float inv, float m, const uin
   top = R + 1;
   base1 = (e_lo << 7) - 1;
   if (2 * half > kLutCountWords || (COUNTERS ? kLutCountWords + 2 * half : 2 * half) > cap) return false;
-  for (int idx = threadIdx.x; idx < 2 * half; idx += kBlock) {
+  const int idx0 = static_cast<int>(threadIdx.x) - first_thread;
+  for (int idx = idx0 < 0 ? 2 * half : idx0; idx < 2 * half; idx += kBlock - first_thread) {
     const int sgn = idx >= half ? 1 : 0;
     const int c = idx - sgn * half;
     float e;

@@ -243,6 +243,16 @@ __device__ __forceinline__ ets_f32x4 coherent_load4(const float4* ptr) {
   asm volatile("global_load_dwordx4 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=v"(v) : "v"(ptr) : "memory");
   return v;
 }
+// Four of them requested together (one trip to memory for a wave that reads four slots per lane).
+__device__ __forceinline__ void coherent_load4x4(const float4* p0, const float4* p1, const float4* p2, const float4* p3,
+                                                 ets_f32x4& v0, ets_f32x4& v1, ets_f32x4& v2, ets_f32x4& v3) {
+  asm volatile(
+      "global_load_dwordx4 %0, %4, off sc1\n\tglobal_load_dwordx4 %1, %5, off sc1\n\t"
+      "global_load_dwordx4 %2, %6, off sc1\n\tglobal_load_dwordx4 %3, %7, off sc1\n\ts_waitcnt vmcnt(0)"
+      : "=&v"(v0), "=&v"(v1), "=&v"(v2), "=&v"(v3)
+      : "v"(p0), "v"(p1), "v"(p2), "v"(p3)
+      : "memory");
+}
 struct SlotMax {
   float M, M2;  // the slot's largest x = logit * inv_temperature (NaN entries ignored), and the largest of the other 63 lanes
 };
@@ -363,6 +373,9 @@ struct Pass2Shared {
   uint32_t list_count;        // candidates this workgroup has listed
   uint32_t top_mass[32];      // the slots' two largest exps, added up per binade (bin j: [2^-j, 2^(1-j))), in units of 2^-20
   uint32_t top_all[32];       // the whole mass of the slots, by the binade of their largest exp, in units of 2^-10 (rounded up)
+  // what the first wave worked out on its own (FUSED): row maximum, approximate total, serial slots, NaN row, done
+  float pro_m, pro_total;
+  uint32_t pro_serial, pro_nan, pro_done;
 };
 
 // One wave, one slot: e[] are the lane's 8 entries; `cls` is the slot's entry of Pass2Shared::cls.
@@ -659,6 +672,18 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
   int early_lut = -1;      // FUSED: the expf table was built for early_m already (1: usable, 0: not)
   float early_m = 0.0f;
   float held0[8], held1[8], held2[8], held3[8];  // FUSED: the wave's slots, read once (named one by one: they stay in registers)
+  bool pro_early = false;  // FUSED: the first wave does the row-level work on its own while the others build the table
+  // (FUSED) Given up on the others: their slots from the logits (whoever stores a slot's three values stores the same bits).
+  auto alone = [&]() {
+    for (int s = wave; s < ns; s += kWaves) {
+      if (s >= s_begin && s < s_end) continue;
+      float v[8];
+      load_slot_lane<DT>(logits, s, lane, V, fill, v, p.row.fused);
+      split_pass1_slot<true>(p, row, s, v, inv);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+  };
   if constexpr (FUSED) {
     if (s_mine < s_end) load_slot_lane<DT>(logits, s_mine, lane, V, fill, held0, p.row.fused);
     if (s_mine + kWaves < s_end) load_slot_lane<DT>(logits, s_mine + kWaves, lane, V, fill, held1, p.row.fused);
@@ -716,17 +741,6 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
       __syncthreads();
       return met;
     };
-    // Given up on the others: their slots from the logits (whoever stores a slot's three values stores the same bits).
-    auto alone = [&]() {
-      for (int s = wave; s < ns; s += kWaves) {
-        if (s >= s_begin && s < s_end) continue;
-        float v[8];
-        load_slot_lane<DT>(logits, s, lane, V, fill, v, p.row.fused);
-        split_pass1_slot<true>(p, row, s, v, inv);
-      }
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      __syncthreads();
-    };
     bool on_my_own = !all_there(arrive_max);
     if (timers) cf1 = wall_clock64();
     float m_early;
@@ -743,68 +757,25 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
       const float x_first = load_logit<DT>(logits, 0, p.row.fused) * inv;
       if (x_first != x_first) m_early = x_first;
     }
+    early_m = m_early;
+    pro_early = !on_my_own;
     if constexpr (DT == kDtypeBFloat16) {
-      if (m_early > kNegInf && m_early < kInf)
+      if (!pro_early && m_early > kNegInf && m_early < kInf)
         early_lut = build_exp_lut<false>(lut_mem, kLutCountWords, inv, m_early, sm.exp2tab, lut_base1, lut_top, lut_half) ? 1 : 0;
-      early_m = m_early;
     }
-    if (!on_my_own && !all_there(arrive_sum)) alone();
-    if (timers) cf2 = wall_clock64();
+    if (on_my_own && timers) cf2 = wall_clock64();
   } else {
     if (s_mine < s_end) load_slot_lane<DT>(logits, s_mine, lane, V, fill, l, p.row.fused);
   }
 
-  // ---- row maximum (sampler.cpp:191-197) from the slots' maxima
-  float m = -kInf;
-  bool any_nan = false;
-  float first_max = 0.0f, first_sum = 0.0f, first_max2 = -kInf;  // the scan below starts with the same slots
-  // (FUSED: other workgroups of this launch stored these)
-  // a slot's maximum, second maximum and sum
-  auto slot_values = [&](int s, float& mx, float& mx2, float& sum) {
-    if constexpr (FUSED) {
-      const ets_f32x4 v = coherent_load4(slot_pack + s);
-      mx = v.x;
-      mx2 = v.y;
-      sum = v.z;
-    } else {
-      mx = slot_max[s];
-      sum = slot_sum[s];
-      mx2 = TOPP ? slot_max2[s] : -kInf;
-    }
-  };
-  for (int s = tid; s < ns; s += kBlock) {
-    float v, v2, vs;
-    slot_values(s, v, v2, vs);
-    if (s == tid) {
-      first_max = v;
-      first_sum = vs;
-      first_max2 = v2;
-    }
-    any_nan = any_nan || (v != v);
-    m = __builtin_fmaxf(m, v);
-  }
-  m = wave_max_ignoring_nan(m);
-  const uint64_t nan_ballot = __ballot(any_nan);
-  if (lane == 0) {
-    sm.red_f[wave] = m;
-    sm.red_u[wave] = nan_ballot ? 1u : 0u;
-  }
-  __syncthreads();
-  m = sm.red_f[0];
-  uint32_t nan_any = sm.red_u[0];
-  for (int w = 1; w < kWaves; ++w) {
-    m = (sm.red_f[w] > m) ? sm.red_f[w] : m;
-    nan_any |= sm.red_u[w];
-  }
-  const float x0 = load_logit<DT>(logits, 0, p.row.fused) * inv;
-  if (x0 != x0) m = x0;  // max_val starts at x[0]; nothing compares greater than NaN
-  const bool row_nan = nan_any != 0u || !(m > -kInf && m < kInf);
-  if (row_nan) {  // one NaN addend poisons the sum: the finish kernel needs nothing else
-    if (part == 0 && tid == 0) p.row_state[row] = {0u, m, 1u, 0.0f, 0, 0, 0, 0u};
-    return;
-  }
-  __syncthreads();
-  if (timers) c1 = wall_clock64();
+  // ---- The row-level work of every workgroup of the row: the row maximum from the slots' maxima
+  //      (sampler.cpp:191-197), the approximate running sums in front of every slot and, from them,
+  //      the binades the sequential sum can be in at the two ends of each slot.  A slot that cannot be
+  //      placed inside one binade (or one of two neighbours) is resolved in order by the finish kernel
+  //      and gets a prepared-slot index.  Two forms of it, the same arithmetic in the same order (all
+  //      workgroups of a row must arrive at the same classes and indices, whichever form each takes):
+  //      by the whole workgroup, a slot per lane; and (FUSED) by the first wave alone, sixty-four
+  //      slots at a time, with no barrier, while the other waves build the expf table.
   RowDivisor walk_div = {};
   float walk_scale = 1.0f;
   if (WALK) {
@@ -812,53 +783,33 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
     walk_div = row_divisor(S);
     walk_scale = 1.0f / S;  // (the approximate sums only place the running sum in a binade)
   }
-
-  // ---- approximate running sums in front of every slot; from them, the binades the sequential
-  //      sum can be in at the two ends of each slot.  A slot that cannot be placed inside one
-  //      binade (or one of two neighbours) is resolved in order by the finish kernel and gets a
-  //      prepared-slot index.
-  float carry = 0.0f;
-  uint32_t serial_before = 0u;
-  for (int base = 0; base < ns; base += kBlock) {
-    const int s = base + tid;
-    float a = 0.0f;
-    if (s < ns) {
-      float sum = first_sum, smax = first_max, smax2_in = first_max2;
-      if (base != 0) slot_values(s, smax, smax2_in, sum);
-      const float f = sum > 0.0f ? fast_exp2((smax - m) * kLog2e) : 0.0f;  // exp of the slot's largest entry
-      a = sum > 0.0f ? sum * f : 0.0f;
-      if (WALK) a *= walk_scale;
-      if (TOPP) sh.top[s] = f * 1.0001f;  // (the hardware's exp2 is within 1e-5 of the exact exp)
-      if (TOPP && f > 0.0f) {
-        // lower bounds of the exact exps of the slot's two largest entries, into the bins of their
-        // binades (integers: every workgroup of the row arrives at the same totals)
-        const float smax2 = smax2_in;
-        const float f2 = smax2 > -kInf ? fast_exp2((smax2 - m) * kLog2e) : 0.0f;
-        const float below[2] = {f * 0.9999f, f2 * 0.9999f};
+  // a slot's approximate mass in units of exp(-m); notes the bound of its largest exp and, for top-p
+  // rows, lower bounds of its two largest exps by binade
+  auto slot_mass = [&](int s, float sum, float smax, float smax2, float m_row) -> float {
+    const float f = sum > 0.0f ? fast_exp2((smax - m_row) * kLog2e) : 0.0f;  // exp of the slot's largest entry
+    float a = sum > 0.0f ? sum * f : 0.0f;
+    if (WALK) a *= walk_scale;
+    if (TOPP) sh.top[s] = f * 1.0001f;  // (the hardware's exp2 is within 1e-5 of the exact exp)
+    if (TOPP && f > 0.0f) {
+      // lower bounds of the exact exps of the slot's two largest entries, into the bins of their
+      // binades (integers: every workgroup of the row arrives at the same totals)
+      const float f2 = smax2 > -kInf ? fast_exp2((smax2 - m_row) * kLog2e) : 0.0f;
+      const float below[2] = {f * 0.9999f, f2 * 0.9999f};
 #pragma unroll
-        for (int q = 0; q < 2; ++q) {
-          const int j = 127 - static_cast<int>(__float_as_uint(below[q]) >> 23);
-          if (below[q] > 0.0f && j >= 0 && j < 32) atomicAdd(&sh.top_mass[j], static_cast<uint32_t>(below[q] * 1048576.0f));
-          // a top-k row counts them by histogram bucket (the histogram is not in use yet)
-          if (row_topk && below[q] > 0.0f) atomicAdd(&sh.hist[hist_bucket(__float_as_uint(below[q]))], 1u);
-        }
-        // the slot's whole mass (at most 512), rounded up: what bounds how many of its entries reach a cut
-        const int j0 = 127 - static_cast<int>(__float_as_uint(below[0]) >> 23);
-        if (j0 >= 0 && j0 < 32) atomicAdd(&sh.top_all[j0], static_cast<uint32_t>(a * 1024.0f) + 1u);
+      for (int q = 0; q < 2; ++q) {
+        const int j = 127 - static_cast<int>(__float_as_uint(below[q]) >> 23);
+        if (below[q] > 0.0f && j >= 0 && j < 32) atomicAdd(&sh.top_mass[j], static_cast<uint32_t>(below[q] * 1048576.0f));
+        // a top-k row counts them by histogram bucket (the histogram is not in use yet)
+        if (row_topk && below[q] > 0.0f) atomicAdd(&sh.hist[hist_bucket(__float_as_uint(below[q]))], 1u);
       }
+      // the slot's whole mass (at most 512), rounded up: what bounds how many of its entries reach a cut
+      const int j0 = 127 - static_cast<int>(__float_as_uint(below[0]) >> 23);
+      if (j0 >= 0 && j0 < 32) atomicAdd(&sh.top_all[j0], static_cast<uint32_t>(a * 1024.0f) + 1u);
     }
-    const float incl = wave_scan_inclusive_f32(a, lane);
-    if (lane == 63) sm.group_total[0][wave] = incl;
-    __syncthreads();
-    float before = carry, all = carry;
-    for (int w = 0; w < kWaves; ++w) {
-      if (w == wave) before = all;
-      all += sm.group_total[0][w];
-    }
-    const float a_out = before + incl;
-    const float a_in = before + lane_before_f32(incl);
-    if (s < ns) sh.upto[s + 1] = a_out;
-    carry = all;
+    return a;
+  };
+  // the class of slot s from the approximate sums at its two ends: kb_lo | kb_hi << 8 | kind << 16 | bit 30
+  auto slot_class = [&](int s, float a_in, float a_out) -> uint32_t {
     const float lo = a_in * (1.0f - split_eps(s * kSlot));
     const float hi = a_out * (1.0f + split_eps((s + 1) * kSlot));
     const uint32_t kb_lo = __float_as_uint(lo > 0.0f ? lo : 0.0f) >> 23, kb_hi = __float_as_uint(hi) >> 23;
@@ -872,23 +823,196 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
         kind = kSlotDual;
       }
     }
-    const bool serial = s < ns && s > 0 && kind == kSlotSerial;  // (slot 0 is worked out in this kernel)
-    const uint64_t serial_ballot = __ballot(serial);
-    if (lane == 0) sm.red_u[wave] = static_cast<uint32_t>(__popcll(serial_ballot));
-    __syncthreads();
-    uint32_t rank = serial_before;
-    uint32_t chunk_total = 0u;
-    for (int w = 0; w < kWaves; ++w) {
-      if (w < wave) rank += sm.red_u[w];
-      chunk_total += sm.red_u[w];
-    }
-    rank += static_cast<uint32_t>(__popcll(serial_ballot & ((1ull << lane) - 1ull)));
     // (bit 30: the approximate sum in front of the slot lies in the upper of the two binades)
     const uint32_t in_hi = (__float_as_uint(a_in) >> 23) > kb_lo ? 1u << 30 : 0u;
-    if (s < ns) sh.cls[s] = (kb_lo & 255u) | ((kb_hi > 255u ? 255u : kb_hi) << 8) | (kind << 16) | ((rank & 0x7ffu) << 19) | in_hi;
-    serial_before += chunk_total;
+    return (kb_lo & 255u) | ((kb_hi > 255u ? 255u : kb_hi) << 8) | (kind << 16) | in_hi;
+  };
+
+  float m = -kInf;
+  float a_total = 0.0f;
+  uint32_t serial_before = 0u;
+  bool row_nan = false;
+  bool pro_done = false;
+  if constexpr (FUSED) {
+    if (pro_early) {
+      if (wave == 0) {
+        // (the second hand-over: every slot's maximum and sum; lane 0 polls, a bounded number of times)
+        int met = 0;
+        if (lane == 0) {
+          for (int spin = 0; spin < p.spin_limit; ++spin) {
+            if (__hip_atomic_load(p.arrive + 2 * lrow + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= static_cast<uint32_t>(n_parts)) {
+              met = 1;
+              break;
+            }
+            __builtin_amdgcn_s_sleep(2);
+          }
+        }
+        met = __builtin_amdgcn_readfirstlane(met);
+        if (met) {
+          // the slots' values, parked in LDS where the results will go (four slots of a lane per trip to memory)
+          float mm = -kInf;
+          bool nanf = false;
+          for (int base = 0; base < ns; base += 256) {
+            ets_f32x4 v[4];
+            const int s0 = base + lane;
+            coherent_load4x4(slot_pack + min(s0, ns - 1), slot_pack + min(s0 + 64, ns - 1), slot_pack + min(s0 + 128, ns - 1),
+                             slot_pack + min(s0 + 192, ns - 1), v[0], v[1], v[2], v[3]);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+              const int s = s0 + 64 * k;
+              if (s < ns) {
+                sh.top[s] = v[k].x;
+                sh.cls[s] = __float_as_uint(v[k].y);
+                sh.upto[s + 1] = v[k].z;
+                nanf = nanf || (v[k].x != v[k].x);
+                mm = __builtin_fmaxf(mm, v[k].x);
+              }
+            }
+          }
+          mm = wave_max_ignoring_nan(mm);
+          const bool nan_any = __ballot(nanf) != 0ull;
+          const float x0 = load_logit<DT>(logits, 0, p.row.fused) * inv;
+          if (x0 != x0) mm = x0;  // max_val starts at x[0]; nothing compares greater than NaN
+          const bool nan_row = nan_any || !(mm > -kInf && mm < kInf);
+          float run = 0.0f;
+          uint32_t serials = 0u;
+          if (!nan_row) {
+            for (int c0 = 0; c0 < ns; c0 += 64) {
+              const int s = c0 + lane;
+              float a = 0.0f;
+              if (s < ns) a = slot_mass(s, sh.upto[s + 1], sh.top[s], __uint_as_float(sh.cls[s]), mm);
+              const float incl = wave_scan_inclusive_f32(a, lane);
+              const float before = run;
+              run = run + readlane_f32(incl, 63);
+              const float a_out = before + incl;
+              const float a_in = before + lane_before_f32(incl);
+              const uint32_t cls = slot_class(s, a_in, a_out);
+              const bool serial = s < ns && s > 0 && ((cls >> 16) & 7u) == kSlotSerial;  // (slot 0 is worked out in this kernel)
+              const uint64_t serial_ballot = __ballot(serial);
+              const uint32_t rank = serials + static_cast<uint32_t>(__popcll(serial_ballot & ((1ull << lane) - 1ull)));
+              if (s < ns) {
+                sh.upto[s + 1] = a_out;
+                sh.cls[s] = cls | ((rank & 0x7ffu) << 19);
+              }
+              serials += static_cast<uint32_t>(__popcll(serial_ballot));
+            }
+          }
+          if (lane == 0) {
+            sh.pro_m = mm;
+            sh.pro_total = run;
+            sh.pro_serial = serials;
+            sh.pro_nan = nan_row ? 1u : 0u;
+          }
+        }
+        if (lane == 0) sh.pro_done = met ? 1u : 0u;
+      }
+      if constexpr (DT == kDtypeBFloat16) {
+        // (the table's entries are dealt to the other waves; the first one only works out where it lies)
+        if (early_m > -kInf && early_m < kInf)
+          early_lut = build_exp_lut<false>(lut_mem, kLutCountWords, inv, early_m, sm.exp2tab, lut_base1, lut_top, lut_half, 64) ? 1 : 0;
+      }
+      __syncthreads();
+      pro_done = sh.pro_done != 0u;
+      if (pro_done) {
+        m = sh.pro_m;
+        a_total = sh.pro_total;
+        serial_before = sh.pro_serial;
+        row_nan = sh.pro_nan != 0u;
+      } else {
+        alone();  // (given up on the others' sums: their slots from the logits, then the form below)
+      }
+      if (timers) cf2 = wall_clock64();
+    }
   }
-  const float a_total = carry;
+  float first_max = 0.0f, first_sum = 0.0f, first_max2 = -kInf;  // the scan below starts with the same slots
+  // (FUSED: other workgroups of this launch stored these) a slot's maximum, second maximum and sum
+  auto slot_values = [&](int s, float& mx, float& mx2, float& sum) {
+    if constexpr (FUSED) {
+      const ets_f32x4 v = coherent_load4(slot_pack + s);
+      mx = v.x;
+      mx2 = v.y;
+      sum = v.z;
+    } else {
+      mx = slot_max[s];
+      sum = slot_sum[s];
+      mx2 = TOPP ? slot_max2[s] : -kInf;
+    }
+  };
+  if (!pro_done) {
+    bool any_nan = false;
+    for (int s = tid; s < ns; s += kBlock) {
+      float v, v2, vs;
+      slot_values(s, v, v2, vs);
+      if (s == tid) {
+        first_max = v;
+        first_sum = vs;
+        first_max2 = v2;
+      }
+      any_nan = any_nan || (v != v);
+      m = __builtin_fmaxf(m, v);
+    }
+    m = wave_max_ignoring_nan(m);
+    const uint64_t nan_ballot = __ballot(any_nan);
+    if (lane == 0) {
+      sm.red_f[wave] = m;
+      sm.red_u[wave] = nan_ballot ? 1u : 0u;
+    }
+    __syncthreads();
+    m = sm.red_f[0];
+    uint32_t nan_any = sm.red_u[0];
+    for (int w = 1; w < kWaves; ++w) {
+      m = (sm.red_f[w] > m) ? sm.red_f[w] : m;
+      nan_any |= sm.red_u[w];
+    }
+    const float x0 = load_logit<DT>(logits, 0, p.row.fused) * inv;
+    if (x0 != x0) m = x0;  // max_val starts at x[0]; nothing compares greater than NaN
+    row_nan = nan_any != 0u || !(m > -kInf && m < kInf);
+  }
+  if (row_nan) {  // one NaN addend poisons the sum: the finish kernel needs nothing else
+    if (part == 0 && tid == 0) p.row_state[row] = {0u, m, 1u, 0.0f, 0, 0, 0, 0u};
+    return;
+  }
+  __syncthreads();
+  if (timers) c1 = wall_clock64();
+  if (!pro_done) {
+    float carry = 0.0f;
+    for (int base = 0; base < ns; base += kBlock) {
+      const int s = base + tid;
+      float a = 0.0f;
+      if (s < ns) {
+        float sum = first_sum, smax = first_max, smax2 = first_max2;
+        if (base != 0) slot_values(s, smax, smax2, sum);
+        a = slot_mass(s, sum, smax, smax2, m);
+      }
+      const float incl = wave_scan_inclusive_f32(a, lane);
+      if (lane == 63) sm.group_total[0][wave] = incl;
+      __syncthreads();
+      float before = carry, all = carry;
+      for (int w = 0; w < kWaves; ++w) {
+        if (w == wave) before = all;
+        all += sm.group_total[0][w];
+      }
+      const float a_out = before + incl;
+      const float a_in = before + lane_before_f32(incl);
+      if (s < ns) sh.upto[s + 1] = a_out;
+      carry = all;
+      const uint32_t cls = slot_class(s, a_in, a_out);
+      const bool serial = s < ns && s > 0 && ((cls >> 16) & 7u) == kSlotSerial;  // (slot 0 is worked out in this kernel)
+      const uint64_t serial_ballot = __ballot(serial);
+      if (lane == 0) sm.red_u[wave] = static_cast<uint32_t>(__popcll(serial_ballot));
+      __syncthreads();
+      uint32_t rank = serial_before;
+      uint32_t chunk_total = 0u;
+      for (int w = 0; w < kWaves; ++w) {
+        if (w < wave) rank += sm.red_u[w];
+        chunk_total += sm.red_u[w];
+      }
+      rank += static_cast<uint32_t>(__popcll(serial_ballot & ((1ull << lane) - 1ull)));
+      if (s < ns) sh.cls[s] = cls | ((rank & 0x7ffu) << 19);
+      serial_before += chunk_total;
+    }
+    a_total = carry;
+  }
   if (timers) c2 = wall_clock64();
 
   // ---- bf16 rows: expf by bit pattern
