@@ -673,6 +673,7 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
   float early_m = 0.0f;
   float held0[8], held1[8], held2[8], held3[8];  // FUSED: the wave's slots, read once (named one by one: they stay in registers)
   bool pro_early = false;  // FUSED: the first wave does the row-level work on its own while the others build the table
+  float x_first = 0.0f;    // FUSED: x[0], asked for with the slots
   // (FUSED) Given up on the others: their slots from the logits (whoever stores a slot's three values stores the same bits).
   auto alone = [&]() {
     for (int s = wave; s < ns; s += kWaves) {
@@ -689,81 +690,22 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
     if (s_mine + kWaves < s_end) load_slot_lane<DT>(logits, s_mine + kWaves, lane, V, fill, held1, p.row.fused);
     if (s_mine + 2 * kWaves < s_end) load_slot_lane<DT>(logits, s_mine + 2 * kWaves, lane, V, fill, held2, p.row.fused);
     if (s_mine + 3 * kWaves < s_end) load_slot_lane<DT>(logits, s_mine + 3 * kWaves, lane, V, fill, held3, p.row.fused);
-    // ---- pass 1 for these slots (the host sends no launch with an infinite inverse temperature here),
-    //      in two steps, each handed to the row's other workgroups as soon as it is done: the
-    //      workgroup's largest x first -- the row maximum is all the expf table needs, and the table is
-    //      built while the second step's values are still on their way --, then every slot's maximum
-    //      and approximate sum.  What the workgroups exchange is stored and read with device-scope
-    //      accesses that go through to memory one by one, complete (the wait below) before lane 0
-    //      counts the workgroup in; no fence of device scope, which would write back or discard the
-    //      die's whole L2 (microseconds, when every workgroup of the die does it).
-    const float kNegInf = -kInf;
-    SlotMax x0m = {kNegInf, kNegInf}, x1m = x0m, x2m = x0m, x3m = x0m;
-    if (s_mine < s_end) x0m = split_pass1_max(held0, inv);
-    if (s_mine + kWaves < s_end) x1m = split_pass1_max(held1, inv);
-    if (s_mine + 2 * kWaves < s_end) x2m = split_pass1_max(held2, inv);
-    if (s_mine + 3 * kWaves < s_end) x3m = split_pass1_max(held3, inv);
-    if (lane == 0) sm.red_f[wave] = __builtin_fmaxf(__builtin_fmaxf(x0m.M, x1m.M), __builtin_fmaxf(x2m.M, x3m.M));
-    __syncthreads();
-    uint32_t* const arrive_max = p.arrive + 2 * lrow;
-    uint32_t* const arrive_sum = arrive_max + 1;
-    float* const part_max = p.part_max + static_cast<int64_t>(lrow) * kMaxRowWorkgroups;
-    if (tid == 0) {
-      float mw = sm.red_f[0];
-      for (int w = 1; w < kWaves; ++w) mw = __builtin_fmaxf(mw, sm.red_f[w]);
-      coherent_store(part_max + part, mw);
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      __hip_atomic_fetch_add(arrive_max, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    if (s_mine < s_end) split_pass1_sum<true>(p, row, s_mine, held0, inv, x0m);
-    if (s_mine + kWaves < s_end) split_pass1_sum<true>(p, row, s_mine + kWaves, held1, inv, x1m);
-    if (s_mine + 2 * kWaves < s_end) split_pass1_sum<true>(p, row, s_mine + 2 * kWaves, held2, inv, x2m);
-    if (s_mine + 3 * kWaves < s_end) split_pass1_sum<true>(p, row, s_mine + 3 * kWaves, held3, inv, x3m);
+    x_first = load_logit<DT>(logits, 0, p.row.fused) * inv;  // (max_val starts at x[0]: a NaN there stays)
+    // ---- pass 1 for these slots (the host sends no launch with an infinite inverse temperature here):
+    //      every slot's maximum, second maximum and approximate sum, handed to the row's other
+    //      workgroups.  What the workgroups exchange is stored and read with device-scope accesses
+    //      that go through to memory one by one, complete (the wait below) before lane 0 counts the
+    //      workgroup in; no fence of device scope, which would write back or discard the die's whole
+    //      L2 (microseconds, when every workgroup of the die does it).
+    if (s_mine < s_end) split_pass1_slot<true>(p, row, s_mine, held0, inv);
+    if (s_mine + kWaves < s_end) split_pass1_slot<true>(p, row, s_mine + kWaves, held1, inv);
+    if (s_mine + 2 * kWaves < s_end) split_pass1_slot<true>(p, row, s_mine + 2 * kWaves, held2, inv);
+    if (s_mine + 3 * kWaves < s_end) split_pass1_slot<true>(p, row, s_mine + 3 * kWaves, held3, inv);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     if (timers) cf0 = wall_clock64();
     __syncthreads();
-    if (tid == 0) __hip_atomic_fetch_add(arrive_sum, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    // One lane polls a counter, a bounded number of times; every lane learns the outcome.
-    auto all_there = [&](uint32_t* counter) -> bool {
-      if (tid == 0) {
-        int met = 0;
-        for (int spin = 0; spin < p.spin_limit; ++spin) {
-          if (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= static_cast<uint32_t>(n_parts)) {
-            met = 1;
-            break;
-          }
-          __builtin_amdgcn_s_sleep(2);
-        }
-        sm.flag = met;
-      }
-      __syncthreads();
-      const bool met = sm.flag != 0;
-      __syncthreads();
-      return met;
-    };
-    bool on_my_own = !all_there(arrive_max);
-    if (timers) cf1 = wall_clock64();
-    float m_early;
-    if (on_my_own) {
-      alone();
-      m_early = kNegInf;
-      for (int s = lane; s < ns; s += 64) m_early = __builtin_fmaxf(m_early, coherent_load4(slot_pack + s).x);  // (ignores NaN)
-      m_early = wave_max_ignoring_nan(m_early);
-    } else {
-      m_early = lane < n_parts ? coherent_load(part_max + lane) : kNegInf;
-      m_early = wave_max_ignoring_nan(m_early);
-    }
-    {
-      const float x_first = load_logit<DT>(logits, 0, p.row.fused) * inv;
-      if (x_first != x_first) m_early = x_first;
-    }
-    early_m = m_early;
-    pro_early = !on_my_own;
-    if constexpr (DT == kDtypeBFloat16) {
-      if (!pro_early && m_early > kNegInf && m_early < kInf)
-        early_lut = build_exp_lut<false>(lut_mem, kLutCountWords, inv, m_early, sm.exp2tab, lut_base1, lut_top, lut_half) ? 1 : 0;
-    }
-    if (on_my_own && timers) cf2 = wall_clock64();
+    if (tid == 0) __hip_atomic_fetch_add(p.arrive + 2 * lrow + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    pro_early = true;
   } else {
     if (s_mine < s_end) load_slot_lane<DT>(logits, s_mine, lane, V, fill, l, p.row.fused);
   }
@@ -836,7 +778,7 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
   if constexpr (FUSED) {
     if (pro_early) {
       if (wave == 0) {
-        // (the second hand-over: every slot's maximum and sum; lane 0 polls, a bounded number of times)
+        // (the hand-over: lane 0 polls the row's counter, a bounded number of times)
         int met = 0;
         if (lane == 0) {
           for (int spin = 0; spin < p.spin_limit; ++spin) {
@@ -871,16 +813,28 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
           }
           mm = wave_max_ignoring_nan(mm);
           const bool nan_any = __ballot(nanf) != 0ull;
-          const float x0 = load_logit<DT>(logits, 0, p.row.fused) * inv;
-          if (x0 != x0) mm = x0;  // max_val starts at x[0]; nothing compares greater than NaN
-          const bool nan_row = nan_any || !(mm > -kInf && mm < kInf);
-          float run = 0.0f;
-          uint32_t serials = 0u;
-          if (!nan_row) {
+          if (x_first != x_first) mm = x_first;  // max_val starts at x[0]; nothing compares greater than NaN
+          if (lane == 0) {
+            sh.pro_m = mm;
+            sh.pro_nan = (nan_any || !(mm > -kInf && mm < kInf)) ? 1u : 0u;
+          }
+        }
+        if (lane == 0) sh.pro_done = met ? 1u : 0u;
+      }
+      __syncthreads();
+      if (timers) cf1 = wall_clock64();
+      pro_done = sh.pro_done != 0u;
+      if (pro_done) {
+        m = sh.pro_m;
+        row_nan = sh.pro_nan != 0u;
+        if (!row_nan) {
+          if (wave == 0) {
+            float run = 0.0f;
+            uint32_t serials = 0u;
             for (int c0 = 0; c0 < ns; c0 += 64) {
               const int s = c0 + lane;
               float a = 0.0f;
-              if (s < ns) a = slot_mass(s, sh.upto[s + 1], sh.top[s], __uint_as_float(sh.cls[s]), mm);
+              if (s < ns) a = slot_mass(s, sh.upto[s + 1], sh.top[s], __uint_as_float(sh.cls[s]), m);
               const float incl = wave_scan_inclusive_f32(a, lane);
               const float before = run;
               run = run + readlane_f32(incl, 63);
@@ -896,30 +850,22 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
               }
               serials += static_cast<uint32_t>(__popcll(serial_ballot));
             }
+            if (lane == 0) {
+              sh.pro_total = run;
+              sh.pro_serial = serials;
+            }
           }
-          if (lane == 0) {
-            sh.pro_m = mm;
-            sh.pro_total = run;
-            sh.pro_serial = serials;
-            sh.pro_nan = nan_row ? 1u : 0u;
+          if constexpr (DT == kDtypeBFloat16) {
+            // (the table's entries are dealt to the other waves; the first one only works out where it lies)
+            early_m = m;
+            early_lut = build_exp_lut<false>(lut_mem, kLutCountWords, inv, m, sm.exp2tab, lut_base1, lut_top, lut_half, 64) ? 1 : 0;
           }
+          __syncthreads();
+          a_total = sh.pro_total;
+          serial_before = sh.pro_serial;
         }
-        if (lane == 0) sh.pro_done = met ? 1u : 0u;
-      }
-      if constexpr (DT == kDtypeBFloat16) {
-        // (the table's entries are dealt to the other waves; the first one only works out where it lies)
-        if (early_m > -kInf && early_m < kInf)
-          early_lut = build_exp_lut<false>(lut_mem, kLutCountWords, inv, early_m, sm.exp2tab, lut_base1, lut_top, lut_half, 64) ? 1 : 0;
-      }
-      __syncthreads();
-      pro_done = sh.pro_done != 0u;
-      if (pro_done) {
-        m = sh.pro_m;
-        a_total = sh.pro_total;
-        serial_before = sh.pro_serial;
-        row_nan = sh.pro_nan != 0u;
       } else {
-        alone();  // (given up on the others' sums: their slots from the logits, then the form below)
+        alone();  // (given up on the others: their slots from the logits, then the form below)
       }
       if (timers) cf2 = wall_clock64();
     }
