@@ -123,7 +123,8 @@ ets_status ensure_split(ets_sampler* s) {
   const size_t o_list = take(list_entries * sizeof(uint64_t));
   ETS_HIP(s, hipMalloc(&s->d_split, at));
   char* base = static_cast<char*>(s->d_split);
-  ETS_HIP(s, hipMemset(base + o_arrive, 0, rows * 2 * sizeof(uint32_t)));  // (0 between launches)
+  ETS_HIP(s, hipMemset(base + o_arrive, 0, rows * 2 * sizeof(uint32_t)));  // (launches are numbered from 1)
+  ETS_HIP(s, hipMemset(base + o_pack, 0, rows * sp.ns_stride * sizeof(float4)));  // (no record carries a launch's tag yet)
   sp.arrive = reinterpret_cast<uint32_t*>(base + o_arrive);
   sp.part_max = reinterpret_cast<float*>(base + o_part);
   sp.slot_pack = reinterpret_cast<float4*>(base + o_pack);
@@ -386,6 +387,7 @@ ets_status sample_device(ets_sampler* s, const void* d_logits, int32_t dtype, in
 // up once per device (at the first handle created there) and kept.
 constexpr size_t kStaticScratchBytes = size_t{32} << 20;
 constexpr int kStaticArriveRows = 1024;
+constexpr size_t kStaticPackBytes = 320 << 10;  // (256 workgroups x 64 slots x 16 bytes, and the rows' padding)
 static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 std::mutex g_static_mutex;
@@ -426,10 +428,15 @@ size_t layout_static(const ets_sampler* s, int32_t dtype, int32_t rows, char* ba
     return base + here;
   };
   wb->tickets = reinterpret_cast<uint32_t*>(take(16 * sizeof(uint32_t)));  // always the array's first bytes: 0 between launches
-  // (the same bytes whatever the call's sizes: 0 between launches, like the tickets.  A call of more
-  // rows than this holds does not use the fused launch.)
+  // (the same bytes whatever the call's sizes: the launches' number, and the slot values that the
+  // workgroups of a fused launch hand to each other -- bytes that never hold anything else, so that what
+  // a reader finds there is a whole record of some launch or the zeros the array starts with.  A fused
+  // launch has at most one workgroup per compute unit and 64 slots per workgroup; a call whose rows
+  // need more does not use it.)
   sp.arrive = reinterpret_cast<uint32_t*>(take(kStaticArriveRows * 2 * sizeof(uint32_t)));
   wb->arrive_rows = kStaticArriveRows;
+  sp.slot_pack = reinterpret_cast<float4*>(take(kStaticPackBytes));
+  wb->pack_bytes = kStaticPackBytes;
   sp.slot_max = reinterpret_cast<float*>(take(r * sp.ns_stride * sizeof(float)));
   sp.slot_max2 = reinterpret_cast<float*>(take(r * sp.ns_stride * sizeof(float)));
   sp.slot_sum = reinterpret_cast<float*>(take(r * sp.ns_stride * sizeof(float)));
@@ -439,7 +446,6 @@ size_t layout_static(const ets_sampler* s, int32_t dtype, int32_t rows, char* ba
   sp.walk = reinterpret_cast<float2*>(take(r * sizeof(float2)));
   sp.list_count = reinterpret_cast<uint32_t*>(take(r * ets::kMaxRowWorkgroups * sizeof(uint32_t)));
   sp.part_max = reinterpret_cast<float*>(take(r * ets::kMaxRowWorkgroups * sizeof(float)));
-  sp.slot_pack = reinterpret_cast<float4*>(take(r * sp.ns_stride * sizeof(float4)));
   sp.hist = reinterpret_cast<uint32_t*>(take(r * g * ets::kHistBuckets * sizeof(uint32_t)));
   sp.phist = reinterpret_cast<uint32_t*>(take(r * g * phist_words * sizeof(uint32_t)));
   sp.list = reinterpret_cast<uint64_t*>(take(r * g * list_region(sp.ns, g) * sizeof(uint64_t)));

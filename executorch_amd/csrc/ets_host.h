@@ -25,7 +25,8 @@ struct WorkBuffers {
   int64_t scratch_stride = 0;
   uint64_t* partials = nullptr;  // [rows, kMaxSplits] arg-max partial results
   int max_row_wgs = 0;           // workgroups of pass 2 per row, at most
-  int arrive_rows = 0;           // rows the fused launch's counters are laid out for
+  int arrive_rows = 0;           // rows `arrive` is laid out for
+  size_t pack_bytes = 0;         // bytes set aside for the slot values a fused launch's workgroups hand to each other
 };
 
 struct ets_sampler {
@@ -55,7 +56,7 @@ struct ets_sampler {
   void* d_phist = nullptr;  // pattern histograms of 16-bit rows, allocated on their first use
   bool cfg_inv_ordinary = false;  // per-row parameters of the call in progress: every inverse temperature is finite
   int32_t beside_rows = 0;  // rows of other launches that run beside this one on another stream (set for the duration of a call)
-  bool arrive_dirty = false;  // a fused launch was not followed by its finish kernel: the counters are cleared before the next one
+  bool arrive_dirty = false;  // a fused launch was not followed by its finish kernel: the next one is given a number of its own first
   ets::SplitParams split = {};
   // per-row sampling parameters of ets_sampler_sample_batch_configs(): pinned host staging buffers
   // that take turns (a call fills the next one and waits only if the upload made from it

@@ -150,10 +150,10 @@ struct SplitParams {
                         //   counters per word, from order key RowState::key_cut upwards
   int32_t phist_words;  // words per (row, workgroup) region; 0 disables the pattern histogram
   float2* walk;         // [rows] multinomial rows: the exact softmax sum and the coin, between the two chains
-  uint32_t* arrive;     // [rows, 2] the fused launch: workgroups of the row that have stored their largest x, and their
-                        //   slots' maxima and sums (0 before a launch; the finish kernel puts them back)
-  float* part_max;      // [rows, kMaxRowWorkgroups] the fused launch: every workgroup's largest x
-  int32_t spin_limit;   // the fused launch: polls of `arrive` after which a workgroup stops waiting for the others
+  uint32_t* arrive;     // the fused launch: word 0 numbers the launches on these buffers (the finish kernel adds one; see
+                        //   coherent_store4)
+  float* part_max;      // (not in use)
+  int32_t spin_limit;   // the fused launch: reads of the row's slot values after which a workgroup stops waiting for the others
   uint64_t* timers;     // phase clocks (profiling), or null
   int32_t list_region;  // entries per region
   int32_t short_lists;  // 1: pass 2 may list only the largest candidates of a peaked row (see RowState::listed_buckets)
@@ -234,8 +234,19 @@ __device__ __forceinline__ float coherent_load(const float* ptr) {
 // of four bytes (every such store is charged a partial line behind L2).  The compiler does not count
 // these accesses: the load waits for its own result, the stores are waited for where the others are.
 typedef float ets_f32x4 __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ void coherent_store4(float4* ptr, float a, float b, float c) {
-  const ets_f32x4 v = {a, b, c, 0.0f};
+// The fourth word is a tag by which the reader knows the three values of THIS launch from whatever the
+// sixteen bytes held before: the launch's number (SplitParams::arrive[0] + 1, which the finish kernel
+// advances, so no two launches on the same buffers share one) mixed with the values themselves.  A record
+// of an earlier launch never carries this launch's tag, whatever its values; a record that is not there yet
+// reads as that earlier record (or as the zeros the buffer starts with, whose tag would be 0 + the mix of
+// zeros = 0, which no launch uses).  The sixteen bytes travel as one request; were a read ever to see part
+// of a store, the mix of the values would have to make up for the difference between two tags.
+__device__ __forceinline__ uint32_t pack_tag(uint32_t launch, float a, float b, float c) {
+  const uint32_t ua = __float_as_uint(a), ub = __float_as_uint(b), uc = __float_as_uint(c);
+  return launch ^ (ua * 0x9E3779B1u) ^ ((ub << 13) | (ub >> 19)) ^ (((uc << 7) | (uc >> 25)) * 0x85EBCA77u);
+}
+__device__ __forceinline__ void coherent_store4(float4* ptr, float a, float b, float c, uint32_t launch) {
+  const ets_f32x4 v = {a, b, c, __uint_as_float(pack_tag(launch, a, b, c))};
   asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(ptr), "v"(v) : "memory");
 }
 __device__ __forceinline__ ets_f32x4 coherent_load4(const float4* ptr) {
@@ -279,7 +290,8 @@ __device__ __forceinline__ SlotMax split_pass1_max(const float (&v)[8], float in
   return {float_of_max_key(Mk), float_of_max_key(wave_max_u32(lane == holder ? float_max_key(-kInf) : xk))};
 }
 template <bool COHERENT = false>
-__device__ __forceinline__ void split_pass1_sum(const SplitParams& p, int row, int s, const float (&v)[8], float inv_u, SlotMax x) {
+__device__ __forceinline__ void split_pass1_sum(const SplitParams& p, int row, int s, const float (&v)[8], float inv_u, SlotMax x,
+                                                uint32_t launch = 0u) {
   const int lane = threadIdx.x & 63;
   const float kInf = __uint_as_float(0x7f800000u);
   const float c1 = inv_u * kLog2e;
@@ -308,7 +320,7 @@ __device__ __forceinline__ void split_pass1_sum(const SplitParams& p, int row, i
   if (lane == 0) {
     const int64_t at = static_cast<int64_t>(row) * p.ns_stride + s;
     if (COHERENT) {
-      coherent_store4(p.slot_pack + at, any_nan ? __uint_as_float(0x7fc00000u) : M, x.M2, sum);
+      coherent_store4(p.slot_pack + at, any_nan ? __uint_as_float(0x7fc00000u) : M, x.M2, sum, launch);
     } else {
       p.slot_max[at] = any_nan ? __uint_as_float(0x7fc00000u) : M;
       p.slot_max2[at] = x.M2;
@@ -317,8 +329,9 @@ __device__ __forceinline__ void split_pass1_sum(const SplitParams& p, int row, i
   }
 }
 template <bool COHERENT = false>
-__device__ __forceinline__ void split_pass1_slot(const SplitParams& p, int row, int s, const float (&v)[8], float inv_u) {
-  split_pass1_sum<COHERENT>(p, row, s, v, inv_u, split_pass1_max(v, inv_u));
+__device__ __forceinline__ void split_pass1_slot(const SplitParams& p, int row, int s, const float (&v)[8], float inv_u,
+                                                 uint32_t launch = 0u) {
+  split_pass1_sum<COHERENT>(p, row, s, v, inv_u, split_pass1_max(v, inv_u), launch);
 }
 
 // grid = (ceil(ns / (4 SLOTS)), rows), 256 lanes: every wave takes SLOTS slots, all loads issued first.
@@ -672,6 +685,7 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
   int early_lut = -1;      // FUSED: the expf table was built for early_m already (1: usable, 0: not)
   float early_m = 0.0f;
   float held0[8], held1[8], held2[8], held3[8];  // FUSED: the wave's slots, read once (named one by one: they stay in registers)
+  const uint32_t launch = FUSED ? p.arrive[0] + 1u : 0u;  // FUSED: the number this launch tags what it hands over with
   bool pro_early = false;  // FUSED: the first wave does the row-level work on its own while the others build the table
   float x_first = 0.0f;    // FUSED: x[0], asked for with the slots
   // (FUSED) Given up on the others: their slots from the logits (whoever stores a slot's three values stores the same bits).
@@ -680,7 +694,7 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
       if (s >= s_begin && s < s_end) continue;
       float v[8];
       load_slot_lane<DT>(logits, s, lane, V, fill, v, p.row.fused);
-      split_pass1_slot<true>(p, row, s, v, inv);
+      split_pass1_slot<true>(p, row, s, v, inv, launch);
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
@@ -693,18 +707,15 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
     x_first = load_logit<DT>(logits, 0, p.row.fused) * inv;  // (max_val starts at x[0]: a NaN there stays)
     // ---- pass 1 for these slots (the host sends no launch with an infinite inverse temperature here):
     //      every slot's maximum, second maximum and approximate sum, handed to the row's other
-    //      workgroups.  What the workgroups exchange is stored and read with device-scope accesses
-    //      that go through to memory one by one, complete (the wait below) before lane 0 counts the
-    //      workgroup in; no fence of device scope, which would write back or discard the die's whole
-    //      L2 (microseconds, when every workgroup of the die does it).
-    if (s_mine < s_end) split_pass1_slot<true>(p, row, s_mine, held0, inv);
-    if (s_mine + kWaves < s_end) split_pass1_slot<true>(p, row, s_mine + kWaves, held1, inv);
-    if (s_mine + 2 * kWaves < s_end) split_pass1_slot<true>(p, row, s_mine + 2 * kWaves, held2, inv);
-    if (s_mine + 3 * kWaves < s_end) split_pass1_slot<true>(p, row, s_mine + 3 * kWaves, held3, inv);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    //      workgroups: stored with device-scope accesses that go through to memory one by one (no
+    //      fence of device scope, which would write back or discard the die's whole L2: microseconds,
+    //      when every workgroup of the die does it), each with a tag that tells the reader that
+    //      it is there (coherent_store4); no counter, and nobody waits for its own stores.
+    if (s_mine < s_end) split_pass1_slot<true>(p, row, s_mine, held0, inv, launch);
+    if (s_mine + kWaves < s_end) split_pass1_slot<true>(p, row, s_mine + kWaves, held1, inv, launch);
+    if (s_mine + 2 * kWaves < s_end) split_pass1_slot<true>(p, row, s_mine + 2 * kWaves, held2, inv, launch);
+    if (s_mine + 3 * kWaves < s_end) split_pass1_slot<true>(p, row, s_mine + 3 * kWaves, held3, inv, launch);
     if (timers) cf0 = wall_clock64();
-    __syncthreads();
-    if (tid == 0) __hip_atomic_fetch_add(p.arrive + 2 * lrow + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     pro_early = true;
   } else {
     if (s_mine < s_end) load_slot_lane<DT>(logits, s_mine, lane, V, fill, l, p.row.fused);
@@ -778,22 +789,17 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
   if constexpr (FUSED) {
     if (pro_early) {
       if (wave == 0) {
-        // (the hand-over: lane 0 polls the row's counter, a bounded number of times)
+        // (the hand-over: the slots' values are read until every one carries this launch's tag, a bounded
+        // number of times; they are parked in LDS where the results will go, four slots of a lane per
+        // trip to memory)
         int met = 0;
-        if (lane == 0) {
-          for (int spin = 0; spin < p.spin_limit; ++spin) {
-            if (__hip_atomic_load(p.arrive + 2 * lrow + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= static_cast<uint32_t>(n_parts)) {
-              met = 1;
-              break;
-            }
-            __builtin_amdgcn_s_sleep(2);
-          }
-        }
-        met = __builtin_amdgcn_readfirstlane(met);
-        if (met) {
-          // the slots' values, parked in LDS where the results will go (four slots of a lane per trip to memory)
-          float mm = -kInf;
-          bool nanf = false;
+        float mm = -kInf;
+        bool nanf = false;
+        for (int spin = 0; spin < p.spin_limit && !met; ++spin) {
+          if (spin != 0) __builtin_amdgcn_s_sleep(2);
+          mm = -kInf;
+          nanf = false;
+          bool missing = false;
           for (int base = 0; base < ns; base += 256) {
             ets_f32x4 v[4];
             const int s0 = base + lane;
@@ -803,6 +809,7 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
             for (int k = 0; k < 4; ++k) {
               const int s = s0 + 64 * k;
               if (s < ns) {
+                missing = missing || __float_as_uint(v[k].w) != pack_tag(launch, v[k].x, v[k].y, v[k].z);
                 sh.top[s] = v[k].x;
                 sh.cls[s] = __float_as_uint(v[k].y);
                 sh.upto[s + 1] = v[k].z;
@@ -811,6 +818,9 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
               }
             }
           }
+          met = __ballot(missing) == 0ull ? 1 : 0;
+        }
+        if (met) {
           mm = wave_max_ignoring_nan(mm);
           const bool nan_any = __ballot(nanf) != 0ull;
           if (x_first != x_first) mm = x_first;  // max_val starts at x[0]; nothing compares greater than NaN
@@ -1131,6 +1141,12 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
     t[2] = c3 - c2;
     t[3] = wall_clock64() - c3;
   }
+}
+
+// After a fused launch that was not followed by its finish kernel: the next one gets a number of its own.
+template <int DT>
+__global__ void split_launch_number_kernel(uint32_t* arrive) {
+  if (threadIdx.x == 0 && blockIdx.x == 0) arrive[0] = arrive[0] + 1u;
 }
 
 // ---- finish ---------------------------------------------------------------------------------------
@@ -2651,7 +2667,8 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
     for (int k = 0; k < 4; ++k) early_hist[k] = hist_in[(k < p.row_wgs ? k : 0) * kHistBuckets + tid];
   }
   const RowState rs = p.row_state[row];
-  if (tid < 2 && p.arrive) p.arrive[2 * lrow + tid] = 0u;  // (the fused launch's counters, for the next launch)
+  // (the number by which the fused launch tags what its workgroups hand over: the next launch gets another)
+  if (lrow == 0 && tid == 0 && p.arrive) atomicAdd(p.arrive, 1u);
   const float m = rs.m;
   const bool row_nan = rs.nan != 0u;
   const float cutoff = (1.0f - topp) / static_cast<float>(V - 1);  // sampler.cpp:136

@@ -80,12 +80,16 @@ ets_status launch_split(ets_sampler* s, const ets::RowParams& p, int32_t rows, h
   const bool inv_ordinary = p.row_cfg ? s->cfg_inv_ordinary : abs_inv < 3.0e38f;
   const bool fused = !TOPK && (!extras || (ETS_PHASE_CLOCKS && p.probs == nullptr)) && fuse_env != 0 && inv_ordinary && s->beside_rows == 0 && sp.arrive != nullptr &&
                      static_cast<int64_t>(rows) * sp.row_wgs <= (s->num_cus > 0 ? s->num_cus : 0) &&
-                     per_wg_slots <= ets::kFusedSlots * ets::kWaves && (!s->wb || rows <= s->wb->arrive_rows);
+                     per_wg_slots <= ets::kFusedSlots * ets::kWaves &&
+                     (!s->wb || static_cast<size_t>(rows) * sp.ns_stride * sizeof(float4) <= s->wb->pack_bytes);
   bool* dirty = arrive_dirty_flag(s);
   if (fused) {
     if constexpr (!TOPK) {
-      if (*dirty) ETS_HIP(s, hipMemsetAsync(sp.arrive, 0, 2 * sizeof(uint32_t) * static_cast<size_t>(s->wb ? s->wb->arrive_rows : s->max_batch), stream));
-      *dirty = true;  // (until this call's finish kernel, which clears the counters, has been launched)
+      if (*dirty) {
+        hipLaunchKernelGGL(ets::split_launch_number_kernel<DT>, dim3(1), dim3(64), 0, stream, sp.arrive);
+        ETS_HIP(s, hipGetLastError());
+      }
+      *dirty = true;  // (until this call's finish kernel, which numbers the next launch, has been launched)
       sp.spin_limit = spin_env < 0 ? 0 : spin_env;
       static std::atomic<size_t> set_bytes_f[kMaxDevices];
       constexpr bool kClocks = ETS_PHASE_CLOCKS != 0;  // (a profiling build: the fused kernel with its phase clocks)

@@ -340,30 +340,39 @@ def test_nuclei_of_hundreds_to_thousands_of_keys(oracle, dev, mode):
                 assert f32_bits(np.float32(rec["cumulative"][b])) == f32_bits(np.float32(ex[b].cumulative)), (kind, temperature, topp, b)
 
 
-@pytest.mark.parametrize("setting", ["fused", "fused_nobody_waits", "three_launches"])
+@pytest.mark.parametrize("setting", ["fused", "fused_one_read", "fused_nobody_waits", "three_launches"])
 @pytest.mark.parametrize("name,rows", [("cfg2", 64), ("cfg2", 8), ("cfg2", 1), ("cfg5", 16), ("cfg3", 24), ("cfg1", 1)])
 def test_pass1_inside_pass2(oracle, dev, monkeypatch, setting, name, rows):
     """Plain top-p launches whose workgroups are all resident run pass 1 inside pass 2: the row's
-    workgroups hand their slots' maxima and sums to one another through device memory and wait for
-    one another a bounded number of polls.  With the bound at 0 nobody waits: every workgroup works
-    the whole row's maxima and sums out itself.  Tokens and coin states must equal the oracle's either
-    way, and those of the three separate launches."""
+    workgroups hand their slots' maxima and sums to one another through device memory, each record
+    tagged with the launch's number, and read one another's a bounded number of times.  With the bound
+    at 0 nobody waits: every workgroup works the whole row's maxima and sums out itself; with the
+    bound at 1 some do and some do not.  Tokens and coin states must equal the oracle's either way,
+    and those of the three separate launches.  The same handle serves every step, with other logits
+    each time: the records of the step before are still where this step's are looked for."""
     if setting == "fused_nobody_waits":
         monkeypatch.setenv("ETS_FUSE_SPIN_LIMIT", "0")
+    if setting == "fused_one_read":
+        monkeypatch.setenv("ETS_FUSE_SPIN_LIMIT", "1")
     if setting == "three_launches":
         monkeypatch.setenv("ETS_FUSE", "0")
     w = W.WORKLOADS[name]
-    for step in range(2):
+    s = ea.Sampler(w.vocab, w.temperature, w.topp, w.coin_seed, max_batch=rows)
+    for step in range(3):
         x = W.logits(w, step, rows)
-        s = ea.Sampler(w.vocab, w.temperature, w.topp, w.coin_seed + 17 * step, max_batch=rows)
         states = s.get_rng_states(rows).copy()
         got = s.sample_batch(to_device(x, w.dtype, dev)).cpu().numpy()  # (no debug records: the fused launch)
         want, _ = oracle.sample_rows(x, w.dtype, oracle.inv_temperature(w.temperature), w.topp, 0, states, mode=oracle.MODE_UPCAST,
                                      tie=oracle.TIE_STABLE, threads=8)
         assert np.array_equal(got, want), (setting, name, rows, step)
         assert np.array_equal(s.get_rng_states(rows), states)
-        # the same handle again: the counters of the hand-over were put back
-        got2 = s.sample_batch(to_device(x, w.dtype, dev)).cpu().numpy()
-        want2, _ = oracle.sample_rows(x, w.dtype, oracle.inv_temperature(w.temperature), w.topp, 0, states, mode=oracle.MODE_UPCAST,
-                                      tie=oracle.TIE_STABLE, threads=8)
-        assert np.array_equal(got2, want2), (setting, name, rows, step, "second call")
+        # fewer rows on the same handle
+        if rows > 1:
+            fewer = (rows + 1) // 2
+            x2 = x[:fewer][::-1].copy()
+            states2 = s.get_rng_states(fewer).copy()
+            got2 = s.sample_batch(to_device(x2, w.dtype, dev)).cpu().numpy()
+            want2, _ = oracle.sample_rows(x2, w.dtype, oracle.inv_temperature(w.temperature), w.topp, 0, states2, mode=oracle.MODE_UPCAST,
+                                          tie=oracle.TIE_STABLE, threads=8)
+            assert np.array_equal(got2, want2), (setting, name, rows, step, "second call")
+            assert np.array_equal(s.get_rng_states(fewer), states2)

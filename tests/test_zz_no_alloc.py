@@ -108,3 +108,19 @@ def test_two_handles_take_turns_on_one_stream(dev):
         got_b = b.sample_batch_static(xb)  # (queued behind a's launches, before they have run)
         assert np.array_equal(got_a.cpu().numpy(), a_ref.sample_batch(xa).cpu().numpy())
         assert np.array_equal(got_b.cpu().numpy(), b_ref.sample_batch(xb).cpu().numpy())
+
+
+def test_handles_of_different_shapes_take_turns(dev):
+    """Handles of different vocabulary sizes and calls of different numbers of rows lay the static array
+    out differently; what one call's workgroups handed to each other stays where the next call's look
+    for theirs (the launches are told apart by their number).  Fresh logits at every step."""
+    shapes = ((50264, 8, W.DTYPE_BFLOAT16), (32000, 5, W.DTYPE_FLOAT), (128256, 8, W.DTYPE_BFLOAT16), (50264, 3, W.DTYPE_HALF))
+    refs = [ea.Sampler(V, 0.7, 0.9, 11 + i, max_batch=8) for i, (V, _, _) in enumerate(shapes)]
+    stas = [ea.Sampler(V, 0.7, 0.9, 11 + i, max_batch=8) for i, (V, _, _) in enumerate(shapes)]
+    for step in range(4):
+        for i, (V, rows, dtype) in enumerate(shapes):
+            x = to_device(rows_of(V, rows, dtype, 100 * step + i, step % 2 == 0), dtype, dev)
+            got = stas[i].sample_batch_static(x).cpu().numpy()
+            want = refs[i].sample_batch(x).cpu().numpy()
+            assert np.array_equal(got, want), (step, i, got, want)
+            assert np.array_equal(stas[i].get_rng_states()[:rows], refs[i].get_rng_states()[:rows])
