@@ -376,3 +376,43 @@ def test_pass1_inside_pass2(oracle, dev, monkeypatch, setting, name, rows):
                                           tie=oracle.TIE_STABLE, threads=8)
             assert np.array_equal(got2, want2), (setting, name, rows, step, "second call")
             assert np.array_equal(s.get_rng_states(fewer), states2)
+
+
+@pytest.mark.parametrize("name,rows", [("cfg2", 64), ("cfg2", 8)])
+def test_fused_step_replayed_from_a_graph(oracle, dev, name, rows):
+    """One call captured into a HIP graph and replayed: every replay runs the launch with pass 1 inside
+    pass 2 with the same kernel arguments, so what tells this replay's hand-over from the last one's
+    lives in device memory (the launch number, which the finish kernel advances).  Other logits are
+    copied into the captured input before every replay, with the program's own eager work and
+    synchronisations between replays; every replay against the oracle."""
+    w = W.WORKLOADS[name]
+    s = ea.Sampler(w.vocab, w.temperature, w.topp, w.coin_seed, max_batch=rows)
+    x0 = W.logits(w, 0, rows)
+    dx = to_device(x0, w.dtype, dev)
+    out = torch.empty(rows, dtype=torch.int32, device=dev)
+    side = torch.cuda.Stream(device=dev)
+    with torch.cuda.stream(side):
+        s.sample_batch(dx, out=out)  # (warm: buffers allocated, kernel attributes set)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=side):
+            s.sample_batch(dx, out=out)
+    torch.cuda.synchronize()
+    for step in range(1, 5):
+        x = W.logits(w, step, rows)
+        dx.copy_(to_device(x, w.dtype, dev))
+        states = s.get_rng_states(rows).copy()
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        got = out.cpu().numpy()
+        want, _ = oracle.sample_rows(x, w.dtype, oracle.inv_temperature(w.temperature), w.topp, 0, states, mode=oracle.MODE_UPCAST,
+                                     tie=oracle.TIE_STABLE, threads=8)
+        assert np.array_equal(got, want), (name, rows, step)
+        assert np.array_equal(s.get_rng_states(rows), states)
+        # eager work of the same handle between the replays
+        if step == 2:
+            eager = s.sample_batch(dx).cpu().numpy()
+            want2, _ = oracle.sample_rows(x, w.dtype, oracle.inv_temperature(w.temperature), w.topp, 0, states, mode=oracle.MODE_UPCAST,
+                                          tie=oracle.TIE_STABLE, threads=8)
+            assert np.array_equal(eager, want2), (name, rows, step, "eager")
