@@ -564,9 +564,12 @@ constexpr int kLutCountWords = 12288;  // a table entry's counter sits 48 KiB ab
 // finite in the way the bounds need, or when the table would not fit in `cap` floats.
 // COUNTERS = false builds the table alone (`cap` then only has to hold its 2 * half floats).
 // The threads from `first_thread` on share the entries; the ones before it only learn where the table lies.
+// `seen`, when given, is a byte per eight consecutive 16-bit patterns (8192 bytes): only the entries of
+// patterns whose byte is set are worked out (and the two ends, which stand for many patterns); the others
+// are left as they are, for a caller that will only look up patterns it has marked.
 template <bool COUNTERS = true>
 __device__ bool build_exp_lut(float* lut, int cap, float inv, float m, const uint64_t* tab, int& base1, int& top,
-                              int& half, int first_thread = 0) {
+                              int& half, int first_thread = 0, const uint8_t* seen = nullptr) {
   const float kInf = __uint_as_float(0x7f800000u);
   if (!(inv > 0.0f && inv < kInf && m > -kInf && m < kInf)) return false;
   const uint32_t ib = __float_as_uint(inv);
@@ -602,6 +605,7 @@ __device__ bool build_exp_lut(float* lut, int cap, float inv, float m, const uin
         d = -m;
       } else {
         const uint32_t pattern = (static_cast<uint32_t>(sgn) << 15) | static_cast<uint32_t>(base1 + c);
+        if (seen != nullptr && seen[pattern >> 3] == 0) continue;
         const float l = __uint_as_float(pattern << 16);
         d = l * inv - m;
       }

@@ -389,6 +389,7 @@ struct Pass2Shared {
   // what the first wave worked out on its own (FUSED): row maximum, approximate total, serial slots, NaN row, done
   float pro_m, pro_total;
   uint32_t pro_serial, pro_nan, pro_done;
+  uint32_t seen[2048];  // (FUSED, bf16) a byte per eight consecutive 16-bit patterns: some entry of this workgroup has one of them
 };
 
 // One wave, one slot: e[] are the lane's 8 entries; `cls` is the slot's entry of Pass2Shared::cls.
@@ -664,6 +665,10 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
     sh.top_mass[tid] = 0u;
     sh.top_all[tid] = 0u;
   }
+  if (FUSED && DT == kDtypeBFloat16) {
+    sh.seen[tid] = 0u;
+    sh.seen[tid + kBlock] = 0u;
+  }
   // 16-bit rows: entries per bit pattern, behind the expf table
   constexpr bool kPatterns = TOPP && (DT == kDtypeBFloat16 || DT == kDtypeHalf);
   uint32_t* ph = reinterpret_cast<uint32_t*>(lut_mem + (DT == kDtypeBFloat16 ? kLutCountWords : 0));
@@ -715,6 +720,21 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
     if (s_mine + kWaves < s_end) split_pass1_slot<true>(p, row, s_mine + kWaves, held1, inv, launch);
     if (s_mine + 2 * kWaves < s_end) split_pass1_slot<true>(p, row, s_mine + 2 * kWaves, held2, inv, launch);
     if (s_mine + 3 * kWaves < s_end) split_pass1_slot<true>(p, row, s_mine + 3 * kWaves, held3, inv, launch);
+    if constexpr (DT == kDtypeBFloat16) {
+      // the bit patterns among this workgroup's entries: the expf table is built for these alone (while
+      // the other workgroups' values are on their way there is nothing else to do)
+      __syncthreads();  // (the marks were cleared by other waves)
+      auto mark = [&](const float (&v)[8]) {
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+          reinterpret_cast<uint8_t*>(sh.seen)[__float_as_uint(v[k]) >> 19] = 1;
+        }
+      };
+      if (s_mine < s_end) mark(held0);
+      if (s_mine + kWaves < s_end) mark(held1);
+      if (s_mine + 2 * kWaves < s_end) mark(held2);
+      if (s_mine + 3 * kWaves < s_end) mark(held3);
+    }
     if (timers) cf0 = wall_clock64();
     pro_early = true;
   } else {
@@ -868,7 +888,7 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
           if constexpr (DT == kDtypeBFloat16) {
             // (the table's entries are dealt to the other waves; the first one only works out where it lies)
             early_m = m;
-            early_lut = build_exp_lut<false>(lut_mem, kLutCountWords, inv, m, sm.exp2tab, lut_base1, lut_top, lut_half, 64) ? 1 : 0;
+            early_lut = build_exp_lut<false>(lut_mem, kLutCountWords, inv, m, sm.exp2tab, lut_base1, lut_top, lut_half, 64, reinterpret_cast<const uint8_t*>(sh.seen)) ? 1 : 0;
           }
           __syncthreads();
           a_total = sh.pro_total;
