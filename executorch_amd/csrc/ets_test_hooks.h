@@ -44,6 +44,12 @@ ETS_API ets_status ets_test_signal_floor(uint32_t* d_words, int32_t hops, int32_
  * ets_sampler_sample_batch_static() has none of them.  HOST pointer to four int32. */
 ETS_API ets_status ets_test_handle_buffers(const ets_sampler* s, int32_t* out);
 
+/* The number of the next launch with pass 1 inside pass 2 on the handle's own work buffers (the word its
+ * workgroups tag their hand-over with; waits for the device).  With `mark_unfinished` the handle is left as
+ * if its last such launch had not been followed by its finish kernel: the next one must then be given a
+ * number of its own first. */
+ETS_API ets_status ets_test_fused_launch_number(ets_sampler* s, int32_t mark_unfinished, uint32_t* out);
+
 /* The message of the calling thread's last failed hook. */
 ETS_API const char* ets_test_last_error(void);
 

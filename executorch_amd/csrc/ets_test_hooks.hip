@@ -225,6 +225,18 @@ ets_status ets_test_handle_buffers(const ets_sampler* s, int32_t* out) {
   return ETS_OK;
 }
 
+ets_status ets_test_fused_launch_number(ets_sampler* s, int32_t mark_unfinished, uint32_t* out) {
+  if (!s || !out) return hook_fail(ETS_INVALID_ARGUMENT, "ets_test_fused_launch_number: null pointer");
+  if (!s->d_split) return hook_fail(ETS_INVALID_STATE, "ets_test_fused_launch_number: the handle has not sampled several workgroups a row yet");
+  int prev = -1;
+  const bool switched = hipGetDevice(&prev) == hipSuccess && prev != s->device && hipSetDevice(s->device) == hipSuccess;
+  const hipError_t e = hipMemcpy(out, s->split.arrive, sizeof(uint32_t), hipMemcpyDeviceToHost);
+  if (switched) (void)hipSetDevice(prev);
+  if (e != hipSuccess) return hook_fail(ETS_INTERNAL, hipGetErrorString(e));
+  if (mark_unfinished) s->arrive_dirty = true;
+  return ETS_OK;
+}
+
 const char* ets_test_last_error(void) { return g_hook_error.c_str(); }
 
 }  // extern "C"

@@ -416,3 +416,38 @@ def test_fused_step_replayed_from_a_graph(oracle, dev, name, rows):
             want2, _ = oracle.sample_rows(x, w.dtype, oracle.inv_temperature(w.temperature), w.topp, 0, states, mode=oracle.MODE_UPCAST,
                                           tie=oracle.TIE_STABLE, threads=8)
             assert np.array_equal(eager, want2), (name, rows, step, "eager")
+
+
+def test_a_launch_without_its_finish_kernel_does_not_lend_its_number(oracle, dev):
+    """The workgroups of a launch with pass 1 inside pass 2 tag what they hand over with the launch's
+    number, which the finish kernel advances.  A launch whose finish kernel was never issued (an error
+    between the two) leaves the number as it was: the handle remembers, and the next such launch is given
+    a number of its own before it starts.  Forced here through the test hook; tokens against the oracle."""
+    import ctypes
+    from executorch_amd import _capi
+    w = W.WORKLOADS["cfg2"]
+    rows = 8
+    s = ea.Sampler(w.vocab, w.temperature, w.topp, w.coin_seed, max_batch=rows)
+
+    def number(mark):
+        out = ctypes.c_uint32(0)
+        assert _capi.hooks().ets_test_fused_launch_number(s._h, mark, ctypes.byref(out)) == _capi.OK
+        return out.value
+
+    def step(k):
+        x = W.logits(w, k, rows)
+        states = s.get_rng_states(rows).copy()
+        got = s.sample_batch(to_device(x, w.dtype, dev)).cpu().numpy()
+        want, _ = oracle.sample_rows(x, w.dtype, oracle.inv_temperature(w.temperature), w.topp, 0, states, mode=oracle.MODE_UPCAST,
+                                     tie=oracle.TIE_STABLE, threads=8)
+        assert np.array_equal(got, want), k
+        assert np.array_equal(s.get_rng_states(rows), states)
+
+    step(0)
+    n1 = number(0)
+    step(1)
+    assert number(1) == n1 + 1  # (one launch, one number; and the handle is marked)
+    step(2)
+    assert number(0) == n1 + 3  # (a number skipped, then the launch's own)
+    step(3)
+    assert number(0) == n1 + 4
