@@ -618,6 +618,70 @@ __device__ bool build_exp_lut(float* lut, int cap, float inv, float m, const uin
   return true;
 }
 
+// The same table for a caller that has marked the patterns it will look up (`seen`: a byte per eight
+// consecutive 16-bit patterns, 8192 bytes, 8-byte aligned) and builds with the waves from the second on:
+// the table is cut into chunks of 64 consecutive patterns; every wave finds out which chunks hold a marked
+// pattern (two reads of eight mark bytes per lane, two ballots) and the builders take those chunks in turn,
+// so that each has the same number of them to work out, whatever the row looks like.  Unmarked chunks are
+// left as they are.  More than 128 chunks: the general routine.
+__device__ bool build_exp_lut_marked(float* lut, int cap, float inv, float m, const uint64_t* tab, int& base1, int& top,
+                                     int& half, const uint8_t* seen) {
+  const float kInf = __uint_as_float(0x7f800000u);
+  if (!(inv > 0.0f && inv < kInf && m > -kInf && m < kInf)) return false;
+  const int ei = static_cast<int>(__float_as_uint(inv) >> 23);
+  if (ei == 0) return false;
+  const uint32_t mb = __float_as_uint(__builtin_fabsf(m));
+  const int em = (mb >> 23) ? static_cast<int>(mb >> 23) : 1;
+  int e_lo = em - ei + 100;  // (the bounds of build_exp_lut)
+  if (e_lo < 0) e_lo = 0;
+  const int et = static_cast<int>(__float_as_uint(__builtin_fabsf(m) + 104.0f) >> 23);
+  int e_hi = et - ei + 128;
+  if (e_hi > 254) e_hi = 254;
+  if (e_hi < e_lo) return false;
+  const int R = (e_hi - e_lo + 1) * 128;
+  const int per_half = R >> 6, n_chunks = 2 * per_half;
+  if (n_chunks > 128) return build_exp_lut<false>(lut, cap, inv, m, tab, base1, top, half, 64, seen);
+  half = R + 2;
+  top = R + 1;
+  base1 = (e_lo << 7) - 1;
+  if (2 * half > kLutCountWords || 2 * half > cap) return false;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (wave == 0) return true;  // (takes no part: where the table lies)
+  const int builders = kBlock / 64 - 1, me = wave - 1;
+  auto first_pattern = [&](int k) -> uint32_t {
+    const int sgn = k >= per_half ? 1 : 0;
+    return (static_cast<uint32_t>(sgn) << 15) | static_cast<uint32_t>((e_lo << 7) + 64 * (k - sgn * per_half));
+  };
+  auto marked = [&](int k) -> bool {
+    return k < n_chunks && *reinterpret_cast<const uint64_t*>(seen + (first_pattern(k) >> 3)) != 0ull;
+  };
+  const uint64_t need0 = __ballot(marked(lane)), need1 = __ballot(marked(lane + 64));
+  const uint64_t below = (1ull << lane) - 1ull;
+  const int rank0 = __popcll(need0 & below), rank1 = __popcll(need0) + __popcll(need1 & below);
+  uint64_t mine[2] = {__ballot(((need0 >> lane) & 1ull) && rank0 % builders == me),
+                      __ballot(((need1 >> lane) & 1ull) && rank1 % builders == me)};
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    while (mine[h] != 0ull) {
+      const int k = 64 * h + __builtin_ctzll(mine[h]);
+      mine[h] &= mine[h] - 1ull;
+      const uint32_t pattern = first_pattern(k) + static_cast<uint32_t>(lane);
+      const int sgn = static_cast<int>(pattern >> 15);
+      const int c = static_cast<int>(pattern & 0x7fffu) - base1;
+      const float l = __uint_as_float(pattern << 16);
+      const float d = __builtin_fminf(__builtin_fmaxf(l * inv - m, -104.0f), 0.0f);  // positive only for patterns that cannot occur
+      lut[sgn * half + c] = expf_core(d, tab);
+    }
+  }
+  if (wave == 1 && lane < 4) {  // the two ends of each half: the patterns below and beyond the table's
+    const int sgn = lane >> 1;
+    const bool beyond = (lane & 1) != 0;
+    const float tiny = expf_core(__builtin_fminf(__builtin_fmaxf(-m, -104.0f), 0.0f), tab);
+    lut[sgn * half + (beyond ? top : 0)] = beyond ? (sgn ? 0.0f : 1.0f) : tiny;
+  }
+  return true;
+}
+
 // Table slot of one bf16 pattern (16 bits: sign, 8 exponent bits, 7 mantissa bits).
 __device__ __forceinline__ int lut_slot(uint32_t mag15, uint32_t sgn, int base1, int top, int half) {
   const int c = min(max(static_cast<int>(mag15), base1), base1 + top);

@@ -389,7 +389,7 @@ struct Pass2Shared {
   // what the first wave worked out on its own (FUSED): row maximum, approximate total, serial slots, NaN row, done
   float pro_m, pro_total;
   uint32_t pro_serial, pro_nan, pro_done;
-  uint32_t seen[2048];  // (FUSED, bf16) a byte per eight consecutive 16-bit patterns: some entry of this workgroup has one of them
+  alignas(8) uint32_t seen[2048];  // (FUSED, bf16) a byte per eight consecutive 16-bit patterns: some entry of this workgroup has one of them
 };
 
 // One wave, one slot: e[] are the lane's 8 entries; `cls` is the slot's entry of Pass2Shared::cls.
@@ -888,7 +888,8 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
           if constexpr (DT == kDtypeBFloat16) {
             // (the table's entries are dealt to the other waves; the first one only works out where it lies)
             early_m = m;
-            early_lut = build_exp_lut<false>(lut_mem, kLutCountWords, inv, m, sm.exp2tab, lut_base1, lut_top, lut_half, 64, reinterpret_cast<const uint8_t*>(sh.seen)) ? 1 : 0;
+            early_lut = build_exp_lut_marked(lut_mem, kLutCountWords, inv, m, sm.exp2tab, lut_base1, lut_top, lut_half,
+                                             reinterpret_cast<const uint8_t*>(sh.seen)) ? 1 : 0;
           }
           __syncthreads();
           a_total = sh.pro_total;
