@@ -116,7 +116,6 @@ ets_status ensure_split(ets_sampler* s) {
   const size_t o_walk = take(rows * sizeof(float2));
   const size_t o_count = take(rows * ets::kMaxRowWorkgroups * sizeof(uint32_t));
   const size_t o_arrive = take(rows * 2 * sizeof(uint32_t));
-  const size_t o_part = take(rows * ets::kMaxRowWorkgroups * sizeof(float));
   const size_t o_pack = take(rows * sp.ns_stride * sizeof(float4));
   const size_t o_timers = take(rows * 12 * sizeof(uint64_t));
   const size_t o_hist = take(row_wgs * ets::kHistBuckets * sizeof(uint32_t));
@@ -126,7 +125,6 @@ ets_status ensure_split(ets_sampler* s) {
   ETS_HIP(s, hipMemset(base + o_arrive, 0, rows * 2 * sizeof(uint32_t)));  // (launches are numbered from 1)
   ETS_HIP(s, hipMemset(base + o_pack, 0, rows * sp.ns_stride * sizeof(float4)));  // (no record carries a launch's tag yet)
   sp.arrive = reinterpret_cast<uint32_t*>(base + o_arrive);
-  sp.part_max = reinterpret_cast<float*>(base + o_part);
   sp.slot_pack = reinterpret_cast<float4*>(base + o_pack);
   sp.slot_max = reinterpret_cast<float*>(base + o_max);
   sp.slot_max2 = reinterpret_cast<float*>(base + o_max2);
@@ -445,7 +443,6 @@ size_t layout_static(const ets_sampler* s, int32_t dtype, int32_t rows, char* ba
   sp.row_state = reinterpret_cast<ets::RowState*>(take(r * sizeof(ets::RowState)));
   sp.walk = reinterpret_cast<float2*>(take(r * sizeof(float2)));
   sp.list_count = reinterpret_cast<uint32_t*>(take(r * ets::kMaxRowWorkgroups * sizeof(uint32_t)));
-  sp.part_max = reinterpret_cast<float*>(take(r * ets::kMaxRowWorkgroups * sizeof(float)));
   sp.hist = reinterpret_cast<uint32_t*>(take(r * g * ets::kHistBuckets * sizeof(uint32_t)));
   sp.phist = reinterpret_cast<uint32_t*>(take(r * g * phist_words * sizeof(uint32_t)));
   sp.list = reinterpret_cast<uint64_t*>(take(r * g * list_region(sp.ns, g) * sizeof(uint64_t)));

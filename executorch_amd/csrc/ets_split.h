@@ -152,7 +152,6 @@ struct SplitParams {
   float2* walk;         // [rows] multinomial rows: the exact softmax sum and the coin, between the two chains
   uint32_t* arrive;     // the fused launch: word 0 numbers the launches on these buffers (the finish kernel adds one; see
                         //   coherent_store4)
-  float* part_max;      // (not in use)
   int32_t spin_limit;   // the fused launch: reads of the row's slot values after which a workgroup stops waiting for the others
   uint64_t* timers;     // phase clocks (profiling), or null
   int32_t list_region;  // entries per region
