@@ -288,7 +288,9 @@ __device__ __forceinline__ SlotMax split_pass1_max(const float (&v)[8], float in
   const int holder = __ffsll(static_cast<long long>(holds)) - 1;  // (some lane holds the maximum)
   return {float_of_max_key(Mk), float_of_max_key(wave_max_u32(lane == holder ? float_max_key(-kInf) : xk))};
 }
-template <bool COHERENT = false>
+// COHERENT: the three values as one tagged record for the other workgroups of the launch (coherent_store4);
+// PLAIN_TOO: and in the three arrays as well, for a later launch that reads them there.
+template <bool COHERENT = false, bool PLAIN_TOO = false>
 __device__ __forceinline__ void split_pass1_sum(const SplitParams& p, int row, int s, const float (&v)[8], float inv_u, SlotMax x,
                                                 uint32_t launch = 0u) {
   const int lane = threadIdx.x & 63;
@@ -318,19 +320,18 @@ __device__ __forceinline__ void split_pass1_sum(const SplitParams& p, int row, i
   const bool any_nan = ordinary ? sum != sum : __ballot(nan) != 0ull;
   if (lane == 0) {
     const int64_t at = static_cast<int64_t>(row) * p.ns_stride + s;
-    if (COHERENT) {
-      coherent_store4(p.slot_pack + at, any_nan ? __uint_as_float(0x7fc00000u) : M, x.M2, sum, launch);
-    } else {
+    if (COHERENT) coherent_store4(p.slot_pack + at, any_nan ? __uint_as_float(0x7fc00000u) : M, x.M2, sum, launch);
+    if (!COHERENT || PLAIN_TOO) {
       p.slot_max[at] = any_nan ? __uint_as_float(0x7fc00000u) : M;
       p.slot_max2[at] = x.M2;
       p.slot_sum[at] = sum;
     }
   }
 }
-template <bool COHERENT = false>
+template <bool COHERENT = false, bool PLAIN_TOO = false>
 __device__ __forceinline__ void split_pass1_slot(const SplitParams& p, int row, int s, const float (&v)[8], float inv_u,
                                                  uint32_t launch = 0u) {
-  split_pass1_sum<COHERENT>(p, row, s, v, inv_u, split_pass1_max(v, inv_u), launch);
+  split_pass1_sum<COHERENT, PLAIN_TOO>(p, row, s, v, inv_u, split_pass1_max(v, inv_u), launch);
 }
 
 // grid = (ceil(ns / (4 SLOTS)), rows), 256 lanes: every wave takes SLOTS slots, all loads issued first.
@@ -714,11 +715,12 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
     //      workgroups: stored with device-scope accesses that go through to memory one by one (no
     //      fence of device scope, which would write back or discard the die's whole L2: microseconds,
     //      when every workgroup of the die does it), each with a tag that tells the reader that
-    //      it is there (coherent_store4); no counter, and nobody waits for its own stores.
-    if (s_mine < s_end) split_pass1_slot<true>(p, row, s_mine, held0, inv, launch);
-    if (s_mine + kWaves < s_end) split_pass1_slot<true>(p, row, s_mine + kWaves, held1, inv, launch);
-    if (s_mine + 2 * kWaves < s_end) split_pass1_slot<true>(p, row, s_mine + 2 * kWaves, held2, inv, launch);
-    if (s_mine + 3 * kWaves < s_end) split_pass1_slot<true>(p, row, s_mine + 3 * kWaves, held3, inv, launch);
+    //      it is there (coherent_store4); no counter, and nobody waits for its own stores.  (A multinomial
+    //      row's second sweep is a launch of its own, which reads the values where pass 1 leaves them.)
+    if (s_mine < s_end) split_pass1_slot<true, !TOPP>(p, row, s_mine, held0, inv, launch);
+    if (s_mine + kWaves < s_end) split_pass1_slot<true, !TOPP>(p, row, s_mine + kWaves, held1, inv, launch);
+    if (s_mine + 2 * kWaves < s_end) split_pass1_slot<true, !TOPP>(p, row, s_mine + 2 * kWaves, held2, inv, launch);
+    if (s_mine + 3 * kWaves < s_end) split_pass1_slot<true, !TOPP>(p, row, s_mine + 3 * kWaves, held3, inv, launch);
     if constexpr (DT == kDtypeBFloat16) {
       // the bit patterns among this workgroup's entries: the expf table is built for these alone (while
       // the other workgroups' values are on their way there is nothing else to do)
@@ -3085,6 +3087,8 @@ __global__ void __launch_bounds__(kWalkBlock) split_walk_kernel(SplitParams p, u
   const int row = p.row.row_map ? p.row.row_map[blockIdx.x] : blockIdx.x;
   const RowState rs = p.row_state[row];
   if (tid < 32) exp2tab[tid] = kExp2Table[tid];
+  // (the number by which a launch with pass 1 inside pass 2 tags what its workgroups hand over: the next one gets another)
+  if (PHASE == 0 && blockIdx.x == 0 && tid == 0 && p.arrive) atomicAdd(p.arrive, 1u);
   auto toss = [&]() {  // one coin per call (sampler.cpp:237, 210-220)
     uint64_t st = p.row.rng[row];
     st ^= st >> 12;

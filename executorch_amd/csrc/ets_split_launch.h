@@ -33,6 +33,26 @@ inline ets_status check_row_wgs(ets_sampler* s, int row_wgs) {
   return ETS_OK;
 }
 
+// Whether a launch of `rows` rows may run pass 1 inside pass 2 (every workgroup resident at once, a wave's
+// slots in its registers, finite temperatures, nothing beside it on another stream, room for the records
+// that the workgroups hand to each other); `spin_limit`: how often a workgroup reads the others' records
+// before it works their slots out itself.  ETS_FUSE=0 switches it off, ETS_FUSE_SPIN_LIMIT sets the limit
+// (read at every launch, so that a test can switch between them inside one process).
+inline bool fused_launch_fits(const ets_sampler* s, const ets::SplitParams& sp, const ets::RowParams& p, int32_t rows, int32_t* spin_limit) {
+  const char* const fuse_text = std::getenv("ETS_FUSE");
+  const int fuse_env = fuse_text ? std::atoi(fuse_text) : 1;
+  const char* const spin_text = std::getenv("ETS_FUSE_SPIN_LIMIT");
+  const int spin_env = spin_text ? std::atoi(spin_text) : (1 << 13);  // (about ten milliseconds; the usual wait is a read or two)
+  *spin_limit = spin_env < 0 ? 0 : spin_env;
+  const int per_wg_slots = ((sp.ns + sp.row_wgs - 1) / sp.row_wgs + ets::kWaves - 1) / ets::kWaves * ets::kWaves;
+  const float abs_inv = p.inv_temperature < 0.0f ? -p.inv_temperature : p.inv_temperature;
+  // (rows with parameters of their own: the caller has looked at their temperatures)
+  const bool inv_ordinary = p.row_cfg ? s->cfg_inv_ordinary : abs_inv < 3.0e38f;
+  return fuse_env != 0 && inv_ordinary && s->beside_rows == 0 && sp.arrive != nullptr &&
+         static_cast<int64_t>(rows) * sp.row_wgs <= (s->num_cus > 0 ? s->num_cus : 0) && per_wg_slots <= ets::kFusedSlots * ets::kWaves &&
+         (!s->wb || static_cast<size_t>(rows) * sp.ns_stride * sizeof(float4) <= s->wb->pack_bytes);
+}
+
 // The three launches for top-p (and, with TOPK, top-k) rows.
 // TOPK: some row may be a top-k row (the kernels of a launch without one leave that case out).
 template <int DT, bool TOPK>
@@ -64,24 +84,10 @@ ets_status launch_split(ets_sampler* s, const ets::RowParams& p, int32_t rows, h
   const size_t lut_bytes = (DT == ets::kDtypeBFloat16 ? sizeof(float) * ets::kLutCountWords : 0) + sizeof(uint32_t) * sp.phist_words;
   // (a launch that neither writes the probabilities nor fills the phase clocks runs kernels without those branches)
   const bool extras = sp.timers != nullptr || p.probs != nullptr;
-  // Pass 1 inside pass 2 (one read of the logits, one launch fewer) when every workgroup of the launch
-  // is resident at once and a wave's slots fit its registers: plain top-p launches with one
-  // temperature, a finite one.  ETS_FUSE=0 switches it off; ETS_FUSE_SPIN_LIMIT sets how often a
-  // workgroup polls for the others of its row before it works their slots out itself (0: at once).
-  // (read at every launch, so that a test can switch between them inside one process)
-  const char* const fuse_text = std::getenv("ETS_FUSE");
-  const int fuse_env = fuse_text ? std::atoi(fuse_text) : 1;
-  const char* const spin_text = std::getenv("ETS_FUSE_SPIN_LIMIT");
-  const int spin_env = spin_text ? std::atoi(spin_text) : (1 << 13);  // (about ten milliseconds; the usual wait is a few polls)
-  const int per_wg_slots = ((sp.ns + sp.row_wgs - 1) / sp.row_wgs + ets::kWaves - 1) / ets::kWaves * ets::kWaves;
-  const float abs_inv = p.inv_temperature < 0.0f ? -p.inv_temperature : p.inv_temperature;
-  // (rows with parameters of their own: the caller has looked at their temperatures; a launch that
-  // shares the compute units with one on another stream may not have all its workgroups resident)
-  const bool inv_ordinary = p.row_cfg ? s->cfg_inv_ordinary : abs_inv < 3.0e38f;
-  const bool fused = !TOPK && (!extras || (ETS_PHASE_CLOCKS && p.probs == nullptr)) && fuse_env != 0 && inv_ordinary && s->beside_rows == 0 && sp.arrive != nullptr &&
-                     static_cast<int64_t>(rows) * sp.row_wgs <= (s->num_cus > 0 ? s->num_cus : 0) &&
-                     per_wg_slots <= ets::kFusedSlots * ets::kWaves &&
-                     (!s->wb || static_cast<size_t>(rows) * sp.ns_stride * sizeof(float4) <= s->wb->pack_bytes);
+  // Pass 1 inside pass 2 (one read of the logits, one launch fewer): plain top-p launches that fit
+  // (fused_launch_fits) and ask for neither probabilities nor debug records.
+  int32_t spin_limit = 0;
+  const bool fused = !TOPK && (!extras || (ETS_PHASE_CLOCKS && p.probs == nullptr)) && fused_launch_fits(s, sp, p, rows, &spin_limit);
   bool* dirty = arrive_dirty_flag(s);
   if (fused) {
     if constexpr (!TOPK) {
@@ -90,7 +96,7 @@ ets_status launch_split(ets_sampler* s, const ets::RowParams& p, int32_t rows, h
         ETS_HIP(s, hipGetLastError());
       }
       *dirty = true;  // (until this call's finish kernel, which numbers the next launch, has been launched)
-      sp.spin_limit = spin_env < 0 ? 0 : spin_env;
+      sp.spin_limit = spin_limit;
       static std::atomic<size_t> set_bytes_f[kMaxDevices];
       constexpr bool kClocks = ETS_PHASE_CLOCKS != 0;  // (a profiling build: the fused kernel with its phase clocks)
       st = allow_dynamic_lds(s, reinterpret_cast<const void*>(&ets::split_pass2_kernel<DT, true, false, false, kClocks, true>), lut_bytes, set_bytes_f);
@@ -160,7 +166,7 @@ ets_status launch_split(ets_sampler* s, const ets::RowParams& p, int32_t rows, h
   return ETS_OK;
 }
 
-// Multinomial rows: five launches (ets_split.h, split_walk_kernel).
+// Multinomial rows: five launches (ets_split.h, split_walk_kernel); four when pass 1 runs inside the first pass 2.
 template <int DT>
 ets_status launch_split_walk(ets_sampler* s, const ets::RowParams& p, int32_t rows, hipStream_t stream) {
   ets_status st = ETS_OK;
@@ -177,8 +183,14 @@ ets_status launch_split_walk(ets_sampler* s, const ets::RowParams& p, int32_t ro
   st = check_row_wgs(s, sp.row_wgs);
   if (st != ETS_OK) return st;
   sp.list_region = 0;
-  launch_split_pass1<DT>(sp, rows, stream);
-  ETS_HIP(s, hipGetLastError());
+  // (pass 1 inside the first pass 2 when the launch fits: four launches instead of five)
+  int32_t spin_limit = 0;
+  const bool fused = fused_launch_fits(s, sp, p, rows, &spin_limit);
+  bool* dirty = arrive_dirty_flag(s);
+  if (!fused) {
+    launch_split_pass1<DT>(sp, rows, stream);
+    ETS_HIP(s, hipGetLastError());
+  }
   const size_t lut_bytes = DT == ets::kDtypeBFloat16 ? sizeof(float) * ets::kLutCountWords : 0;
   // the walk kernel's LDS: the row's records and as many prepared slots as fit beside them
   const uint32_t walk_lds = static_cast<uint32_t>(ets::chain_rec_bytes(sp.ns) + 16 * sizeof(ets::PrepSlot));
@@ -191,10 +203,25 @@ ets_status launch_split_walk(ets_sampler* s, const ets::RowParams& p, int32_t ro
   if (st != ETS_OK) return st;
   st = allow_dynamic_lds(s, reinterpret_cast<const void*>(&ets::split_walk_kernel<DT, 1>), walk_lds, set_k1);
   if (st != ETS_OK) return st;
-  hipLaunchKernelGGL((ets::split_pass2_kernel<DT, false, false>), dim3(sp.row_wgs, rows), dim3(ets::kBlock), lut_bytes, stream, sp);
+  if (fused) {
+    if (*dirty) {
+      hipLaunchKernelGGL(ets::split_launch_number_kernel<DT>, dim3(1), dim3(64), 0, stream, sp.arrive);
+      ETS_HIP(s, hipGetLastError());
+    }
+    *dirty = true;  // (until the first walk kernel, which numbers the next launch, has been launched)
+    sp.spin_limit = spin_limit;
+    static std::atomic<size_t> set_fused[kMaxDevices];
+    st = allow_dynamic_lds(s, reinterpret_cast<const void*>(&ets::split_pass2_kernel<DT, false, false, false, true, true>), lut_bytes, set_fused);
+    if (st != ETS_OK) return st;
+    hipLaunchKernelGGL((ets::split_pass2_kernel<DT, false, false, false, true, true>), dim3(sp.row_wgs * rows), dim3(ets::kBlock), lut_bytes,
+                       stream, sp);
+  } else {
+    hipLaunchKernelGGL((ets::split_pass2_kernel<DT, false, false>), dim3(sp.row_wgs, rows), dim3(ets::kBlock), lut_bytes, stream, sp);
+  }
   ETS_HIP(s, hipGetLastError());
   hipLaunchKernelGGL((ets::split_walk_kernel<DT, 0>), dim3(rows), dim3(ets::kWalkBlock), walk_lds, stream, sp, walk_lds);
   ETS_HIP(s, hipGetLastError());
+  if (fused) *dirty = false;
   hipLaunchKernelGGL((ets::split_pass2_kernel<DT, false, true>), dim3(sp.row_wgs, rows), dim3(ets::kBlock), lut_bytes, stream, sp);
   ETS_HIP(s, hipGetLastError());
   hipLaunchKernelGGL((ets::split_walk_kernel<DT, 1>), dim3(rows), dim3(ets::kWalkBlock), walk_lds, stream, sp, walk_lds);

@@ -114,7 +114,8 @@ ETS_API ets_status ets_sampler_set_topp(ets_sampler* s, float topp);
  * the call runs beside it: the first two are then one kernel, whose workgroups hand each
  * other their results with bounded waits);
  * top-k rows with k <= ceil(vocab / 512) the same three launches, larger k one workgroup per row;
- * multinomial rows (top_p <= 0 or >= 1) FIVE launches, or one workgroup per row when the
+ * multinomial rows (top_p <= 0 or >= 1) FIVE launches (four under the same conditions: the
+ * first two are one kernel then, too), or one workgroup per row when the
  * probabilities are asked for.  All launches of a call go to the call's stream, in order.
  * Work buffers of that path are allocated at the first call that needs them and kept: per row of
  * max_batch about 16 bytes x ceil(vocab / 512) slots x 2 + 40 prepared slots of 2.6 KB, plus per

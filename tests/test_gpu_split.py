@@ -341,9 +341,10 @@ def test_nuclei_of_hundreds_to_thousands_of_keys(oracle, dev, mode):
 
 
 @pytest.mark.parametrize("setting", ["fused", "fused_one_read", "fused_nobody_waits", "three_launches"])
-@pytest.mark.parametrize("name,rows", [("cfg2", 64), ("cfg2", 8), ("cfg2", 1), ("cfg5", 16), ("cfg3", 24), ("cfg1", 1)])
+@pytest.mark.parametrize("name,rows", [("cfg2", 64), ("cfg2", 8), ("cfg2", 1), ("cfg5", 16), ("cfg3", 24), ("cfg1", 1), ("cfg4", 16), ("cfg4", 3)])
 def test_pass1_inside_pass2(oracle, dev, monkeypatch, setting, name, rows):
-    """Plain top-p launches whose workgroups are all resident run pass 1 inside pass 2: the row's
+    """Plain top-p launches (and the first of a multinomial row's two sweeps: cfg4) whose workgroups are all
+    resident run pass 1 inside pass 2: the row's
     workgroups hand their slots' maxima and sums to one another through device memory, each record
     tagged with the launch's number, and read one another's a bounded number of times.  With the bound
     at 0 nobody waits: every workgroup works the whole row's maxima and sums out itself; with the
