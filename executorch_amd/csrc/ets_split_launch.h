@@ -87,10 +87,10 @@ ets_status launch_split(ets_sampler* s, const ets::RowParams& p, int32_t rows, h
   // Pass 1 inside pass 2 (one read of the logits, one launch fewer): plain top-p launches that fit
   // (fused_launch_fits) and ask for neither probabilities nor debug records.
   int32_t spin_limit = 0;
-  const bool fused = !TOPK && (!extras || (ETS_PHASE_CLOCKS && p.probs == nullptr)) && fused_launch_fits(s, sp, p, rows, &spin_limit);
+  const bool fused = (!extras || (ETS_PHASE_CLOCKS && p.probs == nullptr)) && fused_launch_fits(s, sp, p, rows, &spin_limit);
   bool* dirty = arrive_dirty_flag(s);
   if (fused) {
-    if constexpr (!TOPK) {
+    {
       if (*dirty) {
         hipLaunchKernelGGL(ets::split_launch_number_kernel<DT>, dim3(1), dim3(64), 0, stream, sp.arrive);
         ETS_HIP(s, hipGetLastError());
@@ -99,9 +99,9 @@ ets_status launch_split(ets_sampler* s, const ets::RowParams& p, int32_t rows, h
       sp.spin_limit = spin_limit;
       static std::atomic<size_t> set_bytes_f[kMaxDevices];
       constexpr bool kClocks = ETS_PHASE_CLOCKS != 0;  // (a profiling build: the fused kernel with its phase clocks)
-      st = allow_dynamic_lds(s, reinterpret_cast<const void*>(&ets::split_pass2_kernel<DT, true, false, false, kClocks, true>), lut_bytes, set_bytes_f);
+      st = allow_dynamic_lds(s, reinterpret_cast<const void*>(&ets::split_pass2_kernel<DT, true, false, TOPK, kClocks, true>), lut_bytes, set_bytes_f);
       if (st != ETS_OK) return st;
-      hipLaunchKernelGGL((ets::split_pass2_kernel<DT, true, false, false, kClocks, true>), dim3(sp.row_wgs * rows), dim3(ets::kBlock), lut_bytes,
+      hipLaunchKernelGGL((ets::split_pass2_kernel<DT, true, false, TOPK, kClocks, true>), dim3(sp.row_wgs * rows), dim3(ets::kBlock), lut_bytes,
                          stream, sp);
     }
   } else {

@@ -113,7 +113,7 @@ ETS_API ets_status ets_sampler_set_topp(ets_sampler* s, float topp);
  * temperature of the launch is finite, no probabilities are asked for and no other launch of
  * the call runs beside it: the first two are then one kernel, whose workgroups hand each
  * other their results with bounded waits);
- * top-k rows with k <= ceil(vocab / 512) the same three launches, larger k one workgroup per row;
+ * top-k rows with k <= ceil(vocab / 512) the same three (or two) launches, larger k one workgroup per row;
  * multinomial rows (top_p <= 0 or >= 1) FIVE launches (four under the same conditions: the
  * first two are one kernel then, too), or one workgroup per row when the
  * probabilities are asked for.  All launches of a call go to the call's stream, in order.

@@ -452,3 +452,28 @@ def test_a_launch_without_its_finish_kernel_does_not_lend_its_number(oracle, dev
     assert number(0) == n1 + 3  # (a number skipped, then the launch's own)
     step(3)
     assert number(0) == n1 + 4
+
+
+@pytest.mark.parametrize("setting", ["fused", "fused_one_read", "fused_nobody_waits", "three_launches"])
+def test_pass1_inside_pass2_top_k_rows(oracle, dev, monkeypatch, setting):
+    """The same for launches with top-k rows (sampler.cpp:72-120, :239): top-k 40 and top-k 3 with the
+    workload's top-p, and top-k alone (top-p 1)."""
+    if setting == "fused_nobody_waits":
+        monkeypatch.setenv("ETS_FUSE_SPIN_LIMIT", "0")
+    if setting == "fused_one_read":
+        monkeypatch.setenv("ETS_FUSE_SPIN_LIMIT", "1")
+    if setting == "three_launches":
+        monkeypatch.setenv("ETS_FUSE", "0")
+    w = W.WORKLOADS["cfg2"]
+    rows = 16
+    for topk, topp in ((40, w.topp), (3, w.topp), (40, 1.0)):
+        s = ea.Sampler(w.vocab, w.temperature, topp, w.coin_seed, max_batch=rows)
+        s.set_topk(topk)
+        for step in range(2):
+            x = W.logits(w, step, rows)
+            states = s.get_rng_states(rows).copy()
+            got = s.sample_batch(to_device(x, w.dtype, dev)).cpu().numpy()
+            want, _ = oracle.sample_rows(x, w.dtype, oracle.inv_temperature(w.temperature), topp, topk, states, mode=oracle.MODE_UPCAST,
+                                         tie=oracle.TIE_STABLE, threads=8)
+            assert np.array_equal(got, want), (setting, topk, topp, step)
+            assert np.array_equal(s.get_rng_states(rows), states)
