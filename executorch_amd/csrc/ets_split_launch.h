@@ -42,7 +42,10 @@ inline bool fused_launch_fits(const ets_sampler* s, const ets::SplitParams& sp, 
   const char* const fuse_text = std::getenv("ETS_FUSE");
   const int fuse_env = fuse_text ? std::atoi(fuse_text) : 1;
   const char* const spin_text = std::getenv("ETS_FUSE_SPIN_LIMIT");
-  const int spin_env = spin_text ? std::atoi(spin_text) : (1 << 13);  // (about ten milliseconds; the usual wait is a read or two)
+  // (256 reads are about 0.4 ms: the usual wait is a read or two, and a launch whose workgroups cannot all be
+  // resident -- another launch of the same kind on another stream holds the compute units -- should not stall
+  // for long before its workgroups help themselves, which costs them some twenty microseconds)
+  const int spin_env = spin_text ? std::atoi(spin_text) : 256;
   *spin_limit = spin_env < 0 ? 0 : spin_env;
   const int per_wg_slots = ((sp.ns + sp.row_wgs - 1) / sp.row_wgs + ets::kWaves - 1) / ets::kWaves * ets::kWaves;
   const float abs_inv = p.inv_temperature < 0.0f ? -p.inv_temperature : p.inv_temperature;

@@ -477,3 +477,38 @@ def test_pass1_inside_pass2_top_k_rows(oracle, dev, monkeypatch, setting):
                                          tie=oracle.TIE_STABLE, threads=8)
             assert np.array_equal(got, want), (setting, topk, topp, step)
             assert np.array_equal(s.get_rng_states(rows), states)
+
+
+def test_two_handles_on_two_streams_at_once(oracle, dev):
+    """Two launches with pass 1 inside pass 2 at the same time, from two handles on two streams: each was
+    sized to fill the compute units on its own, so the workgroups of one can hold the units that the other's
+    are waiting for.  Nobody waits for ever (the reads of the others' records are bounded, and a workgroup
+    that gives up works the row out itself): tokens and coin states equal the oracle's, call after call."""
+    w = W.WORKLOADS["cfg2"]
+    rows = 64
+    a = ea.Sampler(w.vocab, w.temperature, w.topp, 11, max_batch=rows)
+    b = ea.Sampler(w.vocab, w.temperature, w.topp, 22, max_batch=rows)
+    xs = [W.logits(w, step, rows) for step in range(3)]
+    dxs = [to_device(x, w.dtype, dev) for x in xs]
+    sa, sb = torch.cuda.Stream(device=dev), torch.cuda.Stream(device=dev)
+    outs_a = [torch.empty(rows, dtype=torch.int32, device=dev) for _ in xs]
+    outs_b = [torch.empty(rows, dtype=torch.int32, device=dev) for _ in xs]
+    a.sample_batch(dxs[0], out=outs_a[0])  # (warm: buffers allocated, kernel attributes set)
+    b.sample_batch(dxs[0], out=outs_b[0])
+    torch.cuda.synchronize()
+    states_a, states_b = a.get_rng_states(rows).copy(), b.get_rng_states(rows).copy()
+    for k in range(len(xs)):
+        with torch.cuda.stream(sa):
+            a.sample_batch(dxs[k], out=outs_a[k])
+        with torch.cuda.stream(sb):
+            b.sample_batch(dxs[k], out=outs_b[k])
+    torch.cuda.synchronize()
+    for k, x in enumerate(xs):
+        want_a, _ = oracle.sample_rows(x, w.dtype, oracle.inv_temperature(w.temperature), w.topp, 0, states_a, mode=oracle.MODE_UPCAST,
+                                       tie=oracle.TIE_STABLE, threads=8)
+        want_b, _ = oracle.sample_rows(x, w.dtype, oracle.inv_temperature(w.temperature), w.topp, 0, states_b, mode=oracle.MODE_UPCAST,
+                                       tie=oracle.TIE_STABLE, threads=8)
+        assert np.array_equal(outs_a[k].cpu().numpy(), want_a), ("a", k)
+        assert np.array_equal(outs_b[k].cpu().numpy(), want_b), ("b", k)
+    assert np.array_equal(a.get_rng_states(rows), states_a)
+    assert np.array_equal(b.get_rng_states(rows), states_b)
