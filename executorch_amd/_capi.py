@@ -88,6 +88,7 @@ TEST_HOOKS = {
     "ets_test_last_error": (C.c_char_p, []),
     "ets_test_handle_buffers": (C.c_int32, [C.c_void_p, C.c_void_p]),
     "ets_test_fused_launch_number": (C.c_int32, [C.c_void_p, C.c_int32, C.c_void_p]),
+    "ets_test_set_fused_launch_number": (C.c_int32, [C.c_void_p, C.c_uint32]),
     "ets_test_expf": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p]),
     "ets_test_seq_sum": (C.c_int32, [C.c_void_p, C.c_int32, C.c_float, C.c_float, C.c_void_p, C.c_void_p, C.c_void_p]),
     "ets_test_split_timers": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int32]),

@@ -238,8 +238,15 @@ typedef float ets_f32x4 __attribute__((ext_vector_type(4)));
 // advances, so no two launches on the same buffers share one) mixed with the values themselves.  A record
 // of an earlier launch never carries this launch's tag, whatever its values; a record that is not there yet
 // reads as that earlier record (or as the zeros the buffer starts with, whose tag would be 0 + the mix of
-// zeros = 0, which no launch uses).  The sixteen bytes travel as one request; were a read ever to see part
+// zeros = 0, which no launch uses: next_launch_number).  The sixteen bytes travel as one request; were a read ever to see part
 // of a store, the mix of the values would have to make up for the difference between two tags.
+// The next launch's number, by the one thread of a launch that advances it.  The word never holds 2^32 - 1, so
+// that no launch has the number 0, for which the zeros that the records start as would pass for a record.
+// (After 2^32 - 1 launches on the same buffers the numbers come round.)
+__device__ __forceinline__ void next_launch_number(uint32_t* word) {
+  const uint32_t v = *word + 1u;
+  *word = v == 0xffffffffu ? 0u : v;
+}
 __device__ __forceinline__ uint32_t pack_tag(uint32_t launch, float a, float b, float c) {
   const uint32_t ua = __float_as_uint(a), ub = __float_as_uint(b), uc = __float_as_uint(c);
   return launch ^ (ua * 0x9E3779B1u) ^ ((ub << 13) | (ub >> 19)) ^ (((uc << 7) | (uc >> 25)) * 0x85EBCA77u);
@@ -1168,7 +1175,7 @@ __global__ void __launch_bounds__(kBlock, ETS_PASS2_WAVES_PER_EU) split_pass2_ke
 // After a fused launch that was not followed by its finish kernel: the next one gets a number of its own.
 template <int DT>
 __global__ void split_launch_number_kernel(uint32_t* arrive) {
-  if (threadIdx.x == 0 && blockIdx.x == 0) arrive[0] = arrive[0] + 1u;
+  if (threadIdx.x == 0 && blockIdx.x == 0) next_launch_number(arrive);
 }
 
 // ---- finish ---------------------------------------------------------------------------------------
@@ -2690,7 +2697,7 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
   }
   const RowState rs = p.row_state[row];
   // (the number by which the fused launch tags what its workgroups hand over: the next launch gets another)
-  if (lrow == 0 && tid == 0 && p.arrive) atomicAdd(p.arrive, 1u);
+  if (lrow == 0 && tid == 0 && p.arrive) next_launch_number(p.arrive);
   const float m = rs.m;
   const bool row_nan = rs.nan != 0u;
   const float cutoff = (1.0f - topp) / static_cast<float>(V - 1);  // sampler.cpp:136
@@ -3088,7 +3095,7 @@ __global__ void __launch_bounds__(kWalkBlock) split_walk_kernel(SplitParams p, u
   const RowState rs = p.row_state[row];
   if (tid < 32) exp2tab[tid] = kExp2Table[tid];
   // (the number by which a launch with pass 1 inside pass 2 tags what its workgroups hand over: the next one gets another)
-  if (PHASE == 0 && blockIdx.x == 0 && tid == 0 && p.arrive) atomicAdd(p.arrive, 1u);
+  if (PHASE == 0 && blockIdx.x == 0 && tid == 0 && p.arrive) next_launch_number(p.arrive);
   auto toss = [&]() {  // one coin per call (sampler.cpp:237, 210-220)
     uint64_t st = p.row.rng[row];
     st ^= st >> 12;

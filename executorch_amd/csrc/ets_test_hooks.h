@@ -50,6 +50,9 @@ ETS_API ets_status ets_test_handle_buffers(const ets_sampler* s, int32_t* out);
  * number of its own first. */
 ETS_API ets_status ets_test_fused_launch_number(ets_sampler* s, int32_t mark_unfinished, uint32_t* out);
 
+/* Sets that word (waits for the device): for a test of the numbers coming round after 2^32 - 1 launches. */
+ETS_API ets_status ets_test_set_fused_launch_number(ets_sampler* s, uint32_t value);
+
 /* The message of the calling thread's last failed hook. */
 ETS_API const char* ets_test_last_error(void);
 

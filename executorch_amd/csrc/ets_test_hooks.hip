@@ -237,6 +237,17 @@ ets_status ets_test_fused_launch_number(ets_sampler* s, int32_t mark_unfinished,
   return ETS_OK;
 }
 
+ets_status ets_test_set_fused_launch_number(ets_sampler* s, uint32_t value) {
+  if (!s) return hook_fail(ETS_INVALID_ARGUMENT, "ets_test_set_fused_launch_number: null pointer");
+  if (!s->d_split) return hook_fail(ETS_INVALID_STATE, "ets_test_set_fused_launch_number: the handle has not sampled several workgroups a row yet");
+  int prev = -1;
+  const bool switched = hipGetDevice(&prev) == hipSuccess && prev != s->device && hipSetDevice(s->device) == hipSuccess;
+  const hipError_t e = hipMemcpy(s->split.arrive, &value, sizeof(uint32_t), hipMemcpyHostToDevice);
+  if (switched) (void)hipSetDevice(prev);
+  if (e != hipSuccess) return hook_fail(ETS_INTERNAL, hipGetErrorString(e));
+  return ETS_OK;
+}
+
 const char* ets_test_last_error(void) { return g_hook_error.c_str(); }
 
 }  // extern "C"

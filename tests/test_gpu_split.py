@@ -512,3 +512,36 @@ def test_two_handles_on_two_streams_at_once(oracle, dev):
         assert np.array_equal(outs_b[k].cpu().numpy(), want_b), ("b", k)
     assert np.array_equal(a.get_rng_states(rows), states_a)
     assert np.array_equal(b.get_rng_states(rows), states_b)
+
+
+def test_launch_numbers_come_round(oracle, dev):
+    """After 2^32 - 1 launches the launch numbers start again; the number 0, for which the zeros that the
+    records of never-used rows still hold would pass for records, is left out.  The word is set close to the
+    end through the test hook; a small batch first, then the handle's full batch (rows whose records are
+    still zeros) on the launches around the turn; tokens against the oracle."""
+    import ctypes
+    from executorch_amd import _capi
+    w = W.WORKLOADS["cfg2"]
+    rows = 16
+    s = ea.Sampler(w.vocab, w.temperature, w.topp, w.coin_seed, max_batch=rows)
+
+    def number():
+        out = ctypes.c_uint32(0)
+        assert _capi.hooks().ets_test_fused_launch_number(s._h, 0, ctypes.byref(out)) == _capi.OK
+        return out.value
+
+    def step(k, n):
+        x = W.logits(w, k, n)
+        states = s.get_rng_states(n).copy()
+        got = s.sample_batch(to_device(x, w.dtype, dev)).cpu().numpy()
+        want, _ = oracle.sample_rows(x, w.dtype, oracle.inv_temperature(w.temperature), w.topp, 0, states, mode=oracle.MODE_UPCAST,
+                                     tie=oracle.TIE_STABLE, threads=8)
+        assert np.array_equal(got, want), (k, n)
+
+    step(0, 2)  # (the work buffers exist now; rows 2 .. 15 have never been used)
+    assert _capi.hooks().ets_test_set_fused_launch_number(s._h, 0xFFFFFFFC) == _capi.OK
+    seen = []
+    for k in range(1, 6):
+        step(k, rows if k >= 2 else 2)
+        seen.append(number())
+    assert seen == [0xFFFFFFFD, 0xFFFFFFFE, 0, 1, 2], [hex(v) for v in seen]
