@@ -621,9 +621,9 @@ __device__ bool build_exp_lut(float* lut, int cap, float inv, float m, const uin
 // The same table for a caller that has marked the patterns it will look up (`seen`: a byte per eight
 // consecutive 16-bit patterns, 8192 bytes, 8-byte aligned) and builds with the waves from the second on:
 // the table is cut into chunks of 64 consecutive patterns; every wave finds out which chunks hold a marked
-// pattern (two reads of eight mark bytes per lane, two ballots) and the builders take those chunks in turn,
-// so that each has the same number of them to work out, whatever the row looks like.  Unmarked chunks are
-// left as they are.  More than 128 chunks: the general routine.
+// pattern (three reads of eight mark bytes per lane, three ballots: a table that fits has at most 192
+// chunks) and the builders take those chunks in turn, so that each has the same number of them to work out,
+// whatever the row looks like.  Unmarked chunks are left as they are.
 __device__ bool build_exp_lut_marked(float* lut, int cap, float inv, float m, const uint64_t* tab, int& base1, int& top,
                                      int& half, const uint8_t* seen) {
   const float kInf = __uint_as_float(0x7f800000u);
@@ -640,11 +640,11 @@ __device__ bool build_exp_lut_marked(float* lut, int cap, float inv, float m, co
   if (e_hi < e_lo) return false;
   const int R = (e_hi - e_lo + 1) * 128;
   const int per_half = R >> 6, n_chunks = 2 * per_half;
-  if (n_chunks > 128) return build_exp_lut<false>(lut, cap, inv, m, tab, base1, top, half, 64, seen);
   half = R + 2;
   top = R + 1;
   base1 = (e_lo << 7) - 1;
   if (2 * half > kLutCountWords || 2 * half > cap) return false;
+  static_assert(kLutCountWords <= 192 * 64, "three ballots cover the chunks of a table that fits");
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   if (wave == 0) return true;  // (takes no part: where the table lies)
   const int builders = kBlock / 64 - 1, me = wave - 1;
@@ -655,13 +655,15 @@ __device__ bool build_exp_lut_marked(float* lut, int cap, float inv, float m, co
   auto marked = [&](int k) -> bool {
     return k < n_chunks && *reinterpret_cast<const uint64_t*>(seen + (first_pattern(k) >> 3)) != 0ull;
   };
-  const uint64_t need0 = __ballot(marked(lane)), need1 = __ballot(marked(lane + 64));
+  const uint64_t need0 = __ballot(marked(lane)), need1 = __ballot(marked(lane + 64)), need2 = __ballot(marked(lane + 128));
   const uint64_t below = (1ull << lane) - 1ull;
-  const int rank0 = __popcll(need0 & below), rank1 = __popcll(need0) + __popcll(need1 & below);
-  uint64_t mine[2] = {__ballot(((need0 >> lane) & 1ull) && rank0 % builders == me),
-                      __ballot(((need1 >> lane) & 1ull) && rank1 % builders == me)};
+  const int rank0 = __popcll(need0 & below), rank1 = __popcll(need0) + __popcll(need1 & below),
+            rank2 = __popcll(need0) + __popcll(need1) + __popcll(need2 & below);
+  uint64_t mine[3] = {__ballot(((need0 >> lane) & 1ull) && rank0 % builders == me),
+                      __ballot(((need1 >> lane) & 1ull) && rank1 % builders == me),
+                      __ballot(((need2 >> lane) & 1ull) && rank2 % builders == me)};
 #pragma unroll
-  for (int h = 0; h < 2; ++h) {
+  for (int h = 0; h < 3; ++h) {
     while (mine[h] != 0ull) {
       const int k = 64 * h + __builtin_ctzll(mine[h]);
       mine[h] &= mine[h] - 1ull;
