@@ -2712,6 +2712,7 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
   int n_listed = 0;
   HistPlan plan = {-1, 0, 0, 0};
   bool lists_ok = false;
+  bool topk_few = false;
   if (!row_nan) {
     // ---- how many candidates the workgroups of pass 2 listed; their histograms, added up
     if (tid < 64) {
@@ -2784,6 +2785,10 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
     lists_ok = fs.overflow == 0u;
     plan = split_plan(fs.hist, rs.a_total, topp, cutoff, V, &fs.plan, sm);
     if (timers) t1 = wall_clock64();
+    // (a top-k row whose lists hold at most 64 entries, at least topk of them: one wave can draw it)
+    const int32_t row_topk_early = !TOPK ? 0 : (p.row.row_cfg ? p.row.row_cfg[row].topk : p.row.topk);
+    topk_few = TOPK && row_topk_early > 0 && row_topk_early < V && lists_ok && rs.listed_buckets != 0u && rs.listed_buckets != kNoLists &&
+               n_listed >= row_topk_early && n_listed <= 64;
     if (wave == 0) {
       if (!chained) {
         float sum;
@@ -2811,6 +2816,15 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
 #endif
       } else if (lane == 0) {
         sm.bc_sum = fs.pre_sum[lrow - r_first];
+      }
+    } else if (TOPK && topk_few) {
+      // ---- the second wave, meanwhile: the listed entries of a top-k row, all of them
+      if (wave == 1) {
+        for (int g = 0; g < p.row_wgs; ++g) {
+          const uint64_t* src = p.list + (static_cast<int64_t>(lrow) * p.row_wgs + g) * p.list_region;
+          const int c = static_cast<int>(fs.count[g]);
+          if (lane < c) fs.sel[fs.offset[g] + lane] = src[lane];
+        }
       }
     } else if (lists_ok && plan.b_sel >= 0 && plan.n_sel <= 64) {
       // ---- the other waves, meanwhile: one pass over the listed candidates picks out those of the
@@ -2845,9 +2859,11 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
   //      everything as it was, coin state included, and the row takes the steps below.
   if constexpr (!EXTRAS) {
     const int32_t row_topk = !TOPK ? 0 : (p.row.row_cfg ? p.row.row_cfg[row].topk : p.row.topk);
-    const bool small_tail = !row_nan && p.row.debug == nullptr && !(TOPK && row_topk > 0 && row_topk < V) && lists_ok &&
-                            rs.listed_buckets != 0u && plan.b_sel >= 0 && plan.n_sel >= 1 && plan.n_sel <= 64 &&
-                            fs.sel_count == static_cast<uint32_t>(plan.n_sel) && plan.b_sel < static_cast<int>(rs.listed_buckets);
+    const bool is_topk = TOPK && row_topk > 0 && row_topk < V;
+    const bool small_tail = !row_nan && p.row.debug == nullptr && lists_ok &&
+                            (is_topk ? topk_few
+                                     : (rs.listed_buckets != 0u && plan.b_sel >= 0 && plan.n_sel >= 1 && plan.n_sel <= 64 &&
+                                        fs.sel_count == static_cast<uint32_t>(plan.n_sel) && plan.b_sel < static_cast<int>(rs.listed_buckets)));
     if (small_tail) {
       if (wave == 0) {
         uint64_t st = (static_cast<uint64_t>(readlane_u32(static_cast<uint32_t>(coin_state >> 32), 0)) << 32) |
@@ -2858,19 +2874,23 @@ __global__ void __launch_bounds__(kBlock) split_finish_kernel(SplitParams p) {
         const uint32_t u = static_cast<uint32_t>((st * 0x2545F4914F6CDD1Dull) >> 32);
         const float coin1 = static_cast<float>(u >> 8) / 16777216.0f;
         const RowDivisor div = row_divisor(S);
-        const int n_sel = plan.n_sel;
+        const int n_sel = is_topk ? n_listed : plan.n_sel;
         bool is_in = true;
         uint64_t key = ~0ull;
         if (lane < n_sel) {
           const uint64_t ent = fs.sel[lane];
           const float pj = div_row(__uint_as_float(static_cast<uint32_t>(ent >> 32)), div);
-          is_in = pj >= cutoff;  // sampler.cpp:137-143
+          is_in = is_topk || pj >= cutoff;  // sampler.cpp:137-143 (every entry is a candidate of a top-k draw)
           key = cand_key(pj, static_cast<int>(static_cast<uint32_t>(ent)));
         }
         int pos = -2, last_idx = 0;
         float mass = 0.0f, r = 0.0f;
         uint32_t tok = 0u;
-        if (__ballot(!is_in) == 0ull) {
+        if (TOPK && is_topk) {
+          // (sampler.cpp:72-120: the first topk of the sorted entries; what is not listed lies below the lists' floor)
+          const float list_floor = __uint_as_float(0x3F800000u - (rs.listed_buckets << 17) + 1u);
+          pos = small_wave_core(key, n_sel, n_sel, topp, coin1, row_topk, div_row(list_floor, div), last_idx, mass, r, tok);
+        } else if (__ballot(!is_in) == 0ull) {
           // (more candidates exist than the lists hold; entries outside the selection have exps up to the edge of the next bucket)
           pos = small_wave_core(key, n_sel, 0x7fffffff, topp, coin1, 0, div_row(hist_edge(plan.b_sel + 1), div), last_idx, mass, r, tok);
         }

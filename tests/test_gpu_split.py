@@ -545,3 +545,34 @@ def test_launch_numbers_come_round(oracle, dev):
         step(k, rows if k >= 2 else 2)
         seen.append(number())
     assert seen == [0xFFFFFFFD, 0xFFFFFFFE, 0, 1, 2], [hex(v) for v in seen]
+
+
+@pytest.mark.parametrize("topk", [1, 2, 7, 40, 63, 64, 65, 200])
+def test_top_k_rows_with_short_lists(oracle, dev, topk):
+    """A top-k row whose lists hold at most 64 entries (at least k of them) is drawn by the finish kernel's
+    first wave alone; longer lists, and k beyond 64, take the steps of the whole workgroup.  Peaked rows,
+    rows of few distinct values (ties at the k-th place, broken by index) and rows with a dominant entry,
+    with top-p 0.9 and with top-p 1; tokens and coin states against the oracle."""
+    V, rows = 128256, 8
+    rng = np.random.default_rng(1000 + topk)
+    peaked = (rng.standard_normal((rows, V)) * 1.0).astype(np.float32)
+    for b in range(rows):
+        peaked[b, rng.choice(V, size=24, replace=False)] += 8.0
+    few = rng.integers(0, 6, (rows, V)).astype(np.float32)
+    for b in range(rows):
+        few[b, rng.choice(V, size=30, replace=False)] = 9.0  # (thirty equal largest entries)
+    dominant = (rng.standard_normal((rows, V)) * 0.5).astype(np.float32)
+    dominant[:, 77] = 30.0
+    for kind, x32 in (("peaked", peaked), ("few", few), ("dominant", dominant)):
+        x = W.to_storage(x32, W.DTYPE_BFLOAT16)
+        dx = to_device(x, W.DTYPE_BFLOAT16, dev)
+        for topp in (0.9, 1.0):
+            s = ea.Sampler(V, 0.7, topp, 5 + topk, max_batch=rows)
+            s.set_topk(topk)
+            for step in range(2):
+                states = s.get_rng_states(rows).copy()
+                got = s.sample_batch(dx).cpu().numpy()
+                want, _ = oracle.sample_rows(x, W.DTYPE_BFLOAT16, oracle.inv_temperature(0.7), topp, topk, states, mode=oracle.MODE_UPCAST,
+                                             tie=oracle.TIE_STABLE, threads=8)
+                assert np.array_equal(got, want), (kind, topk, topp, step)
+                assert np.array_equal(s.get_rng_states(rows), states)
